@@ -1,0 +1,66 @@
+"""Build recipe: compiles the gfx950 backend and the host runtime in-tree with hipcc.
+
+  libmi355_backend.so   HIP kernels + the C ABI of include/mi355_abi.h
+  libmirage_runtime.so  the mirage:: host API (C++) + its C facade for ctypes
+
+Run as `python -m attention_superoptimizer_amd.build`.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+INCLUDE = os.path.join(ROOT, "include")
+BACKEND_LIB = os.path.join(HERE, "libmi355_backend.so")
+RUNTIME_LIB = os.path.join(HERE, "libmirage_runtime.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops off: packed FP32 forms have produced silent wrong results on these boxes
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
+
+
+def _sources(sub, exts):
+    d = os.path.join(CSRC, sub)
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(exts))
+
+
+def _run(cmd):
+    print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_backend():
+    srcs = _sources("backend", (".hip", ".cc"))
+    objs = []
+    for s in srcs:
+        o = os.path.splitext(s)[0] + ".o"
+        lang = ["-x", "hip"] if s.endswith(".hip") else []
+        _run([HIPCC] + DEVICE_FLAGS + ["-I", INCLUDE, "-I", os.path.join(CSRC, "backend"), "-c"] + lang + [s, "-o", o])
+        objs.append(o)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", BACKEND_LIB] + objs)
+
+
+def build_runtime():
+    srcs = _sources("host", (".cc",))
+    if not srcs:
+        return
+    _run(["g++", "-O2", "-fPIC", "-std=c++17", "-shared", "-D__HIP_PLATFORM_AMD__",
+          "-I", INCLUDE, "-I", "/opt/rocm/include", "-o", RUNTIME_LIB] + srcs +
+         ["-L" + HERE, "-lmi355_backend", "-Wl,-rpath,$ORIGIN"])
+
+
+def main():
+    build_backend()
+    if os.path.isdir(os.path.join(CSRC, "host")):
+        build_runtime()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,81 @@
+// Shared state and helpers of the gfx950 backend (internal; not part of the ABI).
+#pragma once
+
+#include "mi355_abi.h"
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+namespace mi355 {
+
+// Fingerprint ring constants (reference include/mirage/type.h:26-34).
+constexpr uint32_t FP_P = 227;
+constexpr uint32_t FP_Q = 113;
+constexpr uint32_t FP_EXP_BASE = 3;
+constexpr uint32_t FP_PQ = 25651;
+constexpr uint32_t FP_P_MUL_Q_MOD_1 = 227;
+constexpr uint32_t FP_Q_MUL_P_MOD_1 = 25425;
+
+// Operator type codes (reference include/mirage/type.h:50-62, 79-103).
+enum : int {
+  KN_EXP_OP = 1007,
+  KN_ADD_OP = 1008,
+  KN_MUL_OP = 1009,
+  KN_DIV_OP = 1010,
+  KN_SILU_OP = 1011,  // extension
+  TB_INPUT_OP = 2001,
+  TB_OUTPUT_OP = 2002,
+  TB_MATMUL_OP = 2003,
+  TB_EXP_OP = 2007,
+  TB_ADD_OP = 2008,
+  TB_MUL_OP = 2009,
+  TB_DIV_OP = 2010,
+  TB_SILU_OP = 2012,  // extension
+  TB_REDUCTION_0_OP = 2101,
+  TB_REDUCTION_2_TO_DIMX_OP = 2106,
+  TB_CONCAT_0_OP = 2200,
+  TB_CONCAT_2_OP = 2202,
+};
+
+struct State {
+  bool ready = false;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  char *arena = nullptr;
+  size_t arena_bytes = 0;
+  // device copies of the lookup tables, reference layout
+  uint16_t *exp_tbl = nullptr, *div_p = nullptr, *div_q = nullptr;
+  int *flag = nullptr;        // 4-byte device scratch for mi355_fp_equal
+  int *flag_host = nullptr;   // pinned mirror
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  int max_lds = 65536;
+  mi355_launch_info last_launch{};
+};
+
+State &state();
+int fail(int code, char const *fmt, ...);
+
+#define MI355_HIP(expr)                                                             \
+  do {                                                                              \
+    hipError_t e_ = (expr);                                                         \
+    if (e_ != hipSuccess) {                                                         \
+      return ::mi355::fail(MI355_ERR_HIP, "%s failed: %s (%s:%d)", #expr,           \
+                           hipGetErrorString(e_), __FILE__, __LINE__);              \
+    }                                                                               \
+  } while (0)
+
+#define MI355_REQUIRE_INIT()                                                        \
+  do {                                                                              \
+    if (!::mi355::state().ready) {                                                  \
+      return ::mi355::fail(MI355_ERR_NOT_INITIALISED, "mi355_init has not run");    \
+    }                                                                               \
+  } while (0)
+
+// x mod 25651 / 227 / 113 for 32-bit x.  The compiler lowers `%` by a constant to
+// a multiply-high; kept as functions so every kernel spells it the same way.
+__device__ __forceinline__ uint32_t mod_pq(uint32_t x) { return x % FP_PQ; }
+__device__ __forceinline__ uint32_t mod_p(uint32_t x) { return x % FP_P; }
+__device__ __forceinline__ uint32_t mod_q(uint32_t x) { return x % FP_Q; }
+
+}  // namespace mi355

@@ -1,0 +1,439 @@
+// Kernel-level fingerprint operators over Z_25651 = Z_227 x Z_113 (uint16 storage).
+//
+// Integer only, no matrix cores.  The matmul does not repeat the reference's
+// `(r + a*b) % 25651` per multiply-accumulate: it splits every operand into its
+// residues modulo 227 and 113 (both fit a byte), packs four consecutive k into
+// one dword, accumulates with the packed 4x8-bit dot instruction in each
+// residue field, and recombines once per output with the reference's own CRT
+// multipliers.  (sum a*b) mod 25651 is fixed by its two residues, so the result
+// is bit-identical for operands < 25651.
+#include "common.h"
+
+namespace mi355 {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+
+// ---- inputs (reference src/kernel/cuda/input_kernel.cu:56-61) ------------------
+__global__ void fp_fill_iota_kernel(uint16_t *fp, size_t n) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    fp[i] = static_cast<uint16_t>(i % FP_PQ);
+  }
+}
+
+__global__ void fp_fill_uniform_kernel(uint16_t *fp, size_t n, uint64_t seed) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    fp[i] = static_cast<uint16_t>(splitmix64(seed + i) % FP_PQ);
+  }
+}
+
+// ---- matmul (reference src/kernel/cuda/matmul_kernel.cu:145-173) ---------------
+__device__ __forceinline__ void residues4(uint32_t v0, uint32_t v1, uint32_t v2, uint32_t v3,
+                                          uint32_t &pp, uint32_t &qq) {
+  pp = (v0 % FP_P) | ((v1 % FP_P) << 8) | ((v2 % FP_P) << 16) | ((v3 % FP_P) << 24);
+  qq = (v0 % FP_Q) | ((v1 % FP_Q) << 8) | ((v2 % FP_Q) << 16) | ((v3 % FP_Q) << 24);
+}
+
+// Block tile (16*RM) x 64 outputs, 32 k per step; thread (ty, tx) owns rows
+// ty*RM.. and columns tx*4...  LDS holds the residue-packed tiles:
+//   Ap[f][kq][row]  one dword = residues of A[row][4kq..4kq+3] in field f
+//   Bp[f][kq][col]  one dword = residues of B[4kq..4kq+3][col]
+template <int RM>
+__global__ __launch_bounds__(kThreads) void fp_matmul_kernel(uint16_t const *__restrict__ A,
+                                                            uint16_t const *__restrict__ B,
+                                                            uint16_t *__restrict__ C, int m,
+                                                            int n, int k) {
+  constexpr int TM = 16 * RM, TN = 64, TKQ = 8;
+  __shared__ uint32_t Ap[2][TKQ][TM];
+  __shared__ uint32_t Bp[2][TKQ][TN];
+  int const tid = threadIdx.x;
+  int const tx = tid % 16, ty = tid / 16;
+  int const col0 = blockIdx.x * TN, row0 = blockIdx.y * TM;
+  size_t const b = blockIdx.z;
+  A += b * (size_t)m * k;
+  B += b * (size_t)k * n;
+  C += b * (size_t)m * n;
+  uint32_t accp[RM][4], accq[RM][4];
+#pragma unroll
+  for (int i = 0; i < RM; i++) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      accp[i][j] = 0;
+      accq[i][j] = 0;
+    }
+  }
+  int const num_kt = (k + 31) / 32;
+  for (int kt = 0; kt < num_kt; kt++) {
+    int const k0 = kt * 32;
+    // stage A: TM rows x 8 packed dwords
+    for (int e = tid; e < TM * TKQ; e += kThreads) {
+      int r = e / TKQ, kq = e % TKQ;
+      int gr = row0 + r, gk = k0 + kq * 4;
+      uint32_t v[4] = {0, 0, 0, 0};
+      if (gr < m) {
+        uint16_t const *p = A + (size_t)gr * k + gk;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          if (gk + j < k) {
+            v[j] = p[j];
+          }
+        }
+      }
+      uint32_t pp, qq;
+      residues4(v[0], v[1], v[2], v[3], pp, qq);
+      Ap[0][kq][r] = pp;
+      Ap[1][kq][r] = qq;
+    }
+    // stage B: 8 packed k-groups x 64 columns (coalesced along n)
+    for (int e = tid; e < TKQ * TN; e += kThreads) {
+      int kq = e / TN, c = e % TN;
+      int gc = col0 + c, gk = k0 + kq * 4;
+      uint32_t v[4] = {0, 0, 0, 0};
+      if (gc < n) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          if (gk + j < k) {
+            v[j] = B[(size_t)(gk + j) * n + gc];
+          }
+        }
+      }
+      uint32_t pp, qq;
+      residues4(v[0], v[1], v[2], v[3], pp, qq);
+      Bp[0][kq][c] = pp;
+      Bp[1][kq][c] = qq;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kq = 0; kq < TKQ; kq++) {
+      uint32_t bp[4], bq[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        bp[j] = Bp[0][kq][tx * 4 + j];
+        bq[j] = Bp[1][kq][tx * 4 + j];
+      }
+#pragma unroll
+      for (int i = 0; i < RM; i++) {
+        uint32_t ap = Ap[0][kq][ty * RM + i];
+        uint32_t aq = Ap[1][kq][ty * RM + i];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          accp[i][j] = __builtin_amdgcn_udot4(ap, bp[j], accp[i][j], false);
+          accq[i][j] = __builtin_amdgcn_udot4(aq, bq[j], accq[i][j], false);
+        }
+      }
+    }
+    __syncthreads();
+    // 32 k add at most 32*226^2 < 2^21 per step: fold well before 2^32
+    if ((kt & 1023) == 1023) {
+#pragma unroll
+      for (int i = 0; i < RM; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          accp[i][j] %= FP_P;
+          accq[i][j] %= FP_Q;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RM; i++) {
+    int gr = row0 + ty * RM + i;
+    if (gr >= m) {
+      continue;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      int gc = col0 + tx * 4 + j;
+      if (gc < n) {
+        uint32_t rp = accp[i][j] % FP_P, rq = accq[i][j] % FP_Q;
+        C[(size_t)gr * n + gc] =
+            static_cast<uint16_t>((rp * FP_Q_MUL_P_MOD_1 + rq * FP_P_MUL_Q_MOD_1) % FP_PQ);
+      }
+    }
+  }
+}
+
+// ---- element-wise ---------------------------------------------------------------
+struct FpTables {
+  uint16_t const *exp_tbl, *div_p, *div_q;
+};
+
+__device__ __forceinline__ uint32_t fp_exp_value(FpTables t, uint32_t x) {
+  // reference element_unary_kernel.cu:85-89
+  return (t.exp_tbl[x % FP_Q] * FP_Q_MUL_P_MOD_1) % FP_PQ;
+}
+
+__device__ __forceinline__ uint32_t fp_div_value(FpTables t, uint32_t x, uint32_t y) {
+  // reference element_binary_kernel.cu:155-160
+  uint32_t z = (x % FP_P) * t.div_p[y % FP_P] * FP_Q_MUL_P_MOD_1 +
+               (x % FP_Q) * t.div_q[y % FP_Q] * FP_P_MUL_Q_MOD_1;
+  return z % FP_PQ;
+}
+
+__device__ __forceinline__ uint32_t fp_silu_value(FpTables t, uint32_t x) {
+  // extension: x / (1 + exp(-x)) from the ring primitives above
+  uint32_t neg = (FP_PQ - x) % FP_PQ;
+  uint32_t den = (1u + fp_exp_value(t, neg)) % FP_PQ;
+  return fp_div_value(t, x, den);
+}
+
+__global__ void fp_unary_kernel(int op, FpTables t, uint16_t const *__restrict__ in,
+                                uint16_t *__restrict__ out, size_t n) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    uint32_t x = in[i];
+    out[i] = static_cast<uint16_t>(op == KN_EXP_OP ? fp_exp_value(t, x) : fp_silu_value(t, x));
+  }
+}
+
+struct Dims4 {
+  int nd;
+  int d1[4], d2[4], od[4];
+};
+
+__global__ void fp_binary_kernel(int op, FpTables t, uint16_t const *__restrict__ in1,
+                                 uint16_t const *__restrict__ in2, uint16_t *__restrict__ out,
+                                 Dims4 D, size_t n) {
+  size_t gid = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; gid < n; gid += stride) {
+    // reference element_binary_kernel.cu:108-116
+    size_t i = gid, s1 = 1, i1 = 0, s2 = 1, i2 = 0;
+    for (int d = D.nd - 1; d >= 0; d--) {
+      i1 += (i % D.d1[d]) * s1;
+      i2 += (i % D.d2[d]) * s2;
+      s1 *= D.d1[d];
+      s2 *= D.d2[d];
+      i /= D.od[d];
+    }
+    uint32_t x = in1[i1], y = in2[i2], z;
+    if (op == KN_ADD_OP) {
+      z = (x + y) % FP_PQ;
+    } else if (op == KN_MUL_OP) {
+      z = (x * y) % FP_PQ;
+    } else {
+      z = fp_div_value(t, x, y);
+    }
+    out[gid] = static_cast<uint16_t>(z);
+  }
+}
+
+// ---- reduction (reference src/kernel/cuda/reduction_kernel.cu:80-108) ----------
+// out[i] = sum_k in[(i / os) * is + i % os + k * os]; sums of uint16 are folded
+// every 32768 terms so the 32-bit accumulator cannot wrap.
+__global__ void fp_reduce_kernel(uint16_t const *__restrict__ in, uint16_t *__restrict__ out,
+                                 size_t n_out, int factor, int in_stride, int out_stride) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  if (i >= n_out) {
+    return;
+  }
+  size_t base = (i / out_stride) * (size_t)in_stride + i % out_stride;
+  uint32_t r = 0;
+  for (int k = 0; k < factor; k++) {
+    r += in[base + (size_t)k * out_stride];
+    if ((k & 32767) == 32767) {
+      r %= FP_PQ;
+    }
+  }
+  out[i] = static_cast<uint16_t>(r % FP_PQ);
+}
+
+// rows of contiguous elements (out_stride == 1): one wavefront per output
+__global__ void fp_reduce_rows_kernel(uint16_t const *__restrict__ in, uint16_t *__restrict__ out,
+                                      size_t n_out, int factor) {
+  int const lane = threadIdx.x % 64;
+  size_t row = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) / 64;
+  if (row >= n_out) {
+    return;
+  }
+  uint16_t const *p = in + row * (size_t)factor;
+  uint32_t r = 0;
+  int it = 0;
+  for (int k = lane; k < factor; k += 64) {
+    r += p[k];
+    if ((++it & 32767) == 0) {
+      r %= FP_PQ;
+    }
+  }
+  r %= FP_PQ;
+  for (int off = 32; off > 0; off >>= 1) {
+    r += __shfl_down(r, off, 64);
+  }
+  if (lane == 0) {
+    out[row] = static_cast<uint16_t>(r % FP_PQ);
+  }
+}
+
+// ---- compare (reference src/kernel/cuda/device_tensor_kernel.cu:42-49) ---------
+__global__ void set_flag_kernel(int *flag, int v) { *flag = v; }
+
+__global__ void fp_equal_kernel(uint16_t const *__restrict__ a, uint16_t const *__restrict__ b,
+                                size_t n, int *flag) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  bool differ = false;
+  for (; i < n; i += stride) {
+    differ |= (a[i] != b[i]);
+  }
+  if (differ) {
+    *flag = 0;  // every writer stores the same value
+  }
+}
+
+static inline int grid_for(size_t n, int per_block = kThreads, int cap = 8192) {
+  size_t g = (n + per_block - 1) / per_block;
+  if (g < 1) {
+    g = 1;
+  }
+  if (g > (size_t)cap) {
+    g = cap;
+  }
+  return static_cast<int>(g);
+}
+
+static inline FpTables tables() {
+  State &s = state();
+  return FpTables{s.exp_tbl, s.div_p, s.div_q};
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_fp_fill_iota(uint16_t *fp, size_t n) {
+  MI355_REQUIRE_INIT();
+  if (n == 0) {
+    return MI355_OK;
+  }
+  fp_fill_iota_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(fp, n);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_fill_uniform(uint16_t *fp, size_t n, uint64_t seed) {
+  MI355_REQUIRE_INIT();
+  if (n == 0) {
+    return MI355_OK;
+  }
+  fp_fill_uniform_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(fp, n, seed);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch,
+                               int m, int n, int k) {
+  MI355_REQUIRE_INIT();
+  if (batch < 0 || m < 0 || n < 0 || k < 0) {
+    return fail(MI355_ERR_INVALID, "negative matmul extent");
+  }
+  if (batch == 0 || m == 0 || n == 0) {
+    return MI355_OK;
+  }
+  if (batch > 65535) {
+    return fail(MI355_ERR_UNSUPPORTED, "batch %d exceeds grid.z", batch);
+  }
+  hipStream_t st = state().stream;
+  if (m >= 128) {
+    dim3 grid((n + 63) / 64, (m + 127) / 128, batch);
+    fp_matmul_kernel<8><<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
+  } else if (m >= 33) {
+    dim3 grid((n + 63) / 64, (m + 63) / 64, batch);
+    fp_matmul_kernel<4><<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
+  } else {
+    dim3 grid((n + 63) / 64, (m + 15) / 16, batch);
+    fp_matmul_kernel<1><<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
+  }
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_unary(int op, uint16_t const *in, uint16_t *out, size_t n) {
+  MI355_REQUIRE_INIT();
+  if (op != KN_EXP_OP && op != KN_SILU_OP) {
+    return fail(MI355_ERR_UNSUPPORTED, "unary fingerprint op %d", op);
+  }
+  if (n == 0) {
+    return MI355_OK;
+  }
+  fp_unary_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(op, tables(), in, out, n);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_binary(int op, uint16_t const *in1, int const *dims1,
+                               uint16_t const *in2, int const *dims2, uint16_t *out,
+                               int const *dims_out, int num_dims) {
+  MI355_REQUIRE_INIT();
+  if (op != KN_ADD_OP && op != KN_MUL_OP && op != KN_DIV_OP) {
+    return fail(MI355_ERR_UNSUPPORTED, "binary fingerprint op %d", op);
+  }
+  if (num_dims < 1 || num_dims > 4) {
+    return fail(MI355_ERR_INVALID, "num_dims %d out of range", num_dims);
+  }
+  Dims4 D{};
+  D.nd = num_dims;
+  size_t n = 1;
+  for (int d = 0; d < num_dims; d++) {
+    D.d1[d] = dims1[d];
+    D.d2[d] = dims2[d];
+    D.od[d] = dims_out[d];
+    if (dims1[d] <= 0 || dims2[d] <= 0 || dims_out[d] <= 0 ||
+        (dims1[d] != dims_out[d] && dims1[d] != 1) ||
+        (dims2[d] != dims_out[d] && dims2[d] != 1)) {
+      return fail(MI355_ERR_INVALID, "dim %d is not broadcastable", d);
+    }
+    n *= (size_t)dims_out[d];
+  }
+  fp_binary_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(op, tables(), in1, in2, out, D,
+                                                               n);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_reduce(uint16_t const *in, uint16_t *out, size_t n_out, int factor,
+                               int in_stride, int out_stride) {
+  MI355_REQUIRE_INIT();
+  if (factor <= 0 || in_stride <= 0 || out_stride <= 0 ||
+      (size_t)out_stride * factor != (size_t)in_stride) {
+    return fail(MI355_ERR_INVALID, "reduction strides do not match the factor");
+  }
+  if (n_out == 0) {
+    return MI355_OK;
+  }
+  hipStream_t st = state().stream;
+  if (out_stride == 1 && factor >= 64) {
+    size_t blocks = (n_out * 64 + kThreads - 1) / kThreads;
+    fp_reduce_rows_kernel<<<(unsigned)blocks, kThreads, 0, st>>>(in, out, n_out, factor);
+  } else {
+    size_t blocks = (n_out + kThreads - 1) / kThreads;
+    fp_reduce_kernel<<<(unsigned)blocks, kThreads, 0, st>>>(in, out, n_out, factor, in_stride,
+                                                            out_stride);
+  }
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, int *equal) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  set_flag_kernel<<<1, 1, 0, s.stream>>>(s.flag, 1);
+  if (n > 0) {
+    fp_equal_kernel<<<grid_for(n, kThreads, 2048), kThreads, 0, s.stream>>>(a, b, n, s.flag);
+  }
+  MI355_HIP(hipGetLastError());
+  MI355_HIP(hipMemcpyAsync(s.flag_host, s.flag, sizeof(int), hipMemcpyDeviceToHost, s.stream));
+  MI355_HIP(hipStreamSynchronize(s.stream));
+  *equal = *s.flag_host;
+  return MI355_OK;
+}

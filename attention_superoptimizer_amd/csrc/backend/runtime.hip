@@ -1,0 +1,195 @@
+// Lifetime, memory and timing entry points of the gfx950 backend.
+//
+// Stands in for the device half of the reference's DeviceMemoryManager
+// (src/kernel/device_memory_manager.cu:26-96): one arena allocation, the three
+// fingerprint lookup tables, and the event pairs every profile() uses.
+#include "common.h"
+#include <cstring>
+#include <vector>
+
+namespace mi355 {
+
+static State g_state;
+static char g_error[512] = "";
+
+State &state() { return g_state; }
+
+int fail(int code, char const *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" char const *mi355_last_error(void) { return g_error; }
+
+extern "C" int mi355_is_initialised(void) { return state().ready ? 1 : 0; }
+
+extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
+  State &s = state();
+  if (s.ready) {
+    if (arena_base != nullptr) {
+      *arena_base = s.arena;
+    }
+    if (arena_bytes > s.arena_bytes) {
+      return fail(MI355_ERR_INVALID, "backend already initialised with a smaller arena");
+    }
+    return MI355_OK;
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0) {
+    return fail(MI355_ERR_NO_DEVICE, "no HIP device visible (%s)",
+                e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+  }
+  MI355_HIP(hipSetDevice(0));
+  hipDeviceProp_t prop;
+  MI355_HIP(hipGetDeviceProperties(&prop, 0));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    return fail(MI355_ERR_NO_DEVICE, "device 0 is %s; this backend is built for gfx950 only",
+                prop.gcnArchName);
+  }
+  int optin = 0;
+  if (hipDeviceGetAttribute(&optin, hipDeviceAttributeMaxSharedMemoryPerBlock, 0) == hipSuccess &&
+      optin > 0) {
+    s.max_lds = optin;
+  }
+  MI355_HIP(hipStreamCreate(&s.stream));  // default priority
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.arena), arena_bytes));
+  s.arena_bytes = arena_bytes;
+  // Tables: exp[i] = 3^i mod 227 (i < 113); div_p / div_q = modular inverses with
+  // entries 0 and 1 both mapped to 1 (device_memory_manager.cu:41-90).
+  uint16_t exp_h[FP_Q], divp_h[FP_P], divq_h[FP_Q];
+  exp_h[0] = 1;
+  for (uint32_t i = 1; i < FP_Q; i++) {
+    exp_h[i] = static_cast<uint16_t>((exp_h[i - 1] * FP_EXP_BASE) % FP_P);
+  }
+  if ((exp_h[FP_Q - 1] * FP_EXP_BASE) % FP_P != 1) {
+    return fail(MI355_ERR_INVALID, "exp base does not have order Q modulo P");
+  }
+  auto inverse_table = [](uint16_t *t, uint32_t mod) {
+    for (uint32_t i = 0; i < mod; i++) {
+      t[i] = 1;
+      for (uint32_t j = 1; j < mod; j++) {
+        if ((i * j) % mod == 1) {
+          t[i] = static_cast<uint16_t>(j);
+        }
+      }
+    }
+  };
+  inverse_table(divp_h, FP_P);
+  inverse_table(divq_h, FP_Q);
+  uint16_t *tbl = nullptr;
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&tbl), 1024));
+  s.exp_tbl = tbl;         // 113 entries, 226 B -> next at 240 B
+  s.div_p = tbl + 120;     // 227 entries, 454 B -> next at 704 B
+  s.div_q = tbl + 352;     // 113 entries
+  MI355_HIP(hipMemcpy(s.exp_tbl, exp_h, sizeof(exp_h), hipMemcpyHostToDevice));
+  MI355_HIP(hipMemcpy(s.div_p, divp_h, sizeof(divp_h), hipMemcpyHostToDevice));
+  MI355_HIP(hipMemcpy(s.div_q, divq_h, sizeof(divq_h), hipMemcpyHostToDevice));
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.flag), 256));
+  MI355_HIP(hipHostMalloc(reinterpret_cast<void **>(&s.flag_host), 256, hipHostMallocDefault));
+  MI355_HIP(hipEventCreate(&s.ev0));
+  MI355_HIP(hipEventCreate(&s.ev1));
+  s.ready = true;
+  if (arena_base != nullptr) {
+    *arena_base = s.arena;
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_shutdown(void) {
+  State &s = state();
+  if (!s.ready) {
+    return MI355_OK;
+  }
+  MI355_HIP(hipStreamSynchronize(s.stream));
+  MI355_HIP(hipEventDestroy(s.ev0));
+  MI355_HIP(hipEventDestroy(s.ev1));
+  MI355_HIP(hipFree(s.arena));
+  MI355_HIP(hipFree(s.exp_tbl));
+  MI355_HIP(hipFree(s.flag));
+  MI355_HIP(hipHostFree(s.flag_host));
+  MI355_HIP(hipStreamDestroy(s.stream));
+  s = State{};
+  return MI355_OK;
+}
+
+extern "C" int mi355_get_device_info(mi355_device_info *info) {
+  MI355_REQUIRE_INIT();
+  if (info == nullptr) {
+    return fail(MI355_ERR_INVALID, "null info");
+  }
+  hipDeviceProp_t prop;
+  MI355_HIP(hipGetDeviceProperties(&prop, state().device));
+  memset(info, 0, sizeof(*info));
+  strncpy(info->name, prop.name, sizeof(info->name) - 1);
+  strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+  info->compute_units = prop.multiProcessorCount;
+  info->clock_mhz = prop.clockRate / 1000;
+  info->memory_clock_mhz = prop.memoryClockRate / 1000;
+  info->lds_bytes_per_block = state().max_lds;
+  info->total_memory = prop.totalGlobalMem;
+  return MI355_OK;
+}
+
+extern "C" int mi355_get_tables(void const **exp_tbl, void const **div_p, void const **div_q) {
+  MI355_REQUIRE_INIT();
+  *exp_tbl = state().exp_tbl;
+  *div_p = state().div_p;
+  *div_q = state().div_q;
+  return MI355_OK;
+}
+
+extern "C" int mi355_memcpy_h2d(void *dst, void const *src, size_t bytes) {
+  MI355_REQUIRE_INIT();
+  MI355_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, state().stream));
+  MI355_HIP(hipStreamSynchronize(state().stream));
+  return MI355_OK;
+}
+
+extern "C" int mi355_memcpy_d2h(void *dst, void const *src, size_t bytes) {
+  MI355_REQUIRE_INIT();
+  MI355_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, state().stream));
+  MI355_HIP(hipStreamSynchronize(state().stream));
+  return MI355_OK;
+}
+
+extern "C" int mi355_memset(void *dst, int value, size_t bytes) {
+  MI355_REQUIRE_INIT();
+  MI355_HIP(hipMemsetAsync(dst, value, bytes, state().stream));
+  return MI355_OK;
+}
+
+extern "C" int mi355_sync(void) {
+  MI355_REQUIRE_INIT();
+  MI355_HIP(hipStreamSynchronize(state().stream));
+  return MI355_OK;
+}
+
+extern "C" int mi355_timer_start(void) {
+  MI355_REQUIRE_INIT();
+  MI355_HIP(hipEventRecord(state().ev0, state().stream));
+  return MI355_OK;
+}
+
+extern "C" int mi355_timer_stop(float *ms) {
+  MI355_REQUIRE_INIT();
+  MI355_HIP(hipEventRecord(state().ev1, state().stream));
+  MI355_HIP(hipEventSynchronize(state().ev1));
+  MI355_HIP(hipEventElapsedTime(ms, state().ev0, state().ev1));
+  return MI355_OK;
+}
+
+extern "C" int mi355_last_launch(mi355_launch_info *info) {
+  if (info == nullptr) {
+    return fail(MI355_ERR_INVALID, "null info");
+  }
+  *info = state().last_launch;
+  return MI355_OK;
+}

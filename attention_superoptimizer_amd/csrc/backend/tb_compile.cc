@@ -1,0 +1,411 @@
+// Host-side lowering of an mi355_plan (the reference's NewKernelParams bytecode,
+// produced by threadblock::Graph::get_new_kernel_params, reference
+// src/threadblock/graph.cc:68-432) into a DevProgram for the interpreter kernels.
+#include "common.h"
+#include "tb_program.h"
+
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <vector>
+
+namespace mi355 {
+
+namespace {
+
+struct TensorInfo {
+  int rows = 0, cols = 0;
+  int def_op = 0, last_use = 0;
+  bool persistent = false;
+  bool as_a = false, as_b = false;
+  int bytes = 0;
+};
+
+std::string fmt(char const *f, ...) {
+  char buf[256];
+  va_list ap;
+  va_start(ap, f);
+  vsnprintf(buf, sizeof(buf), f, ap);
+  va_end(ap);
+  return buf;
+}
+
+int round_up(int x, int a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+
+int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,
+                 PlanExtents &ext, std::string &err) {
+  memset(&prog, 0, sizeof(prog));
+  memset(&ext, 0, sizeof(ext));
+  if (plan.num_operators < 1 || plan.num_operators > MI355_MAX_OPERATORS ||
+      plan.num_parameters < 0 || plan.num_parameters > MI355_MAX_PARAMETERS ||
+      plan.num_dmem_inputs < 0 || plan.num_dmem_inputs > MI355_MAX_DMEM_INPUTS ||
+      plan.num_dmem_outputs < 0 || plan.num_dmem_outputs > MI355_MAX_DMEM_OUTPUTS) {
+    err = "plan counts out of range";
+    return MI355_ERR_INVALID;
+  }
+  for (int g = 0; g < 3; g++) {
+    if (plan.grid_dim[g] < 1) {
+      err = "grid_dim must be positive";
+      return MI355_ERR_INVALID;
+    }
+    prog.grid[g] = plan.grid_dim[g];
+  }
+  if (plan.grid_dim[1] > 65535 || plan.grid_dim[2] > 65535) {
+    err = "grid_dim.y/z exceed 65535";
+    return MI355_ERR_UNSUPPORTED;
+  }
+  if (plan.forloop_range < 1) {
+    err = "forloop_range must be positive";
+    return MI355_ERR_INVALID;
+  }
+  int const F = plan.forloop_range;
+  prog.forloop_range = F;
+  prog.num_ops = plan.num_operators;
+
+  std::vector<TensorInfo> T;
+  std::map<int, int> by_offset;  // plan smem offset -> tensor id (latest definition)
+  auto lookup = [&](int voff, int op) -> int {
+    auto it = by_offset.find(voff);
+    if (it == by_offset.end()) {
+      return -1;
+    }
+    T[it->second].last_use = op;
+    return it->second;
+  };
+  auto define = [&](int voff, int rows, int cols, int op) -> int {
+    if ((int)T.size() >= kMaxTensors) {
+      return -1;
+    }
+    TensorInfo ti;
+    ti.rows = rows;
+    ti.cols = cols;
+    ti.def_op = op;
+    ti.last_use = op;
+    T.push_back(ti);
+    by_offset[voff] = (int)T.size() - 1;
+    return (int)T.size() - 1;
+  };
+
+  int const *P = plan.parameters;
+  int pi = 0, n_in = 0, n_out = 0;
+  int const out_start = plan.num_operators - plan.num_dmem_outputs;
+  for (int o = 0; o < plan.num_operators; o++) {
+    DevOp &d = prog.ops[o];
+    d.src0 = d.src1 = d.dst = -1;
+    int const t = plan.operator_types[o];
+    auto need = [&](int n) { return pi + n <= plan.num_parameters; };
+    if (t == TB_INPUT_OP) {
+      if (!need(19) || n_in >= plan.num_dmem_inputs || o != n_in) {
+        err = "input loader out of place or truncated";
+        return MI355_ERR_INVALID;
+      }
+      int const *q = P + pi;
+      pi += 19;
+      d.kind = DOP_LOAD;
+      d.io = n_in++;
+      for (int g = 0; g < 3; g++) {
+        d.row_bs[g] = q[g];
+        d.col_bs[g] = q[3 + g];
+        d.g_bs[g] = q[8 + g];
+      }
+      d.row_fs = q[6];
+      d.col_fs = q[7];
+      d.g_fs = q[11];
+      d.d_rows = q[12];
+      d.d_cols = q[13];
+      int rows = q[14], cols = q[15];
+      if (rows < 1 || cols < 1 || d.d_rows < 1 || d.d_cols < 1) {
+        err = "input tile shape must be positive";
+        return MI355_ERR_INVALID;
+      }
+      d.dst = define(q[18], rows, cols, o);
+      d.hoist = (F == 1) || (d.row_fs == 0 && d.col_fs == 0 && d.g_fs == 0);
+      long long max_row = (long long)(F - 1) * d.row_fs + rows - 1;
+      long long max_col = (long long)(F - 1) * d.col_fs + cols - 1;
+      long long max_g = (long long)(F - 1) * d.g_fs;
+      bool al = cols % 8 == 0 && d.d_cols % 8 == 0 && d.col_fs % 8 == 0 && d.g_fs % 8 == 0;
+      for (int g = 0; g < 3; g++) {
+        long long b = plan.grid_dim[g] - 1;
+        if (d.row_bs[g] < 0 || d.col_bs[g] < 0 || d.g_bs[g] < 0) {
+          err = "negative loader stride";
+          return MI355_ERR_INVALID;
+        }
+        max_row += b * d.row_bs[g];
+        max_col += b * d.col_bs[g];
+        max_g += b * d.g_bs[g];
+        al = al && d.col_bs[g] % 8 == 0 && d.g_bs[g] % 8 == 0;
+      }
+      if (d.row_fs < 0 || d.col_fs < 0 || d.g_fs < 0) {
+        err = "negative loader stride";
+        return MI355_ERR_INVALID;
+      }
+      if (max_row >= d.d_rows || max_col >= d.d_cols) {
+        err = fmt("input %d: tile walks outside its %dx%d matrix", d.io, d.d_rows, d.d_cols);
+        return MI355_ERR_INVALID;
+      }
+      d.vec8 = al ? 1 : 0;
+      ext.in_elems[d.io] = max_g + max_row * d.d_cols + max_col + 1;
+    } else if (t == TB_OUTPUT_OP) {
+      if (!need(17) || o < out_start) {
+        err = "output saver out of place or truncated";
+        return MI355_ERR_INVALID;
+      }
+      int const *q = P + pi;
+      pi += 17;
+      d.kind = DOP_OUTPUT;
+      d.io = n_out++;
+      for (int g = 0; g < 3; g++) {
+        d.row_bs[g] = q[g];
+        d.col_bs[g] = q[3 + g];
+        d.g_bs[g] = q[6 + g];
+      }
+      d.d_rows = q[9];
+      d.d_cols = q[10];
+      int rows = q[11], cols = q[12];
+      d.src0 = lookup(q[15], o);
+      if (d.src0 < 0 || T[d.src0].rows != rows || T[d.src0].cols != cols) {
+        err = "output saver input does not name a tile of its shape";
+        return MI355_ERR_INVALID;
+      }
+      d.dst = define(q[16], rows, cols, o);
+      long long max_row = rows - 1, max_col = cols - 1, max_g = 0;
+      bool al = cols % 8 == 0 && d.d_cols % 8 == 0;
+      for (int g = 0; g < 3; g++) {
+        long long b = plan.grid_dim[g] - 1;
+        if (d.row_bs[g] < 0 || d.col_bs[g] < 0 || d.g_bs[g] < 0) {
+          err = "negative saver stride";
+          return MI355_ERR_INVALID;
+        }
+        max_row += b * d.row_bs[g];
+        max_col += b * d.col_bs[g];
+        max_g += b * d.g_bs[g];
+        al = al && d.col_bs[g] % 8 == 0 && d.g_bs[g] % 8 == 0;
+      }
+      if (max_row >= d.d_rows || max_col >= d.d_cols) {
+        err = fmt("output %d: tile walks outside its %dx%d matrix", d.io, d.d_rows, d.d_cols);
+        return MI355_ERR_INVALID;
+      }
+      d.vec8 = al ? 1 : 0;
+      ext.out_elems[d.io] = max_g + max_row * d.d_cols + max_col + 1;
+    } else if (t == TB_MATMUL_OP) {
+      if (!need(6)) {
+        err = "matmul truncated";
+        return MI355_ERR_INVALID;
+      }
+      int m = P[pi], n = P[pi + 1], k = P[pi + 2];
+      d.kind = DOP_MATMUL;
+      d.src0 = lookup(P[pi + 3], o);
+      d.src1 = lookup(P[pi + 4], o);
+      if (d.src0 < 0 || d.src1 < 0 || T[d.src0].rows != m || T[d.src0].cols != k ||
+          T[d.src1].rows != k || T[d.src1].cols != n || m < 1 || n < 1 || k < 1) {
+        err = "matmul operands do not match m, n, k";
+        return MI355_ERR_INVALID;
+      }
+      T[d.src0].as_a = true;
+      T[d.src1].as_b = true;
+      d.dst = define(P[pi + 5], m, n, o);
+      pi += 6;
+    } else if (t == TB_EXP_OP || t == TB_SILU_OP) {
+      if (!need(2)) {
+        err = "unary truncated";
+        return MI355_ERR_INVALID;
+      }
+      d.kind = DOP_UNARY;
+      d.sub = t;
+      d.src0 = lookup(P[pi], o);
+      if (d.src0 < 0 || T[d.src0].rows * T[d.src0].cols != P[pi + 1]) {
+        err = "unary operand does not match its element count";
+        return MI355_ERR_INVALID;
+      }
+      d.dst = d.src0;  // in place (reference src/threadblock/element_unary.cc:46)
+      pi += 2;
+    } else if (t == TB_ADD_OP || t == TB_MUL_OP || t == TB_DIV_OP) {
+      if (!need(9)) {
+        err = "binary truncated";
+        return MI355_ERR_INVALID;
+      }
+      int const *q = P + pi;
+      pi += 9;
+      if (q[0] != 1 || q[3] != 1) {
+        err = "binary operands with a leading dim > 1 are not supported";
+        return MI355_ERR_UNSUPPORTED;
+      }
+      d.kind = DOP_BINARY;
+      d.sub = t;
+      d.src0 = lookup(q[6], o);
+      d.src1 = lookup(q[7], o);
+      if (d.src0 < 0 || d.src1 < 0 || T[d.src0].rows != q[1] || T[d.src0].cols != q[2] ||
+          T[d.src1].rows != q[4] || T[d.src1].cols != q[5]) {
+        err = "binary operands do not match their shapes";
+        return MI355_ERR_INVALID;
+      }
+      int rows = std::max(q[1], q[4]), cols = std::max(q[2], q[5]);
+      if ((q[1] != rows && q[1] != 1) || (q[4] != rows && q[4] != 1) ||
+          (q[2] != cols && q[2] != 1) || (q[5] != cols && q[5] != 1)) {
+        err = "binary operands are not broadcastable";
+        return MI355_ERR_INVALID;
+      }
+      d.dst = define(q[8], rows, cols, o);
+    } else if (t >= TB_REDUCTION_0_OP && t <= TB_REDUCTION_2_TO_DIMX_OP) {
+      if (!need(5)) {
+        err = "reduction truncated";
+        return MI355_ERR_INVALID;
+      }
+      int n_o = P[pi], deg = P[pi + 1], inner = P[pi + 2];
+      d.kind = DOP_REDUCE;
+      d.src0 = lookup(P[pi + 3], o);
+      if (d.src0 < 0 || n_o < 1 || deg < 1 || inner < 1) {
+        err = "reduction operand missing";
+        return MI355_ERR_INVALID;
+      }
+      int R = T[d.src0].rows, C = T[d.src0].cols;
+      int orows, ocols;
+      if (n_o % R == 0 && inner == n_o / R && (long long)inner * deg == C) {
+        orows = R;  // reduce along columns down to `inner` columns
+        ocols = inner;
+      } else if (inner == n_o && n_o % C == 0 && (long long)(n_o / C) * deg == R) {
+        orows = n_o / C;  // reduce along rows
+        ocols = C;
+      } else {
+        err = "reduction shape is not a row or column reduction of a 2-D tile";
+        return MI355_ERR_UNSUPPORTED;
+      }
+      d.red_deg = deg;
+      d.red_inner = inner;
+      d.dst = define(P[pi + 4], orows, ocols, o);
+      pi += 5;
+    } else if (t >= TB_CONCAT_0_OP && t <= TB_CONCAT_2_OP) {
+      if (!need(7)) {
+        err = "concat truncated";
+        return MI355_ERR_INVALID;
+      }
+      int n_o = P[pi], a = P[pi + 1], b = P[pi + 2], inner = P[pi + 3];
+      d.kind = DOP_CONCAT;
+      d.src0 = lookup(P[pi + 4], o);
+      d.src1 = lookup(P[pi + 5], o);
+      if (d.src0 < 0 || d.src1 < 0) {
+        err = "concat operand missing";
+        return MI355_ERR_INVALID;
+      }
+      TensorInfo const &A = T[d.src0], &B = T[d.src1];
+      int orows, ocols;
+      if (inner == 1 && A.cols == a && B.cols == b && A.rows == B.rows) {
+        orows = A.rows;
+        ocols = a + b;
+      } else if (inner == A.cols && A.cols == B.cols && A.rows == a && B.rows == b) {
+        orows = a + b;
+        ocols = A.cols;
+      } else {
+        err = "concat is not along the rows or columns of a 2-D tile";
+        return MI355_ERR_UNSUPPORTED;
+      }
+      if (n_o != orows * ocols) {
+        err = "concat element count mismatch";
+        return MI355_ERR_INVALID;
+      }
+      d.cat_a = a;
+      d.cat_b = b;
+      d.cat_inner = inner;
+      d.dst = define(P[pi + 6], orows, ocols, o);
+      pi += 7;
+    } else {
+      err = fmt("unsupported thread-block operator %d", t);
+      return MI355_ERR_UNSUPPORTED;
+    }
+    if (d.dst < 0) {
+      err = "too many tensors in one thread-block graph";
+      return MI355_ERR_UNSUPPORTED;
+    }
+  }
+  if (pi != plan.num_parameters || n_in != plan.num_dmem_inputs ||
+      n_out != plan.num_dmem_outputs) {
+    err = "parameter stream does not match the operator list";
+    return MI355_ERR_INVALID;
+  }
+
+  // ---- layouts ---------------------------------------------------------------
+  prog.num_tensors = (int)T.size();
+  for (int i = 0; i < prog.num_tensors; i++) {
+    DevTensor &dt = prog.t[i];
+    TensorInfo &ti = T[i];
+    dt.rows = ti.rows;
+    dt.cols = ti.cols;
+    if (!f16) {
+      dt.rs = ti.cols;
+      dt.cs = 1;
+      ti.bytes = round_up(ti.rows * ti.cols * 2, 16);
+    } else if (ti.as_b && !ti.as_a) {
+      // k-contiguous for the matrix-core B operand: column-major, padded columns
+      dt.rs = 1;
+      dt.cs = ti.rows >= 8 ? round_up(ti.rows, 8) + 8 : ti.rows;
+      ti.bytes = round_up(dt.cs * ti.cols * 2, 16);
+    } else {
+      dt.cs = 1;
+      dt.rs = ti.cols >= 8 ? round_up(ti.cols, 8) + 8 : ti.cols;
+      ti.bytes = round_up(dt.rs * ti.rows * 2, 16);
+    }
+  }
+  // persistent tiles: accumulators and hoisted loads stay live over the whole loop
+  for (int o = 0; o < prog.num_ops; o++) {
+    DevOp const &d = prog.ops[o];
+    if (d.kind == DOP_OUTPUT || (d.kind == DOP_LOAD && d.hoist)) {
+      T[d.dst].persistent = true;
+    }
+  }
+  // ---- LDS placement: persistent tiles first, the rest by first fit over their
+  // [definition, last use] interval inside one iteration
+  int top = kTableBytes;
+  for (int i = 0; i < prog.num_tensors; i++) {
+    if (T[i].persistent) {
+      prog.t[i].off = top;
+      top += T[i].bytes;
+    }
+  }
+  int const base = top;
+  int peak = top;
+  struct Live {
+    int off, bytes, id;
+  };
+  std::vector<Live> live;
+  for (int o = 0; o < prog.num_ops; o++) {
+    for (int i = 0; i < prog.num_tensors; i++) {
+      if (T[i].persistent || T[i].def_op != o) {
+        continue;
+      }
+      std::sort(live.begin(), live.end(), [](Live const &a, Live const &b) { return a.off < b.off; });
+      int off = base;
+      for (Live const &l : live) {
+        if (off + T[i].bytes <= l.off) {
+          break;
+        }
+        off = std::max(off, l.off + l.bytes);
+      }
+      prog.t[i].off = off;
+      live.push_back(Live{off, T[i].bytes, i});
+      peak = std::max(peak, off + T[i].bytes);
+    }
+    live.erase(std::remove_if(live.begin(), live.end(),
+                              [&](Live const &l) { return T[l.id].last_use <= o; }),
+               live.end());
+  }
+  prog.lds_bytes = peak;
+  if (peak > max_lds) {
+    err = fmt("thread-block graph needs %d bytes of LDS, the device offers %d", peak, max_lds);
+    return MI355_ERR_UNSUPPORTED;
+  }
+  // LDS writes of 16 bytes need 8-element row strides on the destination
+  for (int o = 0; o < prog.num_ops; o++) {
+    DevOp &d = prog.ops[o];
+    if (d.kind == DOP_LOAD && f16 && (prog.t[d.dst].cs != 1 || prog.t[d.dst].rs % 8 != 0)) {
+      d.vec8 = d.vec8 ? 2 : 0;  // 2: vector global read, scalar LDS scatter
+    }
+    if (d.kind == DOP_OUTPUT && f16 && (prog.t[d.dst].cs != 1 || prog.t[d.dst].rs % 8 != 0)) {
+      d.vec8 = 0;
+    }
+  }
+  return MI355_OK;
+}
+
+}  // namespace mi355

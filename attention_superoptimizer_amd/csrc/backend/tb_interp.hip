@@ -1,0 +1,654 @@
+// The customized-op interpreters: one workgroup per logical thread block walks
+// the thread-block graph once per for-loop iteration with every tile in LDS.
+//
+//   fp_interp_kernel   uint16 over Z_25651, integer only
+//                      (reference compute_customizedop_fingerprint,
+//                       src/kernel/cuda/customized_kernel.cu:307-603)
+//   f16_interp_kernel  fp16 tiles, fp32 math, matmul on the matrix cores
+//                      (reference customized_kernel_function, :39-305, with the
+//                       arithmetic the reference's generated programs define,
+//                       src/kernel/triton_code_gen.cc:223-333)
+#include "common.h"
+#include "tb_program.h"
+
+#include <string>
+
+namespace mi355 {
+
+constexpr int kInterpThreads = 256;
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+struct TileOrigin {
+  long long base;  // element offset of the batch slice
+  int row0, col0;
+};
+
+__device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it) {
+  TileOrigin o;
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  o.row0 = bx * op.row_bs[0] + by * op.row_bs[1] + bz * op.row_bs[2] + it * op.row_fs;
+  o.col0 = bx * op.col_bs[0] + by * op.col_bs[1] + bz * op.col_bs[2] + it * op.col_fs;
+  o.base = (long long)bx * op.g_bs[0] + (long long)by * op.g_bs[1] + (long long)bz * op.g_bs[2] +
+           (long long)it * op.g_fs;
+  return o;
+}
+
+// ===========================================================================
+// uint16 interpreter
+// ===========================================================================
+// LDS table block: [0,113) exp premultiplied by the CRT lift, [128,355) div_p,
+// [384,497) div_q
+__device__ __forceinline__ uint32_t lds_exp(uint16_t const *tbl, uint32_t x) {
+  return tbl[x % FP_Q];
+}
+__device__ __forceinline__ uint32_t lds_div(uint16_t const *tbl, uint32_t x, uint32_t y) {
+  uint32_t z = (x % FP_P) * tbl[128 + y % FP_P] * FP_Q_MUL_P_MOD_1 +
+               (x % FP_Q) * tbl[384 + y % FP_Q] * FP_P_MUL_Q_MOD_1;
+  return z % FP_PQ;
+}
+__device__ __forceinline__ uint32_t lds_silu(uint16_t const *tbl, uint32_t x) {
+  uint32_t neg = (FP_PQ - x) % FP_PQ;
+  uint32_t den = (1u + lds_exp(tbl, neg)) % FP_PQ;
+  return lds_div(tbl, x, den);
+}
+
+__global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
+    DevProgram const P, uint16_t const *__restrict__ g_exp, uint16_t const *__restrict__ g_divp,
+    uint16_t const *__restrict__ g_divq) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  uint16_t *tbl = reinterpret_cast<uint16_t *>(lds);
+  int const tid = threadIdx.x;
+  for (int i = tid; i < (int)FP_Q; i += kInterpThreads) {
+    tbl[i] = static_cast<uint16_t>((g_exp[i] * FP_Q_MUL_P_MOD_1) % FP_PQ);
+    tbl[384 + i] = g_divq[i];
+  }
+  for (int i = tid; i < (int)FP_P; i += kInterpThreads) {
+    tbl[128 + i] = g_divp[i];
+  }
+  __syncthreads();
+  int const F = P.forloop_range;
+  for (int it = 0; it < F; it++) {
+    for (int o = 0; o < P.num_ops; o++) {
+      DevOp const &op = P.ops[o];
+      switch (op.kind) {
+        case DOP_LOAD: {
+          if (op.hoist && it > 0) {
+            break;
+          }
+          DevTensor const &t = P.t[op.dst];
+          uint16_t *s = reinterpret_cast<uint16_t *>(lds + t.off);
+          TileOrigin org = tile_origin(op, it);
+          uint16_t const *g = static_cast<uint16_t const *>(P.in[op.io]) + org.base;
+          if (op.vec8) {
+            int const cpr = t.cols / 8, n = t.rows * cpr;
+            for (int e = tid; e < n; e += kInterpThreads) {
+              int r = e / cpr, c = (e % cpr) * 8;
+              uint4v v = *reinterpret_cast<uint4v const *>(
+                  g + (long long)(org.row0 + r) * op.d_cols + org.col0 + c);
+              *reinterpret_cast<uint4v *>(s + r * t.cols + c) = v;
+            }
+          } else {
+            int const n = t.rows * t.cols;
+            for (int e = tid; e < n; e += kInterpThreads) {
+              int r = e / t.cols, c = e % t.cols;
+              s[e] = g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c];
+            }
+          }
+          break;
+        }
+        case DOP_MATMUL: {
+          // reference matmul.h:773-804; the modulus is applied every 4 products
+          // (4 * 25650^2 + 25650 < 2^32), same ring value as reducing each step
+          DevTensor const &ta = P.t[op.src0], &tb = P.t[op.src1], &tc = P.t[op.dst];
+          uint16_t const *A = reinterpret_cast<uint16_t const *>(lds + ta.off);
+          uint16_t const *B = reinterpret_cast<uint16_t const *>(lds + tb.off);
+          uint16_t *C = reinterpret_cast<uint16_t *>(lds + tc.off);
+          int const m = ta.rows, k = ta.cols, n = tb.cols;
+          if (n % 4 == 0) {
+            int const n4 = n / 4, total = m * n4;
+            for (int e = tid; e < total; e += kInterpThreads) {
+              int row = e / n4, c0 = (e % n4) * 4;
+              uint32_t acc[4] = {0, 0, 0, 0};
+              uint16_t const *ap = A + row * k;
+              uint16_t const *bp = B + c0;
+              int kk = 0;
+              for (; kk + 4 <= k; kk += 4) {
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                  uint32_t a = ap[kk + u];
+                  uint2 bv = *reinterpret_cast<uint2 const *>(bp + (kk + u) * n);
+                  acc[0] += a * (bv.x & 0xffffu);
+                  acc[1] += a * (bv.x >> 16);
+                  acc[2] += a * (bv.y & 0xffffu);
+                  acc[3] += a * (bv.y >> 16);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  acc[j] %= FP_PQ;
+                }
+              }
+              for (; kk < k; kk++) {
+                uint32_t a = ap[kk];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  acc[j] = (acc[j] + a * bp[kk * n + j]) % FP_PQ;
+                }
+              }
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                C[row * n + c0 + j] = static_cast<uint16_t>(acc[j]);
+              }
+            }
+          } else {
+            int const total = m * n;
+            for (int e = tid; e < total; e += kInterpThreads) {
+              int row = e / n, col = e % n;
+              uint32_t acc = 0;
+              for (int kk = 0; kk < k; kk++) {
+                acc = (acc + (uint32_t)A[row * k + kk] * B[kk * n + col]) % FP_PQ;
+              }
+              C[e] = static_cast<uint16_t>(acc);
+            }
+          }
+          break;
+        }
+        case DOP_UNARY: {
+          DevTensor const &t = P.t[op.dst];
+          uint16_t *p = reinterpret_cast<uint16_t *>(lds + t.off);
+          int const n = t.rows * t.cols;
+          if (op.sub == TB_EXP_OP) {
+            for (int e = tid; e < n; e += kInterpThreads) {
+              p[e] = static_cast<uint16_t>(lds_exp(tbl, p[e]));
+            }
+          } else {
+            for (int e = tid; e < n; e += kInterpThreads) {
+              p[e] = static_cast<uint16_t>(lds_silu(tbl, p[e]));
+            }
+          }
+          break;
+        }
+        case DOP_BINARY: {
+          // reference element_binary.h:86-105 (broadcast by `% dim`)
+          DevTensor const &t1 = P.t[op.src0], &t2 = P.t[op.src1], &to = P.t[op.dst];
+          uint16_t const *x1 = reinterpret_cast<uint16_t const *>(lds + t1.off);
+          uint16_t const *x2 = reinterpret_cast<uint16_t const *>(lds + t2.off);
+          uint16_t *y = reinterpret_cast<uint16_t *>(lds + to.off);
+          int const n = to.rows * to.cols;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int r = e / to.cols, c = e % to.cols;
+            uint32_t a = x1[(r % t1.rows) * t1.cols + c % t1.cols];
+            uint32_t b = x2[(r % t2.rows) * t2.cols + c % t2.cols];
+            uint32_t z;
+            if (op.sub == TB_DIV_OP) {
+              z = lds_div(tbl, a, b);
+            } else if (op.sub == TB_ADD_OP) {
+              z = (a + b) % FP_PQ;
+            } else {
+              z = (a * b) % FP_PQ;
+            }
+            y[e] = static_cast<uint16_t>(z);
+          }
+          break;
+        }
+        case DOP_REDUCE: {
+          // reference reduction.h:147-156; uint16 terms are summed unreduced in
+          // 32 bits and folded every 32768 terms
+          DevTensor const &ti = P.t[op.src0], &to = P.t[op.dst];
+          uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + ti.off);
+          uint16_t *y = reinterpret_cast<uint16_t *>(lds + to.off);
+          int const n = to.rows * to.cols, deg = op.red_deg, inner = op.red_inner;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int pos = (e / inner) * (inner * deg) + e % inner;
+            uint32_t r = 0;
+            for (int kk = 0; kk < deg; kk++, pos += inner) {
+              r += x[pos];
+              if ((kk & 32767) == 32767) {
+                r %= FP_PQ;
+              }
+            }
+            y[e] = static_cast<uint16_t>(r % FP_PQ);
+          }
+          break;
+        }
+        case DOP_CONCAT: {
+          // reference concat.h:90-101
+          DevTensor const &to = P.t[op.dst];
+          uint16_t const *A = reinterpret_cast<uint16_t const *>(lds + P.t[op.src0].off);
+          uint16_t const *B = reinterpret_cast<uint16_t const *>(lds + P.t[op.src1].off);
+          uint16_t *y = reinterpret_cast<uint16_t *>(lds + to.off);
+          int const n = to.rows * to.cols, a = op.cat_a, b = op.cat_b, inner = op.cat_inner;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int in_i = e % inner, cd = (e / inner) % (a + b), outer = (e / inner) / (a + b);
+            y[e] = cd < a ? A[in_i + cd * inner + outer * inner * a]
+                          : B[in_i + (cd - a) * inner + outer * inner * b];
+          }
+          break;
+        }
+        case DOP_OUTPUT: {
+          // reference output_saver.h:373-401 (accumulate) and :418-447 (store)
+          DevTensor const &ti = P.t[op.src0], &ta = P.t[op.dst];
+          uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + ti.off);
+          uint16_t *acc = reinterpret_cast<uint16_t *>(lds + ta.off);
+          int const n = ta.rows * ta.cols;
+          bool const last = (it == F - 1);
+          TileOrigin org = tile_origin(op, 0);
+          uint16_t *g = static_cast<uint16_t *>(P.out[op.io]) + org.base;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            uint32_t v = x[e];
+            if (it > 0) {
+              v = (v + acc[e]) % FP_PQ;
+            }
+            if (last) {
+              int r = e / ta.cols, c = e % ta.cols;
+              g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c] = static_cast<uint16_t>(v);
+            } else {
+              acc[e] = static_cast<uint16_t>(v);
+            }
+          }
+          break;
+        }
+        default:
+          break;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// ===========================================================================
+// fp16 interpreter
+// ===========================================================================
+__device__ __forceinline__ _Float16 *tile_ptr(unsigned char *lds, DevTensor const &t) {
+  return reinterpret_cast<_Float16 *>(lds + t.off);
+}
+
+// C[m][n] = A[m][k] . B[k][n] on the matrix cores.  A is k-contiguous per row
+// (cs == 1), B is k-contiguous per column (rs == 1); both strides are multiples
+// of 8 so every operand fetch is one 16-byte LDS read.  Wavefronts take output
+// tiles round-robin.  Rows past m are clamped on read and masked on write.
+template <int TILE>
+__device__ __forceinline__ void mfma_matmul(unsigned char *lds, DevTensor const &ta,
+                                            DevTensor const &tb, DevTensor const &tc, int wave,
+                                            int lane, int num_waves) {
+  _Float16 const *A = tile_ptr(lds, ta);
+  _Float16 const *B = tile_ptr(lds, tb);
+  _Float16 *C = tile_ptr(lds, tc);
+  int const m = ta.rows, k = ta.cols, n = tb.cols;
+  int const tiles_m = (m + TILE - 1) / TILE, tiles_n = n / TILE;
+  for (int tile = wave; tile < tiles_m * tiles_n; tile += num_waves) {
+    int const tm = tile / tiles_n, tn = tile % tiles_n;
+    if constexpr (TILE == 32) {
+      int arow = tm * 32 + lane % 32;
+      arow = arow < m ? arow : m - 1;
+      _Float16 const *ap = A + arow * ta.rs + 8 * (lane / 32);
+      _Float16 const *bp = B + (tn * 32 + lane % 32) * tb.cs + 8 * (lane / 32);
+      float16v acc;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        acc[i] = 0.0f;
+      }
+      for (int k0 = 0; k0 < k; k0 += 16) {
+        half8 a = *reinterpret_cast<half8 const *>(ap + k0);
+        half8 b = *reinterpret_cast<half8 const *>(bp + k0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int row = tm * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
+        int col = tn * 32 + lane % 32;
+        if (row < m) {
+          C[row * tc.rs + col * tc.cs] = static_cast<_Float16>(acc[r]);
+        }
+      }
+    } else {
+      int arow = tm * 16 + lane % 16;
+      arow = arow < m ? arow : m - 1;
+      _Float16 const *ap = A + arow * ta.rs;
+      _Float16 const *bp = B + (tn * 16 + lane % 16) * tb.cs;
+      float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+      int k0 = 0;
+      for (; k0 + 32 <= k; k0 += 32) {
+        half8 a = *reinterpret_cast<half8 const *>(ap + k0 + 8 * (lane / 16));
+        half8 b = *reinterpret_cast<half8 const *>(bp + k0 + 8 * (lane / 16));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+      }
+      for (; k0 + 16 <= k; k0 += 16) {
+        half4 a = *reinterpret_cast<half4 const *>(ap + k0 + 4 * (lane / 16));
+        half4 b = *reinterpret_cast<half4 const *>(bp + k0 + 4 * (lane / 16));
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        int row = tm * 16 + (lane / 16) * 4 + r;
+        int col = tn * 16 + lane % 16;
+        if (row < m) {
+          C[row * tc.rs + col * tc.cs] = static_cast<_Float16>(acc[r]);
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram const P) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int const tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  int const F = P.forloop_range;
+  for (int it = 0; it < F; it++) {
+    for (int o = 0; o < P.num_ops; o++) {
+      DevOp const &op = P.ops[o];
+      switch (op.kind) {
+        case DOP_LOAD: {
+          if (op.hoist && it > 0) {
+            break;
+          }
+          DevTensor const &t = P.t[op.dst];
+          _Float16 *s = tile_ptr(lds, t);
+          TileOrigin org = tile_origin(op, it);
+          _Float16 const *g = static_cast<_Float16 const *>(P.in[op.io]) + org.base;
+          if (op.vec8) {
+            int const cpr = t.cols / 8, n = t.rows * cpr;
+            for (int e = tid; e < n; e += kInterpThreads) {
+              int r = e / cpr, c = (e % cpr) * 8;
+              half8 v = *reinterpret_cast<half8 const *>(
+                  g + (long long)(org.row0 + r) * op.d_cols + org.col0 + c);
+              if (op.vec8 == 1) {
+                *reinterpret_cast<half8 *>(s + r * t.rs + c) = v;
+              } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                  s[r * t.rs + (c + j) * t.cs] = v[j];
+                }
+              }
+            }
+          } else {
+            int const n = t.rows * t.cols;
+            for (int e = tid; e < n; e += kInterpThreads) {
+              int r = e / t.cols, c = e % t.cols;
+              s[r * t.rs + c * t.cs] = g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c];
+            }
+          }
+          break;
+        }
+        case DOP_MATMUL: {
+          DevTensor const &ta = P.t[op.src0], &tb = P.t[op.src1], &tc = P.t[op.dst];
+          int const m = ta.rows, k = ta.cols, n = tb.cols;
+          bool const fast = ta.cs == 1 && tb.rs == 1 && ta.rs % 8 == 0 && tb.cs % 8 == 0 &&
+                            k % 16 == 0 && n % 16 == 0;
+          if (fast && m % 32 == 0 && n % 32 == 0) {
+            mfma_matmul<32>(lds, ta, tb, tc, wave, lane, kInterpThreads / 64);
+          } else if (fast) {
+            mfma_matmul<16>(lds, ta, tb, tc, wave, lane, kInterpThreads / 64);
+          } else {
+            _Float16 const *A = tile_ptr(lds, ta);
+            _Float16 const *B = tile_ptr(lds, tb);
+            _Float16 *C = tile_ptr(lds, tc);
+            for (int e = tid; e < m * n; e += kInterpThreads) {
+              int row = e / n, col = e % n;
+              float acc = 0.0f;
+              for (int kk = 0; kk < k; kk++) {
+                acc += static_cast<float>(A[row * ta.rs + kk * ta.cs]) *
+                       static_cast<float>(B[kk * tb.rs + col * tb.cs]);
+              }
+              C[row * tc.rs + col * tc.cs] = static_cast<_Float16>(acc);
+            }
+          }
+          break;
+        }
+        case DOP_UNARY: {
+          DevTensor const &t = P.t[op.dst];
+          _Float16 *p = tile_ptr(lds, t);
+          int const n = t.rows * t.cols;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int r = e / t.cols, c = e % t.cols;
+            _Float16 *q = p + r * t.rs + c * t.cs;
+            float x = static_cast<float>(*q);
+            float y = (op.sub == TB_EXP_OP) ? __expf(x) : x / (1.0f + __expf(-x));
+            *q = static_cast<_Float16>(y);
+          }
+          break;
+        }
+        case DOP_BINARY: {
+          DevTensor const &t1 = P.t[op.src0], &t2 = P.t[op.src1], &to = P.t[op.dst];
+          _Float16 const *x1 = tile_ptr(lds, t1);
+          _Float16 const *x2 = tile_ptr(lds, t2);
+          _Float16 *y = tile_ptr(lds, to);
+          int const n = to.rows * to.cols;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int r = e / to.cols, c = e % to.cols;
+            float a = static_cast<float>(x1[(r % t1.rows) * t1.rs + (c % t1.cols) * t1.cs]);
+            float b = static_cast<float>(x2[(r % t2.rows) * t2.rs + (c % t2.cols) * t2.cs]);
+            float z = (op.sub == TB_DIV_OP) ? a / b : (op.sub == TB_ADD_OP) ? a + b : a * b;
+            y[r * to.rs + c * to.cs] = static_cast<_Float16>(z);
+          }
+          break;
+        }
+        case DOP_REDUCE: {
+          DevTensor const &ti = P.t[op.src0], &to = P.t[op.dst];
+          _Float16 const *x = tile_ptr(lds, ti);
+          _Float16 *y = tile_ptr(lds, to);
+          int const n = to.rows * to.cols, deg = op.red_deg, inner = op.red_inner;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int pos = (e / inner) * (inner * deg) + e % inner;
+            float r = 0.0f;
+            for (int kk = 0; kk < deg; kk++, pos += inner) {
+              r += static_cast<float>(x[(pos / ti.cols) * ti.rs + (pos % ti.cols) * ti.cs]);
+            }
+            y[(e / to.cols) * to.rs + (e % to.cols) * to.cs] = static_cast<_Float16>(r);
+          }
+          break;
+        }
+        case DOP_CONCAT: {
+          DevTensor const &t1 = P.t[op.src0], &t2 = P.t[op.src1], &to = P.t[op.dst];
+          _Float16 const *A = tile_ptr(lds, t1);
+          _Float16 const *B = tile_ptr(lds, t2);
+          _Float16 *y = tile_ptr(lds, to);
+          int const n = to.rows * to.cols;
+          bool const along_cols = (op.cat_inner == 1 && t1.rows == to.rows);
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int r = e / to.cols, c = e % to.cols;
+            _Float16 v;
+            if (along_cols) {
+              v = c < t1.cols ? A[r * t1.rs + c * t1.cs] : B[r * t2.rs + (c - t1.cols) * t2.cs];
+            } else {
+              v = r < t1.rows ? A[r * t1.rs + c * t1.cs] : B[(r - t1.rows) * t2.rs + c * t2.cs];
+            }
+            y[r * to.rs + c * to.cs] = v;
+          }
+          break;
+        }
+        case DOP_OUTPUT: {
+          // accumulators start at zero and take `acc + x`, rounded to fp16 every
+          // iteration (triton_code_gen.cc:223-232); stored once after the loop
+          DevTensor const &ti = P.t[op.src0], &ta = P.t[op.dst];
+          _Float16 const *x = tile_ptr(lds, ti);
+          _Float16 *acc = tile_ptr(lds, ta);
+          int const n = ta.rows * ta.cols;
+          bool const last = (it == F - 1);
+          TileOrigin org = tile_origin(op, 0);
+          _Float16 *g = static_cast<_Float16 *>(P.out[op.io]) + org.base;
+          for (int e = tid; e < n; e += kInterpThreads) {
+            int r = e / ta.cols, c = e % ta.cols;
+            float v = static_cast<float>(x[r * ti.rs + c * ti.cs]);
+            if (it > 0) {
+              v += static_cast<float>(acc[r * ta.rs + c * ta.cs]);
+            }
+            _Float16 h = static_cast<_Float16>(v);
+            if (last) {
+              g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c] = h;
+            } else {
+              acc[r * ta.rs + c * ta.cs] = h;
+            }
+          }
+          break;
+        }
+        default:
+          break;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// ===========================================================================
+// launchers
+// ===========================================================================
+static int prepare(mi355_plan const *plan, void const *const *inputs, void *const *outputs,
+                   bool f16, DevProgram &prog) {
+  if (plan == nullptr || inputs == nullptr || outputs == nullptr) {
+    return fail(MI355_ERR_INVALID, "null argument");
+  }
+  PlanExtents ext;
+  std::string err;
+  int rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err);
+  if (rc != MI355_OK) {
+    return fail(rc, "%s", err.c_str());
+  }
+  for (int i = 0; i < plan->num_dmem_inputs; i++) {
+    if (inputs[i] == nullptr) {
+      return fail(MI355_ERR_INVALID, "input %d is null", i);
+    }
+    prog.in[i] = inputs[i];
+  }
+  for (int i = 0; i < plan->num_dmem_outputs; i++) {
+    if (outputs[i] == nullptr) {
+      return fail(MI355_ERR_INVALID, "output %d is null", i);
+    }
+    prog.out[i] = outputs[i];
+  }
+  // 16-byte global accesses also need 16-byte aligned base pointers
+  for (int o = 0; o < prog.num_ops; o++) {
+    DevOp &d = prog.ops[o];
+    if (d.kind == DOP_LOAD && d.vec8 && (reinterpret_cast<uintptr_t>(prog.in[d.io]) & 15) != 0) {
+      d.vec8 = 0;
+    }
+  }
+  return MI355_OK;
+}
+
+static int launch(DevProgram const &prog, bool f16) {
+  State &s = state();
+  dim3 grid(prog.grid[0], prog.grid[1], prog.grid[2]);
+  static int fp_lds_set = 0, f16_lds_set = 0;
+  int &cur = f16 ? f16_lds_set : fp_lds_set;
+  if (prog.lds_bytes > 65536 && prog.lds_bytes > cur) {
+    if (f16) {
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(f16_interp_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, s.max_lds));
+    } else {
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_interp_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, s.max_lds));
+    }
+    cur = s.max_lds;
+  }
+  if (f16) {
+    f16_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream>>>(prog);
+  } else {
+    fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream>>>(prog, s.exp_tbl,
+                                                                          s.div_p, s.div_q);
+  }
+  MI355_HIP(hipGetLastError());
+  s.last_launch.kernel_id = f16 ? MI355_KERNEL_F16_INTERP : MI355_KERNEL_FP_INTERP;
+  s.last_launch.workgroups = prog.grid[0] * prog.grid[1] * prog.grid[2];
+  s.last_launch.threads = kInterpThreads;
+  s.last_launch.lds_bytes = prog.lds_bytes;
+  s.last_launch.row_split = 1;
+  return MI355_OK;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_plan_extents(mi355_plan const *plan, long long *in_elems,
+                                  long long *out_elems, int *lds_bytes_fp, int *lds_bytes_f16) {
+  if (plan == nullptr) {
+    return fail(MI355_ERR_INVALID, "null plan");
+  }
+  DevProgram prog;
+  PlanExtents ext;
+  std::string err;
+  int rc = compile_plan(*plan, false, 1 << 30, prog, ext, err);
+  if (rc != MI355_OK) {
+    return fail(rc, "%s", err.c_str());
+  }
+  for (int i = 0; i < MI355_MAX_DMEM_INPUTS; i++) {
+    if (in_elems != nullptr) {
+      in_elems[i] = ext.in_elems[i];
+    }
+    if (out_elems != nullptr) {
+      out_elems[i] = ext.out_elems[i];
+    }
+  }
+  if (lds_bytes_fp != nullptr) {
+    *lds_bytes_fp = prog.lds_bytes;
+  }
+  if (lds_bytes_f16 != nullptr) {
+    rc = compile_plan(*plan, true, 1 << 30, prog, ext, err);
+    if (rc != MI355_OK) {
+      return fail(rc, "%s", err.c_str());
+    }
+    *lds_bytes_f16 = prog.lds_bytes;
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,
+                                   void *const *outputs) {
+  MI355_REQUIRE_INIT();
+  DevProgram prog;
+  int rc = prepare(plan, inputs, outputs, false, prog);
+  if (rc != MI355_OK) {
+    return rc;
+  }
+  return launch(prog, false);
+}
+
+extern "C" int mi355_customized_run(mi355_plan const *plan, void const *const *inputs,
+                                    void *const *outputs) {
+  MI355_REQUIRE_INIT();
+  DevProgram prog;
+  int rc = prepare(plan, inputs, outputs, true, prog);
+  if (rc != MI355_OK) {
+    return rc;
+  }
+  return launch(prog, true);
+}
+
+extern "C" int mi355_customized_profile(mi355_plan const *plan, void const *const *inputs,
+                                        void *const *outputs, int fingerprint, int warmup,
+                                        int iters, float *ms) {
+  MI355_REQUIRE_INIT();
+  if (iters < 1 || warmup < 0 || ms == nullptr) {
+    return fail(MI355_ERR_INVALID, "bad iteration counts");
+  }
+  DevProgram prog;
+  int rc = prepare(plan, inputs, outputs, fingerprint == 0, prog);
+  if (rc != MI355_OK) {
+    return rc;
+  }
+  State &s = state();
+  for (int i = 0; i < warmup; i++) {
+    rc = launch(prog, fingerprint == 0);
+    if (rc != MI355_OK) {
+      return rc;
+    }
+  }
+  MI355_HIP(hipEventRecord(s.ev0, s.stream));
+  for (int i = 0; i < iters; i++) {
+    rc = launch(prog, fingerprint == 0);
+    if (rc != MI355_OK) {
+      return rc;
+    }
+  }
+  MI355_HIP(hipEventRecord(s.ev1, s.stream));
+  MI355_HIP(hipEventSynchronize(s.ev1));
+  float total = 0.0f;
+  MI355_HIP(hipEventElapsedTime(&total, s.ev0, s.ev1));
+  *ms = total / iters;
+  return MI355_OK;
+}

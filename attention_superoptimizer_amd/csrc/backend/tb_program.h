@@ -1,0 +1,72 @@
+// Device program of one customized op: what the host-side lowering hands to
+// the interpreter kernels.  Built from an mi355_plan (the reference's flat-int
+// NewKernelParams bytecode) by compile_plan(): operands are resolved to tensor
+// records, every tensor gets a physical LDS placement from a liveness scan
+// (the plan's own offsets only name tensors: they are a bump allocation with no
+// reuse and would not fit the larger plans into 160 KB), loop-invariant loads
+// are hoisted, and each tensor gets the LDS layout its consumers want.
+#pragma once
+
+#include "mi355_abi.h"
+#include <cstdint>
+#include <string>
+
+namespace mi355 {
+
+constexpr int kMaxTensors = 24;
+constexpr int kTableBytes = 1024;  // fingerprint tables at the bottom of LDS
+
+enum DevOpKind : int {
+  DOP_LOAD = 1,
+  DOP_MATMUL = 2,
+  DOP_UNARY = 3,
+  DOP_BINARY = 4,
+  DOP_REDUCE = 5,
+  DOP_CONCAT = 6,
+  DOP_OUTPUT = 7,
+};
+
+// A 2-D tile in LDS: element (r, c) lives at byte offset off + 2 * (r*rs + c*cs).
+struct DevTensor {
+  int off;
+  int rows, cols;
+  int rs, cs;
+};
+
+struct DevOp {
+  int kind;
+  int sub;             // UNARY / BINARY: the TB_* operator code
+  int src0, src1, dst; // tensor ids (-1 when unused)
+  int io;              // LOAD: input slot; OUTPUT: output slot
+  int hoist;           // LOAD: loop invariant, executed at iteration 0 only
+  int vec8;            // LOAD / OUTPUT: every row segment is 16-byte aligned in global memory
+  int row_bs[3], col_bs[3], row_fs, col_fs;  // block / for-loop strides of the tile origin
+  int g_bs[3], g_fs;                         // block / for-loop strides of the batch offset
+  int d_rows, d_cols;                        // matrix shape of the device tensor
+  int red_deg, red_inner;                    // REDUCE (flat row-major rule of the reference)
+  int cat_a, cat_b, cat_inner;               // CONCAT
+};
+
+struct DevProgram {
+  int num_ops, num_tensors;
+  int forloop_range;
+  int lds_bytes;  // dynamic LDS to request (tables included)
+  int grid[3];
+  DevTensor t[kMaxTensors];
+  DevOp ops[MI355_MAX_OPERATORS];
+  void const *in[MI355_MAX_DMEM_INPUTS];
+  void *out[MI355_MAX_DMEM_OUTPUTS];
+};
+
+struct PlanExtents {
+  long long in_elems[MI355_MAX_DMEM_INPUTS];   // 1 + largest element index read
+  long long out_elems[MI355_MAX_DMEM_OUTPUTS]; // 1 + largest element index written
+};
+
+// Lowers `plan` for the uint16 interpreter (f16 == false: plain row-major tiles)
+// or the fp16 interpreter (f16 == true: padded rows, B operands k-contiguous).
+// Returns MI355_OK or an error code with `err` set.
+int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,
+                 PlanExtents &ext, std::string &err);
+
+}  // namespace mi355

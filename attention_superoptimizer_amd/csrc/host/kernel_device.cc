@@ -1,0 +1,320 @@
+// Device half of every kernel-level operator: fingerprint(), profile(), run() and
+// DTensor::has_same_fingerprint.  In the reference these live in
+// src/kernel/cuda/*.cu and call CUDA / cuBLAS directly; here they bind the C ABI of
+// mi355_abi.h and nothing else touches HIP.  fingerprint() enqueues on the backend
+// stream without a device-wide sync (the reference syncs after every operator);
+// has_same_fingerprint and profile synchronise.
+#include "mi355_abi.h"
+#include "mirage/kernel/device_memory_manager.h"
+#include "mirage/kernel/graph.h"
+#include "mirage/utils/hip_types.h"
+
+#include <cstring>
+
+namespace mirage {
+namespace kernel {
+
+using namespace mirage::type;
+
+#define MI355_CALL(expr) MIRAGE_CHECK((expr) == MI355_OK, mi355_last_error())
+
+// ---- compare (reference src/kernel/cuda/device_tensor_kernel.cu:22-53) ---------------
+bool DTensor::has_same_fingerprint(DTensor const &ref) const {
+  if (data_type != ref.data_type || layout != ref.layout || num_dims != ref.num_dims) {
+    return false;
+  }
+  for (int i = 0; i < num_dims; i++) {
+    if (dim[i] != ref.dim[i]) {
+      return false;
+    }
+  }
+  require_device("has_same_fingerprint");
+  int equal = 0;
+  MI355_CALL(mi355_fp_equal(fp_ptr, ref.fp_ptr, num_elements(), &equal));
+  return equal != 0;
+}
+
+// ---- input (reference src/kernel/cuda/input_kernel.cu:40-72) ----------------------------
+bool KNInputOp::profile(ProfileResult &profile) {
+  require_device("KNInputOp::profile");
+  DTensor const &t = output_tensors[0];
+  MIRAGE_CHECK(t.data_type == DT_FLOAT16, "only fp16 inputs are supported");
+  MI355_CALL(mi355_f16_fill_iota(t.data_ptr, t.num_elements(), t.dim[t.num_dims - 1]));
+  MI355_CALL(mi355_sync());
+  profile.run_time = 0.0f;
+  return true;
+}
+
+bool KNInputOp::fingerprint(void) {
+  require_device("KNInputOp::fingerprint");
+  DTensor const &t = output_tensors[0];
+  MI355_CALL(mi355_fp_fill_iota(t.fp_ptr, t.num_elements()));
+  return true;
+}
+
+// ---- matmul (reference src/kernel/cuda/matmul_kernel.cu:28-203) --------------------------
+static void matmul_extents(DTensor const &A, DTensor const &B, int &batch, int &m, int &n,
+                           int &k) {
+  int const nd = A.num_dims;
+  m = A.dim[nd - 2];
+  k = A.dim[nd - 1];
+  n = B.dim[nd - 1];
+  batch = 1;
+  for (int i = 0; i < nd - 2; i++) {
+    batch *= A.dim[i];
+  }
+}
+
+bool KNMatmulOp::profile(ProfileResult &result) {
+  require_device("KNMatmulOp::profile");
+  int batch, m, n, k;
+  matmul_extents(input_tensors[0], input_tensors[1], batch, m, n, k);
+  int const iters = 16;
+  MI355_CALL(mi355_f16_matmul(input_tensors[0].data_ptr, input_tensors[1].data_ptr,
+                              output_tensors[0].data_ptr, batch, m, n, k));
+  MI355_CALL(mi355_timer_start());
+  for (int i = 0; i < iters; i++) {
+    MI355_CALL(mi355_f16_matmul(input_tensors[0].data_ptr, input_tensors[1].data_ptr,
+                                output_tensors[0].data_ptr, batch, m, n, k));
+  }
+  float ms = 0.0f;
+  MI355_CALL(mi355_timer_stop(&ms));
+  result.run_time = ms / iters;
+  return true;
+}
+
+bool KNMatmulOp::fingerprint(void) {
+  require_device("KNMatmulOp::fingerprint");
+  int batch, m, n, k;
+  matmul_extents(input_tensors[0], input_tensors[1], batch, m, n, k);
+  MI355_CALL(mi355_fp_matmul(input_tensors[0].fp_ptr, input_tensors[1].fp_ptr,
+                             output_tensors[0].fp_ptr, batch, m, n, k));
+  return true;
+}
+
+// ---- element-wise unary (reference src/kernel/cuda/element_unary_kernel.cu:44-112) -------
+bool KNElementUnaryOp::profile(ProfileResult &result) {
+  require_device("KNElementUnaryOp::profile");
+  size_t const n = input_tensors[0].num_elements();
+  int const iters = ProfileResult::NUM_ITERATIONS;
+  MI355_CALL(mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
+  MI355_CALL(mi355_timer_start());
+  for (int i = 0; i < iters; i++) {
+    MI355_CALL(
+        mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
+  }
+  float ms = 0.0f;
+  MI355_CALL(mi355_timer_stop(&ms));
+  result.run_time = ms / iters;
+  return true;
+}
+
+bool KNElementUnaryOp::fingerprint(void) {
+  require_device("KNElementUnaryOp::fingerprint");
+  MI355_CALL(mi355_fp_unary(op_type, input_tensors[0].fp_ptr, output_tensors[0].fp_ptr,
+                            input_tensors[0].num_elements()));
+  return true;
+}
+
+// ---- element-wise binary (reference src/kernel/cuda/element_binary_kernel.cu:53-199) -----
+bool KNElementBinaryOp::profile(ProfileResult &result) {
+  require_device("KNElementBinaryOp::profile");
+  DTensor const &a = input_tensors[0], &b = input_tensors[1], &o = output_tensors[0];
+  int const iters = 16;
+  MI355_CALL(mi355_f16_binary(op_type, a.data_ptr, a.dim, b.data_ptr, b.dim, o.data_ptr, o.dim,
+                              o.num_dims));
+  MI355_CALL(mi355_timer_start());
+  for (int i = 0; i < iters; i++) {
+    MI355_CALL(mi355_f16_binary(op_type, a.data_ptr, a.dim, b.data_ptr, b.dim, o.data_ptr,
+                                o.dim, o.num_dims));
+  }
+  float ms = 0.0f;
+  MI355_CALL(mi355_timer_stop(&ms));
+  result.run_time = ms / iters;
+  return true;
+}
+
+bool KNElementBinaryOp::fingerprint(void) {
+  require_device("KNElementBinaryOp::fingerprint");
+  DTensor const &a = input_tensors[0], &b = input_tensors[1], &o = output_tensors[0];
+  MI355_CALL(
+      mi355_fp_binary(op_type, a.fp_ptr, a.dim, b.fp_ptr, b.dim, o.fp_ptr, o.dim, o.num_dims));
+  return true;
+}
+
+// ---- reduction (reference src/kernel/cuda/reduction_kernel.cu:45-133) --------------------
+static void reduction_strides(DTensor const &in, DTensor const &out, int dim, int &factor,
+                              int &in_stride, int &out_stride) {
+  out_stride = 1;
+  in_stride = 1;
+  for (int i = dim; i < out.num_dims; i++) {
+    out_stride *= out.dim[i];
+    in_stride *= in.dim[i];
+  }
+  factor = in.dim[dim] / out.dim[dim];
+  MIRAGE_CHECK(out_stride * factor == in_stride, "reduction strides disagree");
+}
+
+bool KNReductionOp::profile(ProfileResult &result) {
+  require_device("KNReductionOp::profile");
+  int factor, is, os;
+  reduction_strides(input_tensors[0], output_tensors[0], reduction_dim_idx, factor, is, os);
+  size_t const n = output_tensors[0].num_elements();
+  int const iters = ProfileResult::NUM_ITERATIONS;
+  MI355_CALL(mi355_f16_reduce(input_tensors[0].data_ptr, output_tensors[0].data_ptr, n, factor,
+                              is, os));
+  MI355_CALL(mi355_timer_start());
+  for (int i = 0; i < iters; i++) {
+    MI355_CALL(mi355_f16_reduce(input_tensors[0].data_ptr, output_tensors[0].data_ptr, n,
+                                factor, is, os));
+  }
+  float ms = 0.0f;
+  MI355_CALL(mi355_timer_stop(&ms));
+  result.run_time = ms / iters;
+  return true;
+}
+
+bool KNReductionOp::fingerprint(void) {
+  require_device("KNReductionOp::fingerprint");
+  int factor, is, os;
+  reduction_strides(input_tensors[0], output_tensors[0], reduction_dim_idx, factor, is, os);
+  MI355_CALL(mi355_fp_reduce(input_tensors[0].fp_ptr, output_tensors[0].fp_ptr,
+                             output_tensors[0].num_elements(), factor, is, os));
+  return true;
+}
+
+// ---- customized (reference src/kernel/cuda/customized_kernel.cu:605-678) -----------------
+struct LoweredOp {
+  mi355_plan plan;
+  void const *inputs[MI355_MAX_DMEM_INPUTS];
+  void *outputs[MI355_MAX_DMEM_OUTPUTS];
+};
+
+static LoweredOp lower(KNCustomizedOp const &op, bool fingerprint) {
+  mirage::threadblock::NewKernelParams p = op.bgraph.get_new_kernel_params(fingerprint);
+  LoweredOp l;
+  std::memset(&l, 0, sizeof(l));
+  l.plan.grid_dim[0] = op.bgraph.grid_dim.x;
+  l.plan.grid_dim[1] = op.bgraph.grid_dim.y;
+  l.plan.grid_dim[2] = op.bgraph.grid_dim.z;
+  l.plan.block_dim[0] = op.bgraph.block_dim.x;
+  l.plan.block_dim[1] = op.bgraph.block_dim.y;
+  l.plan.block_dim[2] = op.bgraph.block_dim.z;
+  l.plan.forloop_range = op.bgraph.forloop_range;
+  l.plan.reduction_dimx = op.bgraph.reduction_dimx;
+  l.plan.smem_bytes = (int)op.bgraph.smem_offset;
+  l.plan.num_operators = p.num_operators;
+  l.plan.num_parameters = p.num_parameters;
+  l.plan.num_dmem_inputs = p.num_dmem_inputs;
+  l.plan.num_dmem_outputs = p.num_dmem_outputs;
+  for (int i = 0; i < p.num_operators; i++) {
+    l.plan.operator_types[i] = p.operator_types[i];
+  }
+  std::memcpy(l.plan.parameters, p.parameters, sizeof(int) * p.num_parameters);
+  for (int i = 0; i < p.num_dmem_inputs; i++) {
+    l.inputs[i] = p.dmem_input_ptrs[i];
+  }
+  for (int i = 0; i < p.num_dmem_outputs; i++) {
+    l.outputs[i] = p.dmem_output_ptrs[i];
+  }
+  // every tile the program touches must lie inside its device tensor
+  long long in_ext[MI355_MAX_DMEM_INPUTS], out_ext[MI355_MAX_DMEM_OUTPUTS];
+  MI355_CALL(mi355_plan_extents(&l.plan, in_ext, out_ext, nullptr, nullptr));
+  int ii = 0, oo = 0;
+  for (mirage::threadblock::TBOperator *t : op.bgraph.operators) {
+    if (t->op_type == TB_INPUT_OP) {
+      auto *in = static_cast<mirage::threadblock::TBInputOp *>(t);
+      MIRAGE_CHECK(in_ext[ii] <= (long long)in->dtensor.num_elements(),
+                   "input loader would read past its tensor");
+      ii++;
+    } else if (t->op_type == TB_OUTPUT_OP) {
+      auto *out = static_cast<mirage::threadblock::TBOutputOp *>(t);
+      MIRAGE_CHECK(out_ext[oo] <= (long long)out->dtensor.num_elements(),
+                   "output saver would write past its tensor");
+      oo++;
+    }
+  }
+  return l;
+}
+
+void KNCustomizedOp::run() {
+  require_device("KNCustomizedOp::run");
+  LoweredOp l = lower(*this, false);
+  MI355_CALL(mi355_customized_run(&l.plan, l.inputs, l.outputs));
+}
+
+bool KNCustomizedOp::profile(ProfileResult &result) {
+  require_device("KNCustomizedOp::profile");
+  LoweredOp l = lower(*this, false);
+  float ms = 0.0f;
+  MI355_CALL(mi355_customized_profile(&l.plan, l.inputs, l.outputs, 0,
+                                      ProfileResult::NUM_WARPUP_ITERATIONS,
+                                      ProfileResult::NUM_ITERATIONS, &ms));
+  result.run_time = ms;
+  return true;
+}
+
+bool KNCustomizedOp::fingerprint(void) {
+  require_device("KNCustomizedOp::fingerprint");
+  LoweredOp l = lower(*this, true);
+  MI355_CALL(mi355_customized_fp(&l.plan, l.inputs, l.outputs));
+  return true;
+}
+
+}  // namespace kernel
+}  // namespace mirage
+
+// ---- one fp16 execution of any operator (extension: the reference only offers
+// profile(), which runs an operator hundreds of times) -----------------------------------
+namespace mirage {
+namespace kernel {
+
+void execute_once(KNOperator *op) {
+  require_device("execute_once");
+  using namespace mirage::type;
+  switch (op->op_type) {
+    case KN_INPUT_OP:
+      break;  // inputs hold whatever the caller wrote
+    case KN_MATMUL_OP: {
+      int batch, m, n, k;
+      matmul_extents(op->input_tensors[0], op->input_tensors[1], batch, m, n, k);
+      MI355_CALL(mi355_f16_matmul(op->input_tensors[0].data_ptr, op->input_tensors[1].data_ptr,
+                                  op->output_tensors[0].data_ptr, batch, m, n, k));
+      break;
+    }
+    case KN_EXP_OP:
+    case KN_SILU_OP:
+      MI355_CALL(mi355_f16_unary(op->op_type, op->input_tensors[0].data_ptr,
+                                 op->output_tensors[0].data_ptr,
+                                 op->input_tensors[0].num_elements()));
+      break;
+    case KN_ADD_OP:
+    case KN_MUL_OP:
+    case KN_DIV_OP: {
+      DTensor const &a = op->input_tensors[0], &b = op->input_tensors[1],
+                    &o = op->output_tensors[0];
+      MI355_CALL(mi355_f16_binary(op->op_type, a.data_ptr, a.dim, b.data_ptr, b.dim, o.data_ptr,
+                                  o.dim, o.num_dims));
+      break;
+    }
+    case KN_REDUCTION_0_OP:
+    case KN_REDUCTION_1_OP:
+    case KN_REDUCTION_2_OP: {
+      auto *r = static_cast<KNReductionOp *>(op);
+      int factor, is, os;
+      reduction_strides(op->input_tensors[0], op->output_tensors[0], r->reduction_dim_idx,
+                        factor, is, os);
+      MI355_CALL(mi355_f16_reduce(op->input_tensors[0].data_ptr, op->output_tensors[0].data_ptr,
+                                  op->output_tensors[0].num_elements(), factor, is, os));
+      break;
+    }
+    case KN_CUSTOMIZED_OP:
+      static_cast<KNCustomizedOp *>(op)->run();
+      break;
+    default:
+      MIRAGE_CHECK(false, "operator cannot be executed");
+  }
+}
+
+}  // namespace kernel
+}  // namespace mirage

@@ -1,0 +1,257 @@
+"""Python mirror of the mirage:: host API (the reference's PyGraph,
+python/mirage/_cython/core.pyx:180-236), bound over the C facade with ctypes.
+
+    g = KNGraph()
+    Q = g.new_input((2, 256, 64)); K = g.new_input((2, 64, 4096)); ...
+    out, = g.customized([Q, K, V], plan)      # plan: dict, see workloads.py
+    g.fingerprint_all(); g.operators ...
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from . import _native as N
+
+DT_FLOAT16 = 921
+DMEM_LAYOUT = {"DmemRowMajor": 100, "DmemColumnMajor": 101}
+SMEM_LAYOUT = {
+    "SmemRowMajor": 200, "SmemColumnMajor": 201,
+    "SmemRowMajorTensorOpMultiplicand_Crosswise16": 202,
+    "SmemRowMajorTensorOpMultiplicand_Crosswise32": 203,
+    "SmemRowMajorTensorOpMultiplicand_Crosswise64": 204,
+    "SmemColumnMajorTensorOpMultiplicand_Crosswise16": 205,
+    "SmemColumnMajorTensorOpMultiplicand_Crosswise32": 206,
+    "SmemColumnMajorTensorOpMultiplicand_Crosswise64": 207,
+}
+KN_OP = {"exp": 1007, "add": 1008, "mul": 1009, "div": 1010, "silu": 1011}
+TB_OP = {
+    "tb_matmul_op": 2003, "tb_exp_op": 2007, "tb_add_op": 2008, "tb_mul_op": 2009,
+    "tb_div_op": 2010, "tb_silu_op": 2012,
+    "tb_reduction_0_op": 2101, "tb_reduction_1_op": 2102, "tb_reduction_2_op": 2103,
+    "tb_reduction_0_to_dimx_op": 2104, "tb_reduction_1_to_dimx_op": 2105,
+    "tb_reduction_2_to_dimx_op": 2106,
+    "tb_concat_0_op": 2200, "tb_concat_1_op": 2201, "tb_concat_2_op": 2202,
+}
+
+
+class InfeasibleOperator(RuntimeError):
+    """create_* returned nullptr: shapes disagree or a budget is exhausted."""
+
+
+def set_smem_budget(nbytes: int) -> None:
+    """threadblock::Graph::set_smem_budget."""
+    N.runtime().mirage_set_smem_budget(int(nbytes))
+
+
+def device_ready() -> bool:
+    return bool(N.runtime().mirage_device_ready())
+
+
+class DTensor:
+    """Handle of a mirage::kernel::DTensor owned by an operator of a KNGraph."""
+
+    def __init__(self, handle: int):
+        self._h = ctypes.c_void_p(handle)
+        nd, dt, lay = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        dims = (ctypes.c_int * 4)()
+        guid = ctypes.c_longlong()
+        N.runtime().mirage_tensor_info(self._h, nd, dims, dt, lay, guid)
+        self.dims = tuple(dims[i] for i in range(nd.value))
+        self.data_type, self.layout, self.guid = dt.value, lay.value, guid.value
+
+    @property
+    def num_elements(self) -> int:
+        return int(np.prod(self.dims))
+
+    def device_ptr(self, fingerprint: bool) -> int:
+        return N.runtime().mirage_tensor_ptr(self._h, 1 if fingerprint else 0)
+
+    def write_fingerprint(self, a: np.ndarray) -> None:
+        a = np.ascontiguousarray(a, dtype=np.uint16)
+        assert a.size == self.num_elements
+        rc = N.runtime().mirage_tensor_write(self._h, 1, a.ctypes.data_as(ctypes.c_void_p), a.nbytes)
+        assert rc == 0, N.last_error()
+
+    def read_fingerprint(self) -> np.ndarray:
+        a = np.empty(self.dims, np.uint16)
+        rc = N.runtime().mirage_tensor_read(self._h, 1, a.ctypes.data_as(ctypes.c_void_p), a.nbytes)
+        assert rc == 0, N.last_error()
+        return a
+
+    def write_data(self, a: np.ndarray) -> None:
+        a = np.ascontiguousarray(a, dtype=np.float16)
+        assert a.size == self.num_elements
+        rc = N.runtime().mirage_tensor_write(self._h, 0, a.ctypes.data_as(ctypes.c_void_p), a.nbytes)
+        assert rc == 0, N.last_error()
+
+    def read_data(self) -> np.ndarray:
+        a = np.empty(self.dims, np.float16)
+        rc = N.runtime().mirage_tensor_read(self._h, 0, a.ctypes.data_as(ctypes.c_void_p), a.nbytes)
+        assert rc == 0, N.last_error()
+        return a
+
+    def has_same_fingerprint(self, other: "DTensor") -> bool:
+        return bool(N.runtime().mirage_tensor_same_fingerprint(self._h, other._h))
+
+
+def _c_plan(plan: dict) -> N.MirageCPlan:
+    p = N.MirageCPlan()
+    n_in = len(plan["input_map"])
+    assert n_in <= 4 and len(plan["ops"]) <= 16
+    for i in range(3):
+        p.grid_dim[i] = plan["grid_dim"][i]
+        p.block_dim[i] = plan.get("block_dim", [128, 1, 1])[i]
+        p.output_map[i] = plan["output_map"][i]
+    p.forloop_range = plan["forloop_range"]
+    p.reduction_dimx = plan.get("reduction_dimx", 64)
+    p.num_inputs = n_in
+    lay = plan.get("input_smem_layouts") or ["SmemRowMajor"] * n_in
+    for i in range(n_in):
+        for j in range(3):
+            p.input_map[i][j] = plan["input_map"][i][j]
+        p.forloop_dim[i] = plan["forloop_dim"][i]
+        p.input_smem_layout[i] = SMEM_LAYOUT[lay[i]] if isinstance(lay[i], str) else int(lay[i])
+    p.num_ops = len(plan["ops"])
+    for i, (name, operands) in enumerate(plan["ops"]):
+        p.op_type[i] = TB_OP[name] if isinstance(name, str) else int(name)
+        assert len(operands) <= 2
+        p.op_num_operands[i] = len(operands)
+        for j, (a, b) in enumerate(operands):
+            p.op_operands[i][j][0] = a
+            p.op_operands[i][j][1] = b
+    return p
+
+
+class KNGraph:
+    """mirage::kernel::Graph."""
+
+    def __init__(self):
+        self._rt = N.runtime()
+        self._g = ctypes.c_void_p(self._rt.mirage_graph_create())
+
+    def close(self):
+        if self._g is not None:
+            self._rt.mirage_graph_destroy(self._g)
+            self._g = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        # graphs share one LIFO arena: destruction order is the caller's business
+        pass
+
+    def _wrap(self, handle, what) -> DTensor:
+        if not handle:
+            raise InfeasibleOperator(what)
+        return DTensor(handle)
+
+    @property
+    def num_operators(self) -> int:
+        return self._rt.mirage_graph_num_operators(self._g)
+
+    def new_input(self, dims: Sequence[int], dtype: int = DT_FLOAT16,
+                  layout: str = "DmemRowMajor") -> DTensor:
+        d = (ctypes.c_int * len(dims))(*dims)
+        return self._wrap(self._rt.mirage_graph_new_input(self._g, d, len(dims), dtype,
+                                                          DMEM_LAYOUT[layout]), "new_input")
+
+    def matmul(self, A: DTensor, B: DTensor) -> DTensor:
+        return self._wrap(self._rt.mirage_graph_matmul(self._g, A._h, B._h), "matmul")
+
+    def _unary(self, name, A):
+        return self._wrap(self._rt.mirage_graph_unary(self._g, KN_OP[name], A._h), name)
+
+    def _binary(self, name, A, B):
+        return self._wrap(self._rt.mirage_graph_binary(self._g, KN_OP[name], A._h, B._h), name)
+
+    def exp(self, A): return self._unary("exp", A)
+    def silu(self, A): return self._unary("silu", A)
+    def add(self, A, B): return self._binary("add", A, B)
+    def mul(self, A, B): return self._binary("mul", A, B)
+    def div(self, A, B): return self._binary("div", A, B)
+
+    def reduction(self, A: DTensor, dim: int, size: int = 1) -> DTensor:
+        return self._wrap(self._rt.mirage_graph_reduction(self._g, A._h, dim, size), "reduction")
+
+    def customized(self, inputs: List[DTensor], plan: dict) -> List[DTensor]:
+        cp = _c_plan(plan)
+        ins = (ctypes.c_void_p * len(inputs))(*[t._h for t in inputs])
+        outs = (ctypes.c_void_p * 4)()
+        n = self._rt.mirage_graph_customized(self._g, ins, len(inputs), ctypes.byref(cp), outs, 4)
+        if n < 0:
+            raise InfeasibleOperator("customized")
+        return [DTensor(outs[i]) for i in range(n)]
+
+    def pop_operator(self) -> None:
+        assert self._rt.mirage_graph_pop_operator(self._g) == 0
+
+    # ---- per-operator device work ------------------------------------------------
+    def op_type(self, idx: int) -> int:
+        return self._rt.mirage_op_type(self._g, idx)
+
+    def outputs(self, idx: int) -> List[DTensor]:
+        n = self._rt.mirage_op_num_outputs(self._g, idx)
+        return [DTensor(self._rt.mirage_op_output(self._g, idx, j)) for j in range(n)]
+
+    def fingerprint(self, idx: int) -> None:
+        assert self._rt.mirage_op_fingerprint(self._g, idx) == 0
+
+    def fingerprint_all(self, skip_inputs: bool = False) -> None:
+        """op->fingerprint() for every operator, as the reference's verify loop does
+        (src/search/search.cc:601-603)."""
+        for i in range(self.num_operators):
+            if skip_inputs and self.op_type(i) == 1001:
+                continue
+            self.fingerprint(i)
+
+    def execute(self, idx: int) -> None:
+        assert self._rt.mirage_op_execute(self._g, idx) == 0
+
+    def execute_all(self) -> None:
+        for i in range(self.num_operators):
+            self.execute(i)
+
+    def profile(self, idx: int) -> float:
+        """Mean milliseconds per launch (reference profile() protocol)."""
+        return float(self._rt.mirage_op_profile(self._g, idx))
+
+    def lowered(self, idx: int, fingerprint: bool = True) -> N.Mi355Plan:
+        p = N.Mi355Plan()
+        rc = self._rt.mirage_op_lowered(self._g, idx, 1 if fingerprint else 0, ctypes.byref(p), None)
+        assert rc == 0
+        return p
+
+
+def build_from_spec(spec: List[dict], graph: Optional[KNGraph] = None):
+    """Builds a graph spec (see workloads.py) through the host API.
+    Returns (graph, per-operator lists of output tensors)."""
+    g = graph or KNGraph()
+    vals: List[List[DTensor]] = []
+
+    def get(ref):
+        return vals[ref[0]][ref[1]]
+
+    for op in spec:
+        k = op["op"]
+        if k == "input":
+            vals.append([g.new_input(op["dims"], DT_FLOAT16, op.get("layout", "DmemRowMajor"))])
+        elif k == "matmul":
+            vals.append([g.matmul(get(op["in"][0]), get(op["in"][1]))])
+        elif k in ("exp", "silu"):
+            vals.append([g._unary(k, get(op["in"][0]))])
+        elif k in ("add", "mul", "div"):
+            vals.append([g._binary(k, get(op["in"][0]), get(op["in"][1]))])
+        elif k == "reduction":
+            vals.append([g.reduction(get(op["in"][0]), op["dim"], op.get("size", 1))])
+        elif k == "customized":
+            vals.append(g.customized([get(r) for r in op["in"]], op["plan"]))
+        else:
+            raise ValueError(k)
+    return g, vals

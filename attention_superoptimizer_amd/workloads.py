@@ -1,0 +1,312 @@
+"""Catalogue of mugraph workloads as plain data (graph specs).
+
+A graph spec is a list of kernel-level ops; entry i describes operator i:
+  {"op": "input", "dims": [...], "layout": "DmemRowMajor" | "DmemColumnMajor"}
+  {"op": "matmul" | "exp" | "silu" | "add" | "mul" | "div", "in": [[op, ts], ...]}
+  {"op": "reduction", "in": [[op, ts]], "dim": d, "size": s}
+  {"op": "customized", "in": [[op, ts], ...], "plan": {...}}
+A plan uses the field names of mirage::threadblock::ExecutionPlan
+(reference include/mirage/threadblock/graph.h:28-53); thread-block ops are
+named as in the reference's JSON ("tb_matmul_op", ...), and each op's operand
+list holds (operator index inside the thread-block graph, tensor index) pairs,
+input loaders occupying the first slots.
+
+`REFERENCE_EXAMPLES` restates the hand-written plans of the reference's
+cpp_examples/*.cc (batch size 1): each pairs a mugraph with the un-fused kernel
+graph it must be fingerprint-equal to.  `BASELINE_CONFIGS` are the five
+benchmark configurations.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Tuple
+
+ROW, COL = "DmemRowMajor", "DmemColumnMajor"
+
+
+def _inp(dims, layout=ROW):
+    return {"op": "input", "dims": list(dims), "layout": layout}
+
+
+def _plan(grid, F, imaps, fdims, omap, ops, dimx=64, block=(128, 1, 1), layouts=None):
+    p = {
+        "grid_dim": list(grid), "block_dim": list(block), "forloop_range": F,
+        "reduction_dimx": dimx, "input_map": [list(m) for m in imaps],
+        "forloop_dim": list(fdims), "output_map": list(omap),
+        "ops": [[n, [list(x) for x in idx]] for n, idx in ops],
+    }
+    p["input_smem_layouts"] = list(layouts) if layouts else ["SmemRowMajor"] * len(imaps)
+    return p
+
+
+def attention_reference(q, k, v) -> List[dict]:
+    """matmul -> exp -> reduction(2) -> div -> matmul, the un-fused graph every
+    attention example of the reference compares against
+    (e.g. cpp_examples/group_query_attn_inc_decode.cc:16-27)."""
+    return [
+        _inp(q), _inp(k, COL), _inp(v, COL),
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "exp", "in": [[3, 0]]},
+        {"op": "reduction", "in": [[4, 0]], "dim": 2, "size": 1},
+        {"op": "div", "in": [[4, 0], [5, 0]]},
+        {"op": "matmul", "in": [[6, 0], [2, 0]]},
+    ]
+
+
+ATT_OPS = [
+    ("tb_matmul_op", [(0, 0), (1, 0)]),
+    ("tb_exp_op", [(3, 0)]),
+    ("tb_matmul_op", [(4, 0), (2, 0)]),
+    ("tb_reduction_2_op", [(4, 0)]),
+]
+COMBINE_OPS = [
+    ("tb_reduction_2_to_dimx_op", [(0, 0)]),
+    ("tb_reduction_2_op", [(1, 0)]),
+    ("tb_div_op", [(2, 0), (3, 0)]),
+]
+
+
+def attention_two_stage(q, k, v, q_imap, omap1, grid1, F, imap2, grid2) -> List[dict]:
+    """The reference's split-KV plan: op1 accumulates numerator and denominator
+    per KV block, op2 folds the partial numerators (reduction_to_dimx), the
+    partial denominators (reduction) and divides."""
+    return [
+        _inp(q), _inp(k, COL), _inp(v, COL),
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0]],
+         "plan": _plan(grid1, F, [q_imap, (0, 2, -1), (0, 1, -1)], (-1, 2, 1), omap1, ATT_OPS)},
+        {"op": "customized", "in": [[3, 0], [3, 1]],
+         "plan": _plan(grid2, 1, [imap2, imap2], (-1, -1), imap2, COMBINE_OPS)},
+    ]
+
+
+def _att(q, kv_len, q_imap, omap1, grid1, F, imap2, grid2):
+    b = q[0]
+    k, v = [b, 64, kv_len], [b, kv_len, 64]
+    return attention_two_stage(q, k, v, q_imap, omap1, grid1, F, imap2, grid2), \
+        attention_reference(q, k, v)
+
+
+def lora_example():
+    """cpp_examples/lora.cc:8-67."""
+    ref = [
+        _inp([16, 256]), _inp([256, 4096], COL), _inp([256, 16], COL), _inp([16, 4096], COL),
+        {"op": "matmul", "in": [[0, 0], [2, 0]]},
+        {"op": "matmul", "in": [[4, 0], [3, 0]]},
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "add", "in": [[6, 0], [5, 0]]},
+    ]
+    g = [
+        _inp([16, 256]), _inp([256, 4096], COL), _inp([256, 16], COL), _inp([16, 4096], COL),
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0], [3, 0]],
+         "plan": _plan((128, 1, 1), 2,
+                       [(-1, -1, -1), (1, -1, -1), (-1, -1, -1), (1, -1, -1)], (1, 0, 0, -1),
+                       (1, -1, -1),
+                       [("tb_matmul_op", [(0, 0), (2, 0)]),
+                        ("tb_concat_1_op", [(0, 0), (4, 0)]),
+                        ("tb_concat_0_op", [(1, 0), (3, 0)]),
+                        ("tb_matmul_op", [(5, 0), (6, 0)])])},
+    ]
+    return g, ref
+
+
+def mlp_example():
+    """cpp_examples/mlp.cc:8-76 (reduction_dimx = 8)."""
+    ref = [
+        _inp([16, 8192]), _inp([8192, 8], COL), _inp([8, 8192], COL),
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "exp", "in": [[3, 0]]},
+        {"op": "matmul", "in": [[4, 0], [2, 0]]},
+    ]
+    g = [
+        _inp([16, 8192]), _inp([8192, 8], COL), _inp([8, 8192], COL),
+        {"op": "customized", "in": [[0, 0], [1, 0]],
+         "plan": _plan((32, 1, 1), 1, [(1, -1, -1), (0, -1, -1)], (-1, -1), (1, -1, -1),
+                       [("tb_matmul_op", [(0, 0), (1, 0)])], dimx=8)},
+        {"op": "customized", "in": [[3, 0], [2, 0]],
+         "plan": _plan((64, 1, 1), 1, [(-1, -1, -1), (1, -1, -1)], (-1, -1), (1, -1, -1),
+                       [("tb_reduction_1_to_dimx_op", [(0, 0)]),
+                        ("tb_exp_op", [(2, 0)]),
+                        ("tb_matmul_op", [(3, 0), (1, 0)])], dimx=8)},
+    ]
+    return g, ref
+
+
+def moe_example(experts=8, hidden=4096):
+    """cpp_examples/moe.cc:8-58; `hidden` may be shrunk for CPU-sized tests
+    (it must stay divisible by 32 * 16)."""
+    ins = [_inp([experts, 8, hidden]), _inp([experts, hidden, hidden], COL),
+           _inp([experts, hidden, hidden], COL)]
+    ref = ins + [
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "exp", "in": [[3, 0]]},
+        {"op": "matmul", "in": [[4, 0], [2, 0]]},
+    ]
+    g = ins + [
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "customized", "in": [[3, 0], [2, 0]],
+         "plan": _plan((experts, 32, 1), 16, [(0, -1, -1), (0, 2, -1)], (2, 1), (0, 2, -1),
+                       [("tb_exp_op", [(0, 0)]), ("tb_matmul_op", [(2, 0), (1, 0)])])},
+    ]
+    return g, ref
+
+
+def tiled_matmul(m, n, k, grid, F, a_imap, b_imap, omap) -> Tuple[List[dict], List[dict]]:
+    """One customized op = a tiled GEMM: loader -> matmul -> accumulate -> saver
+    (plan shape of the reference's tests/threadblock/matmul.cu:163-189)."""
+    ref = [_inp([m, k]), _inp([k, n], COL), {"op": "matmul", "in": [[0, 0], [1, 0]]}]
+    g = [_inp([m, k]), _inp([k, n], COL),
+         {"op": "customized", "in": [[0, 0], [1, 0]],
+          "plan": _plan(grid, F, [a_imap, b_imap], (1, 0), omap,
+                        [("tb_matmul_op", [(0, 0), (1, 0)])])}]
+    return g, ref
+
+
+REFERENCE_EXAMPLES: Dict[str, Tuple[List[dict], List[dict]]] = {
+    # name: (mugraph, un-fused reference graph); citations = where the plan is written
+    "dnn": _att([40, 16, 64], 4096, (0, -1, -1), (0, 2, -1), (40, 8, 1), 8,
+                (0, -1, -1), (40, 1, 1)),                       # cpp_examples/dnn.cc:41-88
+    "group_query_attn_inc_decode": _att([2, 8, 64], 4096, (0, -1, -1), (0, 2, -1), (2, 16, 1), 4,
+                                        (0, -1, -1), (2, 1, 1)),  # group_query_attn_inc_decode.cc:47-101
+    "group_query_attn_spec_decode": _att([2, 256, 64], 4096, (0, -1, 1), (0, 2, 1), (2, 16, 4), 4,
+                                         (0, 1, -1), (2, 16, 1)),  # group_query_attn_spec_decode.cc:45-99
+    "group_query_attn_prefill": _att([2, 256, 64], 4096, (0, -1, 1), (0, 2, 1), (2, 16, 4), 4,
+                                     (0, 1, -1), (2, 16, 1)),      # group_query_attn_prefill.cc:45-96
+    "multi_head_attn_inc_decode": _att([32, 16, 64], 4096, (0, -1, -1), (0, 2, -1), (32, 4, 1), 4,
+                                       (0, -1, -1), (32, 1, 1)),   # multi_head_attn_inc_decode.cc:43-95
+    "multi_head_attn_spec_decode": _att([32, 16, 64], 4096, (0, -1, -1), (0, 2, -1), (32, 4, 1), 4,
+                                        (0, -1, -1), (32, 1, 1)),  # multi_head_attn_spec_decode.cc:43-87
+    "multi_head_attn_prefill": _att([32, 256, 64], 1024, (0, -1, 1), (0, 2, 1), (32, 4, 4), 4,
+                                    (0, 1, -1), (32, 8, 1)),       # multi_head_attn_prefill.cc:43-98
+    "multi_query_attn_inc_decode": _att([1, 32, 64], 4096, (0, -1, -1), (0, 2, -1), (1, 8, 1), 4,
+                                        (0, -1, -1), (1, 1, 1)),   # multi_query_attn_inc_decode.cc:45-89
+    "multi_query_attn_spec_decode": _att([1, 1024, 64], 4096, (0, -1, 1), (0, 2, 1), (1, 8, 16), 4,
+                                         (0, 1, -1), (1, 128, 1)),  # multi_query_attn_spec_decode.cc:45-100
+    "multi_query_attn_prefill": _att([1, 4096, 64], 4096, (0, -1, 1), (0, 2, 1), (1, 16, 16), 4,
+                                     (0, 1, -1), (1, 128, 1)),      # multi_query_attn_prefill.cc:45-100
+    "lora": lora_example(),
+    "mlp": mlp_example(),
+    "moe": moe_example(),
+    "tb_matmul_test": tiled_matmul(4096, 4096, 1024, (64, 64, 1), 16, (0, -1, -1), (-1, 1, -1),
+                                   (0, 1, -1)),                  # tests/threadblock/matmul.cu:163-189
+}
+
+
+# ---------------------------------------------------------------------------
+# The five benchmark configurations.
+# ---------------------------------------------------------------------------
+def config1_fused_matmul():
+    """A[64,1024] x B[1024,1024], grid (16,1,1), for-loop 16 over K."""
+    return tiled_matmul(64, 1024, 1024, (16, 1, 1), 16, (-1, -1, -1), (1, -1, -1), (1, -1, -1))
+
+
+def config2_gqa_decode():
+    """GQA incremental decode as ONE customized op: Q[2,256,64] K[2,64,4096]
+    V[2,4096,64], grid (2,16,1), for-loop 4 over the sequence,
+    matmul -> exp -> sum-reduce -> div -> matmul, output [2,256,1024]."""
+    g = [
+        _inp([2, 256, 64]), _inp([2, 64, 4096], COL), _inp([2, 4096, 64], COL),
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0]],
+         "plan": _plan((2, 16, 1), 4, [(0, -1, -1), (0, 2, -1), (0, 1, -1)], (-1, 2, 1),
+                       (0, 2, -1),
+                       [("tb_matmul_op", [(0, 0), (1, 0)]),
+                        ("tb_exp_op", [(3, 0)]),
+                        ("tb_reduction_2_op", [(4, 0)]),
+                        ("tb_div_op", [(4, 0), (5, 0)]),
+                        ("tb_matmul_op", [(6, 0), (2, 0)])])},
+    ]
+    return g, None
+
+
+def config3_mha_prefill(heads=32, seq=2048, hd=128, q_split=16, kv_split=4, F=8):
+    """MHA prefill, non-causal: op1 accumulates exp(QK^T)V and rowsum(exp(QK^T))
+    over a seq-tiled for-loop per (head, kv block, q block); op2 folds the kv
+    blocks and divides (plan shape of cpp_examples/multi_head_attn_prefill.cc:43-98).
+    Default tiling: Q tile [128,128], K/V tiles of 64 keys."""
+    q, k, v = [heads, seq, hd], [heads, hd, seq], [heads, seq, hd]
+    g = [
+        _inp(q), _inp(k, COL), _inp(v, COL),
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0]],
+         "plan": _plan((heads, kv_split, q_split), F,
+                       [(0, -1, 1), (0, 2, -1), (0, 1, -1)], (-1, 2, 1), (0, 2, 1), ATT_OPS,
+                       dimx=hd)},
+        {"op": "customized", "in": [[3, 0], [3, 1]],
+         "plan": _plan((heads, q_split, 1), 1, [(0, 1, -1), (0, 1, -1)], (-1, -1), (0, 1, -1),
+                       COMBINE_OPS, dimx=hd)},
+    ]
+    return g, attention_reference(q, k, v)
+
+
+def config4_lora(m=16, d=4096, r=16, grid=64, F=16):
+    """X[16,4096] W[4096,4096] A[4096,16] B[16,4096]: X.W + (X.A).B as ONE
+    customized op, in the reference's own plan shape (cpp_examples/lora.cc:45-67):
+    per for-loop slice i it forms [X_i | X_i.A_i] . [W_i ; B] and accumulates,
+    which equals X.W + (X.A).B by linearity."""
+    ref = [
+        _inp([m, d]), _inp([d, d], COL), _inp([d, r], COL), _inp([r, d], COL),
+        {"op": "matmul", "in": [[0, 0], [2, 0]]},
+        {"op": "matmul", "in": [[4, 0], [3, 0]]},
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "add", "in": [[6, 0], [5, 0]]},
+    ]
+    g = [
+        _inp([m, d]), _inp([d, d], COL), _inp([d, r], COL), _inp([r, d], COL),
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0], [3, 0]],
+         "plan": _plan((grid, 1, 1), F,
+                       [(-1, -1, -1), (1, -1, -1), (-1, -1, -1), (1, -1, -1)], (1, 0, 0, -1),
+                       (1, -1, -1),
+                       [("tb_matmul_op", [(0, 0), (2, 0)]),
+                        ("tb_concat_1_op", [(0, 0), (4, 0)]),
+                        ("tb_concat_0_op", [(1, 0), (3, 0)]),
+                        ("tb_matmul_op", [(5, 0), (6, 0)])])},
+    ]
+    return g, ref
+
+
+def config5_gated_mlp(m=8, d=4096, h=14336, grid1=224, F1=16, grid2=64, F2=56):
+    """SiLU(X.W1) * (X.W3) . W2 as two customized ops.  SiLU and the
+    thread-block `mul` are extensions the reference does not have.  op1 tiles
+    the hidden dim over the grid and K over the for-loop; because SiLU is not
+    linear it cannot sit inside a K-split loop, so op1 accumulates X.W1 and X.W3
+    and op2 applies silu/mul on the loaded tiles before its matmul."""
+    ref = [
+        _inp([m, d]), _inp([d, h], COL), _inp([d, h], COL), _inp([h, d], COL),
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "silu", "in": [[4, 0]]},
+        {"op": "matmul", "in": [[0, 0], [2, 0]]},
+        {"op": "mul", "in": [[5, 0], [6, 0]]},
+        {"op": "matmul", "in": [[7, 0], [3, 0]]},
+    ]
+    g = [
+        _inp([m, d]), _inp([d, h], COL), _inp([d, h], COL), _inp([h, d], COL),
+        # op1: G = X.W1, U = X.W3 (two outputs), hidden dim over the grid, K over the loop
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0]],
+         "plan": _plan((grid1, 1, 1), F1, [(-1, -1, -1), (1, -1, -1), (1, -1, -1)], (1, 0, 0),
+                       (1, -1, -1),
+                       [("tb_matmul_op", [(0, 0), (1, 0)]),
+                        ("tb_matmul_op", [(0, 0), (2, 0)])])},
+        # op2: (silu(G) * U) . W2, output columns over the grid, hidden dim over the loop
+        {"op": "customized", "in": [[4, 0], [4, 1], [3, 0]],
+         "plan": _plan((grid2, 1, 1), F2, [(-1, -1, -1), (-1, -1, -1), (1, -1, -1)], (1, 1, 0),
+                       (1, -1, -1),
+                       [("tb_silu_op", [(0, 0)]),
+                        ("tb_mul_op", [(3, 0), (1, 0)]),
+                        ("tb_matmul_op", [(4, 0), (2, 0)])])},
+    ]
+    return g, ref
+
+
+BASELINE_CONFIGS = {
+    "C1_fused_matmul": config1_fused_matmul,
+    "C2_gqa_decode": config2_gqa_decode,
+    "C3_mha_prefill": config3_mha_prefill,
+    "C4_lora": config4_lora,
+    "C5a_gated_mlp": config5_gated_mlp,
+}
+
+# fp16 input distributions per config (std of N(0, std)), keyed by input op index
+INPUT_STD = {
+    "C1_fused_matmul": {0: 0.1, 1: 0.1},
+    "C2_gqa_decode": {0: 0.125, 1: 0.125, 2: 0.125},
+    "C3_mha_prefill": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
+    "C4_lora": {0: 1.0, 1: 0.02, 2: 0.02, 3: 0.02},
+    "C5a_gated_mlp": {0: 1.0, 1: 0.02, 2: 0.02, 3: 0.02},
+}

@@ -1,0 +1,176 @@
+/*
+ * mi355_abi.h — C ABI of the MI355X (gfx950) mugraph execution / fingerprint
+ * backend.
+ *
+ * The reference (Mirage) has no C ABI for this path: its host classes call
+ * CUDA directly from .cu member functions.  This header is the boundary those
+ * member functions bind to instead; each entry point names the reference code
+ * it stands in for (paths relative to the reference root).  Plain pointers and
+ * sizes only; every function returns 0 on success and a negative code on
+ * failure, with mi355_last_error() giving the text.  All device pointers must
+ * come from the arena returned by mi355_init() (or any hipMalloc'ed memory).
+ * Work is enqueued on one backend-owned HIP stream; calls are asynchronous
+ * unless stated otherwise.  Single caller thread, like the reference.
+ */
+#ifndef MI355_ABI_H
+#define MI355_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_OK 0
+#define MI355_ERR_NO_DEVICE (-1)
+#define MI355_ERR_HIP (-2)
+#define MI355_ERR_INVALID (-3)
+#define MI355_ERR_UNSUPPORTED (-4)
+#define MI355_ERR_NOT_INITIALISED (-5)
+
+/* Limits of the reference's flat-int program
+ * (include/mirage/threadblock/serializer/kernel_params.h:25-35). */
+#define MI355_MAX_OPERATORS 16
+#define MI355_MAX_PARAMETERS 120
+#define MI355_MAX_DMEM_INPUTS 4
+#define MI355_MAX_DMEM_OUTPUTS 4
+
+/* POD mirror of NewKernelParams plus the launch shape that the reference keeps
+ * on threadblock::Graph (include/mirage/threadblock/graph.h:110-116).
+ * `parameters` is the reference's serialised per-operator bytecode verbatim
+ * (serializer/{input_loader,output_saver,matmul,element_unary,element_binary,
+ * reduction,concat}_serializer.h); `smem_bytes` is bgraph.smem_offset, the size
+ * of the thread-block graph's STensor address space. */
+typedef struct mi355_plan {
+  int grid_dim[3];
+  int block_dim[3]; /* the plan's logical block shape; a hint on this backend */
+  int forloop_range;
+  int reduction_dimx;
+  int smem_bytes;
+  int num_operators;
+  int num_parameters;
+  int num_dmem_inputs;
+  int num_dmem_outputs;
+  int operator_types[MI355_MAX_OPERATORS];
+  int parameters[MI355_MAX_PARAMETERS];
+} mi355_plan;
+
+typedef struct mi355_device_info {
+  char name[128];
+  char arch[64];
+  int compute_units;
+  int clock_mhz;
+  int memory_clock_mhz;
+  int lds_bytes_per_block;
+  size_t total_memory;
+} mi355_device_info;
+
+/* How a customized op was executed (for reporting / tests). */
+typedef struct mi355_launch_info {
+  int kernel_id;        /* MI355_KERNEL_* */
+  int workgroups;       /* physical workgroups launched */
+  int threads;          /* threads per workgroup */
+  int lds_bytes;        /* LDS actually requested */
+  int row_split;        /* workgroups cooperating on one logical thread block */
+} mi355_launch_info;
+
+#define MI355_KERNEL_FP_INTERP 1
+#define MI355_KERNEL_F16_INTERP 2
+
+/* ---- lifetime ------------------------------------------------------------
+ * Replaces DeviceMemoryManager's constructor / destructor
+ * (src/kernel/device_memory_manager.cu:26-96): one device allocation of
+ * `arena_bytes`, the exp / div lookup tables built and uploaded.  The caller
+ * keeps the bump/LIFO bookkeeping (the reference's `offset`) itself. */
+int mi355_init(size_t arena_bytes, void **arena_base);
+int mi355_shutdown(void);
+int mi355_is_initialised(void);
+char const *mi355_last_error(void);
+int mi355_get_device_info(mi355_device_info *info);
+/* Device addresses of the three uint16 tables (113, 227, 113 entries), in the
+ * reference's layout: exp[i] = 3^i mod 227; div_p[i], div_q[i] = inverse of i
+ * with [0] = [1] = 1 (device_memory_manager.cu:41-90). */
+int mi355_get_tables(void const **exp_tbl, void const **div_p, void const **div_q);
+
+/* Blocking copies and sync (the reference uses cudaMemcpy / cudaDeviceSynchronize). */
+int mi355_memcpy_h2d(void *dst, void const *src, size_t bytes);
+int mi355_memcpy_d2h(void *dst, void const *src, size_t bytes);
+int mi355_memset(void *dst, int value, size_t bytes);
+int mi355_sync(void);
+
+/* ---- fingerprint path (uint16 over Z_25651, integer only) ------------------ */
+/* init_input_fingerprint, src/kernel/cuda/input_kernel.cu:56-72: fp[i] = i % 25651 */
+int mi355_fp_fill_iota(uint16_t *fp, size_t n);
+/* seeded inputs: fp[i] = splitmix64(seed + i) % 25651 (no reference counterpart;
+ * the reference's FIXME at input_kernel.cu:59 asks for random inputs) */
+int mi355_fp_fill_uniform(uint16_t *fp, size_t n, uint64_t seed);
+/* compute_matmul_fingerprint, src/kernel/cuda/matmul_kernel.cu:145-203 */
+int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m,
+                    int n, int k);
+/* compute_elementunary_fingerprint, src/kernel/cuda/element_unary_kernel.cu:77-112;
+ * op = KN_EXP_OP (1007) or the silu extension (1011) */
+int mi355_fp_unary(int op, uint16_t const *in, uint16_t *out, size_t n);
+/* compute_elementbinary_fingerprint, src/kernel/cuda/element_binary_kernel.cu:97-199;
+ * op = KN_ADD_OP / KN_MUL_OP / KN_DIV_OP (1008 / 1009 / 1010) */
+int mi355_fp_binary(int op, uint16_t const *in1, int const *dims1, uint16_t const *in2,
+                    int const *dims2, uint16_t *out, int const *dims_out, int num_dims);
+/* compute_reduction_fingerprint, src/kernel/cuda/reduction_kernel.cu:80-133 */
+int mi355_fp_reduce(uint16_t const *in, uint16_t *out, size_t n_out, int factor,
+                    int in_stride, int out_stride);
+/* DTensor::has_same_fingerprint's element loop, src/kernel/cuda/device_tensor_kernel.cu:36-52,
+ * done on the device; writes 1/0 to *equal (blocking: 4 bytes come back, not 2 tensors) */
+int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, int *equal);
+/* KNCustomizedOp::fingerprint + compute_customizedop_fingerprint,
+ * src/kernel/cuda/customized_kernel.cu:307-603,655-678 */
+int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,
+                        void *const *outputs);
+
+/* Host-only check of a plan (no device needed): 1 + the largest element index the
+ * plan reads from each input / writes to each output, and the LDS the two
+ * interpreters would request.  Callers compare the extents with their tensors'
+ * element counts before launching; the reference relies on device asserts
+ * (include/mirage/threadblock/cuda/input_loader.h:463) instead.  Any pointer may
+ * be NULL. */
+int mi355_plan_extents(mi355_plan const *plan, long long *in_elems, long long *out_elems,
+                       int *lds_bytes_fp, int *lds_bytes_f16);
+
+/* ---- fp16 execution path --------------------------------------------------- */
+/* KNCustomizedOp::run + customized_kernel_function,
+ * src/kernel/cuda/customized_kernel.cu:39-305,605-613 */
+int mi355_customized_run(mi355_plan const *plan, void const *const *inputs,
+                         void *const *outputs);
+/* KNCustomizedOp::profile, customized_kernel.cu:615-653: `warmup` untimed then
+ * `iters` timed launches between two events on the backend stream; *ms = mean. */
+int mi355_customized_profile(mi355_plan const *plan, void const *const *inputs,
+                             void *const *outputs, int fingerprint, int warmup, int iters,
+                             float *ms);
+/* What the last mi355_customized_{fp,run,profile} call launched. */
+int mi355_last_launch(mi355_launch_info *info);
+
+/* init_input<half>, src/kernel/cuda/input_kernel.cu:29-54: x[i] = (half)(i % last_dim) */
+int mi355_f16_fill_iota(void *x, size_t n, int last_dim);
+/* seeded N(0, std) inputs rounded to fp16 (counter-based: splitmix64 + Box-Muller) */
+int mi355_f16_fill_normal(void *x, size_t n, float std, uint64_t seed);
+/* KNMatmulOp::profile's GEMM, src/kernel/cuda/matmul_kernel.cu:28-143 (row-major) */
+int mi355_f16_matmul(void const *A, void const *B, void *C, int batch, int m, int n, int k);
+/* execute_elementunary, src/kernel/cuda/element_unary_kernel.cu:30-42 */
+int mi355_f16_unary(int op, void const *in, void *out, size_t n);
+/* execute_elementbinary, src/kernel/cuda/element_binary_kernel.cu:30-51, with the
+ * fingerprint kernel's per-dim broadcast rule so both paths agree on shapes */
+int mi355_f16_binary(int op, void const *in1, int const *dims1, void const *in2,
+                     int const *dims2, void *out, int const *dims_out, int num_dims);
+/* execute_reduction, src/kernel/cuda/reduction_kernel.cu:30-42 is a stand-in in the
+ * reference; this one computes the strided sum the fingerprint kernel defines */
+int mi355_f16_reduce(void const *in, void *out, size_t n_out, int factor, int in_stride,
+                     int out_stride);
+
+/* ---- timing -----------------------------------------------------------------
+ * cudaEvent pairs of every profile() in the reference (e.g. matmul_kernel.cu:63-70). */
+int mi355_timer_start(void);
+int mi355_timer_stop(float *ms); /* blocking */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_ABI_H */
