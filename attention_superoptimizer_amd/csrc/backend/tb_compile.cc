@@ -34,8 +34,22 @@ int round_up(int x, int a) { return (x + a - 1) / a * a; }
 
 }  // namespace
 
+static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int max_lds,
+                               DevProgram &prog, PlanExtents &ext, std::string &err);
+
 int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,
                  PlanExtents &ext, std::string &err) {
+  // fp16 tiles are padded by 8 halfs per row to spread 16-byte reads over the LDS
+  // banks; a graph that only fits unpadded runs unpadded
+  int rc = compile_plan_padded(plan, f16, 8, max_lds, prog, ext, err);
+  if (rc == MI355_ERR_UNSUPPORTED && f16 && prog.lds_bytes > max_lds) {
+    rc = compile_plan_padded(plan, f16, 0, max_lds, prog, ext, err);
+  }
+  return rc;
+}
+
+static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int max_lds,
+                               DevProgram &prog, PlanExtents &ext, std::string &err) {
   memset(&prog, 0, sizeof(prog));
   memset(&ext, 0, sizeof(ext));
   if (plan.num_operators < 1 || plan.num_operators > MI355_MAX_OPERATORS ||
@@ -339,11 +353,11 @@ int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog
     } else if (ti.as_b && !ti.as_a) {
       // k-contiguous for the matrix-core B operand: column-major, padded columns
       dt.rs = 1;
-      dt.cs = ti.rows >= 8 ? round_up(ti.rows, 8) + 8 : ti.rows;
+      dt.cs = ti.rows >= 8 ? round_up(ti.rows, 8) + pad : ti.rows;
       ti.bytes = round_up(dt.cs * ti.cols * 2, 16);
     } else {
       dt.cs = 1;
-      dt.rs = ti.cols >= 8 ? round_up(ti.cols, 8) + 8 : ti.cols;
+      dt.rs = ti.cols >= 8 ? round_up(ti.cols, 8) + pad : ti.cols;
       ti.bytes = round_up(dt.rs * ti.rows * 2, 16);
     }
   }
@@ -352,6 +366,9 @@ int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog
     DevOp const &d = prog.ops[o];
     if (d.kind == DOP_OUTPUT || (d.kind == DOP_LOAD && d.hoist)) {
       T[d.dst].persistent = true;
+    }
+    if (d.kind == DOP_OUTPUT && F == 1) {
+      T[d.dst].bytes = 0;  // a single iteration stores straight from its input tile
     }
   }
   // ---- LDS placement: persistent tiles first, the rest by first fit over their
@@ -373,6 +390,33 @@ int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog
     for (int i = 0; i < prog.num_tensors; i++) {
       if (T[i].persistent || T[i].def_op != o) {
         continue;
+      }
+      // an element-wise result may overwrite an operand of the same shape and
+      // layout that dies here: every thread reads element e before writing it
+      DevOp const &d = prog.ops[o];
+      if (d.kind == DOP_BINARY && d.dst == i) {
+        int alias = -1;
+        for (int src : {d.src0, d.src1}) {
+          if (alias < 0 && src >= 0 && !T[src].persistent && T[src].last_use == o &&
+              T[src].rows == T[i].rows && T[src].cols == T[i].cols &&
+              prog.t[src].rs == prog.t[i].rs && prog.t[src].cs == prog.t[i].cs) {
+            alias = src;
+          }
+        }
+        bool done = false;
+        if (alias >= 0) {
+          for (Live &l : live) {
+            if (l.id == alias) {
+              prog.t[i].off = l.off;
+              l.id = i;
+              done = true;
+              break;
+            }
+          }
+        }
+        if (done) {
+          continue;
+        }
       }
       std::sort(live.begin(), live.end(), [](Live const &a, Live const &b) { return a.off < b.off; });
       int off = base;

@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Headline benchmark: GQA incremental decode as ONE customized op on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one launch of the customized op (config C2 of the benchmark set:
+Q[2,256,64] K[2,64,4096] V[2,4096,64] fp16, grid (2,16,1), for-loop 4,
+matmul -> exp -> sum-reduce -> div -> matmul, output [2,256,1024]) with inputs
+already resident in HBM.  Timing follows the reference's profile() protocol:
+W untimed launches, then K timed launches between two events on the stream the
+kernel runs on (reference src/kernel/cuda/customized_kernel.cu:631-648).
+
+Prints ONE JSON line.  `roofline` prices the kernel against HBM with the
+algorithmic bytes of the op (every input element read once, every output
+element written once); `cpu_baseline` times the scalar C restatement of the same
+op (oracle/, fp32 math with fp16 rounding) on the host cores, as a baseline only.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_FP16_PEAK_TFLOPS = 2500.0
+
+
+def algorithmic_bytes(spec, idx, out_dims):
+    """2 bytes x (distinct input elements + output elements) of customized op `idx`."""
+    n = 0
+    for a, _ in spec[idx]["in"]:
+        n += int(np.prod(spec[a]["dims"])) if spec[a]["op"] == "input" else 0
+    for d in out_dims:
+        n += int(np.prod(d))
+    return 2 * n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1024)
+    ap.add_argument("--warmup", type=int, default=1024)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the other benchmark configurations (printed to stderr)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU (a customized op's grid does not span "
+              "devices); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    from attention_superoptimizer_amd import _native as N
+    from attention_superoptimizer_amd import graph as G
+    from attention_superoptimizer_amd import workloads as W
+
+    if not G.device_ready():
+        print("bench.py: no MI355X backend (host-only runtime)", file=sys.stderr)
+        return 3
+    abi = N.backend()
+    G.set_smem_budget(1 << 20)
+    info = N.Mi355DeviceInfo()
+    assert abi.mi355_get_device_info(ctypes.byref(info)) == 0
+
+    def setup(name):
+        spec, _ = W.BASELINE_CONFIGS[name]()
+        g, vals = G.build_from_spec(spec)
+        for i, op in enumerate(spec):
+            if op["op"] == "input":
+                t = vals[i][0]
+                rc = abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
+                                               ctypes.c_float(W.INPUT_STD[name][i]), 0xC0FFEE00 + i)
+                assert rc == 0, N.last_error()
+        return spec, g, vals
+
+    spec, g, vals = setup("C2_gqa_decode")
+    op_idx = 3
+    # device pointers of the op's inputs / outputs, as the host API hands them over
+    ins = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(False) for a, b in spec[op_idx]["in"]])
+    outs = (ctypes.c_void_p * 4)(*[t.device_ptr(False) for t in vals[op_idx]])
+    plan = g.lowered(op_idx, fingerprint=False)
+
+    ms_ev = ctypes.c_float()
+    assert abi.mi355_sync() == 0
+    t0 = time.perf_counter()
+    rc = abi.mi355_customized_profile(ctypes.byref(plan), ins, outs, 0, args.warmup, 0 + args.steps,
+                                      ctypes.byref(ms_ev))
+    assert rc == 0, N.last_error()
+    assert abi.mi355_sync() == 0
+    t1 = time.perf_counter()
+    # wall clock over exactly K steps: a second, warm, timed-only pass
+    assert abi.mi355_sync() == 0
+    w0 = time.perf_counter()
+    rc = abi.mi355_customized_profile(ctypes.byref(plan), ins, outs, 0, 0, args.steps,
+                                      ctypes.byref(ms_ev))
+    assert rc == 0, N.last_error()
+    assert abi.mi355_sync() == 0
+    w1 = time.perf_counter()
+    ms_wall = (w1 - w0) * 1e3 / args.steps
+    ms_kernel = float(ms_ev.value)
+    launch = N.Mi355LaunchInfo()
+    abi.mi355_last_launch(ctypes.byref(launch))
+
+    out_dims = [list(t.dims) for t in vals[op_idx]]
+    abytes = algorithmic_bytes(spec, op_idx, out_dims)
+    achieved = abytes / (ms_kernel * 1e-3) / 1e9
+    flops = 2 * 2 * (2 * 256 * 64 * 4096)
+
+    result = {
+        "metric": "gqa_decode_customized_op_latency",
+        "value": round(ms_wall * 1e3, 3),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_wall, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "C2 GQA incremental decode, one customized op: Q[2,256,64] K[2,64,4096] "
+                        "V[2,4096,64] fp16 N(0,1)/8, grid (2,16,1), forloop 4, "
+                        "matmul-exp-reduce-div-matmul, out [2,256,1024]",
+            "device": info.name.decode(), "arch": info.arch.decode(),
+            "compute_units": info.compute_units, "clock_mhz": info.clock_mhz,
+            "kernel": {1: "fp_interp", 2: "f16_interp"}.get(launch.kernel_id, str(launch.kernel_id)),
+            "workgroups": launch.workgroups, "threads": launch.threads, "lds_bytes": launch.lds_bytes,
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": None,
+            "kernel_us": round(ms_kernel * 1e3, 3), "algorithmic_bytes": abytes,
+            "mfma_tflops": round(flops / (ms_kernel * 1e-3) / 1e12, 3),
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import evaluate as orc
+        host_in = [vals[a][b].read_data() for a, b in spec[op_idx]["in"]]
+        threads = min(16, os.cpu_count() or 1)
+        c0 = time.perf_counter()
+        gold = orc.customized(spec[op_idx]["plan"], host_in, f16=True, threads=threads)
+        c1 = time.perf_counter()
+        got = vals[op_idx][0].read_data()
+        err = np.abs(got.astype(np.float64) - gold[0].view(np.float16).astype(np.float64))
+        tol = 1e-3 + 1e-2 * np.abs(gold[0].view(np.float16).astype(np.float64))
+        result["cpu_baseline"] = {
+            "value": round((c1 - c0) * 1e6, 1), "unit": "us", "cores": threads, "kind": "port",
+            "sample": "1 evaluation of the same customized op by the scalar C oracle "
+                      "(fp32 math, fp16 rounding per tile), thread blocks split over host threads",
+        }
+        result["parity_vs_oracle"] = bool((err <= tol).all())
+    g.close()
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

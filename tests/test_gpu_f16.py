@@ -1,0 +1,125 @@
+"""GPU parity of the fp16 execution path against the fp16 golden of the CPU oracle.
+
+Tolerance (the bar this backend is held to): |gpu - golden| <= 1e-3 + 1e-2 * |golden|
+element-wise.  The golden is fp32 arithmetic with one fp16 rounding per materialised
+tile and fp16 for-loop accumulators (semantics of the reference's generated
+programs, src/kernel/triton_code_gen.cc:223-333)."""
+import numpy as np
+import pytest
+
+from helpers import assert_f16_close, normal_f16
+from oracle import evaluate as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph_f16(rt, spec, inputs):
+    g, vals = rt.build_from_spec(spec)
+    try:
+        for i, op in enumerate(spec):
+            if op["op"] == "input":
+                vals[i][0].write_data(inputs[i])
+            else:
+                g.execute(i)
+        return [[t.read_data() for t in v] for v in vals]
+    finally:
+        g.close()
+
+
+def _inputs(spec, stds, seed=0):
+    return {i: normal_f16(op["dims"], stds.get(i, 1.0) if isinstance(stds, dict) else stds, seed + i)
+            for i, op in enumerate(spec) if op["op"] == "input"}
+
+
+def _check(rt, spec, ins, what, threads=8):
+    got = _graph_f16(rt, spec, ins)
+    want = orc.eval_graph(spec, "f16", ins, threads=threads)
+    for i in range(len(spec)):
+        if spec[i]["op"] == "input":
+            continue
+        for j, w in enumerate(want[i]):
+            assert_f16_close(got[i][j], w, what=f"{what} op {i} ({spec[i]['op']}) out {j}")
+    return got
+
+
+def test_kernel_level_ops(rt):
+    spec = [
+        {"op": "input", "dims": [3, 70, 96]}, {"op": "input", "dims": [3, 96, 130]},
+        {"op": "input", "dims": [3, 70, 1]},
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "exp", "in": [[3, 0]]},
+        {"op": "reduction", "in": [[4, 0]], "dim": 2, "size": 1},
+        {"op": "div", "in": [[4, 0], [5, 0]]},
+        {"op": "add", "in": [[6, 0], [2, 0]]},
+        {"op": "mul", "in": [[7, 0], [7, 0]]},
+        {"op": "silu", "in": [[8, 0]]},
+        {"op": "reduction", "in": [[9, 0]], "dim": 2, "size": 65},
+        {"op": "reduction", "in": [[9, 0]], "dim": 1, "size": 1},
+    ]
+    _check(rt, spec, _inputs(spec, 0.1), "kernel ops")
+
+
+def test_config1_fused_matmul(rt):
+    from attention_superoptimizer_amd import workloads as W
+    spec, ref = W.config1_fused_matmul()
+    ins = _inputs(spec, W.INPUT_STD["C1_fused_matmul"], 10)
+    got = _check(rt, spec, ins, "C1")
+    # textbook special case: the op is a plain GEMM
+    exact = ins[0].astype(np.float64) @ ins[1].astype(np.float64)
+    assert_f16_close(got[2][0], exact, rtol=1e-2, atol=4e-3, what="C1 vs float64 GEMM")
+
+
+def test_config2_gqa_decode(rt):
+    from attention_superoptimizer_amd import workloads as W
+    spec, _ = W.config2_gqa_decode()
+    ins = _inputs(spec, W.INPUT_STD["C2_gqa_decode"], 20)
+    got = _check(rt, spec, ins, "C2")[3][0]
+    # independent statement: per (head, kv block of 256, tile of 64) softmax-without-max
+    Q, K, V = (ins[i].astype(np.float64) for i in range(3))
+    out = np.zeros((2, 256, 1024))
+    for h in range(2):
+        for blk in range(16):
+            acc = np.zeros((256, 64))
+            for it in range(4):
+                s = blk * 256 + it * 64
+                e = np.exp(Q[h] @ K[h][:, s:s + 64])
+                acc += (e / e.sum(axis=1, keepdims=True)) @ V[h][s:s + 64]
+            out[h][:, blk * 64:(blk + 1) * 64] = acc
+    assert_f16_close(got, out, rtol=1e-2, atol=2e-3, what="C2 vs float64 statement")
+
+
+def test_config3_mha_prefill_small(rt):
+    from attention_superoptimizer_amd import workloads as W
+    spec, ref = W.config3_mha_prefill(heads=2, seq=512, hd=128, q_split=4, kv_split=2, F=4)
+    ins = _inputs(spec, 128 ** -0.5, 30)
+    got = _check(rt, spec, ins, "C3 small")[-1][0]
+    # textbook special case: numerator / denominator = softmax(Q K^T) V
+    Q, K, V = (ins[i].astype(np.float64) for i in range(3))
+    s = Q @ K
+    p = np.exp(s - s.max(axis=-1, keepdims=True))
+    att = (p / p.sum(axis=-1, keepdims=True)) @ V
+    assert_f16_close(got, att, rtol=1e-2, atol=2e-3, what="C3 vs softmax attention")
+
+
+def test_config4_lora(rt):
+    from attention_superoptimizer_amd import workloads as W
+    spec, ref = W.config4_lora()
+    ins = _inputs(spec, W.INPUT_STD["C4_lora"], 40)
+    _check(rt, spec, ins, "C4")
+
+
+def test_config5_gated_mlp_small(rt):
+    from attention_superoptimizer_amd import workloads as W
+    spec, ref = W.config5_gated_mlp(m=8, d=1024, h=3584, grid1=56, F1=4, grid2=16, F2=14)
+    ins = _inputs(spec, W.INPUT_STD["C5a_gated_mlp"], 50)
+    _check(rt, spec, ins, "C5a small")
+
+
+def test_reference_examples_f16(rt):
+    """The reference's example plans, fp16, small-valued inputs so exp stays finite."""
+    from attention_superoptimizer_amd import workloads as W
+    for name in ["group_query_attn_inc_decode", "group_query_attn_spec_decode",
+                 "multi_head_attn_prefill", "lora", "mlp"]:
+        spec, ref = W.REFERENCE_EXAMPLES[name]
+        ins = _inputs(spec, 0.05, 60)
+        _check(rt, spec, ins, name)

@@ -1,0 +1,169 @@
+"""GPU parity of the fingerprint path: HIP kernels (through the C ABI and the
+host API above it) against the CPU oracle, bit for bit."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from helpers import FP_PQ, load_gqa_fixture, uniform_fp
+from oracle import evaluate as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph_fp(rt, spec, inputs=None):
+    """Builds spec through the host API, fingerprints every op, returns per-op outputs."""
+    g, vals = rt.build_from_spec(spec)
+    try:
+        for i, op in enumerate(spec):
+            if op["op"] == "input" and inputs is not None and i in inputs:
+                vals[i][0].write_fingerprint(inputs[i])
+            else:
+                g.fingerprint(i)
+        return [[t.read_fingerprint() for t in v] for v in vals]
+    finally:
+        g.close()
+
+
+@pytest.mark.parametrize("shape", [(1, 16, 64, 48), (3, 70, 33, 129), (2, 256, 64, 4096),
+                                   (1, 5, 7, 3), (1, 130, 200, 72)])
+def test_kernel_matmul_matches_oracle(rt, shape):
+    b, m, n, k = shape
+    A = uniform_fp((b, m, k), 11)
+    B = uniform_fp((b, k, n), 12)
+    spec = [{"op": "input", "dims": [b, m, k]}, {"op": "input", "dims": [b, k, n]},
+            {"op": "matmul", "in": [[0, 0], [1, 0]]}]
+    got = _graph_fp(rt, spec, {0: A, 1: B})[2][0]
+    want = orc.fp_matmul(A, B)
+    assert np.array_equal(got, want)
+
+
+def test_kernel_matmul_extreme_values(rt):
+    """All operands 25650: the largest products, k long enough to need folding."""
+    b, m, n, k = 1, 33, 65, 4100
+    A = np.full((b, m, k), FP_PQ - 1, np.uint16)
+    B = np.full((b, k, n), FP_PQ - 1, np.uint16)
+    spec = [{"op": "input", "dims": [b, m, k]}, {"op": "input", "dims": [b, k, n]},
+            {"op": "matmul", "in": [[0, 0], [1, 0]]}]
+    got = _graph_fp(rt, spec, {0: A, 1: B})[2][0]
+    assert np.all(got == (k * (FP_PQ - 1) ** 2) % FP_PQ)
+
+
+def test_kernel_elementwise_and_reduction(rt):
+    X = uniform_fp((2, 64, 96), 3)
+    Y = uniform_fp((2, 64, 1), 4)
+    Z = uniform_fp((2, 1, 96), 5)
+    spec = [
+        {"op": "input", "dims": [2, 64, 96]}, {"op": "input", "dims": [2, 64, 1]},
+        {"op": "input", "dims": [2, 1, 96]},
+        {"op": "exp", "in": [[0, 0]]},
+        {"op": "div", "in": [[3, 0], [1, 0]]},
+        {"op": "add", "in": [[4, 0], [2, 0]]},
+        {"op": "mul", "in": [[5, 0], [0, 0]]},
+        {"op": "silu", "in": [[6, 0]]},
+        {"op": "reduction", "in": [[7, 0]], "dim": 2, "size": 1},
+        {"op": "reduction", "in": [[7, 0]], "dim": 2, "size": 32},
+        {"op": "reduction", "in": [[7, 0]], "dim": 1, "size": 1},
+        {"op": "reduction", "in": [[7, 0]], "dim": 0, "size": 1},
+        {"op": "div", "in": [[1, 0], [2, 0]]},
+    ]
+    ins = {0: X, 1: Y, 2: Z}
+    got = _graph_fp(rt, spec, ins)
+    want = orc.eval_graph(spec, "fp", ins)
+    for i in range(3, len(spec)):
+        assert np.array_equal(got[i][0], want[i][0]), spec[i]
+
+
+def test_iota_inputs_and_compare(rt):
+    spec = [{"op": "input", "dims": [3, 100, 91]}, {"op": "input", "dims": [3, 100, 91]}]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        g.fingerprint_all()
+        a = vals[0][0].read_fingerprint()
+        assert np.array_equal(a.ravel(), np.arange(a.size) % FP_PQ)
+        assert vals[0][0].has_same_fingerprint(vals[1][0])
+        b = a.copy()
+        b[2, 99, 90] ^= 1
+        vals[1][0].write_fingerprint(b)
+        assert not vals[0][0].has_same_fingerprint(vals[1][0])
+    finally:
+        g.close()
+
+
+def test_uniform_fill_matches_host_generator(rt, abi):
+    spec = [{"op": "input", "dims": [5, 77, 13]}]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        t = vals[0][0]
+        assert abi.mi355_fp_fill_uniform(ctypes.c_void_p(t.device_ptr(True)), t.num_elements, 1234) == 0
+        assert np.array_equal(t.read_fingerprint(), uniform_fp(t.dims, 1234))
+    finally:
+        g.close()
+
+
+def _check_examples(rt, names, random_inputs):
+    from attention_superoptimizer_amd import workloads as W
+    for name in names:
+        spec, ref = W.REFERENCE_EXAMPLES[name]
+        if name == "moe":
+            spec, ref = W.moe_example(8, 1024)
+        if name == "tb_matmul_test":
+            spec, ref = W.tiled_matmul(512, 512, 256, (8, 8, 1), 4, (0, -1, -1), (-1, 1, -1), (0, 1, -1))
+        ins = None
+        if random_inputs:
+            ins = {i: uniform_fp(op["dims"], 100 + i) for i, op in enumerate(spec) if op["op"] == "input"}
+        got = _graph_fp(rt, spec, ins)
+        want = orc.eval_graph(spec, "fp", ins, threads=8)
+        for i, op in enumerate(spec):
+            for j, w in enumerate(want[i]):
+                assert np.array_equal(got[i][j], w), (name, i, j, op["op"])
+        got_ref = _graph_fp(rt, ref, ins)
+        assert np.array_equal(got_ref[-1][0], got[-1][0]), f"{name}: mugraph != un-fused graph on the GPU"
+
+
+def test_reference_examples_iota_inputs(rt):
+    """The reference's own integration checks (cpp_examples/*.cc: has_same_fingerprint of
+    the hand-written mugraph and the un-fused graph), inputs idx % 25651 as there."""
+    _check_examples(rt, ["group_query_attn_inc_decode", "group_query_attn_spec_decode",
+                         "multi_head_attn_inc_decode", "multi_head_attn_prefill",
+                         "multi_query_attn_inc_decode", "multi_query_attn_spec_decode",
+                         "lora", "mlp", "moe", "tb_matmul_test", "dnn"], False)
+
+
+def test_reference_examples_random_inputs(rt):
+    _check_examples(rt, ["group_query_attn_inc_decode", "group_query_attn_prefill",
+                         "multi_head_attn_spec_decode", "lora", "mlp", "moe", "tb_matmul_test"], True)
+
+
+def test_gqa_fixture_graphs(rt):
+    """Every one of the 69 graphs the reference's search verified must fingerprint-equal
+    the computation graph, on the GPU, and match the oracle bit for bit."""
+    fx = load_gqa_fixture()
+    ref_spec = fx["computation_graph"]
+    want = orc.eval_graph(ref_spec, "fp")[-1][0]
+    got_ref = _graph_fp(rt, ref_spec)[-1][0]
+    assert np.array_equal(got_ref, want)
+    for gi, spec in enumerate(fx["generated_graphs"]):
+        got = _graph_fp(rt, spec)[-1][0]
+        assert np.array_equal(got, want), f"fixture graph {gi}"
+
+
+def test_baseline_configs_fingerprint(rt):
+    from attention_superoptimizer_amd import workloads as W
+    cases = {
+        "C1": W.config1_fused_matmul(),
+        "C2": W.config2_gqa_decode(),
+        "C3s": W.config3_mha_prefill(heads=2, seq=512, hd=128, q_split=4, kv_split=2, F=4),
+        "C4": W.config4_lora(),
+        "C5s": W.config5_gated_mlp(m=8, d=1024, h=3584, grid1=56, F1=4, grid2=16, F2=14),
+    }
+    for name, (spec, ref) in cases.items():
+        ins = {i: uniform_fp(op["dims"], 7 + i) for i, op in enumerate(spec) if op["op"] == "input"}
+        got = _graph_fp(rt, spec, ins)
+        want = orc.eval_graph(spec, "fp", ins, threads=8)
+        for i in range(len(spec)):
+            for j, w in enumerate(want[i]):
+                assert np.array_equal(got[i][j], w), (name, i, j)
+        if ref is not None:
+            got_ref = _graph_fp(rt, ref, ins)
+            assert np.array_equal(got_ref[-1][0], got[-1][0]), name
