@@ -70,6 +70,8 @@ ABI = {
     "mi355_is_initialised": (_ci, []),
     "mi355_last_error": (ctypes.c_char_p, []),
     "mi355_get_device_info": (_ci, [ctypes.POINTER(Mi355DeviceInfo)]),
+    "mi355_set_option": (_ci, [_ci, _ci]),
+    "mi355_launch_floor": (_ci, [_ci, _pf]),
     "mi355_get_tables": (_ci, [_pvp, _pvp, _pvp]),
     "mi355_memcpy_h2d": (_ci, [_vp, _vp, _sz]),
     "mi355_memcpy_d2h": (_ci, [_vp, _vp, _sz]),

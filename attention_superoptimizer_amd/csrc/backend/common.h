@@ -51,6 +51,7 @@ struct State {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int max_lds = 65536;
   mi355_launch_info last_launch{};
+  int force_interpreter = 0;
 };
 
 State &state();

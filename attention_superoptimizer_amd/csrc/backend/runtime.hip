@@ -138,6 +138,39 @@ extern "C" int mi355_get_device_info(mi355_device_info *info) {
   return MI355_OK;
 }
 
+extern "C" int mi355_set_option(int option, int value) {
+  if (option == MI355_OPT_FORCE_INTERPRETER) {
+    state().force_interpreter = value;
+    return MI355_OK;
+  }
+  return fail(MI355_ERR_INVALID, "unknown option %d", option);
+}
+
+namespace mi355 {
+__global__ void empty_kernel() {}
+}  // namespace mi355
+
+extern "C" int mi355_launch_floor(int iters, float *us) {
+  MI355_REQUIRE_INIT();
+  if (iters < 1 || us == nullptr) {
+    return fail(MI355_ERR_INVALID, "bad arguments");
+  }
+  State &s = state();
+  for (int i = 0; i < 64; i++) {
+    empty_kernel<<<1, 64, 0, s.stream>>>();
+  }
+  MI355_HIP(hipEventRecord(s.ev0, s.stream));
+  for (int i = 0; i < iters; i++) {
+    empty_kernel<<<1, 64, 0, s.stream>>>();
+  }
+  MI355_HIP(hipEventRecord(s.ev1, s.stream));
+  MI355_HIP(hipEventSynchronize(s.ev1));
+  float ms = 0.0f;
+  MI355_HIP(hipEventElapsedTime(&ms, s.ev0, s.ev1));
+  *us = ms * 1000.0f / iters;
+  return MI355_OK;
+}
+
 extern "C" int mi355_get_tables(void const **exp_tbl, void const **div_p, void const **div_q) {
   MI355_REQUIRE_INIT();
   *exp_tbl = state().exp_tbl;

@@ -160,6 +160,7 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
         return MI355_ERR_INVALID;
       }
       d.vec8 = al ? 1 : 0;
+      d.galign = d.vec8;
       ext.in_elems[d.io] = max_g + max_row * d.d_cols + max_col + 1;
     } else if (t == TB_OUTPUT_OP) {
       if (!need(17) || o < out_start) {
@@ -202,6 +203,7 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
         return MI355_ERR_INVALID;
       }
       d.vec8 = al ? 1 : 0;
+      d.galign = d.vec8;
       ext.out_elems[d.io] = max_g + max_row * d.d_cols + max_col + 1;
     } else if (t == TB_MATMUL_OP) {
       if (!need(6)) {

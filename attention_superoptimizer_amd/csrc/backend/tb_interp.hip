@@ -504,9 +504,31 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   }
   PlanExtents ext;
   std::string err;
-  int rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err);
+  bool const try_fused = f16 && !state().force_interpreter;
+  // a fused kernel keeps tiles in registers, so the interpreter's LDS need does not
+  // bound it: lower without the limit first, and again with it if no fused kernel fits
+  int rc = compile_plan(*plan, f16, try_fused ? (1 << 30) : state().max_lds, prog, ext, err);
   if (rc != MI355_OK) {
     return fail(rc, "%s", err.c_str());
+  }
+  auto bind = [&]() {
+    for (int i = 0; i < plan->num_dmem_inputs; i++) {
+      prog.in[i] = inputs[i];
+    }
+    for (int i = 0; i < plan->num_dmem_outputs; i++) {
+      prog.out[i] = outputs[i];
+    }
+  };
+  if (try_fused) {
+    bind();
+    if (attention_applicable(prog)) {
+      prog.fused = 1;
+    } else {
+      rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err);
+      if (rc != MI355_OK) {
+        return fail(rc, "%s", err.c_str());
+      }
+    }
   }
   for (int i = 0; i < plan->num_dmem_inputs; i++) {
     if (inputs[i] == nullptr) {
@@ -532,6 +554,13 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
 
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
+  if (prog.fused == 1) {
+    int rc = try_launch_attention(prog);
+    if (rc == 1) {
+      return MI355_OK;
+    }
+    return rc < 0 ? rc : fail(MI355_ERR_UNSUPPORTED, "fused attention kernel declined the launch");
+  }
   dim3 grid(prog.grid[0], prog.grid[1], prog.grid[2]);
   static int fp_lds_set = 0, f16_lds_set = 0;
   int &cur = f16 ? f16_lds_set : fp_lds_set;

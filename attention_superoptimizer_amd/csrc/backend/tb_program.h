@@ -39,7 +39,8 @@ struct DevOp {
   int src0, src1, dst; // tensor ids (-1 when unused)
   int io;              // LOAD: input slot; OUTPUT: output slot
   int hoist;           // LOAD: loop invariant, executed at iteration 0 only
-  int vec8;            // LOAD / OUTPUT: every row segment is 16-byte aligned in global memory
+  int vec8;            // LOAD / OUTPUT: 16-byte accesses usable on both the global and LDS side
+  int galign;          // LOAD / OUTPUT: every row segment is 16-byte aligned in global memory
   int row_bs[3], col_bs[3], row_fs, col_fs;  // block / for-loop strides of the tile origin
   int g_bs[3], g_fs;                         // block / for-loop strides of the batch offset
   int d_rows, d_cols;                        // matrix shape of the device tensor
@@ -50,7 +51,8 @@ struct DevOp {
 struct DevProgram {
   int num_ops, num_tensors;
   int forloop_range;
-  int lds_bytes;  // dynamic LDS to request (tables included)
+  int lds_bytes;  // dynamic LDS the interpreter requests (tables included)
+  int fused;      // 1: run by the fused attention kernel instead of the interpreter
   int grid[3];
   DevTensor t[kMaxTensors];
   DevOp ops[MI355_MAX_OPERATORS];
@@ -62,6 +64,12 @@ struct PlanExtents {
   long long in_elems[MI355_MAX_DMEM_INPUTS];   // 1 + largest element index read
   long long out_elems[MI355_MAX_DMEM_OUTPUTS]; // 1 + largest element index written
 };
+
+// Fused register-resident kernels for recognised graph shapes (attn_fused.hip).
+// Returns 1 when `prog` was recognised and launched, 0 when it is not of that
+// family, a negative error code on failure.
+int try_launch_attention(DevProgram const &prog);
+bool attention_applicable(DevProgram const &prog);
 
 // Lowers `plan` for the uint16 interpreter (f16 == false: plain row-major tiles)
 // or the fp16 interpreter (f16 == true: padded rows, B operands k-contiguous).

@@ -77,6 +77,12 @@ typedef struct mi355_launch_info {
 
 #define MI355_KERNEL_FP_INTERP 1
 #define MI355_KERNEL_F16_INTERP 2
+#define MI355_KERNEL_F16_ATTENTION 3 /* fused register-resident attention family */
+
+/* Backend options (mi355_set_option).  FORCE_INTERPRETER = 1 sends every fp16
+ * customized op through the generic LDS interpreter instead of a fused kernel
+ * (both must agree with the oracle; tests run the two against each other). */
+#define MI355_OPT_FORCE_INTERPRETER 1
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor
@@ -88,6 +94,10 @@ int mi355_shutdown(void);
 int mi355_is_initialised(void);
 char const *mi355_last_error(void);
 int mi355_get_device_info(mi355_device_info *info);
+int mi355_set_option(int option, int value);
+/* Mean microseconds per launch of an empty kernel, `iters` launches back to back on
+ * the backend stream: the floor under any per-launch figure (blocking). */
+int mi355_launch_floor(int iters, float *us);
 /* Device addresses of the three uint16 tables (113, 227, 113 entries), in the
  * reference's layout: exp[i] = 3^i mod 227; div_p[i], div_q[i] = inverse of i
  * with [0] = [1] = 1 (device_memory_manager.cu:41-90). */

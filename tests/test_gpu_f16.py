@@ -13,14 +13,34 @@ from oracle import evaluate as orc
 pytestmark = pytest.mark.gpu
 
 
+KERNEL_INTERP, KERNEL_ATTENTION = 2, 3
+_last_kernels = []
+
+
+@pytest.fixture(params=["fused", "interpreter"])
+def path(request, abi):
+    """Every customized op is checked on both fp16 routes: the fused kernel its shape
+    selects (if any) and the generic LDS interpreter."""
+    assert abi.mi355_set_option(1, 1 if request.param == "interpreter" else 0) == 0
+    yield request.param
+    assert abi.mi355_set_option(1, 0) == 0
+
+
 def _graph_f16(rt, spec, inputs):
+    import ctypes
+    from attention_superoptimizer_amd import _native as N
     g, vals = rt.build_from_spec(spec)
+    del _last_kernels[:]
     try:
         for i, op in enumerate(spec):
             if op["op"] == "input":
                 vals[i][0].write_data(inputs[i])
             else:
                 g.execute(i)
+                if op["op"] == "customized":
+                    info = N.Mi355LaunchInfo()
+                    N.backend().mi355_last_launch(ctypes.byref(info))
+                    _last_kernels.append(info.kernel_id)
         return [[t.read_data() for t in v] for v in vals]
     finally:
         g.close()
@@ -69,11 +89,12 @@ def test_config1_fused_matmul(rt):
     assert_f16_close(got[2][0], exact, rtol=1e-2, atol=4e-3, what="C1 vs float64 GEMM")
 
 
-def test_config2_gqa_decode(rt):
+def test_config2_gqa_decode(rt, path):
     from attention_superoptimizer_amd import workloads as W
     spec, _ = W.config2_gqa_decode()
     ins = _inputs(spec, W.INPUT_STD["C2_gqa_decode"], 20)
     got = _check(rt, spec, ins, "C2")[3][0]
+    assert _last_kernels == [KERNEL_ATTENTION if path == "fused" else KERNEL_INTERP]
     # independent statement: per (head, kv block of 256, tile of 64) softmax-without-max
     Q, K, V = (ins[i].astype(np.float64) for i in range(3))
     out = np.zeros((2, 256, 1024))
@@ -88,11 +109,12 @@ def test_config2_gqa_decode(rt):
     assert_f16_close(got, out, rtol=1e-2, atol=2e-3, what="C2 vs float64 statement")
 
 
-def test_config3_mha_prefill_small(rt):
+def test_config3_mha_prefill_small(rt, path):
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config3_mha_prefill(heads=2, seq=512, hd=128, q_split=4, kv_split=2, F=4)
     ins = _inputs(spec, 128 ** -0.5, 30)
     got = _check(rt, spec, ins, "C3 small")[-1][0]
+    assert _last_kernels[0] == (KERNEL_ATTENTION if path == "fused" else KERNEL_INTERP)
     # textbook special case: numerator / denominator = softmax(Q K^T) V
     Q, K, V = (ins[i].astype(np.float64) for i in range(3))
     s = Q @ K
@@ -115,11 +137,26 @@ def test_config5_gated_mlp_small(rt):
     _check(rt, spec, ins, "C5a small")
 
 
-def test_reference_examples_f16(rt):
+def test_reference_examples_f16(rt, path):
     """The reference's example plans, fp16, small-valued inputs so exp stays finite."""
     from attention_superoptimizer_amd import workloads as W
     for name in ["group_query_attn_inc_decode", "group_query_attn_spec_decode",
-                 "multi_head_attn_prefill", "lora", "mlp"]:
+                 "multi_head_attn_inc_decode", "multi_head_attn_prefill",
+                 "multi_query_attn_inc_decode", "dnn", "lora", "mlp"]:
         spec, ref = W.REFERENCE_EXAMPLES[name]
         ins = _inputs(spec, 0.05, 60)
         _check(rt, spec, ins, name)
+        # query tiles with a multiple of 16 rows take the fused kernel (8-row tiles do not)
+        if path == "fused" and name in ("group_query_attn_spec_decode", "multi_head_attn_inc_decode",
+                                        "multi_head_attn_prefill", "multi_query_attn_inc_decode", "dnn"):
+            assert _last_kernels[0] == KERNEL_ATTENTION, name
+
+
+def test_gqa_fixture_graphs_f16(rt, path):
+    """A sample of the 69 recorded GQA graphs in fp16 (K tiles of 256 keys, Q tiles of 16 rows)."""
+    from helpers import load_gqa_fixture
+    fx = load_gqa_fixture()
+    for gi in (0, 17, 25, 29, 44, 68):
+        spec = fx["generated_graphs"][gi]
+        ins = _inputs(spec, 0.05, 70)
+        _check(rt, spec, ins, f"fixture graph {gi}")
