@@ -8,29 +8,38 @@
 // same fp16 rounding points as the generic interpreter, but no intermediate tile
 // ever touches LDS:
 //
-//  * one wavefront owns 16 query rows; a logical thread block's rows are split over
-//    as many workgroups as it takes to fill the chip (the plan's grid is a lower
-//    bound on parallelism, not the launch shape);
+//  * one wavefront owns 16 query rows for one for-loop iteration at a time.  A
+//    workgroup is RG row groups x IP iteration lanes: the IP wavefronts of a row
+//    group work on IP consecutive iterations at once and hand their fp16 results to
+//    the group's first wavefront, which adds them in iteration order (the order the
+//    sequential loop would use).  A logical thread block's rows are split over as
+//    many workgroups as it takes to fill the chip: the plan's grid is a lower bound
+//    on parallelism, not the launch shape;
 //  * S is produced TRANSPOSED (S^T = K^T.Q^T) with 16x16x32 fp16 MFMA, so that each
 //    lane ends up holding four consecutive keys of one query row — exactly the
 //    A-operand layout of the next MFMA.  exp, the row sum (two cross-lane adds) and
-//    the division happen on those accumulator registers; P.V consumes them directly;
+//    the normalisation happen on those accumulator registers; P.V consumes them
+//    directly;
 //  * K tiles arrive [head_dim][keys] and V tiles [keys][dv], both with the MFMA's
 //    reduction index strided in memory, so they are transposed once while being
 //    staged into LDS (four 16-byte global reads -> eight 8-byte LDS writes per 4x8
-//    patch) and every operand fetch is one contiguous LDS read;
-//  * as many for-loop iterations as fit are staged per barrier, so their loads are
-//    in flight together;
+//    patch) and every operand fetch is one contiguous LDS read.  LDS rows are
+//    unpadded; 16-byte chunks are XOR-swizzled with (row ^ row>>3) & 7, which makes
+//    both the transposing writes and the operand reads spread over all banks;
+//  * as many for-loop iterations as fit are staged per barrier, and every load of
+//    a staging step is issued before the first one is waited for;
 //  * the for-loop accumulators live in VGPRs (fp16-rounded each iteration, as the
 //    reference's generated programs do) and are written once, through LDS, as full
 //    16-byte row segments.
 #include "common.h"
 #include "tb_program.h"
+#include <cstdlib>
 
 namespace mi355 {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
@@ -59,46 +68,70 @@ __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int 
   return base + (long long)row0 * t.d_cols + col0;
 }
 
-// src: R x C tile, columns contiguous, row stride ld.  dst[c][r] with row stride LD.
-__device__ __forceinline__ void stage_transposed(_Float16 const *__restrict__ src, int ld, int R,
-                                                 int C, _Float16 *__restrict__ dst, int LD,
-                                                 int tid, int nthreads) {
-  int const cblocks = C / 8, patches = (R / 4) * cblocks;
-  for (int p = tid; p < patches; p += nthreads) {
-    int const cb = p % cblocks, rb = p / cblocks;
-    _Float16 const *s = src + (long long)(4 * rb) * ld + 8 * cb;
-    uint4v x0 = *reinterpret_cast<uint4v const *>(s);
-    uint4v x1 = *reinterpret_cast<uint4v const *>(s + ld);
-    uint4v x2 = *reinterpret_cast<uint4v const *>(s + 2 * (long long)ld);
-    uint4v x3 = *reinterpret_cast<uint4v const *>(s + 3 * (long long)ld);
-    _Float16 *d = dst + (8 * cb) * LD + 4 * rb;
+// Element offset of 16-byte chunk `chunk` of row `row` in a swizzled LDS tile whose
+// rows hold LD halfs (LD a multiple of 64).
+__device__ __forceinline__ int swz_chunk(int row, int chunk, int LD) {
+  return row * LD + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 3);
+}
+
+// A 4 x 8 patch of a tile whose columns are contiguous in memory: rows r..r+3,
+// columns c..c+7, as four 16-byte words.
+struct Patch {
+  uint4v x[4];
+};
+
+__device__ __forceinline__ Patch load_patch(_Float16 const *__restrict__ src, int ld, int cblocks,
+                                            int p) {
+  int const cb = p % cblocks, rb = p / cblocks;
+  _Float16 const *s = src + (long long)(4 * rb) * ld + 8 * cb;
+  Patch q;
+  q.x[0] = *reinterpret_cast<uint4v const *>(s);
+  q.x[1] = *reinterpret_cast<uint4v const *>(s + ld);
+  q.x[2] = *reinterpret_cast<uint4v const *>(s + 2 * (long long)ld);
+  q.x[3] = *reinterpret_cast<uint4v const *>(s + 3 * (long long)ld);
+  return q;
+}
+
+// Writes the patch transposed into a swizzled tile: dst row c + i holds source
+// rows r..r+3 as four consecutive halfs, i < 8.
+__device__ __forceinline__ void store_patch_transposed(Patch const &q, _Float16 *__restrict__ dst,
+                                                       int LD, int cblocks, int p) {
+  int const cb = p % cblocks, rb = p / cblocks;
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
-      uint2v even, odd;  // columns 2w and 2w+1, rows 0..3
-      even.x = (x0[w] & 0xffffu) | (x1[w] << 16);
-      even.y = (x2[w] & 0xffffu) | (x3[w] << 16);
-      odd.x = (x0[w] >> 16) | (x1[w] & 0xffff0000u);
-      odd.y = (x2[w] >> 16) | (x3[w] & 0xffff0000u);
-      *reinterpret_cast<uint2v *>(d + (2 * w) * LD) = even;
-      *reinterpret_cast<uint2v *>(d + (2 * w + 1) * LD) = odd;
-    }
+  for (int w = 0; w < 4; w++) {
+    uint2v even, odd;  // source columns 2w and 2w+1, rows 0..3
+    even.x = (q.x[0][w] & 0xffffu) | (q.x[1][w] << 16);
+    even.y = (q.x[2][w] & 0xffffu) | (q.x[3][w] << 16);
+    odd.x = (q.x[0][w] >> 16) | (q.x[1][w] & 0xffff0000u);
+    odd.y = (q.x[2][w] >> 16) | (q.x[3][w] & 0xffff0000u);
+    int const row = 8 * cb + 2 * w;
+    *reinterpret_cast<uint2v *>(dst + swz_chunk(row, rb >> 1, LD) + (rb & 1) * 4) = even;
+    *reinterpret_cast<uint2v *>(dst + swz_chunk(row + 1, rb >> 1, LD) + (rb & 1) * 4) = odd;
   }
 }
 
-template <int D, int NK, int DV, bool HAS_DIV>
-__global__ __launch_bounds__(256) void attn_fused_kernel(AttnParams const P) {
-  constexpr int LDK = D + 8;    // K^T rows: [key][head_dim]
-  constexpr int LDV = NK + 8;   // V^T rows: [dv][key]
+// RG row groups of 16 query rows, IP wavefronts per row group working on IP
+// consecutive for-loop iterations.
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
+__global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
+  constexpr int NW = RG * IP, NT = 64 * NW;
+  // staging work per thread and per for-loop iteration, in 4x8 patches
+  constexpr int KP = (D / 4) * (NK / 8), VP = (NK / 4) * (DV / 8);
+  constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
+  // iterations whose loads are issued together (at most 8 patches = 32 x 16 B per thread)
+  constexpr int SG = (8 / (KPT + VPT)) < 1 ? 1 : ((8 / (KPT + VPT)) > 4 ? 4 : (8 / (KPT + VPT)));
+  constexpr int SLOT_DW = DB * 2 + 1;  // one wavefront's iteration result, dwords per lane
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
-  int const tid = threadIdx.x, nthreads = blockDim.x;
-  int const lane = tid % 64, wave = tid / 64, nwaves = nthreads / 64;
+  int const tid = threadIdx.x;
+  int const lane = tid % 64, wave = tid / 64;
+  int const rg = wave / IP, ip = wave % IP;
   int const g = lane / 16, c = lane % 16;
   int const bx = blockIdx.x / P.split, slice = blockIdx.x % P.split;
   int const by = blockIdx.y, bz = blockIdx.z;
-  int const row_base = (slice * nwaves + wave) * 16;  // first query row of this wavefront
+  int const row_base = (slice * RG + rg) * 16;  // first query row of this row group
   int const F = P.forloop_range;
 
   // Q fragments (B operand of S^T): Q[row c][32kk + 8g .. +7], loop invariant
@@ -112,7 +145,9 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(AttnParams const P) {
     }
   }
 
-  _Float16 oacc[DB][4];  // O[row 4g + r][16t + c], fp16 like the reference's accumulators
+  // for-loop accumulators of the row group, held by its first wavefront:
+  // oacc[t][r] = O[row 4g + r][16t + c], fp16 like the reference's accumulators
+  _Float16 oacc[DB][4];
   _Float16 racc = (_Float16)0.0f;
 #pragma unroll
   for (int t = 0; t < DB; t++) {
@@ -122,98 +157,195 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(AttnParams const P) {
     }
   }
 
-  _Float16 *o_stage = reinterpret_cast<_Float16 *>(lds + P.stages * P.lds_stage_bytes);
+  unsigned char *const tail = lds + P.stages * P.lds_stage_bytes;
+  _Float16 *const o_stage = reinterpret_cast<_Float16 *>(tail);
+  uint32_t *const slots = reinterpret_cast<uint32_t *>(tail + RG * 16 * LDO * 2);
 
   for (int it0 = 0; it0 < F; it0 += P.stages) {
     int const n_st = (F - it0) < P.stages ? (F - it0) : P.stages;
     if (it0 > 0) {
       __syncthreads();  // previous chunk fully consumed
     }
-    for (int s = 0; s < n_st; s++) {
-      _Float16 *kt = reinterpret_cast<_Float16 *>(lds + s * P.lds_stage_bytes);
-      _Float16 *vt = kt + NK * LDK;
-      _Float16 const *kg =
-          static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it0 + s);
-      _Float16 const *vg =
-          static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it0 + s);
-      stage_transposed(kg, P.k.d_cols, D, NK, kt, LDK, tid, nthreads);   // [D][NK] -> [NK][D]
-      stage_transposed(vg, P.v.d_cols, NK, DV, vt, LDV, tid, nthreads);  // [NK][DV] -> [DV][NK]
-    }
-    __syncthreads();
-    for (int s = 0; s < n_st; s++) {
-      int const it = it0 + s;
-      _Float16 const *kt = reinterpret_cast<_Float16 const *>(lds + s * P.lds_stage_bytes);
-      _Float16 const *vt = kt + NK * LDK;
-      // ---- S^T = K^T . Q^T, exp, row sum ------------------------------------------
-      half4 e[KB];  // e[j][r] = E[row c][key 16j + 4g + r]
-      float rs = 0.0f;
+    for (int s0 = 0; s0 < n_st; s0 += SG) {
+      // phase 1: every load of up to SG iterations goes out before anything waits
+      Patch kp[SG][KPT], vp[SG][VPT];
 #pragma unroll
-      for (int j = 0; j < KB; j++) {
-        float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+      for (int u = 0; u < SG; u++) {
+        if (s0 + u < n_st) {
+          _Float16 const *kg =
+              static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it0 + s0 + u);
+          _Float16 const *vg =
+              static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it0 + s0 + u);
 #pragma unroll
-        for (int kk = 0; kk < DK; kk++) {
-          half8 a = *reinterpret_cast<half8 const *>(kt + (16 * j + c) * LDK + 32 * kk + 8 * g);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kk], acc, 0, 0, 0);
-        }
+          for (int i = 0; i < KPT; i++) {
+            int p = tid + i * NT;
+            if (KP % NT == 0 || p < KP) {
+              kp[u][i] = load_patch(kg, P.k.d_cols, NK / 8, p);
+            }
+          }
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          _Float16 s16 = static_cast<_Float16>(acc[r]);                       // S tile (fp16)
-          _Float16 e16 = static_cast<_Float16>(__expf(static_cast<float>(s16)));  // E tile
-          e[j][r] = e16;
-          rs += static_cast<float>(e16);
-        }
-      }
-      rs += __shfl_xor(rs, 16, 64);
-      rs += __shfl_xor(rs, 32, 64);
-      _Float16 const r16 = static_cast<_Float16>(rs);  // row-sum tile (fp16)
-      if (HAS_DIV) {
-        float const den = static_cast<float>(r16);
-#pragma unroll
-        for (int j = 0; j < KB; j++) {
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            e[j][r] = static_cast<_Float16>(static_cast<float>(e[j][r]) / den);
+          for (int i = 0; i < VPT; i++) {
+            int p = tid + i * NT;
+            if (VP % NT == 0 || p < VP) {
+              vp[u][i] = load_patch(vg, P.v.d_cols, DV / 8, p);
+            }
           }
         }
-      } else {
-        racc = (it == 0) ? r16
-                         : static_cast<_Float16>(static_cast<float>(racc) + static_cast<float>(r16));
       }
-      // ---- O = P . V: the accumulators of S^T are the A operand as they stand -----
+      // phase 2: transpose in registers, write K^T [NK][D] and V^T [DV][NK]
 #pragma unroll
-      for (int t = 0; t < DB; t++) {
-        float4v o = {0.0f, 0.0f, 0.0f, 0.0f};
-        _Float16 const *vrow = vt + (16 * t + c) * LDV + 4 * g;
+      for (int u = 0; u < SG; u++) {
+        if (s0 + u < n_st) {
+          _Float16 *kt = reinterpret_cast<_Float16 *>(lds + (s0 + u) * P.lds_stage_bytes);
+          _Float16 *vt = kt + NK * D;
 #pragma unroll
-        for (int jj = 0; jj < KB / 2; jj++) {
-          half4 b0 = *reinterpret_cast<half4 const *>(vrow + 32 * jj);
-          half4 b1 = *reinterpret_cast<half4 const *>(vrow + 32 * jj + 16);
-          half8 a = __builtin_shufflevector(e[2 * jj], e[2 * jj + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-          half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
-          o = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, o, 0, 0, 0);
+          for (int i = 0; i < KPT; i++) {
+            int p = tid + i * NT;
+            if (KP % NT == 0 || p < KP) {
+              store_patch_transposed(kp[u][i], kt, D, NK / 8, p);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < VPT; i++) {
+            int p = tid + i * NT;
+            if (VP % NT == 0 || p < VP) {
+              store_patch_transposed(vp[u][i], vt, NK, DV / 8, p);
+            }
+          }
         }
+      }
+    }
+    __syncthreads();
+    // rounds of IP iterations: wavefront `ip` of each row group takes iteration r0 + ip
+    for (int r0 = 0; r0 < n_st; r0 += IP) {
+      int const s = r0 + ip;
+      bool const active = s < n_st;
+      _Float16 o16[DB][4];
+      _Float16 r16 = (_Float16)0.0f;
+      if (active) {
+        _Float16 const *kt = reinterpret_cast<_Float16 const *>(lds + s * P.lds_stage_bytes);
+        _Float16 const *vt = kt + NK * D;
+        // ---- S^T = K^T . Q^T, exp, row sum ----------------------------------------
+        half4 e[KB];  // e[j][r] = E[row c][key 16j + 4g + r]
+        float rs = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          _Float16 o16 = static_cast<_Float16>(o[r]);  // O tile (fp16)
-          oacc[t][r] = (it == 0) ? o16
-                                 : static_cast<_Float16>(static_cast<float>(oacc[t][r]) +
-                                                         static_cast<float>(o16));
+        for (int j = 0; j < KB; j++) {
+          float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int kk = 0; kk < DK; kk++) {
+            half8 a = *reinterpret_cast<half8 const *>(kt + swz_chunk(16 * j + c, 4 * kk + g, D));
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kk], acc, 0, 0, 0);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            _Float16 s16 = static_cast<_Float16>(acc[r]);                           // S tile
+            _Float16 e16 = static_cast<_Float16>(__expf(static_cast<float>(s16)));  // E tile
+            e[j][r] = e16;
+            rs += static_cast<float>(e16);
+          }
         }
+        rs += __shfl_xor(rs, 16, 64);
+        rs += __shfl_xor(rs, 32, 64);
+        r16 = static_cast<_Float16>(rs);  // row-sum tile (fp16)
+        if (HAS_DIV) {
+          // one reciprocal per row, then multiplies: within an fp32 ulp of the division
+          float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
+#pragma unroll
+          for (int j = 0; j < KB; j++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              e[j][r] = static_cast<_Float16>(static_cast<float>(e[j][r]) * inv);
+            }
+          }
+        }
+        // ---- O = P . V: the accumulators of S^T are the A operand as they stand ---
+#pragma unroll
+        for (int t = 0; t < DB; t++) {
+          float4v o = {0.0f, 0.0f, 0.0f, 0.0f};
+          int const vrow = 16 * t + c;
+#pragma unroll
+          for (int jj = 0; jj < KB / 2; jj++) {
+            half4 b0 = *reinterpret_cast<half4 const *>(vt + swz_chunk(vrow, 4 * jj + (g >> 1), NK) +
+                                                        (g & 1) * 4);
+            half4 b1 = *reinterpret_cast<half4 const *>(
+                vt + swz_chunk(vrow, 4 * jj + 2 + (g >> 1), NK) + (g & 1) * 4);
+            half8 a = __builtin_shufflevector(e[2 * jj], e[2 * jj + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+            half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
+            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, o, 0, 0, 0);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            o16[t][r] = static_cast<_Float16>(o[r]);  // O tile (fp16)
+          }
+        }
+      }
+      if (IP > 1) {
+        // hand the iteration's result to the row group's first wavefront
+        if (ip > 0 && active) {
+          uint32_t *slot = slots + ((rg * (IP - 1) + (ip - 1)) * SLOT_DW) * 64 + lane;
+#pragma unroll
+          for (int t = 0; t < DB; t++) {
+            half2v lo = {o16[t][0], o16[t][1]}, hi = {o16[t][2], o16[t][3]};
+            slot[(2 * t) * 64] = __builtin_bit_cast(uint32_t, lo);
+            slot[(2 * t + 1) * 64] = __builtin_bit_cast(uint32_t, hi);
+          }
+          half2v rr = {r16, (_Float16)0.0f};
+          slot[(2 * DB) * 64] = __builtin_bit_cast(uint32_t, rr);
+        }
+        __syncthreads();
+      }
+      if (ip == 0) {
+        // add the round's results in iteration order, rounding to fp16 after each
+        // add exactly as the sequential loop would
+#pragma unroll
+        for (int q = 0; q < IP; q++) {
+          if (r0 + q < n_st) {
+            if (q > 0) {
+              uint32_t const *slot = slots + ((rg * (IP - 1) + (q - 1)) * SLOT_DW) * 64 + lane;
+#pragma unroll
+              for (int t = 0; t < DB; t++) {
+                half2v lo = __builtin_bit_cast(half2v, slot[(2 * t) * 64]);
+                half2v hi = __builtin_bit_cast(half2v, slot[(2 * t + 1) * 64]);
+                o16[t][0] = lo[0];
+                o16[t][1] = lo[1];
+                o16[t][2] = hi[0];
+                o16[t][3] = hi[1];
+              }
+              r16 = __builtin_bit_cast(half2v, slot[(2 * DB) * 64])[0];
+            }
+#pragma unroll
+            for (int t = 0; t < DB; t++) {
+#pragma unroll
+              for (int r = 0; r < 4; r++) {
+                oacc[t][r] = static_cast<_Float16>(static_cast<float>(oacc[t][r]) +
+                                                   static_cast<float>(o16[t][r]));
+              }
+            }
+            if (!HAS_DIV) {
+              racc = static_cast<_Float16>(static_cast<float>(racc) + static_cast<float>(r16));
+            }
+          }
+        }
+      }
+      if (IP > 1) {
+        __syncthreads();  // slots are free again
       }
     }
   }
 
   // ---- store: through LDS so every lane writes a 16-byte row segment ----------------
-  _Float16 *ow = o_stage + wave * 16 * LDO;
+  _Float16 *ow = o_stage + rg * 16 * LDO;
+  if (ip == 0) {
 #pragma unroll
-  for (int t = 0; t < DB; t++) {
+    for (int t = 0; t < DB; t++) {
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      ow[(4 * g + r) * LDO + 16 * t + c] = oacc[t][r];
+      for (int r = 0; r < 4; r++) {
+        ow[(4 * g + r) * LDO + 16 * t + c] = oacc[t][r];
+      }
     }
   }
   __syncthreads();
-  {
+  if (ip == 0) {
     _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
                    tile_offset(P.o, bx, by, bz, 0) + (long long)row_base * P.o.d_cols;
     constexpr int CH = DV / 8;  // 16-byte chunks per row
@@ -222,11 +354,11 @@ __global__ __launch_bounds__(256) void attn_fused_kernel(AttnParams const P) {
       *reinterpret_cast<uint4v *>(og + (long long)rr * P.o.d_cols + cc) =
           *reinterpret_cast<uint4v const *>(ow + rr * LDO + cc);
     }
-  }
-  if (!HAS_DIV && g == 0) {
-    _Float16 *rg = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
-                   tile_offset(P.r, bx, by, bz, 0);
-    rg[(long long)(row_base + c) * P.r.d_cols] = racc;
+    if (!HAS_DIV && g == 0) {
+      _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
+                      tile_offset(P.r, bx, by, bz, 0);
+      rgp[(long long)(row_base + c) * P.r.d_cols] = racc;
+    }
   }
 }
 
@@ -349,30 +481,40 @@ bool match(DevProgram const &P, Match &M) {
   return true;
 }
 
-template <int D, int NK, int DV>
-int launch_shape(AttnParams const &A, bool has_div, dim3 grid, int threads, int lds) {
-  State &s = state();
-  auto set_lds = [&](void const *fn) -> int {
-    if (lds > 65536) {
-      MI355_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    }
-    return MI355_OK;
-  };
-  if (has_div) {
-    int rc = set_lds(reinterpret_cast<void const *>(attn_fused_kernel<D, NK, DV, true>));
-    if (rc != MI355_OK) {
-      return rc;
-    }
-    attn_fused_kernel<D, NK, DV, true><<<grid, threads, lds, s.stream>>>(A);
-  } else {
-    int rc = set_lds(reinterpret_cast<void const *>(attn_fused_kernel<D, NK, DV, false>));
-    if (rc != MI355_OK) {
-      return rc;
-    }
-    attn_fused_kernel<D, NK, DV, false><<<grid, threads, lds, s.stream>>>(A);
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
+int launch_one(AttnParams const &A, dim3 grid, int lds) {
+  auto *fn = attn_fused_kernel<D, NK, DV, HAS_DIV, RG, IP>;
+  static int granted = 0;  // per instantiation
+  if (lds > 65536 && lds > granted) {
+    MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
+    granted = state().max_lds;
   }
+  fn<<<grid, 64 * RG * IP, lds, state().stream>>>(A);
   MI355_HIP(hipGetLastError());
   return 1;
+}
+
+template <int D, int NK, int DV, bool HAS_DIV>
+int launch_waves(AttnParams const &A, dim3 grid, int rg, int ip, int lds) {
+  switch (rg * 16 + ip) {
+    case 1 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 1, 1>(A, grid, lds);
+    case 1 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 1, 2>(A, grid, lds);
+    case 1 * 16 + 4: return launch_one<D, NK, DV, HAS_DIV, 1, 4>(A, grid, lds);
+    case 1 * 16 + 8: return launch_one<D, NK, DV, HAS_DIV, 1, 8>(A, grid, lds);
+    case 2 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 2, 1>(A, grid, lds);
+    case 2 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 2, 2>(A, grid, lds);
+    case 2 * 16 + 4: return launch_one<D, NK, DV, HAS_DIV, 2, 4>(A, grid, lds);
+    case 4 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 4, 1>(A, grid, lds);
+    case 4 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 4, 2>(A, grid, lds);
+    default: return 0;
+  }
+}
+
+template <int D, int NK, int DV>
+int launch_shape(AttnParams const &A, bool has_div, dim3 grid, int rg, int ip, int lds) {
+  return has_div ? launch_waves<D, NK, DV, true>(A, grid, rg, ip, lds)
+                 : launch_waves<D, NK, DV, false>(A, grid, rg, ip, lds);
 }
 
 }  // namespace
@@ -400,38 +542,54 @@ int try_launch_attention(DevProgram const &P) {
   A.o = tile_addr(P.ops[M.out_o], P.out[P.ops[M.out_o].io]);
   A.r = M.out_r >= 0 ? tile_addr(P.ops[M.out_r], P.out[P.ops[M.out_r].io]) : A.o;
   A.forloop_range = P.forloop_range;
-  // wavefronts per workgroup: as many as the tile has 16-row groups, at most 4, fewer
-  // when that is what it takes to put a workgroup on every compute unit
+
+  // Row groups per workgroup: up to 4, fewer when that is what it takes to put a
+  // workgroup on every compute unit.  Iteration lanes: whatever is left of 8
+  // wavefronts, at most the for-loop range.
   int const groups = M.m / 16;
-  int nw = groups >= 4 && groups % 4 == 0 ? 4 : (groups % 2 == 0 ? 2 : 1);
+  int rg = groups % 4 == 0 ? 4 : (groups % 2 == 0 ? 2 : 1);
   long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
-  while (nw > 1 && blocks * (groups / nw) < 256) {
-    nw /= 2;
+  while (rg > 1 && blocks * (groups / rg) < 256) {
+    rg /= 2;
   }
-  A.split = groups / nw;
+  int ip = 1;
+  while (ip * 2 * rg <= 8 && ip * 2 <= P.forloop_range) {
+    ip *= 2;
+  }
+  A.split = groups / rg;
   if ((long long)P.grid[0] * A.split > 2147483647LL) {
     return 0;
   }
-  int const stage_bytes = (M.NK * (M.D + 8) + M.DV * (M.NK + 8)) * 2;
-  int const out_bytes = nw * 16 * (M.DV + 8) * 2;
-  int stages = (96 * 1024 - out_bytes) / stage_bytes;
+  int const stage_bytes = (M.NK * M.D + M.DV * M.NK) * 2;
+  int const tail_bytes = rg * 16 * (M.DV + 8) * 2 + rg * (ip - 1) * (M.DV / 8 + 1) * 64 * 4;
+  int stages = (96 * 1024 - tail_bytes) / stage_bytes;
   stages = stages < 1 ? 1 : (stages > P.forloop_range ? P.forloop_range : stages);
+  if (stages >= ip) {
+    stages -= stages % ip;  // whole rounds per staging step
+  } else {
+    ip = 1;
+    while (ip * 2 <= stages) {
+      ip *= 2;
+    }
+    stages = ip;
+  }
   A.stages = stages;
   A.lds_stage_bytes = stage_bytes;
-  int const lds = stages * stage_bytes + out_bytes;
+  int const lds = stages * stage_bytes + tail_bytes;
   if (lds > s.max_lds) {
     return 0;
   }
   dim3 grid(P.grid[0] * A.split, P.grid[1], P.grid[2]);
+  int const nw = rg * ip;
   int rc;
   if (M.D == 64 && M.NK == 64) {
-    rc = launch_shape<64, 64, 64>(A, M.has_div, grid, nw * 64, lds);
+    rc = launch_shape<64, 64, 64>(A, M.has_div, grid, rg, ip, lds);
   } else if (M.D == 64 && M.NK == 128) {
-    rc = launch_shape<64, 128, 64>(A, M.has_div, grid, nw * 64, lds);
+    rc = launch_shape<64, 128, 64>(A, M.has_div, grid, rg, ip, lds);
   } else if (M.D == 64 && M.NK == 256) {
-    rc = launch_shape<64, 256, 64>(A, M.has_div, grid, nw * 64, lds);
+    rc = launch_shape<64, 256, 64>(A, M.has_div, grid, rg, ip, lds);
   } else {
-    rc = launch_shape<128, 64, 128>(A, M.has_div, grid, nw * 64, lds);
+    rc = launch_shape<128, 64, 128>(A, M.has_div, grid, rg, ip, lds);
   }
   if (rc == 1) {
     s.last_launch.kernel_id = MI355_KERNEL_F16_ATTENTION;
