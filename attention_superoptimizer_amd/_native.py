@@ -76,6 +76,7 @@ ABI = {
     "mi355_memcpy_h2d": (_ci, [_vp, _vp, _sz]),
     "mi355_memcpy_d2h": (_ci, [_vp, _vp, _sz]),
     "mi355_memset": (_ci, [_vp, _ci, _sz]),
+    "mi355_copy": (_ci, [_vp, _vp, _sz]),
     "mi355_sync": (_ci, []),
     "mi355_fp_fill_iota": (_ci, [_vp, _sz]),
     "mi355_fp_fill_uniform": (_ci, [_vp, _sz, _u64]),

@@ -129,8 +129,24 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
   int const lane = tid % 64, wave = tid / 64;
   int const rg = wave / IP, ip = wave % IP;
   int const g = lane / 16, c = lane % 16;
-  int const bx = blockIdx.x / P.split, slice = blockIdx.x % P.split;
-  int const by = blockIdx.y, bz = blockIdx.z;
+  // Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has
+  // its own L2.  Renumber so that each XCD gets a contiguous run of (block, slice)
+  // pairs: the slices of one logical block then share the K / V tiles in one L2
+  // instead of fetching them eight times.
+  int bx, by, bz, slice;
+  {
+    unsigned const gx = gridDim.x, gy = gridDim.y, gz = gridDim.z;
+    unsigned const total = gx * gy * gz;
+    unsigned id = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+    if (total % 8 == 0) {
+      id = (id % 8) * (total / 8) + id / 8;
+    }
+    unsigned const x = id % gx;
+    by = (id / gx) % gy;
+    bz = id / (gx * gy);
+    bx = x / P.split;
+    slice = x % P.split;
+  }
   int const row_base = (slice * RG + rg) * 16;  // first query row of this row group
   int const F = P.forloop_range;
 

@@ -148,7 +148,41 @@ extern "C" int mi355_set_option(int option, int value) {
 
 namespace mi355 {
 __global__ void empty_kernel() {}
+
+// plain device-to-device copy, 16 bytes per lane per step
+__global__ void copy_kernel(uint4 const *__restrict__ src, uint4 *__restrict__ dst, size_t n16,
+                            unsigned char const *__restrict__ src_tail,
+                            unsigned char *__restrict__ dst_tail, int tail) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n16; i += stride) {
+    dst[i] = src[i];
+  }
+  if (blockIdx.x == 0 && (int)threadIdx.x < tail) {
+    dst_tail[threadIdx.x] = src_tail[threadIdx.x];
+  }
+}
 }  // namespace mi355
+
+extern "C" int mi355_copy(void *dst, void const *src, size_t bytes) {
+  MI355_REQUIRE_INIT();
+  if (((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) != 0) {
+    return fail(MI355_ERR_INVALID, "mi355_copy needs 16-byte aligned pointers");
+  }
+  if (bytes == 0) {
+    return MI355_OK;
+  }
+  size_t n16 = bytes / 16;
+  int tail = (int)(bytes % 16);
+  size_t blocks = (n16 + 255) / 256;
+  blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+  copy_kernel<<<(unsigned)blocks, 256, 0, state().stream>>>(
+      static_cast<uint4 const *>(src), static_cast<uint4 *>(dst), n16,
+      static_cast<unsigned char const *>(src) + n16 * 16, static_cast<unsigned char *>(dst) + n16 * 16,
+      tail);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
 
 extern "C" int mi355_launch_floor(int iters, float *us) {
   MI355_REQUIRE_INIT();

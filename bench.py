@@ -49,8 +49,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=1024)
     ap.add_argument("--warmup", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extras", action="store_true",
-                    help="also time the other benchmark configurations (printed to stderr)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="run 16 plain device copies of MIB MiB and exit: the known-size "
+                         "traffic that hardware byte counters are scaled against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (a customized op's grid does not span "
@@ -68,6 +69,19 @@ def main() -> int:
     G.set_smem_budget(1 << 20)
     info = N.Mi355DeviceInfo()
     assert abi.mi355_get_device_info(ctypes.byref(info)) == 0
+
+    if args.calibrate_copy:
+        n = args.calibrate_copy << 20
+        g = G.KNGraph()
+        a = g.new_input((n // 2,))
+        b = g.new_input((n // 2,))
+        for _ in range(16):
+            assert abi.mi355_copy(ctypes.c_void_p(b.device_ptr(False)),
+                                  ctypes.c_void_p(a.device_ptr(False)), n) == 0
+        assert abi.mi355_sync() == 0
+        print(json.dumps({"copy_bytes": n, "launches": 16}))
+        g.close()
+        return 0
 
     def setup(name):
         spec, _ = W.BASELINE_CONFIGS[name]()

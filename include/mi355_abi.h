@@ -107,6 +107,9 @@ int mi355_get_tables(void const **exp_tbl, void const **div_p, void const **div_
 int mi355_memcpy_h2d(void *dst, void const *src, size_t bytes);
 int mi355_memcpy_d2h(void *dst, void const *src, size_t bytes);
 int mi355_memset(void *dst, int value, size_t bytes);
+/* Asynchronous device-to-device copy by a plain kernel (16-byte aligned pointers).
+ * Also the known-size reference that hardware byte counters are scaled against. */
+int mi355_copy(void *dst, void const *src, size_t bytes);
 int mi355_sync(void);
 
 /* ---- fingerprint path (uint16 over Z_25651, integer only) ------------------ */
