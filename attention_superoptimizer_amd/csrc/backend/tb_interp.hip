@@ -523,6 +523,8 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     bind();
     if (attention_applicable(prog)) {
       prog.fused = 1;
+    } else if (gemm_applicable(prog)) {
+      prog.fused = 2;
     } else {
       rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err);
       if (rc != MI355_OK) {
@@ -554,12 +556,12 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
 
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
-  if (prog.fused == 1) {
-    int rc = try_launch_attention(prog);
+  if (prog.fused != 0) {
+    int rc = prog.fused == 1 ? try_launch_attention(prog) : try_launch_gemm(prog);
     if (rc == 1) {
       return MI355_OK;
     }
-    return rc < 0 ? rc : fail(MI355_ERR_UNSUPPORTED, "fused attention kernel declined the launch");
+    return rc < 0 ? rc : fail(MI355_ERR_UNSUPPORTED, "fused kernel declined the launch");
   }
   dim3 grid(prog.grid[0], prog.grid[1], prog.grid[2]);
   static int fp_lds_set = 0, f16_lds_set = 0;

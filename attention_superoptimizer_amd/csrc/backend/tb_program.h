@@ -52,7 +52,7 @@ struct DevProgram {
   int num_ops, num_tensors;
   int forloop_range;
   int lds_bytes;  // dynamic LDS the interpreter requests (tables included)
-  int fused;      // 1: run by the fused attention kernel instead of the interpreter
+  int fused;      // 1 / 2: run by the fused attention / GEMM kernel instead of the interpreter
   int grid[3];
   DevTensor t[kMaxTensors];
   DevOp ops[MI355_MAX_OPERATORS];
@@ -70,6 +70,8 @@ struct PlanExtents {
 // family, a negative error code on failure.
 int try_launch_attention(DevProgram const &prog);
 bool attention_applicable(DevProgram const &prog);
+int try_launch_gemm(DevProgram const &prog);  // gemm_fused.hip, same convention
+bool gemm_applicable(DevProgram const &prog);
 
 // Lowers `plan` for the uint16 interpreter (f16 == false: plain row-major tiles)
 // or the fp16 interpreter (f16 == true: padded rows, B operands k-contiguous).

@@ -13,7 +13,7 @@ from oracle import evaluate as orc
 pytestmark = pytest.mark.gpu
 
 
-KERNEL_INTERP, KERNEL_ATTENTION = 2, 3
+KERNEL_INTERP, KERNEL_ATTENTION, KERNEL_GEMM = 2, 3, 4
 _last_kernels = []
 
 
@@ -79,11 +79,16 @@ def test_kernel_level_ops(rt):
     _check(rt, spec, _inputs(spec, 0.1), "kernel ops")
 
 
-def test_config1_fused_matmul(rt):
+def _expect(path, fused_kernel):
+    return fused_kernel if path == "fused" else KERNEL_INTERP
+
+
+def test_config1_fused_matmul(rt, path):
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config1_fused_matmul()
     ins = _inputs(spec, W.INPUT_STD["C1_fused_matmul"], 10)
     got = _check(rt, spec, ins, "C1")
+    assert _last_kernels == [_expect(path, KERNEL_GEMM)]
     # textbook special case: the op is a plain GEMM
     exact = ins[0].astype(np.float64) @ ins[1].astype(np.float64)
     assert_f16_close(got[2][0], exact, rtol=1e-2, atol=4e-3, what="C1 vs float64 GEMM")
@@ -123,18 +128,52 @@ def test_config3_mha_prefill_small(rt, path):
     assert_f16_close(got, att, rtol=1e-2, atol=2e-3, what="C3 vs softmax attention")
 
 
-def test_config4_lora(rt):
+def test_config4_lora(rt, path):
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config4_lora()
     ins = _inputs(spec, W.INPUT_STD["C4_lora"], 40)
-    _check(rt, spec, ins, "C4")
+    got = _check(rt, spec, ins, "C4")[4][0]
+    assert _last_kernels == [_expect(path, KERNEL_GEMM)]
+    # independent statement: X.W + (X.A).B in float64
+    X, Wm, A, B = (ins[i].astype(np.float64) for i in range(4))
+    assert_f16_close(got, X @ Wm + (X @ A) @ B, rtol=1e-2, atol=4e-3, what="C4 vs float64")
 
 
-def test_config5_gated_mlp_small(rt):
+def test_config5_gated_mlp_small(rt, path):
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config5_gated_mlp(m=8, d=1024, h=3584, grid1=56, F1=4, grid2=16, F2=14)
     ins = _inputs(spec, W.INPUT_STD["C5a_gated_mlp"], 50)
-    _check(rt, spec, ins, "C5a small")
+    got = _check(rt, spec, ins, "C5a small")[-1][0]
+    assert _last_kernels == [_expect(path, KERNEL_GEMM)] * 2
+    X, W1, W3, W2 = (ins[i].astype(np.float64) for i in range(4))
+    gate = X @ W1
+    exact = ((gate / (1 + np.exp(-gate))) * (X @ W3)) @ W2
+    assert_f16_close(got, exact, rtol=2e-2, atol=4e-3, what="C5a vs float64")
+
+
+def test_gemm_family_shapes(rt, path):
+    """for-loop split over workgroups (few blocks) and unsplit (many blocks), 16/32/64-row
+    tiles, exp prologue"""
+    from attention_superoptimizer_amd import workloads as W
+    cases = {
+        "unsplit": W.tiled_matmul(1024, 4096, 128, (16, 64, 1), 2, (0, -1, -1), (-1, 1, -1), (0, 1, -1)),
+        "split": W.tiled_matmul(32, 512, 2048, (8, 1, 1), 16, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),
+        "rows16": W.tiled_matmul(16, 256, 1024, (4, 1, 1), 4, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),
+        "uneven": W.tiled_matmul(64, 128, 448, (2, 1, 1), 7, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),
+    }
+    for name, (spec, ref) in cases.items():
+        ins = _inputs(spec, 0.1, 80)
+        _check(rt, spec, ins, name)
+        assert _last_kernels == [_expect(path, KERNEL_GEMM)], name
+    spec = [
+        {"op": "input", "dims": [16, 1024]}, {"op": "input", "dims": [1024, 256]},
+        {"op": "customized", "in": [[0, 0], [1, 0]], "plan": {
+            "grid_dim": [4, 1, 1], "forloop_range": 8, "input_map": [[-1, -1, -1], [1, -1, -1]],
+            "forloop_dim": [1, 0], "output_map": [1, -1, -1],
+            "ops": [["tb_exp_op", [[0, 0]]], ["tb_matmul_op", [[2, 0], [1, 0]]]]}},
+    ]
+    _check(rt, spec, _inputs(spec, 0.05, 81), "exp prologue")
+    assert _last_kernels == [_expect(path, KERNEL_GEMM)]
 
 
 def test_reference_examples_f16(rt, path):
