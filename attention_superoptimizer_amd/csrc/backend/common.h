@@ -52,12 +52,9 @@ struct State {
   int max_lds = 65536;
   mi355_launch_info last_launch{};
   int force_interpreter = 0;
-  // fused-kernel workspace: per-iteration fp16 products of split for-loops, and one
-  // arrival counter per logical block (zero between launches)
+  // fused-kernel workspace: fp16 range sums of split for-loops
   void *scratch = nullptr;
   size_t scratch_bytes = 0;
-  unsigned *tickets = nullptr;
-  int ticket_count = 0;
 };
 
 State &state();

@@ -15,10 +15,10 @@
 //    of an iteration before it waits for any, so one compute unit keeps several
 //    whole tiles in flight;
 //  * the reference's generated programs round each iteration's product to fp16 and
-//    add it to an fp16 accumulator in iteration order.  To keep exactly that rounding
-//    sequence under the split, workgroups do not pre-add: each writes its per-
-//    iteration fp16 products to a scratch slab, and the last workgroup of the block
-//    to finish (an atomic ticket) adds all of them in iteration order and stores;
+//    add it to an fp16 accumulator in iteration order.  Every workgroup does exactly
+//    that over its own range and writes its fp16 sum to a scratch slab; a second,
+//    tiny launch adds the ranges' sums of each block in range order, again rounding
+//    to fp16 after each add, and stores;
 //  * weight tiles arrive [k][n] with n contiguous while the MFMA wants k contiguous
 //    per lane, so they are transposed once while being staged into LDS (4 x 16 B
 //    global reads -> 8 x 8 B LDS writes per 4x8 patch), into unpadded rows with a
@@ -55,8 +55,7 @@ struct GemmParams {
   int M, KT;         // rows of the activation tile, k extent of one iteration
   int forloop_range;
   int ksplit;        // workgroups per logical block
-  _Float16 *scratch; // [blocks][F][NB][M][64] fp16 products (ksplit > 1)
-  unsigned *tickets; // [blocks]
+  _Float16 *scratch; // [blocks][ksplit][NB][M][64] fp16 range sums (ksplit > 1)
 };
 
 __device__ __forceinline__ long long gtile_offset(GTile const &t, int bx, int by, int bz, int it) {
@@ -260,71 +259,106 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           _Float16 p16 = static_cast<_Float16>(o[mt][r]);  // this iteration's product tile
-          if (P.ksplit == 1) {
-            acc16[b][mt][r] = static_cast<_Float16>(static_cast<float>(acc16[b][mt][r]) +
-                                                    static_cast<float>(p16));
-          } else {
-            int row = 16 * mt + 4 * g + r;
-            if (row < M) {
-              P.scratch[((((long long)block_linear * F + it) * NB + b) * M + row) * 64 + 16 * wave + c] =
-                  p16;
-            }
-          }
+          acc16[b][mt][r] = static_cast<_Float16>(static_cast<float>(acc16[b][mt][r]) +
+                                                  static_cast<float>(p16));
         }
       }
     }
   }
 
   // ---- finish ---------------------------------------------------------------------------
-  if (P.ksplit > 1) {
-    // the last workgroup of the block to arrive adds every iteration's product in order
-    // (the flag lives in the 16 bytes past the tiles: no static LDS beside the
-    // dynamic allocation)
-    unsigned *last = reinterpret_cast<unsigned *>(lb_lds + (LORA ? 64 * 16 : 0));
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-      unsigned t = atomicAdd(&P.tickets[block_linear], 1u);
-      *last = (t == (unsigned)P.ksplit - 1) ? 1u : 0u;
-      if (*last) {
-        P.tickets[block_linear] = 0;  // ready for the next launch
-      }
-    }
-    __syncthreads();
-    if (!*last) {
-      return;
-    }
-    __threadfence();
-#pragma unroll
-    for (int b = 0; b < NB; b++) {
-      GTile const &ot = b == 0 ? P.o0 : P.o1;
-      _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
-      for (int e = tid; e < M * 64; e += NT) {
-        int row = e / 64, col = e % 64;
-        _Float16 acc = (_Float16)0.0f;
-        _Float16 const *sp = P.scratch + (((long long)block_linear * F) * NB + b) * M * 64 + e;
-        for (int it = 0; it < F; it++) {
-          acc = static_cast<_Float16>(static_cast<float>(acc) +
-                                      static_cast<float>(__builtin_nontemporal_load(sp + (long long)it * NB * M * 64)));
-        }
-        og[(long long)row * ot.d_cols + col] = acc;
-      }
-    }
-    return;
-  }
+  // The workgroup's fp16 sums go through LDS so that they leave as 16-byte row
+  // segments: straight to the output when the for-loop was not split, else to this
+  // range's slab of the scratch buffer.
+  constexpr int LDT = 64 + 8;
+  _Float16 *t_lds = reinterpret_cast<_Float16 *>(lds);  // the tiles are dead by now
+  __syncthreads();
 #pragma unroll
   for (int b = 0; b < NB; b++) {
-    GTile const &ot = b == 0 ? P.o0 : P.o1;
-    _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        int row = 16 * mt + 4 * g + r;
-        if (row < M) {
-          og[(long long)row * ot.d_cols + 16 * wave + c] = acc16[b][mt][r];
+        t_lds[(b * 16 * MT + 16 * mt + 4 * g + r) * LDT + 16 * wave + c] = acc16[b][mt][r];
+      }
+    }
+  }
+  __syncthreads();
+  int const chunks = M * 8;  // 16-byte chunks of one [M][64] tile
+  if (P.ksplit == 1) {
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      GTile const &ot = b == 0 ? P.o0 : P.o1;
+      _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
+      for (int e = tid; e < chunks; e += NT) {
+        int row = e / 8, col = (e % 8) * 8;
+        *reinterpret_cast<uint4v *>(og + (long long)row * ot.d_cols + col) =
+            *reinterpret_cast<uint4v const *>(t_lds + (b * 16 * MT + row) * LDT + col);
+      }
+    }
+    return;
+  }
+  // scratch layout: [block][range][NB][M][64]
+  long long const slab = (long long)NB * M * 64;
+  _Float16 *mine = P.scratch + ((long long)block_linear * P.ksplit + ks) * slab;
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
+    for (int e = tid; e < chunks; e += NT) {
+      int row = e / 8, col = (e % 8) * 8;
+      *reinterpret_cast<uint4v *>(mine + (long long)b * M * 64 + row * 64 + col) =
+          *reinterpret_cast<uint4v const *>(t_lds + (b * 16 * MT + row) * LDT + col);
+    }
+  }
+}
+
+// Second pass of a split for-loop: adds the ranges' fp16 sums of every logical block
+// in range order (fp16 rounding after each add, as the sequential loop would) and
+// stores the block's output tile.  A separate launch rather than a last-arriver
+// fix-up: the kernel boundary makes the slabs visible without device-scope fences,
+// which on this part write back and invalidate a whole L2 each time.
+template <int NB>
+__global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
+  int const tid = threadIdx.x, M = P.M;
+  int const bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  int const block_linear = bx + gridDim.x * (by + gridDim.y * bz);
+  long long const slab = (long long)NB * M * 64;
+  _Float16 const *all = P.scratch + (long long)block_linear * P.ksplit * slab;
+  int const chunks = M * 8;
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
+    GTile const &ot = b == 0 ? P.o0 : P.o1;
+    _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
+    for (int e = tid; e < chunks; e += 256) {
+      int row = e / 8, col = (e % 8) * 8;
+      _Float16 const *sp = all + (long long)b * M * 64 + row * 64 + col;
+      half8 acc;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        acc[j] = (_Float16)0.0f;
+      }
+      int q = 0;
+      for (; q + 4 <= P.ksplit; q += 4) {  // four loads in flight, adds in order
+        half8 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          v[u] = *reinterpret_cast<half8 const *>(sp + (long long)(q + u) * slab);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            acc[j] = static_cast<_Float16>(static_cast<float>(acc[j]) + static_cast<float>(v[u][j]));
+          }
         }
       }
+      for (; q < P.ksplit; q++) {
+        half8 v = *reinterpret_cast<half8 const *>(sp + (long long)q * slab);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          acc[j] = static_cast<_Float16>(static_cast<float>(acc[j]) + static_cast<float>(v[j]));
+        }
+      }
+      *reinterpret_cast<half8 *>(og + (long long)row * ot.d_cols + col) = acc;
     }
   }
 }
@@ -459,6 +493,11 @@ bool gmatch(DevProgram const &P, GMatch &G) {
   if (G.lora && (ta.cols != P.t[P.ops[G.la].dst].rows)) {
     return false;
   }
+  for (int i : {G.o0, G.o1}) {
+    if (i >= 0 && (!P.ops[i].galign || (reinterpret_cast<uintptr_t>(P.out[P.ops[i].io]) & 15) != 0)) {
+      return false;
+    }
+  }
   return true;
 }
 
@@ -516,14 +555,15 @@ int try_launch_gemm(DevProgram const &P) {
   ksplit = ksplit < 1 ? 1 : (ksplit > P.forloop_range ? P.forloop_range : ksplit);
   int per = (P.forloop_range + ksplit - 1) / ksplit;
   ksplit = (P.forloop_range + per - 1) / per;  // no empty ranges
-  long long const scratch_elems = blocks * P.forloop_range * G.nb * G.M * 64;
-  if (ksplit > 1 && (scratch_elems * 2 > (long long)s.scratch_bytes || blocks > (long long)s.ticket_count)) {
+  long long const scratch_elems = blocks * ksplit * G.nb * G.M * 64;
+  if (ksplit > 1 && (scratch_elems * 2 > (long long)s.scratch_bytes)) {
     ksplit = 1;
   }
   A.ksplit = ksplit;
   A.scratch = static_cast<_Float16 *>(s.scratch);
-  A.tickets = s.tickets;
-  int const lds = (16 * mt * G.KT + G.nb * 64 * G.KT + (G.lora ? 16 * G.KT + 64 * 16 : 0)) * 2 + 16;
+  int const tile_lds = (16 * mt * G.KT + G.nb * 64 * G.KT + (G.lora ? 16 * G.KT + 64 * 16 : 0)) * 2;
+  int const out_lds = G.nb * 16 * mt * (64 + 8) * 2;
+  int const lds = tile_lds > out_lds ? tile_lds : out_lds;
   if (lds > s.max_lds || (long long)P.grid[0] * ksplit > 2147483647LL) {
     return 0;
   }
@@ -542,6 +582,15 @@ int try_launch_gemm(DevProgram const &P) {
   MI355_GEMM_CASE(1, 1, PRO_SILU_MUL, false)
   MI355_GEMM_CASE(1, 1, PRO_NONE, true)
 #undef MI355_GEMM_CASE
+  if (rc == 1 && ksplit > 1) {
+    dim3 cgrid(P.grid[0], P.grid[1], P.grid[2]);
+    if (G.nb == 1) {
+      gemm_combine_kernel<1><<<cgrid, 256, 0, s.stream>>>(A);
+    } else {
+      gemm_combine_kernel<2><<<cgrid, 256, 0, s.stream>>>(A);
+    }
+    MI355_HIP(hipGetLastError());
+  }
   if (rc == 1) {
     s.last_launch.kernel_id = MI355_KERNEL_F16_GEMM;
     s.last_launch.workgroups = grid.x * grid.y * grid.z;

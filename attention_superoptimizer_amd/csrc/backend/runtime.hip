@@ -97,10 +97,7 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
   MI355_HIP(hipEventCreate(&s.ev0));
   MI355_HIP(hipEventCreate(&s.ev1));
   s.scratch_bytes = (size_t)64 << 20;
-  s.ticket_count = 65536;
   MI355_HIP(hipMalloc(&s.scratch, s.scratch_bytes));
-  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.tickets), s.ticket_count * sizeof(unsigned)));
-  MI355_HIP(hipMemset(s.tickets, 0, s.ticket_count * sizeof(unsigned)));
   s.ready = true;
   if (arena_base != nullptr) {
     *arena_base = s.arena;
@@ -121,7 +118,6 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipFree(s.flag));
   MI355_HIP(hipHostFree(s.flag_host));
   MI355_HIP(hipFree(s.scratch));
-  MI355_HIP(hipFree(s.tickets));
   MI355_HIP(hipStreamDestroy(s.stream));
   s = State{};
   return MI355_OK;
