@@ -57,6 +57,7 @@ struct AttnParams {
   int split;   // workgroups per logical thread block
   int stages;  // for-loop iterations staged per barrier
   int lds_stage_bytes;
+  int perm[3];  // grid dims from fastest to slowest varying in the renumbered workgroup id
 };
 
 __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int by, int bz,
@@ -110,6 +111,40 @@ __device__ __forceinline__ void store_patch_transposed(Patch const &q, _Float16 
   }
 }
 
+// Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has its
+// own L2.  Renumber so that each XCD gets a contiguous run of ids, and unpack the id
+// with the grid dims the K / V tiles do NOT depend on varying fastest (row slices
+// first): workgroups that read the same K / V tiles then sit on one XCD and share
+// one L2 instead of fetching the tiles once per XCD.
+__device__ __forceinline__ void decode_block(AttnParams const &P, int &bx, int &by, int &bz,
+                                             int &slice) {
+  unsigned const ext[3] = {gridDim.x, gridDim.y, gridDim.z};
+  unsigned const total = ext[0] * ext[1] * ext[2];
+  unsigned id = blockIdx.x + ext[0] * (blockIdx.y + ext[1] * blockIdx.z);
+  if (total % 8 == 0) {
+    id = (id % 8) * (total / 8) + id / 8;
+  }
+  unsigned coord[3] = {0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < 3; i++) {
+    int const d = P.perm[i];
+    unsigned const e = d == 0 ? ext[0] : (d == 1 ? ext[1] : ext[2]);
+    unsigned const v = id % e;
+    id /= e;
+    if (d == 0) {
+      coord[0] = v;
+    } else if (d == 1) {
+      coord[1] = v;
+    } else {
+      coord[2] = v;
+    }
+  }
+  bx = coord[0] / P.split;
+  slice = coord[0] % P.split;
+  by = coord[1];
+  bz = coord[2];
+}
+
 // RG row groups of 16 query rows, IP wavefronts per row group working on IP
 // consecutive for-loop iterations.
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
@@ -129,24 +164,8 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
   int const lane = tid % 64, wave = tid / 64;
   int const rg = wave / IP, ip = wave % IP;
   int const g = lane / 16, c = lane % 16;
-  // Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has
-  // its own L2.  Renumber so that each XCD gets a contiguous run of (block, slice)
-  // pairs: the slices of one logical block then share the K / V tiles in one L2
-  // instead of fetching them eight times.
   int bx, by, bz, slice;
-  {
-    unsigned const gx = gridDim.x, gy = gridDim.y, gz = gridDim.z;
-    unsigned const total = gx * gy * gz;
-    unsigned id = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
-    if (total % 8 == 0) {
-      id = (id % 8) * (total / 8) + id / 8;
-    }
-    unsigned const x = id % gx;
-    by = (id / gx) % gy;
-    bz = id / (gx * gy);
-    bx = x / P.split;
-    slice = x % P.split;
-  }
+  decode_block(P, bx, by, bz, slice);
   int const row_base = (slice * RG + rg) * 16;  // first query row of this row group
   int const F = P.forloop_range;
 
@@ -378,6 +397,226 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
   }
 }
 
+// Throughput variant for large problems: every wavefront owns RPW row groups of 16
+// query rows (so each K^T / V^T operand fetched from LDS feeds RPW MFMAs) and walks
+// all for-loop iterations itself; K / V tiles are double-buffered in LDS and the
+// global loads of iteration i+1 are in flight (in registers) while iteration i is on
+// the matrix cores.  One barrier per iteration.
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW>
+__global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P) {
+  constexpr int LDO = DV + 8;
+  constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
+  constexpr int NT = 64 * RG;
+  constexpr int KP = (D / 4) * (NK / 8), VP = (NK / 4) * (DV / 8);
+  constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
+  constexpr int STAGE = (NK * D + DV * NK);  // halfs per buffer
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  _Float16 *const buf = reinterpret_cast<_Float16 *>(lds);
+
+  int const tid = threadIdx.x;
+  int const lane = tid % 64, wave = tid / 64;
+  int const g = lane / 16, c = lane % 16;
+  int bx, by, bz, slice;
+  decode_block(P, bx, by, bz, slice);
+  int const row_base = (slice * RG + wave) * RPW * 16;
+  int const F = P.forloop_range;
+
+  half8 qf[RPW][DK];
+  {
+    _Float16 const *q = static_cast<_Float16 const *>(P.q.ptr) + tile_offset(P.q, bx, by, bz, 0) +
+                        (long long)(row_base + c) * P.q.d_cols + 8 * g;
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+      for (int kk = 0; kk < DK; kk++) {
+        qf[rp][kk] = *reinterpret_cast<half8 const *>(q + (long long)(16 * rp) * P.q.d_cols + 32 * kk);
+      }
+    }
+  }
+  _Float16 oacc[RPW][DB][4];
+  _Float16 racc[RPW];
+#pragma unroll
+  for (int rp = 0; rp < RPW; rp++) {
+    racc[rp] = (_Float16)0.0f;
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        oacc[rp][t][r] = (_Float16)0.0f;
+      }
+    }
+  }
+
+  Patch kp[KPT], vp[VPT];
+  auto issue_loads = [&](int it) {
+    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
+#pragma unroll
+    for (int i = 0; i < KPT; i++) {
+      int p = tid + i * NT;
+      if (KP % NT == 0 || p < KP) {
+        kp[i] = load_patch(kg, P.k.d_cols, NK / 8, p);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+      int p = tid + i * NT;
+      if (VP % NT == 0 || p < VP) {
+        vp[i] = load_patch(vg, P.v.d_cols, DV / 8, p);
+      }
+    }
+  };
+  auto write_tiles = [&](int b) {
+    _Float16 *kt = buf + b * STAGE;
+    _Float16 *vt = kt + NK * D;
+#pragma unroll
+    for (int i = 0; i < KPT; i++) {
+      int p = tid + i * NT;
+      if (KP % NT == 0 || p < KP) {
+        store_patch_transposed(kp[i], kt, D, NK / 8, p);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+      int p = tid + i * NT;
+      if (VP % NT == 0 || p < VP) {
+        store_patch_transposed(vp[i], vt, NK, DV / 8, p);
+      }
+    }
+  };
+
+  issue_loads(0);
+  write_tiles(0);
+  __syncthreads();
+  for (int it = 0; it < F; it++) {
+    if (it + 1 < F) {
+      issue_loads(it + 1);  // in flight while this iteration computes
+    }
+    _Float16 const *kt = buf + (it & 1) * STAGE;
+    _Float16 const *vt = kt + NK * D;
+    // ---- S^T = K^T . Q^T for RPW row groups, exp, row sums ------------------------
+    half4 e[RPW][KB];
+    float rs[RPW];
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+      rs[rp] = 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < KB; j++) {
+      float4v acc[RPW];
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        acc[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+#pragma unroll
+      for (int kk = 0; kk < DK; kk++) {
+        half8 a = *reinterpret_cast<half8 const *>(kt + swz_chunk(16 * j + c, 4 * kk + g, D));
+#pragma unroll
+        for (int rp = 0; rp < RPW; rp++) {
+          acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rp][kk], acc[rp], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          _Float16 s16 = static_cast<_Float16>(acc[rp][r]);
+          _Float16 e16 = static_cast<_Float16>(__expf(static_cast<float>(s16)));
+          e[rp][j][r] = e16;
+          rs[rp] += static_cast<float>(e16);
+        }
+      }
+    }
+    _Float16 r16[RPW];
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+      rs[rp] += __shfl_xor(rs[rp], 16, 64);
+      rs[rp] += __shfl_xor(rs[rp], 32, 64);
+      r16[rp] = static_cast<_Float16>(rs[rp]);
+      if (HAS_DIV) {
+        float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16[rp]));
+#pragma unroll
+        for (int j = 0; j < KB; j++) {
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            e[rp][j][r] = static_cast<_Float16>(static_cast<float>(e[rp][j][r]) * inv);
+          }
+        }
+      } else {
+        racc[rp] = static_cast<_Float16>(static_cast<float>(racc[rp]) + static_cast<float>(r16[rp]));
+      }
+    }
+    // ---- O = P . V ------------------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+      float4v o[RPW];
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+      int const vrow = 16 * t + c;
+#pragma unroll
+      for (int jj = 0; jj < KB / 2; jj++) {
+        half4 b0 = *reinterpret_cast<half4 const *>(vt + swz_chunk(vrow, 4 * jj + (g >> 1), NK) +
+                                                    (g & 1) * 4);
+        half4 b1 = *reinterpret_cast<half4 const *>(vt + swz_chunk(vrow, 4 * jj + 2 + (g >> 1), NK) +
+                                                    (g & 1) * 4);
+        half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int rp = 0; rp < RPW; rp++) {
+          half8 a = __builtin_shufflevector(e[rp][2 * jj], e[rp][2 * jj + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+          o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, o[rp], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          _Float16 o16 = static_cast<_Float16>(o[rp][r]);
+          oacc[rp][t][r] = static_cast<_Float16>(static_cast<float>(oacc[rp][t][r]) +
+                                                 static_cast<float>(o16));
+        }
+      }
+    }
+    if (it + 1 < F) {
+      write_tiles((it + 1) & 1);  // that buffer was last read in iteration it - 1
+    }
+    __syncthreads();
+  }
+
+  // ---- store through LDS (the tile buffers are dead) ----------------------------------
+  _Float16 *ow = buf + wave * RPW * 16 * LDO;
+#pragma unroll
+  for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        ow[(16 * rp + 4 * g + r) * LDO + 16 * t + c] = oacc[rp][t][r];
+      }
+    }
+  }
+  __syncthreads();
+  {
+    _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
+                   tile_offset(P.o, bx, by, bz, 0) + (long long)row_base * P.o.d_cols;
+    constexpr int CH = DV / 8;
+    for (int e2 = lane; e2 < RPW * 16 * CH; e2 += 64) {
+      int rr = e2 / CH, cc = (e2 % CH) * 8;
+      *reinterpret_cast<uint4v *>(og + (long long)rr * P.o.d_cols + cc) =
+          *reinterpret_cast<uint4v const *>(ow + rr * LDO + cc);
+    }
+    if (!HAS_DIV && g == 0) {
+      _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
+                      tile_offset(P.r, bx, by, bz, 0);
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        rgp[(long long)(row_base + 16 * rp + c) * P.r.d_cols] = racc[rp];
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // host: recognise the family in a lowered program and launch
 // ---------------------------------------------------------------------------------------
@@ -533,6 +772,28 @@ int launch_shape(AttnParams const &A, bool has_div, dim3 grid, int rg, int ip, i
                  : launch_waves<D, NK, DV, false>(A, grid, rg, ip, lds);
 }
 
+template <int D, int NK, int DV, bool HAS_DIV, int RG>
+int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
+  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, 2>;
+  if (lds > 65536) {
+    MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  }
+  fn<<<grid, 64 * RG, lds, state().stream>>>(A);
+  MI355_HIP(hipGetLastError());
+  return 1;
+}
+
+template <int D, int NK, int DV>
+int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds) {
+  if (has_div) {
+    return rg == 4 ? launch_stream_one<D, NK, DV, true, 4>(A, grid, lds)
+                   : launch_stream_one<D, NK, DV, true, 2>(A, grid, lds);
+  }
+  return rg == 4 ? launch_stream_one<D, NK, DV, false, 4>(A, grid, lds)
+                 : launch_stream_one<D, NK, DV, false, 2>(A, grid, lds);
+}
+
 }  // namespace
 
 static bool shape_supported(Match const &M) {
@@ -558,6 +819,60 @@ int try_launch_attention(DevProgram const &P) {
   A.o = tile_addr(P.ops[M.out_o], P.out[P.ops[M.out_o].io]);
   A.r = M.out_r >= 0 ? tile_addr(P.ops[M.out_r], P.out[P.ops[M.out_r].io]) : A.o;
   A.forloop_range = P.forloop_range;
+  {
+    // grid dims the K / V tiles do not depend on vary fastest in the workgroup id
+    int n = 0;
+    bool dep[3];
+    for (int d = 0; d < 3; d++) {
+      DevOp const &lk = P.ops[M.k], &lv = P.ops[M.v];
+      dep[d] = lk.row_bs[d] || lk.col_bs[d] || lk.g_bs[d] || lv.row_bs[d] || lv.col_bs[d] || lv.g_bs[d];
+    }
+    for (int d = 0; d < 3; d++) {
+      if (!dep[d]) {
+        A.perm[n++] = d;
+      }
+    }
+    for (int d = 0; d < 3; d++) {
+      if (dep[d]) {
+        A.perm[n++] = d;
+      }
+    }
+  }
+  long long const blocks_all = (long long)P.grid[0] * P.grid[1] * P.grid[2];
+  // ---- throughput variant: enough independent 32-row wavefront slabs to fill the chip
+  // twice over, and a for-loop long enough to pipeline
+  {
+    int const slabs = M.m / 32;
+    int rgs = (M.m % 128 == 0) ? 4 : ((M.m % 64 == 0) ? 2 : 0);
+    bool const shape = (M.D == 64 && M.NK == 64 && M.DV == 64) || (M.D == 128 && M.NK == 64 && M.DV == 128);
+    bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512;
+    if (s.attention_mode == 1) {
+      want = false;
+    } else if (s.attention_mode == 2) {
+      want = rgs != 0 && shape;
+    }
+    if (want) {
+      A.split = slabs / rgs;
+      A.stages = 2;
+      A.lds_stage_bytes = (M.NK * M.D + M.DV * M.NK) * 2;
+      int const out_bytes = rgs * 32 * (M.DV + 8) * 2;
+      int lds = 2 * A.lds_stage_bytes;
+      lds = lds > out_bytes ? lds : out_bytes;
+      if (lds <= s.max_lds && (long long)P.grid[0] * A.split <= 2147483647LL) {
+        dim3 grid(P.grid[0] * A.split, P.grid[1], P.grid[2]);
+        int rc = M.D == 64 ? launch_stream<64, 64, 64>(A, M.has_div, grid, rgs, lds)
+                           : launch_stream<128, 64, 128>(A, M.has_div, grid, rgs, lds);
+        if (rc == 1) {
+          s.last_launch.kernel_id = MI355_KERNEL_F16_ATTENTION;
+          s.last_launch.workgroups = grid.x * grid.y * grid.z;
+          s.last_launch.threads = rgs * 64;
+          s.last_launch.lds_bytes = lds;
+          s.last_launch.row_split = A.split;
+        }
+        return rc;
+      }
+    }
+  }
 
   // Row groups per workgroup: up to 4, fewer when that is what it takes to put a
   // workgroup on every compute unit.  Iteration lanes: whatever is left of 8

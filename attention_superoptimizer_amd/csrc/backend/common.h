@@ -52,6 +52,7 @@ struct State {
   int max_lds = 65536;
   mi355_launch_info last_launch{};
   int force_interpreter = 0;
+  int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
   // fused-kernel workspace: fp16 range sums of split for-loops
   void *scratch = nullptr;
   size_t scratch_bytes = 0;

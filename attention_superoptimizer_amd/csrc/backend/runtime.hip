@@ -146,6 +146,10 @@ extern "C" int mi355_set_option(int option, int value) {
     state().force_interpreter = value;
     return MI355_OK;
   }
+  if (option == MI355_OPT_ATTENTION_MODE && value >= 0 && value <= 2) {
+    state().attention_mode = value;
+    return MI355_OK;
+  }
   return fail(MI355_ERR_INVALID, "unknown option %d", option);
 }
 

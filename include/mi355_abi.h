@@ -84,6 +84,10 @@ typedef struct mi355_launch_info {
  * customized op through the generic LDS interpreter instead of a fused kernel
  * (both must agree with the oracle; tests run the two against each other). */
 #define MI355_OPT_FORCE_INTERPRETER 1
+/* ATTENTION_MODE: 0 = choose by problem size (default), 1 = always the latency
+ * variant of the fused attention kernel, 2 = the throughput variant whenever the
+ * tile shape allows it. */
+#define MI355_OPT_ATTENTION_MODE 2
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor

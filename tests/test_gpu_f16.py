@@ -199,3 +199,22 @@ def test_gqa_fixture_graphs_f16(rt, path):
         spec = fx["generated_graphs"][gi]
         ins = _inputs(spec, 0.05, 70)
         _check(rt, spec, ins, f"fixture graph {gi}")
+
+
+def test_attention_throughput_variant(rt, abi):
+    """the pipelined 32-rows-per-wavefront variant, forced on small problems: both forms,
+    both head sizes"""
+    from attention_superoptimizer_amd import workloads as W
+    assert abi.mi355_set_option(2, 2) == 0
+    try:
+        spec, _ = W.config2_gqa_decode()
+        _check(rt, spec, _inputs(spec, W.INPUT_STD["C2_gqa_decode"], 90), "C2 throughput variant")
+        assert _last_kernels == [KERNEL_ATTENTION]
+        spec, _ = W.config3_mha_prefill(heads=2, seq=512, hd=128, q_split=4, kv_split=2, F=4)
+        _check(rt, spec, _inputs(spec, 128 ** -0.5, 91), "C3 small throughput variant")
+        assert _last_kernels[0] == KERNEL_ATTENTION
+        spec, _ = W.REFERENCE_EXAMPLES["multi_head_attn_prefill"]   # Q tile [64, 64], form B
+        _check(rt, spec, _inputs(spec, 0.05, 92), "mha prefill throughput variant")
+        assert _last_kernels[0] == KERNEL_ATTENTION
+    finally:
+        assert abi.mi355_set_option(2, 0) == 0
