@@ -433,17 +433,18 @@ __global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P
       }
     }
   }
-  _Float16 oacc[RPW][DB][4];
+  // fp16 accumulators, two per register: the per-iteration `acc + x` rounded to fp16
+  // is one packed fp16 add (the exact sum of two fp16 numbers rounded once, which is
+  // what adding in fp32 and rounding gives)
+  half2v oacc[RPW][DB][2];
   _Float16 racc[RPW];
 #pragma unroll
   for (int rp = 0; rp < RPW; rp++) {
     racc[rp] = (_Float16)0.0f;
 #pragma unroll
     for (int t = 0; t < DB; t++) {
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        oacc[rp][t][r] = (_Float16)0.0f;
-      }
+      oacc[rp][t][0] = half2v{(_Float16)0.0f, (_Float16)0.0f};
+      oacc[rp][t][1] = half2v{(_Float16)0.0f, (_Float16)0.0f};
     }
   }
 
@@ -570,12 +571,10 @@ __global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P
       }
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          _Float16 o16 = static_cast<_Float16>(o[rp][r]);
-          oacc[rp][t][r] = static_cast<_Float16>(static_cast<float>(oacc[rp][t][r]) +
-                                                 static_cast<float>(o16));
-        }
+        half2v lo = {static_cast<_Float16>(o[rp][0]), static_cast<_Float16>(o[rp][1])};
+        half2v hi = {static_cast<_Float16>(o[rp][2]), static_cast<_Float16>(o[rp][3])};
+        oacc[rp][t][0] = oacc[rp][t][0] + lo;
+        oacc[rp][t][1] = oacc[rp][t][1] + hi;
       }
     }
     if (it + 1 < F) {
@@ -592,7 +591,7 @@ __global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P
     for (int t = 0; t < DB; t++) {
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        ow[(16 * rp + 4 * g + r) * LDO + 16 * t + c] = oacc[rp][t][r];
+        ow[(16 * rp + 4 * g + r) * LDO + 16 * t + c] = oacc[rp][t][r >> 1][r & 1];
       }
     }
   }
