@@ -418,6 +418,13 @@ __global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P
   int const g = lane / 16, c = lane % 16;
   int bx, by, bz, slice;
   decode_block(P, bx, by, bz, slice);
+  // Swizzled operand addresses = lane part + compile-time part.  For row 16j + c the
+  // swizzle key (row ^ row>>3) & 7 is s0 ^ (2j & 7) with s0 = (c ^ c>>3) & 7, and a
+  // chunk index 4kk + g is 4kk ^ g, so chunk ^ key = (s0 ^ g) ^ (4kk ^ (2j & 7)): one
+  // XOR with a constant per fetch, everything else folds into the instruction offset.
+  int const s0 = (c ^ (c >> 3)) & 7;
+  int const k_lane = c * D, k_sg8 = (s0 ^ g) << 3;            // K^T: row c, 16-byte chunk g
+  int const v_lane = c * NK + (g & 1) * 4, v_sg8 = (s0 ^ (g >> 1)) << 3;  // V^T: 8-byte half chunks
   int const row_base = (slice * RG + wave) * RPW * 16;
   int const F = P.forloop_range;
 
@@ -511,7 +518,8 @@ __global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P
       }
 #pragma unroll
       for (int kk = 0; kk < DK; kk++) {
-        half8 a = *reinterpret_cast<half8 const *>(kt + swz_chunk(16 * j + c, 4 * kk + g, D));
+        half8 a = *reinterpret_cast<half8 const *>(
+            kt + k_lane + 16 * j * D + (k_sg8 ^ (((4 * kk) ^ ((2 * j) & 7)) << 3)));
 #pragma unroll
         for (int rp = 0; rp < RPW; rp++) {
           acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rp][kk], acc[rp], 0, 0, 0);
@@ -555,13 +563,13 @@ __global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P
       for (int rp = 0; rp < RPW; rp++) {
         o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
       }
-      int const vrow = 16 * t + c;
 #pragma unroll
       for (int jj = 0; jj < KB / 2; jj++) {
-        half4 b0 = *reinterpret_cast<half4 const *>(vt + swz_chunk(vrow, 4 * jj + (g >> 1), NK) +
-                                                    (g & 1) * 4);
-        half4 b1 = *reinterpret_cast<half4 const *>(vt + swz_chunk(vrow, 4 * jj + 2 + (g >> 1), NK) +
-                                                    (g & 1) * 4);
+        // row 16t + c, chunks 4jj + (g>>1) and 4jj + 2 + (g>>1)
+        half4 b0 = *reinterpret_cast<half4 const *>(
+            vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj) ^ ((2 * t) & 7)) << 3)));
+        half4 b1 = *reinterpret_cast<half4 const *>(
+            vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj + 2) ^ ((2 * t) & 7)) << 3)));
         half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
         for (int rp = 0; rp < RPW; rp++) {

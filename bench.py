@@ -51,6 +51,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="time only the headline configuration (used under the profiler)")
+    ap.add_argument("--only", default="", metavar="CONFIG",
+                    help="launch every customized op of one configuration --steps times and "
+                         "exit (for use under the profiler), e.g. C3_mha_prefill")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run 16 plain device copies of MIB MiB and exit: the known-size "
                          "traffic that hardware byte counters are scaled against")
@@ -95,6 +98,23 @@ def main() -> int:
                                                ctypes.c_float(W.INPUT_STD[name][i]), 0xC0FFEE00 + i)
                 assert rc == 0, N.last_error()
         return spec, g, vals
+
+    if args.only:
+        spec, g, vals = setup(args.only)
+        out = {}
+        for i, op in enumerate(spec):
+            if op["op"] != "customized":
+                continue
+            pl = g.lowered(i, fingerprint=False)
+            i_p = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(False) for a, b in op["in"]])
+            o_p = (ctypes.c_void_p * 4)(*[t.device_ptr(False) for t in vals[i]])
+            ms = ctypes.c_float()
+            assert abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, args.warmup, args.steps,
+                                                ctypes.byref(ms)) == 0, N.last_error()
+            out[f"op{i}_us"] = round(ms.value * 1e3, 3)
+        print(json.dumps({"config": args.only, **out}))
+        g.close()
+        return 0
 
     spec, g, vals = setup("C2_gqa_decode")
     op_idx = 3
