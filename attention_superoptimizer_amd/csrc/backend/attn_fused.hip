@@ -403,7 +403,7 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
 // global loads of iteration i+1 are in flight (in registers) while iteration i is on
 // the matrix cores.  One barrier per iteration.
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW>
-__global__ __launch_bounds__(64 * RG) void attn_stream_kernel(AttnParams const P) {
+__global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
   constexpr int NT = 64 * RG;
