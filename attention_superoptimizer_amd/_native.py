@@ -57,6 +57,13 @@ class MirageCPlan(ctypes.Structure):
     ]
 
 
+class MirageVerifyStats(ctypes.Structure):
+    """mirage_verify_stats of csrc/host/verify.cc."""
+    _fields_ = [("kernel_ops", ctypes.c_int), ("customized_ops", ctypes.c_int),
+                ("compares", ctypes.c_int), ("fp_bytes", ctypes.c_longlong),
+                ("matmul_macs", ctypes.c_longlong)]
+
+
 # every symbol include/mi355_abi.h declares, with its signature
 _vp, _ci, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64
 _pi = ctypes.POINTER(ctypes.c_int)
@@ -85,6 +92,9 @@ ABI = {
     "mi355_fp_binary": (_ci, [_ci, _vp, _pi, _vp, _pi, _vp, _pi, _ci]),
     "mi355_fp_reduce": (_ci, [_vp, _vp, _sz, _ci, _ci, _ci]),
     "mi355_fp_equal": (_ci, [_vp, _vp, _sz, _pi]),
+    "mi355_fp_equal_reset": (_ci, [_ci, _ci]),
+    "mi355_fp_equal_enqueue": (_ci, [_vp, _vp, _sz, _ci]),
+    "mi355_fp_equal_collect": (_ci, [_ci, _ci, _vp]),
     "mi355_customized_fp": (_ci, [_pplan, _pvp, _pvp]),
     "mi355_plan_extents": (_ci, [_pplan, _pll, _pll, _pi, _pi]),
     "mi355_customized_run": (_ci, [_pplan, _pvp, _pvp]),
@@ -123,6 +133,8 @@ FACADE = {
     "mirage_tensor_write": (_ci, [_vp, _ci, _vp, _sz]),
     "mirage_tensor_read": (_ci, [_vp, _ci, _vp, _sz]),
     "mirage_tensor_same_fingerprint": (_ci, [_vp, _vp]),
+    "mirage_graph_fingerprint": (_ci, [_vp, _u64, ctypes.POINTER(MirageVerifyStats)]),
+    "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_set_smem_budget": (None, [_sz]),
     "mirage_get_smem_budget": (_sz, []),
     "mirage_device_ready": (_ci, []),

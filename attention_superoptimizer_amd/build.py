@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import os
 import subprocess
+from concurrent.futures import ThreadPoolExecutor
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -37,12 +38,15 @@ def _run(cmd):
 
 def build_backend():
     srcs = _sources("backend", (".hip", ".cc"))
-    objs = []
-    for s in srcs:
-        o = os.path.splitext(s)[0] + ".o"
+    objs = [os.path.splitext(s)[0] + ".o" for s in srcs]
+
+    def compile_one(pair):
+        s, o = pair
         lang = ["-x", "hip"] if s.endswith(".hip") else []
         _run([HIPCC] + DEVICE_FLAGS + ["-I", INCLUDE, "-I", os.path.join(CSRC, "backend"), "-c"] + lang + [s, "-o", o])
-        objs.append(o)
+
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        list(pool.map(compile_one, zip(srcs, objs)))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", BACKEND_LIB] + objs)
 
 

@@ -48,6 +48,8 @@ struct State {
   uint16_t *exp_tbl = nullptr, *div_p = nullptr, *div_q = nullptr;
   int *flag = nullptr;        // 4-byte device scratch for mi355_fp_equal
   int *flag_host = nullptr;   // pinned mirror
+  int *cmp_slots = nullptr;   // MI355_COMPARE_SLOTS mismatch flags of deferred compares
+  int *cmp_host = nullptr;    // pinned mirror
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int max_lds = 65536;
   mi355_launch_info last_launch{};

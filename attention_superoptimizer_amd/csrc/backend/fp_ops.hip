@@ -12,6 +12,7 @@
 namespace mi355 {
 
 constexpr int kThreads = 256;
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
   x += 0x9E3779B97F4A7C15ull;
@@ -435,5 +436,83 @@ extern "C" int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, in
   MI355_HIP(hipMemcpyAsync(s.flag_host, s.flag, sizeof(int), hipMemcpyDeviceToHost, s.stream));
   MI355_HIP(hipStreamSynchronize(s.stream));
   *equal = *s.flag_host;
+  return MI355_OK;
+}
+
+// ---- deferred compares: many candidates, one synchronisation ----------------------------
+// Slot i of the device array holds "a mismatch was seen"; nothing comes back to the host
+// until the caller collects a range of slots.
+__global__ void clear_slots_kernel(int *slots, int count) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) {
+    slots[i] = 0;
+  }
+}
+
+__global__ void fp_differ_kernel(uint16_t const *__restrict__ a, uint16_t const *__restrict__ b,
+                                 size_t n, int *slot) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  bool differ = false;
+  size_t const n8 = (((uintptr_t)a | (uintptr_t)b) & 15) == 0 ? n / 8 : 0;
+  for (size_t j = i; j < n8; j += stride) {
+    uint4v x = reinterpret_cast<uint4v const *>(a)[j];
+    uint4v y = reinterpret_cast<uint4v const *>(b)[j];
+    differ |= (x[0] != y[0]) | (x[1] != y[1]) | (x[2] != y[2]) | (x[3] != y[3]);
+  }
+  for (size_t j = n8 * 8 + i; j < n; j += stride) {
+    differ |= (a[j] != b[j]);
+  }
+  if (differ) {
+    *slot = 1;  // every writer stores the same value
+  }
+}
+
+extern "C" int mi355_fp_equal_reset(int first_slot, int count) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (first_slot < 0 || count < 0 || first_slot + count > MI355_COMPARE_SLOTS) {
+    return fail(MI355_ERR_INVALID, "compare slots [%d, %d) out of range", first_slot,
+                first_slot + count);
+  }
+  if (count > 0) {
+    clear_slots_kernel<<<(count + kThreads - 1) / kThreads, kThreads, 0, s.stream>>>(
+        s.cmp_slots + first_slot, count);
+    MI355_HIP(hipGetLastError());
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_equal_enqueue(uint16_t const *a, uint16_t const *b, size_t n, int slot) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (slot < 0 || slot >= MI355_COMPARE_SLOTS) {
+    return fail(MI355_ERR_INVALID, "compare slot %d out of range", slot);
+  }
+  if (n > 0) {
+    fp_differ_kernel<<<grid_for((n + 7) / 8, kThreads, 1024), kThreads, 0, s.stream>>>(
+        a, b, n, s.cmp_slots + slot);
+    MI355_HIP(hipGetLastError());
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (first_slot < 0 || count < 0 || first_slot + count > MI355_COMPARE_SLOTS ||
+      (count > 0 && equal == nullptr)) {
+    return fail(MI355_ERR_INVALID, "compare slots [%d, %d) out of range", first_slot,
+                first_slot + count);
+  }
+  if (count == 0) {
+    return MI355_OK;
+  }
+  MI355_HIP(hipMemcpyAsync(s.cmp_host + first_slot, s.cmp_slots + first_slot,
+                           sizeof(int) * (size_t)count, hipMemcpyDeviceToHost, s.stream));
+  MI355_HIP(hipStreamSynchronize(s.stream));
+  for (int i = 0; i < count; i++) {
+    equal[i] = s.cmp_host[first_slot + i] == 0 ? 1 : 0;
+  }
   return MI355_OK;
 }

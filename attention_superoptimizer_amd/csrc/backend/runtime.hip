@@ -94,6 +94,9 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
   MI355_HIP(hipMemcpy(s.div_q, divq_h, sizeof(divq_h), hipMemcpyHostToDevice));
   MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.flag), 256));
   MI355_HIP(hipHostMalloc(reinterpret_cast<void **>(&s.flag_host), 256, hipHostMallocDefault));
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.cmp_slots), sizeof(int) * MI355_COMPARE_SLOTS));
+  MI355_HIP(hipHostMalloc(reinterpret_cast<void **>(&s.cmp_host), sizeof(int) * MI355_COMPARE_SLOTS,
+                          hipHostMallocDefault));
   MI355_HIP(hipEventCreate(&s.ev0));
   MI355_HIP(hipEventCreate(&s.ev1));
   s.scratch_bytes = (size_t)64 << 20;
@@ -117,6 +120,8 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipFree(s.exp_tbl));
   MI355_HIP(hipFree(s.flag));
   MI355_HIP(hipHostFree(s.flag_host));
+  MI355_HIP(hipFree(s.cmp_slots));
+  MI355_HIP(hipHostFree(s.cmp_host));
   MI355_HIP(hipFree(s.scratch));
   MI355_HIP(hipStreamDestroy(s.stream));
   s = State{};

@@ -211,6 +211,13 @@ class KNGraph:
                 continue
             self.fingerprint(i)
 
+    def fingerprint_seeded(self, input_seed: int) -> dict:
+        """fingerprint() of every operator; input number j holds uniform values drawn
+        from (input_seed, j) when input_seed != 0, `idx % 25651` otherwise."""
+        st = N.MirageVerifyStats()
+        assert self._rt.mirage_graph_fingerprint(self._g, input_seed, ctypes.byref(st)) == 0
+        return _stats(st)
+
     def execute(self, idx: int) -> None:
         assert self._rt.mirage_op_execute(self._g, idx) == 0
 
@@ -227,6 +234,25 @@ class KNGraph:
         rc = self._rt.mirage_op_lowered(self._g, idx, 1 if fingerprint else 0, ctypes.byref(p), None)
         assert rc == 0
         return p
+
+
+def _stats(st) -> dict:
+    return {"kernel_ops": st.kernel_ops, "customized_ops": st.customized_ops,
+            "compares": st.compares, "fp_bytes": st.fp_bytes, "matmul_macs": st.matmul_macs}
+
+
+def verify_batch(candidates: Sequence["KNGraph"], reference: "KNGraph", input_seed: int = 0):
+    """Batched KernelGraphGenerator::verify (reference src/search/search.cc:569-623):
+    fingerprints every candidate and compares its outputs with the (already
+    fingerprinted) outputs of `reference` on the device, one synchronisation for the
+    whole batch.  Returns (list of bool, stats)."""
+    n = len(candidates)
+    arr = (ctypes.c_void_p * n)(*[c._g for c in candidates])
+    eq = (ctypes.c_ubyte * n)()
+    st = N.MirageVerifyStats()
+    rc = N.runtime().mirage_verify_batch(arr, n, reference._g, input_seed, eq, ctypes.byref(st))
+    assert rc == 0
+    return [bool(eq[i]) for i in range(n)], _stats(st)
 
 
 def build_from_spec(spec: List[dict], graph: Optional[KNGraph] = None):

@@ -43,12 +43,97 @@ def algorithmic_bytes(spec, idx, out_dims):
     return 2 * n
 
 
+def _spec_inputs(spec, seed):
+    """Host copies of the inputs verify_batch generates on the device: input number j
+    = splitmix64((seed ^ j << 40) + i) % 25651."""
+    def splitmix(x):
+        x = x + np.uint64(0x9E3779B97F4A7C15)
+        x = (x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return x ^ (x >> np.uint64(31))
+    ins, j = {}, 0
+    for i, op in enumerate(spec):
+        if op["op"] == "input":
+            n = int(np.prod(op["dims"]))
+            with np.errstate(over="ignore"):
+                v = splitmix(np.arange(n, dtype=np.uint64) + np.uint64(seed ^ (j << 40)))
+            ins[i] = (v % np.uint64(25651)).astype(np.uint16).reshape(op["dims"])
+            j += 1
+    return ins
+
+
+def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_problem: int = 64):
+    """Batched verification of 4096 generated candidate mugraphs (8-12 operators, dims in
+    [64, 1024]): per problem the reference graph is fingerprinted once, its candidates are
+    built through the host API (untimed) and verified by ONE verify_batch call (timed, host
+    wall clock: enqueue of every fingerprint kernel and compare + the single sync)."""
+    from attention_superoptimizer_amd import candidates as C
+    probs = C.generate(num_problems=num_problems, per_problem=per_problem)
+    t_build = t_verify = 0.0
+    tot = {"kernel_ops": 0, "customized_ops": 0, "compares": 0, "fp_bytes": 0, "matmul_macs": 0}
+    n = wrong = 0
+    for prob in probs:
+        ref_g, _ = G.build_from_spec(prob["reference"])
+        ref_g.fingerprint_seeded(prob["input_seed"])
+        b0 = time.perf_counter()
+        graphs = [G.build_from_spec(c["spec"])[0] for c in prob["candidates"]]
+        b1 = time.perf_counter()
+        verdicts, st = G.verify_batch(graphs, ref_g, prob["input_seed"])
+        b2 = time.perf_counter()
+        t_build += b1 - b0
+        t_verify += b2 - b1
+        for k in tot:
+            tot[k] += st[k]
+        n += len(graphs)
+        wrong += sum(v != c["expect_equal"] for v, c in zip(verdicts, prob["candidates"]))
+        for gph in reversed(graphs):
+            gph.close()
+        ref_g.close()
+    rec = {
+        "candidates": n, "problems": len(probs), "candidates_per_s": round(n / t_verify, 1),
+        "verify_s": round(t_verify, 4), "host_graph_build_s": round(t_build, 4),
+        "kernel_ops": tot["kernel_ops"], "customized_ops": tot["customized_ops"],
+        "compares": tot["compares"],
+        "fingerprint_GBps": round(tot["fp_bytes"] / t_verify / 1e9, 2),
+        "int_TMACps": round(tot["matmul_macs"] / t_verify / 1e12, 3),
+        "verdicts_as_constructed": wrong == 0,
+        "inputs": "uniform [0, 25651) from (seed, input index)",
+    }
+    if cpu_baseline:
+        # the scalar C restatement over a bounded sample: candidate 0 of every 8th problem,
+        # once on one core and once with one candidate per host thread
+        from concurrent.futures import ThreadPoolExecutor
+        from oracle import evaluate as orc
+        sample = [(p["candidates"][0]["spec"], p["input_seed"]) for p in probs[::8]]
+        ins = [_spec_inputs(sp, seed) for sp, seed in sample]
+        c0 = time.perf_counter()
+        for (sp, _), i_ in zip(sample, ins):
+            orc.eval_graph(sp, "fp", i_, threads=1)
+        c1 = time.perf_counter()
+        cores = min(16, os.cpu_count() or 1)
+        with ThreadPoolExecutor(cores) as pool:
+            list(pool.map(lambda a: orc.eval_graph(a[0][0], "fp", a[1], threads=1), zip(sample, ins)))
+        c2 = time.perf_counter()
+        rec["cpu_baseline"] = {
+            "value": round(len(sample) / (c1 - c0), 2), "unit": "candidates/s", "cores": 1,
+            "all_cores_value": round(len(sample) / (c2 - c1), 2), "all_cores": cores, "kind": "port",
+            "sample": f"{len(sample)} candidates (first candidate of every 8th problem), scalar C "
+                      "oracle, `%` per multiply-accumulate as the reference's kernels do",
+        }
+    return rec
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1024)
     ap.add_argument("--warmup", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fingerprints", action="store_true",
+                    help="skip the batched candidate-verification throughput leg")
+    ap.add_argument("--fingerprints-only", action="store_true",
+                    help="run only the batched candidate-verification leg and print its record "
+                         "(for use under the profiler)")
     ap.add_argument("--headline-only", action="store_true",
                     help="time only the headline configuration (used under the profiler)")
     ap.add_argument("--only", default="", metavar="CONFIG",
@@ -74,6 +159,10 @@ def main() -> int:
     G.set_smem_budget(1 << 20)
     info = N.Mi355DeviceInfo()
     assert abi.mi355_get_device_info(ctypes.byref(info)) == 0
+
+    if args.fingerprints_only:
+        print(json.dumps(fingerprint_throughput(G, False)), flush=True)
+        return 0
 
     if args.calibrate_copy:
         n = args.calibrate_copy << 20
@@ -180,14 +269,17 @@ def main() -> int:
     }
 
     # ---- the other benchmark configurations (reported beside the headline) -----------
-    def flops_of(spec, idx, in_dims):
-        """2*m*n*k per thread-block matmul, summed over blocks and iterations"""
-        from oracle import lowering as _lw  # host-side shape arithmetic only
-        tg = _lw.build_tb_graph(spec[idx]["plan"], in_dims, None, 1 << 30)
-        per_block = sum(2 * o.inputs[0].dims[-2] * o.inputs[0].dims[-1] * o.inputs[1].dims[-1]
-                        for o in tg.operators if o.op_type == _lw.TB_MATMUL_OP)
-        gd = spec[idx]["plan"]["grid_dim"]
-        return per_block * gd[0] * gd[1] * gd[2] * spec[idx]["plan"]["forloop_range"]
+    def flops_of(pl):
+        """2*m*n*k per thread-block matmul of a lowered plan, over blocks and iterations"""
+        width = {2001: 19, 2002: 17, 2003: 6, 2007: 2, 2012: 2, 2008: 9, 2009: 9, 2010: 9}
+        pos, per_block = 0, 0
+        for j in range(pl.num_operators):
+            t = pl.operator_types[j]
+            if t == 2003:
+                m, n, k = pl.parameters[pos], pl.parameters[pos + 1], pl.parameters[pos + 2]
+                per_block += 2 * m * n * k
+            pos += width.get(t, 5 if 2101 <= t <= 2106 else 7)
+        return per_block * pl.grid_dim[0] * pl.grid_dim[1] * pl.grid_dim[2] * pl.forloop_range
 
     others = []
     if not args.headline_only:
@@ -210,7 +302,7 @@ def main() -> int:
                 abi.mi355_last_launch(ctypes.byref(li))
                 nbytes = 2 * (sum(vals2[a][b].num_elements for a, b in op["in"]) +
                               sum(t.num_elements for t in vals2[i]))
-                fl = flops_of(spec2, i, [list(vals2[a][b].dims) for a, b in op["in"]])
+                fl = flops_of(pl)
                 us = ms.value * 1e3
                 rec["ops"].append({"op": i, "us": round(us, 3), "kernel": kname.get(li.kernel_id),
                                    "workgroups": li.workgroups, "algorithmic_bytes": nbytes,
@@ -222,6 +314,10 @@ def main() -> int:
                         "mfma_frac": round(tot_flops / tot_us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)})
             others.append(rec)
         result["other_configs"] = others
+    if not args.headline_only and not args.no_fingerprints:
+        g.close()
+        result["fingerprint_throughput"] = fingerprint_throughput(G, not args.no_cpu_baseline)
+        spec, g, vals = setup("C2_gqa_decode")
     floor = ctypes.c_float()
     if abi.mi355_launch_floor(2048, ctypes.byref(floor)) == 0:
         result["roofline"]["empty_launch_us"] = round(floor.value, 3)

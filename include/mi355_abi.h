@@ -139,6 +139,17 @@ int mi355_fp_reduce(uint16_t const *in, uint16_t *out, size_t n_out, int factor,
 /* DTensor::has_same_fingerprint's element loop, src/kernel/cuda/device_tensor_kernel.cu:36-52,
  * done on the device; writes 1/0 to *equal (blocking: 4 bytes come back, not 2 tensors) */
 int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, int *equal);
+/* The same compare without the round trip, for verifying many candidates
+ * (the verify loop of src/search/search.cc:569-623 calls has_same_fingerprint once per
+ * candidate output and blocks each time).  The backend keeps MI355_COMPARE_SLOTS result
+ * slots on the device: reset a range, enqueue one compare per slot behind the
+ * fingerprint kernels on the backend stream, then collect the range with a single
+ * synchronisation; equal[i] = 1/0 for slot first_slot + i.  A slot that several
+ * compares target reports their conjunction. */
+#define MI355_COMPARE_SLOTS 65536
+int mi355_fp_equal_reset(int first_slot, int count);
+int mi355_fp_equal_enqueue(uint16_t const *a, uint16_t const *b, size_t n, int slot);
+int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal);
 /* KNCustomizedOp::fingerprint + compute_customizedop_fingerprint,
  * src/kernel/cuda/customized_kernel.cu:307-603,655-678 */
 int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,

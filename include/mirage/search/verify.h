@@ -1,0 +1,50 @@
+// Batched probabilistic verification of candidate kernel graphs: the device half
+// of the reference's KernelGraphGenerator::verify / have_same_fingerprint
+// (src/search/search.cc:569-623), restated for many candidates at once.
+//
+// The reference verifies one candidate at a time: fingerprint() of every operator
+// (a device-wide sync after each), then one blocking has_same_fingerprint per
+// output and permutation.  Here every candidate's fingerprint kernels and one
+// on-device compare per (reference output, candidate output) pair are enqueued
+// back to back; the host synchronises once per batch and resolves the output
+// permutations from the compare matrix.
+#pragma once
+
+#include "mirage/kernel/graph.h"
+#include <cstdint>
+#include <vector>
+
+namespace mirage {
+namespace search {
+
+// Tensors of `g` that no operator of `g` consumes, in creation order
+// (search.cc:580-593: `num_consumers[i] == 0`).
+std::vector<mirage::kernel::DTensor> graph_outputs(mirage::kernel::Graph const &g);
+
+struct VerifyStats {
+  int kernel_ops = 0;         // operators fingerprinted (inputs included)
+  int customized_ops = 0;     // of which customized
+  int compares = 0;           // on-device compares enqueued
+  long long fp_bytes = 0;     // 2 B x (input + output elements) over all operators
+  long long matmul_macs = 0;  // m*n*k over kernel-level and thread-block matmuls
+};
+
+// equal[i] = 1 iff candidate i has as many outputs as `reference_outputs` and some
+// permutation of them is fingerprint-equal to the reference outputs (same dtype,
+// layout and dims, search.cc:611-619).  Every operator of every candidate is
+// fingerprinted first.  input_seed == 0 fills inputs as the reference does
+// (`idx % 25651`, src/kernel/cuda/input_kernel.cu:56-61); otherwise input number j of
+// each graph holds uniform values generated from (input_seed, j), so graphs built
+// over the same inputs see the same data.  The reference outputs must already hold
+// their fingerprints.  At most MI355_COMPARE_SLOTS compares per call.
+void verify_batch(std::vector<mirage::kernel::Graph *> const &candidates,
+                  std::vector<mirage::kernel::DTensor> const &reference_outputs,
+                  uint64_t input_seed, std::vector<uint8_t> &equal,
+                  VerifyStats *stats = nullptr);
+
+// fingerprint() of every operator of one graph with the same input convention.
+void fingerprint_graph(mirage::kernel::Graph const &g, uint64_t input_seed,
+                       VerifyStats *stats = nullptr);
+
+}  // namespace search
+}  // namespace mirage
