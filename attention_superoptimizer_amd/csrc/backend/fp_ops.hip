@@ -34,7 +34,11 @@ __global__ void fp_fill_uniform_kernel(uint16_t *fp, size_t n, uint64_t seed) {
   size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
   size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) {
-    fp[i] = static_cast<uint16_t>(splitmix64(seed + i) % FP_PQ);
+    // v % 25651 for 64-bit v through 32-bit arithmetic: 2^32 = 15158 (mod 25651)
+    uint64_t const v = splitmix64(seed + i);
+    uint32_t const hi = static_cast<uint32_t>(v >> 32) % FP_PQ;
+    uint32_t const lo = static_cast<uint32_t>(v) % FP_PQ;
+    fp[i] = static_cast<uint16_t>((hi * 15158u + lo) % FP_PQ);
   }
 }
 

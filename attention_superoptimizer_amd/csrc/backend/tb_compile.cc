@@ -441,6 +441,40 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
     err = fmt("thread-block graph needs %d bytes of LDS, the device offers %d", peak, max_lds);
     return MI355_ERR_UNSUPPORTED;
   }
+  prog.mm_off = peak;
+  prog.splits = 1;
+  for (int o = 0; o < prog.num_ops; o++) {
+    prog.ops[o].mm_kc = 0;
+  }
+  if (!f16 && max_lds <= (1 << 20)) {  // not for a lowering that only sizes the plan
+    // Residue scratch of the packed matmul path: two fields x (m + 4 + n) x kc bytes for
+    // a k chunk of kc.  Each matmul takes the largest chunk that still fits; one that
+    // cannot get even 16 keeps the scalar path.
+    int const device_lds = max_lds;
+    int scratch = 0;
+    for (int o = 0; o < prog.num_ops; o++) {
+      DevOp &d = prog.ops[o];
+      if (d.kind != DOP_MATMUL) {
+        continue;
+      }
+      int const m = prog.t[d.src0].rows, k = prog.t[d.src0].cols, n = prog.t[d.src1].cols;
+      if (m % 4 != 0 || n % 4 != 0 || k % 4 != 0) {
+        continue;
+      }
+      for (int kc = k; kc >= 16 || kc == k; kc /= 2) {
+        if (kc % 4 != 0 || k % kc != 0) {
+          break;
+        }
+        int const need = 2 * kc * (m + 4 + n);
+        if (peak + need <= device_lds) {
+          d.mm_kc = kc;
+          scratch = std::max(scratch, need);
+          break;
+        }
+      }
+    }
+    prog.lds_bytes = peak + scratch;
+  }
   // LDS writes of 16 bytes need 8-element row strides on the destination
   for (int o = 0; o < prog.num_ops; o++) {
     DevOp &d = prog.ops[o];

@@ -11,6 +11,7 @@
 #include "common.h"
 #include "tb_program.h"
 
+#include <algorithm>
 #include <string>
 
 namespace mi355 {
@@ -28,9 +29,9 @@ struct TileOrigin {
   int row0, col0;
 };
 
-__device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it) {
+__device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it, int bx) {
   TileOrigin o;
-  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  int by = blockIdx.y, bz = blockIdx.z;
   o.row0 = bx * op.row_bs[0] + by * op.row_bs[1] + bz * op.row_bs[2] + it * op.row_fs;
   o.col0 = bx * op.col_bs[0] + by * op.col_bs[1] + bz * op.col_bs[2] + it * op.col_fs;
   o.base = (long long)bx * op.g_bs[0] + (long long)by * op.g_bs[1] + (long long)bz * op.g_bs[2] +
@@ -57,6 +58,102 @@ __device__ __forceinline__ uint32_t lds_silu(uint16_t const *tbl, uint32_t x) {
   return lds_div(tbl, x, den);
 }
 
+// C[m][n] = A[m][k] . B[k][n] over Z_25651 without a modulus in the inner loop:
+// every operand is split into its residues modulo 227 and 113 (both fit a byte), four
+// consecutive k are packed into one dword per field, and the packed 4 x 8-bit dot
+// instruction accumulates in each field; one CRT recombination per output and k chunk
+// (reference multipliers, include/mirage/type.h:26-36).  The sum of products modulo
+// 25651 is fixed by its two residues, so the value equals the reference's
+// `(r + a*b) % 25651` chain (matmul.h:773-804) bit for bit.  m, n, k, kc multiples of 4.
+// scratch: Ap[2][kc/4][m + 4] then Bp[2][kc/4][n] dwords; thread tiles are 4 x 4.
+__device__ __forceinline__ uint32_t pack_residues(uint32_t v0, uint32_t v1, uint32_t v2,
+                                                  uint32_t v3, uint32_t mod) {
+  return (v0 % mod) | ((v1 % mod) << 8) | ((v2 % mod) << 16) | ((v3 % mod) << 24);
+}
+
+__device__ void fp_matmul_packed(uint16_t const *A, uint16_t const *B, uint16_t *C, int m, int n,
+                                 int k, int kc, uint32_t *scratch, int tid) {
+  int const kq = kc / 4, lda = m + 4;
+  uint32_t *Ap = scratch, *Bp = scratch + 2 * kq * lda;
+  int const n4 = n / 4, tiles = (m / 4) * n4;
+  for (int k0 = 0; k0 < k; k0 += kc) {
+    if (k0 > 0) {
+      __syncthreads();  // the previous chunk's residues are still being read
+    }
+    for (int e = tid; e < m * kq; e += kInterpThreads) {
+      int const row = e / kq, q = e % kq;
+      uint2 v = *reinterpret_cast<uint2 const *>(A + row * k + k0 + 4 * q);
+      uint32_t v0 = v.x & 0xffffu, v1 = v.x >> 16, v2 = v.y & 0xffffu, v3 = v.y >> 16;
+      Ap[q * lda + row] = pack_residues(v0, v1, v2, v3, FP_P);
+      Ap[(kq + q) * lda + row] = pack_residues(v0, v1, v2, v3, FP_Q);
+    }
+    for (int e = tid; e < kq * (n / 2); e += kInterpThreads) {
+      int const q = e / (n / 2), c2 = (e % (n / 2)) * 2;
+      uint16_t const *bp = B + (k0 + 4 * q) * n + c2;
+      uint32_t w0 = *reinterpret_cast<uint32_t const *>(bp);
+      uint32_t w1 = *reinterpret_cast<uint32_t const *>(bp + n);
+      uint32_t w2 = *reinterpret_cast<uint32_t const *>(bp + 2 * n);
+      uint32_t w3 = *reinterpret_cast<uint32_t const *>(bp + 3 * n);
+      uint2 pp, qq;
+      pp.x = pack_residues(w0 & 0xffffu, w1 & 0xffffu, w2 & 0xffffu, w3 & 0xffffu, FP_P);
+      pp.y = pack_residues(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16, FP_P);
+      qq.x = pack_residues(w0 & 0xffffu, w1 & 0xffffu, w2 & 0xffffu, w3 & 0xffffu, FP_Q);
+      qq.y = pack_residues(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16, FP_Q);
+      *reinterpret_cast<uint2 *>(Bp + q * n + c2) = pp;
+      *reinterpret_cast<uint2 *>(Bp + (kq + q) * n + c2) = qq;
+    }
+    __syncthreads();
+    for (int t = tid; t < tiles; t += kInterpThreads) {
+      int const r0 = (t / n4) * 4, c0 = (t % n4) * 4;
+      uint32_t accp[4][4], accq[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          accp[i][j] = 0;
+          accq[i][j] = 0;
+        }
+      }
+      uint32_t const *ap = Ap + r0, *bp = Bp + c0;
+      for (int q = 0; q < kq; q++) {
+        uint4v a_p = *reinterpret_cast<uint4v const *>(ap + q * lda);
+        uint4v a_q = *reinterpret_cast<uint4v const *>(ap + (kq + q) * lda);
+        uint4v b_p = *reinterpret_cast<uint4v const *>(bp + q * n);
+        uint4v b_q = *reinterpret_cast<uint4v const *>(bp + (kq + q) * n);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            accp[i][j] = __builtin_amdgcn_udot4(a_p[i], b_p[j], accp[i][j], false);
+            accq[i][j] = __builtin_amdgcn_udot4(a_q[i], b_q[j], accq[i][j], false);
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        uint16_t *cp = C + (r0 + i) * n + c0;
+        uint32_t z[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          z[j] = ((accp[i][j] % FP_P) * FP_Q_MUL_P_MOD_1 + (accq[i][j] % FP_Q) * FP_P_MUL_Q_MOD_1) %
+                 FP_PQ;
+        }
+        if (k0 > 0) {
+          uint2 old = *reinterpret_cast<uint2 const *>(cp);
+          z[0] = (z[0] + (old.x & 0xffffu)) % FP_PQ;
+          z[1] = (z[1] + (old.x >> 16)) % FP_PQ;
+          z[2] = (z[2] + (old.y & 0xffffu)) % FP_PQ;
+          z[3] = (z[3] + (old.y >> 16)) % FP_PQ;
+        }
+        uint2 out;
+        out.x = z[0] | (z[1] << 16);
+        out.y = z[2] | (z[3] << 16);
+        *reinterpret_cast<uint2 *>(cp) = out;
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
     DevProgram const P, uint16_t const *__restrict__ g_exp, uint16_t const *__restrict__ g_divp,
     uint16_t const *__restrict__ g_divq) {
@@ -72,17 +169,21 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
   }
   __syncthreads();
   int const F = P.forloop_range;
-  for (int it = 0; it < F; it++) {
+  // a split for-loop: this workgroup covers iterations [it_begin, it_end) of block bx
+  int const bx = blockIdx.x % P.grid[0], split = blockIdx.x / P.grid[0];
+  int const it_begin = (int)((long long)F * split / P.splits);
+  int const it_end = (int)((long long)F * (split + 1) / P.splits);
+  for (int it = it_begin; it < it_end; it++) {
     for (int o = 0; o < P.num_ops; o++) {
       DevOp const &op = P.ops[o];
       switch (op.kind) {
         case DOP_LOAD: {
-          if (op.hoist && it > 0) {
+          if (op.hoist && it > it_begin) {
             break;
           }
           DevTensor const &t = P.t[op.dst];
           uint16_t *s = reinterpret_cast<uint16_t *>(lds + t.off);
-          TileOrigin org = tile_origin(op, it);
+          TileOrigin org = tile_origin(op, it, bx);
           uint16_t const *g = static_cast<uint16_t const *>(P.in[op.io]) + org.base;
           if (op.vec8) {
             int const cpr = t.cols / 8, n = t.rows * cpr;
@@ -109,7 +210,10 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           uint16_t const *B = reinterpret_cast<uint16_t const *>(lds + tb.off);
           uint16_t *C = reinterpret_cast<uint16_t *>(lds + tc.off);
           int const m = ta.rows, k = ta.cols, n = tb.cols;
-          if (n % 4 == 0) {
+          if (op.mm_kc > 0) {
+            fp_matmul_packed(A, B, C, m, n, k, op.mm_kc,
+                             reinterpret_cast<uint32_t *>(lds + P.mm_off), tid);
+          } else if (n % 4 == 0) {
             int const n4 = n / 4, total = m * n4;
             for (int e = tid; e < total; e += kInterpThreads) {
               int row = e / n4, c0 = (e % n4) * 4;
@@ -235,12 +339,14 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + ti.off);
           uint16_t *acc = reinterpret_cast<uint16_t *>(lds + ta.off);
           int const n = ta.rows * ta.cols;
-          bool const last = (it == F - 1);
-          TileOrigin org = tile_origin(op, 0);
-          uint16_t *g = static_cast<uint16_t *>(P.out[op.io]) + org.base;
+          bool const last = (it == it_end - 1);
+          TileOrigin org = tile_origin(op, 0, bx);
+          uint16_t *g = (P.splits > 1 ? P.part[op.io] + (long long)split * P.part_elems[op.io]
+                                      : static_cast<uint16_t *>(P.out[op.io])) +
+                        org.base;
           for (int e = tid; e < n; e += kInterpThreads) {
             uint32_t v = x[e];
-            if (it > 0) {
+            if (it > it_begin) {
               v = (v + acc[e]) % FP_PQ;
             }
             if (last) {
@@ -348,7 +454,7 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           }
           DevTensor const &t = P.t[op.dst];
           _Float16 *s = tile_ptr(lds, t);
-          TileOrigin org = tile_origin(op, it);
+          TileOrigin org = tile_origin(op, it, blockIdx.x);
           _Float16 const *g = static_cast<_Float16 const *>(P.in[op.io]) + org.base;
           if (op.vec8) {
             int const cpr = t.cols / 8, n = t.rows * cpr;
@@ -469,7 +575,7 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           _Float16 *acc = tile_ptr(lds, ta);
           int const n = ta.rows * ta.cols;
           bool const last = (it == F - 1);
-          TileOrigin org = tile_origin(op, 0);
+          TileOrigin org = tile_origin(op, 0, blockIdx.x);
           _Float16 *g = static_cast<_Float16 *>(P.out[op.io]) + org.base;
           for (int e = tid; e < n; e += kInterpThreads) {
             int r = e / ta.cols, c = e % ta.cols;
@@ -497,6 +603,51 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
 // ===========================================================================
 // launchers
 // ===========================================================================
+// out[e] = sum over splits of part[split * n + e] (mod 25651)
+__global__ void fp_combine_splits_kernel(uint16_t const *__restrict__ part,
+                                         uint16_t *__restrict__ out, long long n, int splits) {
+  long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  long long const stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    uint32_t v = 0;
+    for (int s = 0; s < splits; s++) {
+      v += part[(long long)s * n + i];  // splits <= 64: far from 2^32
+    }
+    out[i] = static_cast<uint16_t>(v % FP_PQ);
+  }
+}
+
+// How many workgroups share one logical block's for-loop in the uint16 interpreter.
+// The accumulating saver is a sum over iterations in a ring, so any split of the
+// iteration range gives the same value; small grids are split until the device is full.
+static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outputs) {
+  State &s = state();
+  prog.splits = 1;
+  int const blocks = prog.grid[0] * prog.grid[1] * prog.grid[2];
+  int const F = prog.forloop_range;
+  if (F < 2 || blocks >= 192 || s.scratch == nullptr) {
+    return;
+  }
+  int splits = std::min(std::min(F, 64), (256 + blocks - 1) / blocks);
+  long long elems = 0;
+  for (int i = 0; i < num_outputs; i++) {
+    elems += (ext.out_elems[i] + 7) / 8 * 8;
+  }
+  while (splits > 1 && (size_t)(elems * splits * 2) > s.scratch_bytes) {
+    splits--;
+  }
+  if (splits < 2) {
+    return;
+  }
+  prog.splits = splits;
+  uint16_t *p = static_cast<uint16_t *>(s.scratch);
+  for (int i = 0; i < num_outputs; i++) {
+    prog.part[i] = p;
+    prog.part_elems[i] = ext.out_elems[i];
+    p += (ext.out_elems[i] + 7) / 8 * 8 * splits;
+  }
+}
+
 static int prepare(mi355_plan const *plan, void const *const *inputs, void *const *outputs,
                    bool f16, DevProgram &prog) {
   if (plan == nullptr || inputs == nullptr || outputs == nullptr) {
@@ -544,6 +695,9 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     }
     prog.out[i] = outputs[i];
   }
+  if (!f16) {
+    choose_splits(prog, ext, plan->num_dmem_outputs);
+  }
   // 16-byte global accesses also need 16-byte aligned base pointers
   for (int o = 0; o < prog.num_ops; o++) {
     DevOp &d = prog.ops[o];
@@ -563,7 +717,7 @@ static int launch(DevProgram const &prog, bool f16) {
     }
     return rc < 0 ? rc : fail(MI355_ERR_UNSUPPORTED, "fused kernel declined the launch");
   }
-  dim3 grid(prog.grid[0], prog.grid[1], prog.grid[2]);
+  dim3 grid(prog.grid[0] * (f16 ? 1 : prog.splits), prog.grid[1], prog.grid[2]);
   static int fp_lds_set = 0, f16_lds_set = 0;
   int &cur = f16 ? f16_lds_set : fp_lds_set;
   if (prog.lds_bytes > 65536 && prog.lds_bytes > cur) {
@@ -581,10 +735,21 @@ static int launch(DevProgram const &prog, bool f16) {
   } else {
     fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream>>>(prog, s.exp_tbl,
                                                                           s.div_p, s.div_q);
+    if (prog.splits > 1) {
+      for (int o = 0; o < MI355_MAX_DMEM_OUTPUTS; o++) {
+        if (prog.out[o] == nullptr || prog.part_elems[o] <= 0) {
+          continue;
+        }
+        long long const n = prog.part_elems[o];
+        int const blocks = (int)std::min<long long>((n + 255) / 256, 2048);
+        fp_combine_splits_kernel<<<blocks, 256, 0, s.stream>>>(
+            prog.part[o], static_cast<uint16_t *>(prog.out[o]), n, prog.splits);
+      }
+    }
   }
   MI355_HIP(hipGetLastError());
   s.last_launch.kernel_id = f16 ? MI355_KERNEL_F16_INTERP : MI355_KERNEL_FP_INTERP;
-  s.last_launch.workgroups = prog.grid[0] * prog.grid[1] * prog.grid[2];
+  s.last_launch.workgroups = (int)(grid.x * grid.y * grid.z);
   s.last_launch.threads = kInterpThreads;
   s.last_launch.lds_bytes = prog.lds_bytes;
   s.last_launch.row_split = 1;

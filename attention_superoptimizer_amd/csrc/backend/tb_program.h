@@ -46,6 +46,7 @@ struct DevOp {
   int d_rows, d_cols;                        // matrix shape of the device tensor
   int red_deg, red_inner;                    // REDUCE (flat row-major rule of the reference)
   int cat_a, cat_b, cat_inner;               // CONCAT
+  int mm_kc;  // MATMUL, uint16 interpreter: k chunk of the packed-residue path, 0 = scalar path
 };
 
 struct DevProgram {
@@ -54,6 +55,13 @@ struct DevProgram {
   int lds_bytes;  // dynamic LDS the interpreter requests (tables included)
   int fused;      // 1 / 2: run by the fused attention / GEMM kernel instead of the interpreter
   int grid[3];
+  int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
+  // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
+  // [F*split/splits, F*(split+1)/splits) and stores its sums to part[o] + split*part_elems[o];
+  // a second launch adds the splits (exact in the ring).  splits == 1: stores go to out[].
+  int splits;
+  long long part_elems[MI355_MAX_DMEM_OUTPUTS];
+  uint16_t *part[MI355_MAX_DMEM_OUTPUTS];
   DevTensor t[kMaxTensors];
   DevOp ops[MI355_MAX_OPERATORS];
   void const *in[MI355_MAX_DMEM_INPUTS];
