@@ -61,7 +61,8 @@ class MirageVerifyStats(ctypes.Structure):
     """mirage_verify_stats of csrc/host/verify.cc."""
     _fields_ = [("kernel_ops", ctypes.c_int), ("customized_ops", ctypes.c_int),
                 ("compares", ctypes.c_int), ("fp_bytes", ctypes.c_longlong),
-                ("matmul_macs", ctypes.c_longlong)]
+                ("matmul_macs", ctypes.c_longlong),
+                ("enqueue_seconds", ctypes.c_double), ("wait_seconds", ctypes.c_double)]
 
 
 # every symbol include/mi355_abi.h declares, with its signature
@@ -85,8 +86,10 @@ ABI = {
     "mi355_memset": (_ci, [_vp, _ci, _sz]),
     "mi355_copy": (_ci, [_vp, _vp, _sz]),
     "mi355_sync": (_ci, []),
+    "mi355_queue_select": (_ci, [_ci]),
     "mi355_fp_fill_iota": (_ci, [_vp, _sz]),
     "mi355_fp_fill_uniform": (_ci, [_vp, _sz, _u64]),
+    "mi355_fp_fill_many": (_ci, [_pvp, ctypes.POINTER(_sz), ctypes.POINTER(_u64), _ci, _ci]),
     "mi355_fp_matmul": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci]),
     "mi355_fp_unary": (_ci, [_ci, _vp, _vp, _sz]),
     "mi355_fp_binary": (_ci, [_ci, _vp, _pi, _vp, _pi, _vp, _pi, _ci]),

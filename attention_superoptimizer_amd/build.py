@@ -56,7 +56,7 @@ def build_runtime():
         return
     _run(["g++", "-O2", "-fPIC", "-std=c++17", "-shared", "-D__HIP_PLATFORM_AMD__",
           "-I", INCLUDE, "-I", "/opt/rocm/include", "-o", RUNTIME_LIB] + srcs +
-         ["-L" + HERE, "-lmi355_backend", "-Wl,-rpath,$ORIGIN"])
+         ["-L" + HERE, "-lmi355_backend", "-Wl,-rpath,$ORIGIN", "-pthread"])
 
 
 def main():

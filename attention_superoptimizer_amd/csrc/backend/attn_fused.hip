@@ -752,7 +752,7 @@ int launch_one(AttnParams const &A, dim3 grid, int lds) {
                                   hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
     granted = state().max_lds;
   }
-  fn<<<grid, 64 * RG * IP, lds, state().stream>>>(A);
+  fn<<<grid, 64 * RG * IP, lds, state().stream()>>>(A);
   MI355_HIP(hipGetLastError());
   return 1;
 }
@@ -786,7 +786,7 @@ int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   }
-  fn<<<grid, 64 * RG, lds, state().stream>>>(A);
+  fn<<<grid, 64 * RG, lds, state().stream()>>>(A);
   MI355_HIP(hipGetLastError());
   return 1;
 }

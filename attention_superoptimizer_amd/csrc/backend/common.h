@@ -38,10 +38,16 @@ enum : int {
   TB_CONCAT_2_OP = 2202,
 };
 
+extern thread_local int tls_queue;  // the calling thread's queue, see mi355_queue_select
+
 struct State {
   bool ready = false;
   int device = 0;
-  hipStream_t stream = nullptr;
+  // Work is enqueued on the calling host thread's selected queue (queue 0 unless the
+  // thread chose another); the others exist so independent candidates can overlap their
+  // small kernels and host threads can enqueue side by side.
+  hipStream_t queues[MI355_NUM_QUEUES] = {};
+  hipStream_t stream() const { return queues[tls_queue]; }
   char *arena = nullptr;
   size_t arena_bytes = 0;
   // device copies of the lookup tables, reference layout
@@ -56,11 +62,16 @@ struct State {
   int force_interpreter = 0;
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
   // fused-kernel workspace: fp16 range sums of split for-loops
-  void *scratch = nullptr;
-  size_t scratch_bytes = 0;
+  // (each queue has its own slice of scratch_base, so concurrent queues never share)
+  size_t scratch_bytes = 0;  // per queue
+  char *scratch_base = nullptr;
+  void *scratch() const {
+    return scratch_base == nullptr ? nullptr : scratch_base + (size_t)tls_queue * scratch_bytes;
+  }
 };
 
 State &state();
+int sync_all_queues();
 int fail(int code, char const *fmt, ...);
 
 #define MI355_HIP(expr)                                                             \

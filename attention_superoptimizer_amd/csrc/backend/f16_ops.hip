@@ -190,7 +190,7 @@ extern "C" int mi355_f16_fill_iota(void *x, size_t n, int last_dim) {
   if (n == 0) {
     return MI355_OK;
   }
-  f16_fill_iota_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(
+  f16_fill_iota_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(
       static_cast<_Float16 *>(x), n, last_dim);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
@@ -201,7 +201,7 @@ extern "C" int mi355_f16_fill_normal(void *x, size_t n, float std, uint64_t seed
   if (n == 0) {
     return MI355_OK;
   }
-  f16_fill_normal_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(
+  f16_fill_normal_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(
       static_cast<_Float16 *>(x), n, std, seed);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
@@ -220,7 +220,7 @@ extern "C" int mi355_f16_matmul(void const *A, void const *B, void *C, int batch
     return fail(MI355_ERR_UNSUPPORTED, "batch %d exceeds grid.z", batch);
   }
   dim3 grid((n + 63) / 64, (m + 63) / 64, batch);
-  f16_matmul_kernel<<<grid, kThreads, 0, state().stream>>>(
+  f16_matmul_kernel<<<grid, kThreads, 0, state().stream()>>>(
       static_cast<_Float16 const *>(A), static_cast<_Float16 const *>(B),
       static_cast<_Float16 *>(C), m, n, k);
   MI355_HIP(hipGetLastError());
@@ -235,7 +235,7 @@ extern "C" int mi355_f16_unary(int op, void const *in, void *out, size_t n) {
   if (n == 0) {
     return MI355_OK;
   }
-  f16_unary_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(
+  f16_unary_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(
       op, static_cast<_Float16 const *>(in), static_cast<_Float16 *>(out), n);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
@@ -265,7 +265,7 @@ extern "C" int mi355_f16_binary(int op, void const *in1, int const *dims1, void 
     }
     n *= (size_t)dims_out[d];
   }
-  f16_binary_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(
+  f16_binary_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(
       op, static_cast<_Float16 const *>(in1), static_cast<_Float16 const *>(in2),
       static_cast<_Float16 *>(out), D, n);
   MI355_HIP(hipGetLastError());
@@ -282,7 +282,7 @@ extern "C" int mi355_f16_reduce(void const *in, void *out, size_t n_out, int fac
   if (n_out == 0) {
     return MI355_OK;
   }
-  hipStream_t st = state().stream;
+  hipStream_t st = state().stream();
   if (out_stride == 1 && factor >= 64) {
     size_t blocks = (n_out * 64 + kThreads - 1) / kThreads;
     f16_reduce_rows_kernel<<<(unsigned)blocks, kThreads, 0, st>>>(

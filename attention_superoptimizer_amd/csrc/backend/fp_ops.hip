@@ -9,6 +9,8 @@
 // is bit-identical for operands < 25651.
 #include "common.h"
 
+#include <algorithm>
+
 namespace mi355 {
 
 constexpr int kThreads = 256;
@@ -30,15 +32,61 @@ __global__ void fp_fill_iota_kernel(uint16_t *fp, size_t n) {
   }
 }
 
+__device__ __forceinline__ uint32_t uniform_value(uint64_t seed, size_t i) {
+  // v % 25651 for 64-bit v through 32-bit arithmetic: 2^32 = 15158 (mod 25651)
+  uint64_t const v = splitmix64(seed + i);
+  uint32_t const hi = static_cast<uint32_t>(v >> 32) % FP_PQ;
+  uint32_t const lo = static_cast<uint32_t>(v) % FP_PQ;
+  return (hi * 15158u + lo) % FP_PQ;
+}
+
+// eight values = one 16-byte store per thread and step (fp is 16-byte aligned)
 __global__ void fp_fill_uniform_kernel(uint16_t *fp, size_t n, uint64_t seed) {
-  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-  size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) * 8;
+  size_t const stride = (size_t)gridDim.x * blockDim.x * 8;
   for (; i < n; i += stride) {
-    // v % 25651 for 64-bit v through 32-bit arithmetic: 2^32 = 15158 (mod 25651)
-    uint64_t const v = splitmix64(seed + i);
-    uint32_t const hi = static_cast<uint32_t>(v >> 32) % FP_PQ;
-    uint32_t const lo = static_cast<uint32_t>(v) % FP_PQ;
-    fp[i] = static_cast<uint16_t>((hi * 15158u + lo) % FP_PQ);
+    if (i + 8 <= n) {
+      uint4v w;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        w[j] = uniform_value(seed, i + 2 * j) | (uniform_value(seed, i + 2 * j + 1) << 16);
+      }
+      *reinterpret_cast<uint4v *>(fp + i) = w;
+    } else {
+      for (size_t j = i; j < n; j++) {
+        fp[j] = static_cast<uint16_t>(uniform_value(seed, j));
+      }
+    }
+  }
+}
+
+// All inputs of one graph in a single launch: blockIdx.y names the tensor.
+struct FillMany {
+  uint16_t *ptr[MI355_MAX_FILL_TENSORS];
+  size_t n[MI355_MAX_FILL_TENSORS];
+  uint64_t seed[MI355_MAX_FILL_TENSORS];
+};
+
+__global__ void fp_fill_many_kernel(FillMany const F, int iota) {
+  uint16_t *fp = F.ptr[blockIdx.y];
+  size_t const n = F.n[blockIdx.y];
+  uint64_t const seed = F.seed[blockIdx.y];
+  size_t i = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) * 8;
+  size_t const stride = (size_t)gridDim.x * blockDim.x * 8;
+  for (; i < n; i += stride) {
+    size_t const end = i + 8 <= n ? i + 8 : n;
+    uint32_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t j = i; j < end; j++) {
+      v[j - i] = iota ? static_cast<uint32_t>(j % FP_PQ) : uniform_value(seed, j);
+    }
+    if (end == i + 8) {
+      uint4v w = {v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+      *reinterpret_cast<uint4v *>(fp + i) = w;
+    } else {
+      for (size_t j = i; j < end; j++) {
+        fp[j] = static_cast<uint16_t>(v[j - i]);
+      }
+    }
   }
 }
 
@@ -321,7 +369,7 @@ extern "C" int mi355_fp_fill_iota(uint16_t *fp, size_t n) {
   if (n == 0) {
     return MI355_OK;
   }
-  fp_fill_iota_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(fp, n);
+  fp_fill_iota_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(fp, n);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }
@@ -331,7 +379,37 @@ extern "C" int mi355_fp_fill_uniform(uint16_t *fp, size_t n, uint64_t seed) {
   if (n == 0) {
     return MI355_OK;
   }
-  fp_fill_uniform_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(fp, n, seed);
+  if ((reinterpret_cast<uintptr_t>(fp) & 15) != 0) {
+    return fail(MI355_ERR_INVALID, "fingerprint buffers are 16-byte aligned");
+  }
+  fp_fill_uniform_kernel<<<grid_for((n + 7) / 8), kThreads, 0, state().stream()>>>(fp, n, seed);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_fill_many(uint16_t *const *fp, size_t const *n, uint64_t const *seeds,
+                                  int count, int iota) {
+  MI355_REQUIRE_INIT();
+  if (count < 0 || count > MI355_MAX_FILL_TENSORS || (count > 0 && (fp == nullptr || n == nullptr)) ||
+      (!iota && count > 0 && seeds == nullptr)) {
+    return fail(MI355_ERR_INVALID, "bad tensor list (count %d)", count);
+  }
+  FillMany F{};
+  size_t largest = 0;
+  for (int i = 0; i < count; i++) {
+    if ((reinterpret_cast<uintptr_t>(fp[i]) & 15) != 0) {
+      return fail(MI355_ERR_INVALID, "fingerprint buffers are 16-byte aligned");
+    }
+    F.ptr[i] = fp[i];
+    F.n[i] = n[i];
+    F.seed[i] = iota ? 0 : seeds[i];
+    largest = std::max(largest, n[i]);
+  }
+  if (count == 0 || largest == 0) {
+    return MI355_OK;
+  }
+  dim3 grid(grid_for((largest + 7) / 8, kThreads, 2048), count);
+  fp_fill_many_kernel<<<grid, kThreads, 0, state().stream()>>>(F, iota);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }
@@ -348,7 +426,7 @@ extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C
   if (batch > 65535) {
     return fail(MI355_ERR_UNSUPPORTED, "batch %d exceeds grid.z", batch);
   }
-  hipStream_t st = state().stream;
+  hipStream_t st = state().stream();
   if (m >= 128) {
     dim3 grid((n + 63) / 64, (m + 127) / 128, batch);
     fp_matmul_kernel<8><<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
@@ -371,7 +449,7 @@ extern "C" int mi355_fp_unary(int op, uint16_t const *in, uint16_t *out, size_t 
   if (n == 0) {
     return MI355_OK;
   }
-  fp_unary_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(op, tables(), in, out, n);
+  fp_unary_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(op, tables(), in, out, n);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }
@@ -400,7 +478,7 @@ extern "C" int mi355_fp_binary(int op, uint16_t const *in1, int const *dims1,
     }
     n *= (size_t)dims_out[d];
   }
-  fp_binary_kernel<<<grid_for(n), kThreads, 0, state().stream>>>(op, tables(), in1, in2, out, D,
+  fp_binary_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(op, tables(), in1, in2, out, D,
                                                                n);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
@@ -416,7 +494,7 @@ extern "C" int mi355_fp_reduce(uint16_t const *in, uint16_t *out, size_t n_out, 
   if (n_out == 0) {
     return MI355_OK;
   }
-  hipStream_t st = state().stream;
+  hipStream_t st = state().stream();
   if (out_stride == 1 && factor >= 64) {
     size_t blocks = (n_out * 64 + kThreads - 1) / kThreads;
     fp_reduce_rows_kernel<<<(unsigned)blocks, kThreads, 0, st>>>(in, out, n_out, factor);
@@ -432,13 +510,16 @@ extern "C" int mi355_fp_reduce(uint16_t const *in, uint16_t *out, size_t n_out, 
 extern "C" int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, int *equal) {
   MI355_REQUIRE_INIT();
   State &s = state();
-  set_flag_kernel<<<1, 1, 0, s.stream>>>(s.flag, 1);
+  if (int rc = sync_all_queues()) {  // the operands may come from any queue
+    return rc;
+  }
+  set_flag_kernel<<<1, 1, 0, s.stream()>>>(s.flag, 1);
   if (n > 0) {
-    fp_equal_kernel<<<grid_for(n, kThreads, 2048), kThreads, 0, s.stream>>>(a, b, n, s.flag);
+    fp_equal_kernel<<<grid_for(n, kThreads, 2048), kThreads, 0, s.stream()>>>(a, b, n, s.flag);
   }
   MI355_HIP(hipGetLastError());
-  MI355_HIP(hipMemcpyAsync(s.flag_host, s.flag, sizeof(int), hipMemcpyDeviceToHost, s.stream));
-  MI355_HIP(hipStreamSynchronize(s.stream));
+  MI355_HIP(hipMemcpyAsync(s.flag_host, s.flag, sizeof(int), hipMemcpyDeviceToHost, s.stream()));
+  MI355_HIP(hipStreamSynchronize(s.stream()));
   *equal = *s.flag_host;
   return MI355_OK;
 }
@@ -480,7 +561,7 @@ extern "C" int mi355_fp_equal_reset(int first_slot, int count) {
                 first_slot + count);
   }
   if (count > 0) {
-    clear_slots_kernel<<<(count + kThreads - 1) / kThreads, kThreads, 0, s.stream>>>(
+    clear_slots_kernel<<<(count + kThreads - 1) / kThreads, kThreads, 0, s.stream()>>>(
         s.cmp_slots + first_slot, count);
     MI355_HIP(hipGetLastError());
   }
@@ -494,7 +575,7 @@ extern "C" int mi355_fp_equal_enqueue(uint16_t const *a, uint16_t const *b, size
     return fail(MI355_ERR_INVALID, "compare slot %d out of range", slot);
   }
   if (n > 0) {
-    fp_differ_kernel<<<grid_for((n + 7) / 8, kThreads, 1024), kThreads, 0, s.stream>>>(
+    fp_differ_kernel<<<grid_for((n + 7) / 8, kThreads, 1024), kThreads, 0, s.stream()>>>(
         a, b, n, s.cmp_slots + slot);
     MI355_HIP(hipGetLastError());
   }
@@ -512,9 +593,12 @@ extern "C" int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal)
   if (count == 0) {
     return MI355_OK;
   }
+  if (int rc = sync_all_queues()) {  // compares may sit on any queue
+    return rc;
+  }
   MI355_HIP(hipMemcpyAsync(s.cmp_host + first_slot, s.cmp_slots + first_slot,
-                           sizeof(int) * (size_t)count, hipMemcpyDeviceToHost, s.stream));
-  MI355_HIP(hipStreamSynchronize(s.stream));
+                           sizeof(int) * (size_t)count, hipMemcpyDeviceToHost, s.stream()));
+  MI355_HIP(hipStreamSynchronize(s.stream()));
   for (int i = 0; i < count; i++) {
     equal[i] = s.cmp_host[first_slot + i] == 0 ? 1 : 0;
   }

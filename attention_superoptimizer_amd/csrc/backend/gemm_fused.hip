@@ -509,7 +509,7 @@ int launch_kt(GemmParams const &A, dim3 grid, int lds) {
       MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     }
-    fn<<<grid, 256, lds, s.stream>>>(A);
+    fn<<<grid, 256, lds, s.stream()>>>(A);
     MI355_HIP(hipGetLastError());
     return 1;
   };
@@ -560,7 +560,7 @@ int try_launch_gemm(DevProgram const &P) {
     ksplit = 1;
   }
   A.ksplit = ksplit;
-  A.scratch = static_cast<_Float16 *>(s.scratch);
+  A.scratch = static_cast<_Float16 *>(s.scratch());
   int const tile_lds = (16 * mt * G.KT + G.nb * 64 * G.KT + (G.lora ? 16 * G.KT + 64 * 16 : 0)) * 2;
   int const out_lds = G.nb * 16 * mt * (64 + 8) * 2;
   int const lds = tile_lds > out_lds ? tile_lds : out_lds;
@@ -585,9 +585,9 @@ int try_launch_gemm(DevProgram const &P) {
   if (rc == 1 && ksplit > 1) {
     dim3 cgrid(P.grid[0], P.grid[1], P.grid[2]);
     if (G.nb == 1) {
-      gemm_combine_kernel<1><<<cgrid, 256, 0, s.stream>>>(A);
+      gemm_combine_kernel<1><<<cgrid, 256, 0, s.stream()>>>(A);
     } else {
-      gemm_combine_kernel<2><<<cgrid, 256, 0, s.stream>>>(A);
+      gemm_combine_kernel<2><<<cgrid, 256, 0, s.stream()>>>(A);
     }
     MI355_HIP(hipGetLastError());
   }

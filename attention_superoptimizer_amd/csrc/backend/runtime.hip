@@ -22,6 +22,18 @@ int fail(int code, char const *fmt, ...) {
   return code;
 }
 
+thread_local int tls_queue = 0;
+
+int sync_all_queues() {
+  State &s = state();
+  for (int i = 0; i < MI355_NUM_QUEUES; i++) {
+    if (s.queues[i] != nullptr) {
+      MI355_HIP(hipStreamSynchronize(s.queues[i]));
+    }
+  }
+  return MI355_OK;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -59,7 +71,10 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
       optin > 0) {
     s.max_lds = optin;
   }
-  MI355_HIP(hipStreamCreate(&s.stream));  // default priority
+  for (int i = 0; i < MI355_NUM_QUEUES; i++) {
+    MI355_HIP(hipStreamCreate(&s.queues[i]));  // default priority, all of them
+  }
+  tls_queue = 0;
   MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.arena), arena_bytes));
   s.arena_bytes = arena_bytes;
   // Tables: exp[i] = 3^i mod 227 (i < 113); div_p / div_q = modular inverses with
@@ -99,8 +114,9 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
                           hipHostMallocDefault));
   MI355_HIP(hipEventCreate(&s.ev0));
   MI355_HIP(hipEventCreate(&s.ev1));
-  s.scratch_bytes = (size_t)64 << 20;
-  MI355_HIP(hipMalloc(&s.scratch, s.scratch_bytes));
+  s.scratch_bytes = (size_t)64 << 20;  // per queue
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.scratch_base),
+                      s.scratch_bytes * MI355_NUM_QUEUES));
   s.ready = true;
   if (arena_base != nullptr) {
     *arena_base = s.arena;
@@ -113,7 +129,9 @@ extern "C" int mi355_shutdown(void) {
   if (!s.ready) {
     return MI355_OK;
   }
-  MI355_HIP(hipStreamSynchronize(s.stream));
+  if (int rc = sync_all_queues()) {
+    return rc;
+  }
   MI355_HIP(hipEventDestroy(s.ev0));
   MI355_HIP(hipEventDestroy(s.ev1));
   MI355_HIP(hipFree(s.arena));
@@ -122,8 +140,10 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipHostFree(s.flag_host));
   MI355_HIP(hipFree(s.cmp_slots));
   MI355_HIP(hipHostFree(s.cmp_host));
-  MI355_HIP(hipFree(s.scratch));
-  MI355_HIP(hipStreamDestroy(s.stream));
+  MI355_HIP(hipFree(s.scratch_base));
+  for (int i = 0; i < MI355_NUM_QUEUES; i++) {
+    MI355_HIP(hipStreamDestroy(s.queues[i]));
+  }
   s = State{};
   return MI355_OK;
 }
@@ -188,7 +208,7 @@ extern "C" int mi355_copy(void *dst, void const *src, size_t bytes) {
   int tail = (int)(bytes % 16);
   size_t blocks = (n16 + 255) / 256;
   blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
-  copy_kernel<<<(unsigned)blocks, 256, 0, state().stream>>>(
+  copy_kernel<<<(unsigned)blocks, 256, 0, state().stream()>>>(
       static_cast<uint4 const *>(src), static_cast<uint4 *>(dst), n16,
       static_cast<unsigned char const *>(src) + n16 * 16, static_cast<unsigned char *>(dst) + n16 * 16,
       tail);
@@ -203,13 +223,13 @@ extern "C" int mi355_launch_floor(int iters, float *us) {
   }
   State &s = state();
   for (int i = 0; i < 64; i++) {
-    empty_kernel<<<1, 64, 0, s.stream>>>();
+    empty_kernel<<<1, 64, 0, s.stream()>>>();
   }
-  MI355_HIP(hipEventRecord(s.ev0, s.stream));
+  MI355_HIP(hipEventRecord(s.ev0, s.stream()));
   for (int i = 0; i < iters; i++) {
-    empty_kernel<<<1, 64, 0, s.stream>>>();
+    empty_kernel<<<1, 64, 0, s.stream()>>>();
   }
-  MI355_HIP(hipEventRecord(s.ev1, s.stream));
+  MI355_HIP(hipEventRecord(s.ev1, s.stream()));
   MI355_HIP(hipEventSynchronize(s.ev1));
   float ms = 0.0f;
   MI355_HIP(hipEventElapsedTime(&ms, s.ev0, s.ev1));
@@ -227,39 +247,54 @@ extern "C" int mi355_get_tables(void const **exp_tbl, void const **div_p, void c
 
 extern "C" int mi355_memcpy_h2d(void *dst, void const *src, size_t bytes) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, state().stream));
-  MI355_HIP(hipStreamSynchronize(state().stream));
+  if (int rc = sync_all_queues()) {  // work on any queue may still read dst
+    return rc;
+  }
+  MI355_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, state().stream()));
+  MI355_HIP(hipStreamSynchronize(state().stream()));
   return MI355_OK;
 }
 
 extern "C" int mi355_memcpy_d2h(void *dst, void const *src, size_t bytes) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, state().stream));
-  MI355_HIP(hipStreamSynchronize(state().stream));
+  if (int rc = sync_all_queues()) {  // src may be produced on any queue
+    return rc;
+  }
+  MI355_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, state().stream()));
+  MI355_HIP(hipStreamSynchronize(state().stream()));
+  return MI355_OK;
+}
+
+extern "C" int mi355_queue_select(int queue) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (queue < 0 || queue >= MI355_NUM_QUEUES) {
+    return fail(MI355_ERR_INVALID, "queue %d out of range [0, %d)", queue, MI355_NUM_QUEUES);
+  }
+  tls_queue = queue;
   return MI355_OK;
 }
 
 extern "C" int mi355_memset(void *dst, int value, size_t bytes) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipMemsetAsync(dst, value, bytes, state().stream));
+  MI355_HIP(hipMemsetAsync(dst, value, bytes, state().stream()));
   return MI355_OK;
 }
 
 extern "C" int mi355_sync(void) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipStreamSynchronize(state().stream));
-  return MI355_OK;
+  return sync_all_queues();
 }
 
 extern "C" int mi355_timer_start(void) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipEventRecord(state().ev0, state().stream));
+  MI355_HIP(hipEventRecord(state().ev0, state().stream()));
   return MI355_OK;
 }
 
 extern "C" int mi355_timer_stop(float *ms) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipEventRecord(state().ev1, state().stream));
+  MI355_HIP(hipEventRecord(state().ev1, state().stream()));
   MI355_HIP(hipEventSynchronize(state().ev1));
   MI355_HIP(hipEventElapsedTime(ms, state().ev0, state().ev1));
   return MI355_OK;

@@ -625,7 +625,7 @@ static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outp
   prog.splits = 1;
   int const blocks = prog.grid[0] * prog.grid[1] * prog.grid[2];
   int const F = prog.forloop_range;
-  if (F < 2 || blocks >= 192 || s.scratch == nullptr) {
+  if (F < 2 || blocks >= 192 || s.scratch() == nullptr) {
     return;
   }
   int splits = std::min(std::min(F, 64), (256 + blocks - 1) / blocks);
@@ -640,7 +640,7 @@ static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outp
     return;
   }
   prog.splits = splits;
-  uint16_t *p = static_cast<uint16_t *>(s.scratch);
+  uint16_t *p = static_cast<uint16_t *>(s.scratch());
   for (int i = 0; i < num_outputs; i++) {
     prog.part[i] = p;
     prog.part_elems[i] = ext.out_elems[i];
@@ -731,9 +731,9 @@ static int launch(DevProgram const &prog, bool f16) {
     cur = s.max_lds;
   }
   if (f16) {
-    f16_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream>>>(prog);
+    f16_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog);
   } else {
-    fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream>>>(prog, s.exp_tbl,
+    fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog, s.exp_tbl,
                                                                           s.div_p, s.div_q);
     if (prog.splits > 1) {
       for (int o = 0; o < MI355_MAX_DMEM_OUTPUTS; o++) {
@@ -742,7 +742,7 @@ static int launch(DevProgram const &prog, bool f16) {
         }
         long long const n = prog.part_elems[o];
         int const blocks = (int)std::min<long long>((n + 255) / 256, 2048);
-        fp_combine_splits_kernel<<<blocks, 256, 0, s.stream>>>(
+        fp_combine_splits_kernel<<<blocks, 256, 0, s.stream()>>>(
             prog.part[o], static_cast<uint16_t *>(prog.out[o]), n, prog.splits);
       }
     }
@@ -834,14 +834,14 @@ extern "C" int mi355_customized_profile(mi355_plan const *plan, void const *cons
       return rc;
     }
   }
-  MI355_HIP(hipEventRecord(s.ev0, s.stream));
+  MI355_HIP(hipEventRecord(s.ev0, s.stream()));
   for (int i = 0; i < iters; i++) {
     rc = launch(prog, fingerprint == 0);
     if (rc != MI355_OK) {
       return rc;
     }
   }
-  MI355_HIP(hipEventRecord(s.ev1, s.stream));
+  MI355_HIP(hipEventRecord(s.ev1, s.stream()));
   MI355_HIP(hipEventSynchronize(s.ev1));
   float total = 0.0f;
   MI355_HIP(hipEventElapsedTime(&total, s.ev0, s.ev1));

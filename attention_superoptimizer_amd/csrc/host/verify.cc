@@ -9,7 +9,9 @@
 #include "mirage/utils/hip_types.h"
 
 #include <algorithm>
+#include <chrono>
 #include <numeric>
+#include <thread>
 #include <unordered_set>
 
 namespace mirage {
@@ -71,18 +73,36 @@ static void account(KNOperator const *op, VerifyStats *stats) {
 
 void fingerprint_graph(kernel::Graph const &g, uint64_t input_seed, VerifyStats *stats) {
   kernel::require_device("fingerprint_graph");
+  // inputs depend on nothing: all of them in one launch (batches of MI355_MAX_FILL_TENSORS)
+  uint16_t *ptrs[MI355_MAX_FILL_TENSORS];
+  size_t counts[MI355_MAX_FILL_TENSORS];
+  uint64_t seeds[MI355_MAX_FILL_TENSORS];
+  int pending = 0;
   uint64_t ordinal = 0;
+  auto flush = [&]() {
+    if (pending > 0) {
+      MI355_CALL(mi355_fp_fill_many(ptrs, counts, seeds, pending, input_seed == 0 ? 1 : 0));
+      pending = 0;
+    }
+  };
+  for (KNOperator *op : g.operators) {
+    if (op->op_type != KN_INPUT_OP) {
+      continue;
+    }
+    DTensor const &t = op->output_tensors[0];
+    ptrs[pending] = t.fp_ptr;
+    counts[pending] = t.num_elements();
+    seeds[pending] = input_seed ^ (ordinal << 40);
+    ordinal++;
+    if (++pending == MI355_MAX_FILL_TENSORS) {
+      flush();
+    }
+  }
+  flush();
   for (KNOperator *op : g.operators) {
     account(op, stats);
-    if (op->op_type == KN_INPUT_OP && input_seed != 0) {
-      DTensor const &t = op->output_tensors[0];
-      MI355_CALL(mi355_fp_fill_uniform(t.fp_ptr, t.num_elements(),
-                                       input_seed ^ (ordinal << 40)));
-    } else {
+    if (op->op_type != KN_INPUT_OP) {
       op->fingerprint();
-    }
-    if (op->op_type == KN_INPUT_OP) {
-      ordinal++;
     }
   }
 }
@@ -119,33 +139,70 @@ void verify_batch(std::vector<kernel::Graph *> const &candidates,
     }
   }
   MIRAGE_CHECK(slots <= MI355_COMPARE_SLOTS, "too many compares for one verify_batch call");
+  auto const t0 = std::chrono::steady_clock::now();
   MI355_CALL(mi355_fp_equal_reset(0, slots));
+  // Candidates are independent: deal them over the backend's queues so their small
+  // kernels overlap.  Everything enqueued so far (the reference's fingerprints, the slot
+  // reset) must be complete before another queue may depend on it.
+  MI355_CALL(mi355_sync());
   // which (reference, candidate) output pairs can be equal at all
   std::vector<uint8_t> possible((size_t)slots, 0);
-  for (size_t i = 0; i < n; i++) {
-    fingerprint_graph(*candidates[i], input_seed, stats);
-    if (pend[i].first_slot < 0) {
-      continue;
-    }
-    for (size_t r = 0; r < no; r++) {
-      for (size_t c = 0; c < no; c++) {
-        if (!comparable(reference_outputs[r], pend[i].outputs[c])) {
-          continue;
-        }
-        int const slot = pend[i].first_slot + (int)(r * no + c);
-        possible[slot] = 1;
-        MI355_CALL(mi355_fp_equal_enqueue(reference_outputs[r].fp_ptr,
-                                          pend[i].outputs[c].fp_ptr,
-                                          reference_outputs[r].num_elements(), slot));
-        if (stats != nullptr) {
-          stats->compares++;
-          stats->fp_bytes += 2 * (long long)reference_outputs[r].fingerprint_size();
+  // one host thread per queue: candidate i is lowered and enqueued by thread i % queues
+  int const workers = (int)std::min<size_t>(MI355_NUM_QUEUES, n);
+  std::vector<VerifyStats> local((size_t)std::max(workers, 1));
+  auto work = [&](int w) {
+    MI355_CALL(mi355_queue_select(w));
+    for (size_t i = (size_t)w; i < n; i += (size_t)workers) {
+      fingerprint_graph(*candidates[i], input_seed, &local[w]);
+      if (pend[i].first_slot < 0) {
+        continue;
+      }
+      for (size_t r = 0; r < no; r++) {
+        for (size_t c = 0; c < no; c++) {
+          if (!comparable(reference_outputs[r], pend[i].outputs[c])) {
+            continue;
+          }
+          int const slot = pend[i].first_slot + (int)(r * no + c);
+          possible[slot] = 1;
+          MI355_CALL(mi355_fp_equal_enqueue(reference_outputs[r].fp_ptr,
+                                            pend[i].outputs[c].fp_ptr,
+                                            reference_outputs[r].num_elements(), slot));
+          local[w].compares++;
+          local[w].fp_bytes += 2 * (long long)reference_outputs[r].fingerprint_size();
         }
       }
     }
+  };
+  {
+    std::vector<std::thread> threads;
+    for (int w = 1; w < workers; w++) {
+      threads.emplace_back(work, w);
+    }
+    if (workers > 0) {
+      work(0);
+    }
+    for (std::thread &t : threads) {
+      t.join();
+    }
   }
+  if (stats != nullptr) {
+    for (VerifyStats const &l : local) {
+      stats->kernel_ops += l.kernel_ops;
+      stats->customized_ops += l.customized_ops;
+      stats->compares += l.compares;
+      stats->fp_bytes += l.fp_bytes;
+      stats->matmul_macs += l.matmul_macs;
+    }
+  }
+  MI355_CALL(mi355_queue_select(0));
+  auto const t1 = std::chrono::steady_clock::now();
   std::vector<uint8_t> same((size_t)slots, 0);
   MI355_CALL(mi355_fp_equal_collect(0, slots, same.data()));
+  if (stats != nullptr) {
+    auto const t2 = std::chrono::steady_clock::now();
+    stats->enqueue_seconds += std::chrono::duration<double>(t1 - t0).count();
+    stats->wait_seconds += std::chrono::duration<double>(t2 - t1).count();
+  }
   std::vector<int> perm(no);
   for (size_t i = 0; i < n; i++) {
     if (pend[i].first_slot < 0) {
@@ -175,6 +232,7 @@ extern "C" {
 typedef struct mirage_verify_stats {
   int kernel_ops, customized_ops, compares;
   long long fp_bytes, matmul_macs;
+  double enqueue_seconds, wait_seconds;
 } mirage_verify_stats;
 
 static void export_stats(mirage::search::VerifyStats const &s, mirage_verify_stats *out) {
@@ -184,6 +242,8 @@ static void export_stats(mirage::search::VerifyStats const &s, mirage_verify_sta
     out->compares = s.compares;
     out->fp_bytes = s.fp_bytes;
     out->matmul_macs = s.matmul_macs;
+    out->enqueue_seconds = s.enqueue_seconds;
+    out->wait_seconds = s.wait_seconds;
   }
 }
 

@@ -238,7 +238,8 @@ class KNGraph:
 
 def _stats(st) -> dict:
     return {"kernel_ops": st.kernel_ops, "customized_ops": st.customized_ops,
-            "compares": st.compares, "fp_bytes": st.fp_bytes, "matmul_macs": st.matmul_macs}
+            "compares": st.compares, "fp_bytes": st.fp_bytes, "matmul_macs": st.matmul_macs,
+            "enqueue_seconds": st.enqueue_seconds, "wait_seconds": st.wait_seconds}
 
 
 def verify_batch(candidates: Sequence["KNGraph"], reference: "KNGraph", input_seed: int = 0):

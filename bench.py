@@ -70,7 +70,8 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
     from attention_superoptimizer_amd import candidates as C
     probs = C.generate(num_problems=num_problems, per_problem=per_problem)
     t_build = t_verify = 0.0
-    tot = {"kernel_ops": 0, "customized_ops": 0, "compares": 0, "fp_bytes": 0, "matmul_macs": 0}
+    tot = {"kernel_ops": 0, "customized_ops": 0, "compares": 0, "fp_bytes": 0, "matmul_macs": 0,
+           "enqueue_seconds": 0.0, "wait_seconds": 0.0}
     n = wrong = 0
     for prob in probs:
         ref_g, _ = G.build_from_spec(prob["reference"])
@@ -91,7 +92,8 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
         ref_g.close()
     rec = {
         "candidates": n, "problems": len(probs), "candidates_per_s": round(n / t_verify, 1),
-        "verify_s": round(t_verify, 4), "host_graph_build_s": round(t_build, 4),
+        "verify_s": round(t_verify, 4), "host_enqueue_s": round(tot["enqueue_seconds"], 4),
+        "final_wait_s": round(tot["wait_seconds"], 4), "host_graph_build_s": round(t_build, 4),
         "kernel_ops": tot["kernel_ops"], "customized_ops": tot["customized_ops"],
         "compares": tot["compares"],
         "fingerprint_GBps": round(tot["fp_bytes"] / t_verify / 1e9, 2),

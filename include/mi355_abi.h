@@ -116,6 +116,16 @@ int mi355_memset(void *dst, int value, size_t bytes);
  * Also the known-size reference that hardware byte counters are scaled against. */
 int mi355_copy(void *dst, void const *src, size_t bytes);
 int mi355_sync(void);
+/* The backend owns MI355_NUM_QUEUES in-order queues (HIP streams, all at the default
+ * priority).  Every call enqueues on the queue its host thread selected (queue 0 until the
+ * thread selects another), so host threads can enqueue side by side; work on different
+ * queues may overlap on the device, which is how a batch of independent candidate graphs
+ * fills the chip with its many small kernels (the reference has one stream and a
+ * cudaDeviceSynchronize after every fingerprint launch, customized_kernel.cu:676).
+ * mi355_sync, the memcpy calls and mi355_fp_equal_collect wait for all queues.  The
+ * caller orders dependent work itself: same queue, or a mi355_sync in between. */
+#define MI355_NUM_QUEUES 4
+int mi355_queue_select(int queue);
 
 /* ---- fingerprint path (uint16 over Z_25651, integer only) ------------------ */
 /* init_input_fingerprint, src/kernel/cuda/input_kernel.cu:56-72: fp[i] = i % 25651 */
@@ -123,6 +133,12 @@ int mi355_fp_fill_iota(uint16_t *fp, size_t n);
 /* seeded inputs: fp[i] = splitmix64(seed + i) % 25651 (no reference counterpart;
  * the reference's FIXME at input_kernel.cu:59 asks for random inputs) */
 int mi355_fp_fill_uniform(uint16_t *fp, size_t n, uint64_t seed);
+/* Every input of one graph in a single launch (init_input_fingerprint once per tensor in
+ * the reference, input_kernel.cu:56-72): tensor i gets `idx % 25651` when iota != 0, else
+ * the uniform values of mi355_fp_fill_uniform with seeds[i]. */
+#define MI355_MAX_FILL_TENSORS 8
+int mi355_fp_fill_many(uint16_t *const *fp, size_t const *n, uint64_t const *seeds, int count,
+                       int iota);
 /* compute_matmul_fingerprint, src/kernel/cuda/matmul_kernel.cu:145-203 */
 int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m,
                     int n, int k);

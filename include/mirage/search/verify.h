@@ -27,6 +27,8 @@ struct VerifyStats {
   int compares = 0;           // on-device compares enqueued
   long long fp_bytes = 0;     // 2 B x (input + output elements) over all operators
   long long matmul_macs = 0;  // m*n*k over kernel-level and thread-block matmuls
+  double enqueue_seconds = 0; // host time spent lowering and enqueueing (verify_batch)
+  double wait_seconds = 0;    // host time spent in the final synchronisation
 };
 
 // equal[i] = 1 iff candidate i has as many outputs as `reference_outputs` and some
