@@ -216,6 +216,123 @@ __global__ __launch_bounds__(kThreads) void fp_matmul_kernel(uint16_t const *__r
   }
 }
 
+// Aligned fast path: m, n, k multiples of 64 and 16-byte aligned matrices.  One workgroup
+// owns a 64 x 64 output tile and walks k in chunks of 64.  The raw uint16 of chunk i + 1
+// are in flight in registers while chunk i is multiplied; they are split into residues
+// on their way into LDS (Ap[f][q][row], Bp[f][q][col], one dword = four consecutive k),
+// which is double-buffered, so a chunk costs one barrier.  Thread (ty, tx) owns the
+// 4 x 4 outputs at rows 4*ty, columns 4*tx and keeps both residue sums in registers for
+// the whole k range (64 * 226^2 per chunk: 2^32 is reached after 1300 chunks; sums are
+// folded every 1024).
+__global__ __launch_bounds__(kThreads) void fp_matmul64_kernel(uint16_t const *__restrict__ A,
+                                                              uint16_t const *__restrict__ B,
+                                                              uint16_t *__restrict__ C, int m,
+                                                              int n, int k) {
+  constexpr int LDA = 68, KQ = 16;
+  constexpr int BUF = 2 * KQ * LDA + 2 * KQ * 64;  // dwords per buffer
+  __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF];
+  int const tid = threadIdx.x;
+  size_t const b = blockIdx.z;
+  A += b * (size_t)m * k + (size_t)blockIdx.y * 64 * k;
+  B += b * (size_t)k * n + (size_t)blockIdx.x * 64;
+  C += b * (size_t)m * n + (size_t)blockIdx.y * 64 * n + (size_t)blockIdx.x * 64;
+  // staging roles: A as 2 x (row, 8 consecutive k), B as (4 consecutive k) x 4 columns
+  int const a_row = tid / 8, a_k8 = (tid % 8) * 8;  // second patch: row + 32
+  int const b_q = tid / 16, b_c4 = (tid % 16) * 4;
+  uint4v ra[2];
+  uint2 rb[4];
+  auto fetch = [&](int k0) {
+    ra[0] = *reinterpret_cast<uint4v const *>(A + (size_t)a_row * k + k0 + a_k8);
+    ra[1] = *reinterpret_cast<uint4v const *>(A + (size_t)(a_row + 32) * k + k0 + a_k8);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      rb[j] = *reinterpret_cast<uint2 const *>(B + (size_t)(k0 + 4 * b_q + j) * n + b_c4);
+    }
+  };
+  auto stage = [&](int buf) {
+    uint32_t *Ap = lds + buf * BUF, *Bp = Ap + 2 * KQ * LDA;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      int const row = a_row + 32 * h, q = a_k8 / 4;
+      uint32_t pp, qq;
+      residues4(ra[h][0] & 0xffffu, ra[h][0] >> 16, ra[h][1] & 0xffffu, ra[h][1] >> 16, pp, qq);
+      Ap[q * LDA + row] = pp;
+      Ap[(KQ + q) * LDA + row] = qq;
+      residues4(ra[h][2] & 0xffffu, ra[h][2] >> 16, ra[h][3] & 0xffffu, ra[h][3] >> 16, pp, qq);
+      Ap[(q + 1) * LDA + row] = pp;
+      Ap[(KQ + q + 1) * LDA + row] = qq;
+    }
+    uint32_t bp[4], bq[4];
+    residues4(rb[0].x & 0xffffu, rb[1].x & 0xffffu, rb[2].x & 0xffffu, rb[3].x & 0xffffu, bp[0], bq[0]);
+    residues4(rb[0].x >> 16, rb[1].x >> 16, rb[2].x >> 16, rb[3].x >> 16, bp[1], bq[1]);
+    residues4(rb[0].y & 0xffffu, rb[1].y & 0xffffu, rb[2].y & 0xffffu, rb[3].y & 0xffffu, bp[2], bq[2]);
+    residues4(rb[0].y >> 16, rb[1].y >> 16, rb[2].y >> 16, rb[3].y >> 16, bp[3], bq[3]);
+    *reinterpret_cast<uint4v *>(Bp + b_q * 64 + b_c4) = uint4v{bp[0], bp[1], bp[2], bp[3]};
+    *reinterpret_cast<uint4v *>(Bp + (KQ + b_q) * 64 + b_c4) = uint4v{bq[0], bq[1], bq[2], bq[3]};
+  };
+  int const r0 = (tid / 16) * 4, c0 = (tid % 16) * 4;
+  uint32_t accp[4][4], accq[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      accp[i][j] = 0;
+      accq[i][j] = 0;
+    }
+  }
+  int const chunks = k / 64;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (int ch = 0; ch < chunks; ch++) {
+    if (ch + 1 < chunks) {
+      fetch((ch + 1) * 64);
+    }
+    uint32_t const *ap = lds + (ch & 1) * BUF + r0, *bp = lds + (ch & 1) * BUF + 2 * KQ * LDA + c0;
+#pragma unroll 4
+    for (int q = 0; q < KQ; q++) {
+      uint4v a_p = *reinterpret_cast<uint4v const *>(ap + q * LDA);
+      uint4v a_q = *reinterpret_cast<uint4v const *>(ap + (KQ + q) * LDA);
+      uint4v b_p = *reinterpret_cast<uint4v const *>(bp + q * 64);
+      uint4v b_q = *reinterpret_cast<uint4v const *>(bp + (KQ + q) * 64);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          accp[i][j] = __builtin_amdgcn_udot4(a_p[i], b_p[j], accp[i][j], false);
+          accq[i][j] = __builtin_amdgcn_udot4(a_q[i], b_q[j], accq[i][j], false);
+        }
+      }
+    }
+    if ((ch & 1023) == 1023) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          accp[i][j] %= FP_P;
+          accq[i][j] %= FP_Q;
+        }
+      }
+    }
+    if (ch + 1 < chunks) {
+      stage((ch + 1) & 1);  // that buffer was last read in chunk ch - 1
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    uint32_t z[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      z[j] = ((accp[i][j] % FP_P) * FP_Q_MUL_P_MOD_1 + (accq[i][j] % FP_Q) * FP_P_MUL_Q_MOD_1) % FP_PQ;
+    }
+    uint2 out;
+    out.x = z[0] | (z[1] << 16);
+    out.y = z[2] | (z[3] << 16);
+    *reinterpret_cast<uint2 *>(C + (size_t)(r0 + i) * n + c0) = out;
+  }
+}
+
 // ---- element-wise ---------------------------------------------------------------
 struct FpTables {
   uint16_t const *exp_tbl, *div_p, *div_q;
@@ -427,7 +544,13 @@ extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C
     return fail(MI355_ERR_UNSUPPORTED, "batch %d exceeds grid.z", batch);
   }
   hipStream_t st = state().stream();
-  if (m >= 128) {
+  bool const aligned = m % 64 == 0 && n % 64 == 0 && k % 64 == 0 && k > 0 &&
+                       ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
+                         reinterpret_cast<uintptr_t>(C)) & 15) == 0;
+  if (aligned) {
+    dim3 grid(n / 64, m / 64, batch);
+    fp_matmul64_kernel<<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
+  } else if (m >= 128) {
     dim3 grid((n + 63) / 64, (m + 127) / 128, batch);
     fp_matmul_kernel<8><<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
   } else if (m >= 33) {

@@ -475,6 +475,25 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
     }
     prog.lds_bytes = peak + scratch;
   }
+  for (int i = 0; i < prog.num_tensors; i++) {
+    prog.t[i].mcols = fast_div_magic(prog.t[i].cols);
+    prog.t[i].mcpr = fast_div_magic(prog.t[i].cols / 8);
+  }
+  for (int o = 0; o < prog.num_ops; o++) {
+    DevOp &d = prog.ops[o];
+    d.mg0 = d.mg1 = d.mg2 = 0;
+    if (d.kind == DOP_MATMUL) {
+      int const n = prog.t[d.src1].cols;
+      d.mg0 = fast_div_magic(d.mm_kc / 4);
+      d.mg1 = fast_div_magic(n / 2);
+      d.mg2 = fast_div_magic(n / 4);
+    } else if (d.kind == DOP_REDUCE) {
+      d.mg0 = fast_div_magic(d.red_inner);
+    } else if (d.kind == DOP_CONCAT) {
+      d.mg0 = fast_div_magic(d.cat_inner);
+      d.mg1 = fast_div_magic(d.cat_a + d.cat_b);
+    }
+  }
   // LDS writes of 16 bytes need 8-element row strides on the destination
   for (int o = 0; o < prog.num_ops; o++) {
     DevOp &d = prog.ops[o];

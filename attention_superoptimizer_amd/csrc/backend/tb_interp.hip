@@ -58,6 +58,12 @@ __device__ __forceinline__ uint32_t lds_silu(uint16_t const *tbl, uint32_t x) {
   return lds_div(tbl, x, den);
 }
 
+// Tile index arithmetic without integer division: q = e / d for e * d < 2^32 is one
+// multiply-high with magic = ceil(2^32 / d) (0 stands for d == 1), computed on the host.
+__device__ __forceinline__ int fdiv(int e, uint32_t magic) {
+  return magic ? (int)__umulhi((uint32_t)e, magic) : e;
+}
+
 // C[m][n] = A[m][k] . B[k][n] over Z_25651 without a modulus in the inner loop:
 // every operand is split into its residues modulo 227 and 113 (both fit a byte), four
 // consecutive k are packed into one dword per field, and the packed 4 x 8-bit dot
@@ -72,23 +78,23 @@ __device__ __forceinline__ uint32_t pack_residues(uint32_t v0, uint32_t v1, uint
 }
 
 __device__ void fp_matmul_packed(uint16_t const *A, uint16_t const *B, uint16_t *C, int m, int n,
-                                 int k, int kc, uint32_t *scratch, int tid) {
-  int const kq = kc / 4, lda = m + 4;
+                                 int k, DevOp const &op, uint32_t *scratch, int tid) {
+  int const kc = op.mm_kc, kq = kc / 4, lda = m + 4;
   uint32_t *Ap = scratch, *Bp = scratch + 2 * kq * lda;
-  int const n4 = n / 4, tiles = (m / 4) * n4;
+  int const n2 = n / 2, n4 = n / 4, tiles = (m / 4) * n4;
   for (int k0 = 0; k0 < k; k0 += kc) {
     if (k0 > 0) {
       __syncthreads();  // the previous chunk's residues are still being read
     }
     for (int e = tid; e < m * kq; e += kInterpThreads) {
-      int const row = e / kq, q = e % kq;
+      int const row = fdiv(e, op.mg0), q = e - row * kq;
       uint2 v = *reinterpret_cast<uint2 const *>(A + row * k + k0 + 4 * q);
       uint32_t v0 = v.x & 0xffffu, v1 = v.x >> 16, v2 = v.y & 0xffffu, v3 = v.y >> 16;
       Ap[q * lda + row] = pack_residues(v0, v1, v2, v3, FP_P);
       Ap[(kq + q) * lda + row] = pack_residues(v0, v1, v2, v3, FP_Q);
     }
-    for (int e = tid; e < kq * (n / 2); e += kInterpThreads) {
-      int const q = e / (n / 2), c2 = (e % (n / 2)) * 2;
+    for (int e = tid; e < kq * n2; e += kInterpThreads) {
+      int const q = fdiv(e, op.mg1), c2 = (e - q * n2) * 2;
       uint16_t const *bp = B + (k0 + 4 * q) * n + c2;
       uint32_t w0 = *reinterpret_cast<uint32_t const *>(bp);
       uint32_t w1 = *reinterpret_cast<uint32_t const *>(bp + n);
@@ -104,7 +110,7 @@ __device__ void fp_matmul_packed(uint16_t const *A, uint16_t const *B, uint16_t 
     }
     __syncthreads();
     for (int t = tid; t < tiles; t += kInterpThreads) {
-      int const r0 = (t / n4) * 4, c0 = (t % n4) * 4;
+      int const tr = fdiv(t, op.mg2), r0 = tr * 4, c0 = (t - tr * n4) * 4;
       uint32_t accp[4][4], accq[4][4];
 #pragma unroll
       for (int i = 0; i < 4; i++) {
@@ -154,6 +160,13 @@ __device__ void fp_matmul_packed(uint16_t const *A, uint16_t const *B, uint16_t 
   }
 }
 
+__device__ __forceinline__ uint32_t add_mod_pair(uint32_t a, uint32_t b) {
+  // two uint16 lanes: (a + b) mod 25651 in each
+  uint32_t lo = ((a & 0xffffu) + (b & 0xffffu)) % FP_PQ;
+  uint32_t hi = ((a >> 16) + (b >> 16)) % FP_PQ;
+  return lo | (hi << 16);
+}
+
 __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
     DevProgram const P, uint16_t const *__restrict__ g_exp, uint16_t const *__restrict__ g_divp,
     uint16_t const *__restrict__ g_divq) {
@@ -184,76 +197,50 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           DevTensor const &t = P.t[op.dst];
           uint16_t *s = reinterpret_cast<uint16_t *>(lds + t.off);
           TileOrigin org = tile_origin(op, it, bx);
-          uint16_t const *g = static_cast<uint16_t const *>(P.in[op.io]) + org.base;
+          uint16_t const *g = static_cast<uint16_t const *>(P.in[op.io]) + org.base +
+                              (long long)org.row0 * op.d_cols + org.col0;
           if (op.vec8) {
             int const cpr = t.cols / 8, n = t.rows * cpr;
             for (int e = tid; e < n; e += kInterpThreads) {
-              int r = e / cpr, c = (e % cpr) * 8;
-              uint4v v = *reinterpret_cast<uint4v const *>(
-                  g + (long long)(org.row0 + r) * op.d_cols + org.col0 + c);
+              int const r = fdiv(e, t.mcpr), c = (e - r * cpr) * 8;
+              uint4v v = *reinterpret_cast<uint4v const *>(g + (long long)r * op.d_cols + c);
               *reinterpret_cast<uint4v *>(s + r * t.cols + c) = v;
             }
           } else {
             int const n = t.rows * t.cols;
             for (int e = tid; e < n; e += kInterpThreads) {
-              int r = e / t.cols, c = e % t.cols;
-              s[e] = g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c];
+              int const r = fdiv(e, t.mcols), c = e - r * t.cols;
+              s[e] = g[(long long)r * op.d_cols + c];
             }
           }
           break;
         }
         case DOP_MATMUL: {
-          // reference matmul.h:773-804; the modulus is applied every 4 products
-          // (4 * 25650^2 + 25650 < 2^32), same ring value as reducing each step
+          // reference matmul.h:773-804
           DevTensor const &ta = P.t[op.src0], &tb = P.t[op.src1], &tc = P.t[op.dst];
           uint16_t const *A = reinterpret_cast<uint16_t const *>(lds + ta.off);
           uint16_t const *B = reinterpret_cast<uint16_t const *>(lds + tb.off);
           uint16_t *C = reinterpret_cast<uint16_t *>(lds + tc.off);
           int const m = ta.rows, k = ta.cols, n = tb.cols;
           if (op.mm_kc > 0) {
-            fp_matmul_packed(A, B, C, m, n, k, op.mm_kc,
-                             reinterpret_cast<uint32_t *>(lds + P.mm_off), tid);
-          } else if (n % 4 == 0) {
-            int const n4 = n / 4, total = m * n4;
+            fp_matmul_packed(A, B, C, m, n, k, op, reinterpret_cast<uint32_t *>(lds + P.mm_off),
+                             tid);
+          } else {
+            // shapes the packed path does not take; the modulus is applied every 4
+            // products (4 * 25650^2 + 25650 < 2^32), same ring value as reducing each step
+            int const total = m * n;
             for (int e = tid; e < total; e += kInterpThreads) {
-              int row = e / n4, c0 = (e % n4) * 4;
-              uint32_t acc[4] = {0, 0, 0, 0};
-              uint16_t const *ap = A + row * k;
-              uint16_t const *bp = B + c0;
+              int const row = fdiv(e, tb.mcols), col = e - row * n;
+              uint32_t acc = 0;
               int kk = 0;
               for (; kk + 4 <= k; kk += 4) {
 #pragma unroll
                 for (int u = 0; u < 4; u++) {
-                  uint32_t a = ap[kk + u];
-                  uint2 bv = *reinterpret_cast<uint2 const *>(bp + (kk + u) * n);
-                  acc[0] += a * (bv.x & 0xffffu);
-                  acc[1] += a * (bv.x >> 16);
-                  acc[2] += a * (bv.y & 0xffffu);
-                  acc[3] += a * (bv.y >> 16);
+                  acc += (uint32_t)A[row * k + kk + u] * B[(kk + u) * n + col];
                 }
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                  acc[j] %= FP_PQ;
-                }
+                acc %= FP_PQ;
               }
               for (; kk < k; kk++) {
-                uint32_t a = ap[kk];
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                  acc[j] = (acc[j] + a * bp[kk * n + j]) % FP_PQ;
-                }
-              }
-#pragma unroll
-              for (int j = 0; j < 4; j++) {
-                C[row * n + c0 + j] = static_cast<uint16_t>(acc[j]);
-              }
-            }
-          } else {
-            int const total = m * n;
-            for (int e = tid; e < total; e += kInterpThreads) {
-              int row = e / n, col = e % n;
-              uint32_t acc = 0;
-              for (int kk = 0; kk < k; kk++) {
                 acc = (acc + (uint32_t)A[row * k + kk] * B[kk * n + col]) % FP_PQ;
               }
               C[e] = static_cast<uint16_t>(acc);
@@ -277,16 +264,19 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           break;
         }
         case DOP_BINARY: {
-          // reference element_binary.h:86-105 (broadcast by `% dim`)
+          // reference element_binary.h:86-105; an operand dim is the output's or 1, so the
+          // reference's `% dim` broadcast index is the output index or 0
           DevTensor const &t1 = P.t[op.src0], &t2 = P.t[op.src1], &to = P.t[op.dst];
           uint16_t const *x1 = reinterpret_cast<uint16_t const *>(lds + t1.off);
           uint16_t const *x2 = reinterpret_cast<uint16_t const *>(lds + t2.off);
           uint16_t *y = reinterpret_cast<uint16_t *>(lds + to.off);
           int const n = to.rows * to.cols;
+          int const r1 = t1.rows == to.rows ? t1.cols : 0, c1 = t1.cols == to.cols ? 1 : 0;
+          int const r2 = t2.rows == to.rows ? t2.cols : 0, c2 = t2.cols == to.cols ? 1 : 0;
           for (int e = tid; e < n; e += kInterpThreads) {
-            int r = e / to.cols, c = e % to.cols;
-            uint32_t a = x1[(r % t1.rows) * t1.cols + c % t1.cols];
-            uint32_t b = x2[(r % t2.rows) * t2.cols + c % t2.cols];
+            int const r = fdiv(e, to.mcols), c = e - r * to.cols;
+            uint32_t a = x1[r * r1 + c * c1];
+            uint32_t b = x2[r * r2 + c * c2];
             uint32_t z;
             if (op.sub == TB_DIV_OP) {
               z = lds_div(tbl, a, b);
@@ -306,16 +296,37 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + ti.off);
           uint16_t *y = reinterpret_cast<uint16_t *>(lds + to.off);
           int const n = to.rows * to.cols, deg = op.red_deg, inner = op.red_inner;
-          for (int e = tid; e < n; e += kInterpThreads) {
-            int pos = (e / inner) * (inner * deg) + e % inner;
-            uint32_t r = 0;
-            for (int kk = 0; kk < deg; kk++, pos += inner) {
-              r += x[pos];
-              if ((kk & 32767) == 32767) {
-                r %= FP_PQ;
+          if (inner == 1 && deg >= 64) {
+            // one output per 16 lanes: each lane strides the row, then the lanes fold
+            int const lane16 = tid & 15;
+            for (int e = tid >> 4; e < n; e += kInterpThreads / 16) {
+              uint16_t const *row = x + e * deg;
+              uint32_t r = 0;
+              for (int kk = lane16; kk < deg; kk += 16) {
+                r += row[kk];  // an LDS tile is far too small to overflow 32 bits here
+              }
+              r %= FP_PQ;
+              r += __shfl_xor(r, 8, 16);
+              r += __shfl_xor(r, 4, 16);
+              r += __shfl_xor(r, 2, 16);
+              r += __shfl_xor(r, 1, 16);
+              if (lane16 == 0) {
+                y[e] = static_cast<uint16_t>(r % FP_PQ);
               }
             }
-            y[e] = static_cast<uint16_t>(r % FP_PQ);
+          } else {
+            for (int e = tid; e < n; e += kInterpThreads) {
+              int const outer = fdiv(e, op.mg0);
+              int pos = outer * (inner * deg) + (e - outer * inner);
+              uint32_t r = 0;
+              for (int kk = 0; kk < deg; kk++, pos += inner) {
+                r += x[pos];
+                if ((kk & 32767) == 32767) {
+                  r %= FP_PQ;
+                }
+              }
+              y[e] = static_cast<uint16_t>(r % FP_PQ);
+            }
           }
           break;
         }
@@ -327,7 +338,8 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           uint16_t *y = reinterpret_cast<uint16_t *>(lds + to.off);
           int const n = to.rows * to.cols, a = op.cat_a, b = op.cat_b, inner = op.cat_inner;
           for (int e = tid; e < n; e += kInterpThreads) {
-            int in_i = e % inner, cd = (e / inner) % (a + b), outer = (e / inner) / (a + b);
+            int const ei = fdiv(e, op.mg0), in_i = e - ei * inner;
+            int const outer = fdiv(ei, op.mg1), cd = ei - outer * (a + b);
             y[e] = cd < a ? A[in_i + cd * inner + outer * inner * a]
                           : B[in_i + (cd - a) * inner + outer * inner * b];
           }
@@ -339,21 +351,41 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + ti.off);
           uint16_t *acc = reinterpret_cast<uint16_t *>(lds + ta.off);
           int const n = ta.rows * ta.cols;
-          bool const last = (it == it_end - 1);
+          bool const last = (it == it_end - 1), first = (it == it_begin);
           TileOrigin org = tile_origin(op, 0, bx);
-          uint16_t *g = (P.splits > 1 ? P.part[op.io] + (long long)split * P.part_elems[op.io]
+          uint16_t *g = (P.splits > 1 ? P.part[op.io] + (long long)split * P.part_stride[op.io]
                                       : static_cast<uint16_t *>(P.out[op.io])) +
-                        org.base;
-          for (int e = tid; e < n; e += kInterpThreads) {
-            uint32_t v = x[e];
-            if (it > it_begin) {
-              v = (v + acc[e]) % FP_PQ;
+                        org.base + (long long)org.row0 * op.d_cols + org.col0;
+          if (op.vec8) {
+            int const cpr = ta.cols / 8, n8 = ta.rows * cpr;
+            for (int e = tid; e < n8; e += kInterpThreads) {
+              uint4v v = *reinterpret_cast<uint4v const *>(x + e * 8);
+              if (!first) {
+                uint4v w = *reinterpret_cast<uint4v const *>(acc + e * 8);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  v[j] = add_mod_pair(v[j], w[j]);
+                }
+              }
+              if (last) {
+                int const r = fdiv(e, ta.mcpr), c = (e - r * cpr) * 8;
+                *reinterpret_cast<uint4v *>(g + (long long)r * op.d_cols + c) = v;
+              } else {
+                *reinterpret_cast<uint4v *>(acc + e * 8) = v;
+              }
             }
-            if (last) {
-              int r = e / ta.cols, c = e % ta.cols;
-              g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c] = static_cast<uint16_t>(v);
-            } else {
-              acc[e] = static_cast<uint16_t>(v);
+          } else {
+            for (int e = tid; e < n; e += kInterpThreads) {
+              uint32_t v = x[e];
+              if (!first) {
+                v = (v + acc[e]) % FP_PQ;
+              }
+              if (last) {
+                int const r = fdiv(e, ta.mcols), c = e - r * ta.cols;
+                g[(long long)r * op.d_cols + c] = static_cast<uint16_t>(v);
+              } else {
+                acc[e] = static_cast<uint16_t>(v);
+              }
             }
           }
           break;
@@ -605,13 +637,14 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
 // ===========================================================================
 // out[e] = sum over splits of part[split * n + e] (mod 25651)
 __global__ void fp_combine_splits_kernel(uint16_t const *__restrict__ part,
-                                         uint16_t *__restrict__ out, long long n, int splits) {
+                                         uint16_t *__restrict__ out, long long n,
+                                         long long stride_elems, int splits) {
   long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
   long long const stride = (long long)gridDim.x * blockDim.x;
   for (; i < n; i += stride) {
     uint32_t v = 0;
     for (int s = 0; s < splits; s++) {
-      v += part[(long long)s * n + i];  // splits <= 64: far from 2^32
+      v += part[(long long)s * stride_elems + i];  // splits <= 64: far from 2^32
     }
     out[i] = static_cast<uint16_t>(v % FP_PQ);
   }
@@ -644,7 +677,8 @@ static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outp
   for (int i = 0; i < num_outputs; i++) {
     prog.part[i] = p;
     prog.part_elems[i] = ext.out_elems[i];
-    p += (ext.out_elems[i] + 7) / 8 * 8 * splits;
+    prog.part_stride[i] = (ext.out_elems[i] + 7) / 8 * 8;
+    p += prog.part_stride[i] * splits;
   }
 }
 
@@ -743,7 +777,7 @@ static int launch(DevProgram const &prog, bool f16) {
         long long const n = prog.part_elems[o];
         int const blocks = (int)std::min<long long>((n + 255) / 256, 2048);
         fp_combine_splits_kernel<<<blocks, 256, 0, s.stream()>>>(
-            prog.part[o], static_cast<uint16_t *>(prog.out[o]), n, prog.splits);
+            prog.part[o], static_cast<uint16_t *>(prog.out[o]), n, prog.part_stride[o], prog.splits);
       }
     }
   }

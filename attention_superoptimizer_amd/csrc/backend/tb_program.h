@@ -31,7 +31,14 @@ struct DevTensor {
   int off;
   int rows, cols;
   int rs, cs;
+  uint32_t mcols, mcpr;  // division magics of cols and cols / 8 (see fast_div_magic)
 };
+
+// q = e / d as one multiply-high: magic = ceil(2^32 / d), exact while e * d < 2^32;
+// 0 stands for d == 1.
+inline uint32_t fast_div_magic(int d) {
+  return d <= 1 ? 0u : (uint32_t)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d);
+}
 
 struct DevOp {
   int kind;
@@ -47,6 +54,8 @@ struct DevOp {
   int red_deg, red_inner;                    // REDUCE (flat row-major rule of the reference)
   int cat_a, cat_b, cat_inner;               // CONCAT
   int mm_kc;  // MATMUL, uint16 interpreter: k chunk of the packed-residue path, 0 = scalar path
+  // division magics.  MATMUL: kc / 4, n / 2, n / 4.  REDUCE: inner.  CONCAT: inner, a + b.
+  uint32_t mg0, mg1, mg2;
 };
 
 struct DevProgram {
@@ -61,6 +70,7 @@ struct DevProgram {
   // a second launch adds the splits (exact in the ring).  splits == 1: stores go to out[].
   int splits;
   long long part_elems[MI355_MAX_DMEM_OUTPUTS];
+  long long part_stride[MI355_MAX_DMEM_OUTPUTS];  // part_elems rounded up to 8
   uint16_t *part[MI355_MAX_DMEM_OUTPUTS];
   DevTensor t[kMaxTensors];
   DevOp ops[MI355_MAX_OPERATORS];

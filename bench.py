@@ -73,6 +73,7 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
     tot = {"kernel_ops": 0, "customized_ops": 0, "compares": 0, "fp_bytes": 0, "matmul_macs": 0,
            "enqueue_seconds": 0.0, "wait_seconds": 0.0}
     n = wrong = 0
+    fam = {}
     for prob in probs:
         ref_g, _ = G.build_from_spec(prob["reference"])
         ref_g.fingerprint_seeded(prob["input_seed"])
@@ -83,6 +84,9 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
         b2 = time.perf_counter()
         t_build += b1 - b0
         t_verify += b2 - b1
+        f = fam.setdefault(prob["family"], [0, 0.0])
+        f[0] += len(graphs)
+        f[1] += b2 - b1
         for k in tot:
             tot[k] += st[k]
         n += len(graphs)
@@ -99,6 +103,7 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
         "fingerprint_GBps": round(tot["fp_bytes"] / t_verify / 1e9, 2),
         "int_TMACps": round(tot["matmul_macs"] / t_verify / 1e12, 3),
         "verdicts_as_constructed": wrong == 0,
+        "candidates_per_s_by_family": {k: round(v[0] / v[1], 1) for k, v in sorted(fam.items())},
         "inputs": "uniform [0, 25651) from (seed, input index)",
     }
     if cpu_baseline:

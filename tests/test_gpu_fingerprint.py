@@ -26,7 +26,8 @@ def _graph_fp(rt, spec, inputs=None):
 
 
 @pytest.mark.parametrize("shape", [(1, 16, 64, 48), (3, 70, 33, 129), (2, 256, 64, 4096),
-                                   (1, 5, 7, 3), (1, 130, 200, 72)])
+                                   (1, 5, 7, 3), (1, 130, 200, 72), (3, 64, 128, 64),
+                                   (1, 192, 320, 448)])
 def test_kernel_matmul_matches_oracle(rt, shape):
     b, m, n, k = shape
     A = uniform_fp((b, m, k), 11)
@@ -38,9 +39,11 @@ def test_kernel_matmul_matches_oracle(rt, shape):
     assert np.array_equal(got, want)
 
 
-def test_kernel_matmul_extreme_values(rt):
-    """All operands 25650: the largest products, k long enough to need folding."""
-    b, m, n, k = 1, 33, 65, 4100
+@pytest.mark.parametrize("shape", [(1, 33, 65, 4100), (1, 64, 64, 65536 + 128), (2, 128, 192, 1024)])
+def test_kernel_matmul_extreme_values(rt, shape):
+    """All operands 25650: the largest products, k long enough to need folding (ragged
+    shapes take the general kernel, multiples of 64 the aligned one)."""
+    b, m, n, k = shape
     A = np.full((b, m, k), FP_PQ - 1, np.uint16)
     B = np.full((b, k, n), FP_PQ - 1, np.uint16)
     spec = [{"op": "input", "dims": [b, m, k]}, {"op": "input", "dims": [b, k, n]},
