@@ -216,6 +216,20 @@ __global__ __launch_bounds__(kThreads) void fp_matmul_kernel(uint16_t const *__r
   }
 }
 
+// out[e] = sum over slabs of part[slab * n + e] (mod 25651)
+__global__ void fp_sum_slabs_kernel(uint16_t const *__restrict__ part, uint16_t *__restrict__ out,
+                                    size_t n, int slabs) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t const stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    uint32_t v = 0;
+    for (int s = 0; s < slabs; s++) {
+      v += part[(size_t)s * n + i];  // at most 256 slabs of values < 25651
+    }
+    out[i] = static_cast<uint16_t>(v % FP_PQ);
+  }
+}
+
 // Aligned fast path: m, n, k multiples of 64 and 16-byte aligned matrices.  One workgroup
 // owns a 64 x 64 output tile and walks k in chunks of 64.  The raw uint16 of chunk i + 1
 // are in flight in registers while chunk i is multiplied; they are split into residues
@@ -227,15 +241,23 @@ __global__ __launch_bounds__(kThreads) void fp_matmul_kernel(uint16_t const *__r
 __global__ __launch_bounds__(kThreads) void fp_matmul64_kernel(uint16_t const *__restrict__ A,
                                                               uint16_t const *__restrict__ B,
                                                               uint16_t *__restrict__ C, int m,
-                                                              int n, int k) {
+                                                              int n, int k, int ksplit,
+                                                              uint16_t *__restrict__ part) {
   constexpr int LDA = 68, KQ = 16;
   constexpr int BUF = 2 * KQ * LDA + 2 * KQ * 64;  // dwords per buffer
   __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF];
   int const tid = threadIdx.x;
-  size_t const b = blockIdx.z;
+  // blockIdx.z = batch * ksplit + ks: this workgroup sums chunks [ch_begin, ch_end) and,
+  // when k is split, stores to slab ks of `part` (a second launch adds the slabs)
+  size_t const b = blockIdx.z / ksplit;
+  int const ks = blockIdx.z % ksplit;
+  int const ch_begin = (int)((long long)(k / 64) * ks / ksplit);
+  int const ch_end = (int)((long long)(k / 64) * (ks + 1) / ksplit);
   A += b * (size_t)m * k + (size_t)blockIdx.y * 64 * k;
   B += b * (size_t)k * n + (size_t)blockIdx.x * 64;
-  C += b * (size_t)m * n + (size_t)blockIdx.y * 64 * n + (size_t)blockIdx.x * 64;
+  size_t const batch = gridDim.z / ksplit;
+  C = (ksplit > 1 ? part + (size_t)ks * batch * m * n : C) + b * (size_t)m * n +
+      (size_t)blockIdx.y * 64 * n + (size_t)blockIdx.x * 64;
   // staging roles: A as 2 x (row, 8 consecutive k), B as (4 consecutive k) x 4 columns
   int const a_row = tid / 8, a_k8 = (tid % 8) * 8;  // second patch: row + 32
   int const b_q = tid / 16, b_c4 = (tid % 16) * 4;
@@ -280,12 +302,11 @@ __global__ __launch_bounds__(kThreads) void fp_matmul64_kernel(uint16_t const *_
       accq[i][j] = 0;
     }
   }
-  int const chunks = k / 64;
-  fetch(0);
-  stage(0);
+  fetch(ch_begin * 64);
+  stage(ch_begin & 1);
   __syncthreads();
-  for (int ch = 0; ch < chunks; ch++) {
-    if (ch + 1 < chunks) {
+  for (int ch = ch_begin; ch < ch_end; ch++) {
+    if (ch + 1 < ch_end) {
       fetch((ch + 1) * 64);
     }
     uint32_t const *ap = lds + (ch & 1) * BUF + r0, *bp = lds + (ch & 1) * BUF + 2 * KQ * LDA + c0;
@@ -314,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void fp_matmul64_kernel(uint16_t const *_
         }
       }
     }
-    if (ch + 1 < chunks) {
+    if (ch + 1 < ch_end) {
       stage((ch + 1) & 1);  // that buffer was last read in chunk ch - 1
     }
     __syncthreads();
@@ -548,8 +569,26 @@ extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C
                        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
                          reinterpret_cast<uintptr_t>(C)) & 15) == 0;
   if (aligned) {
-    dim3 grid(n / 64, m / 64, batch);
-    fp_matmul64_kernel<<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
+    // a grid too small for the device also splits k (sums over k ranges add up exactly
+    // in the ring); the range sums go to the queue's scratch and a second launch adds them
+    long long const blocks = (long long)(n / 64) * (m / 64) * batch;
+    size_t const out_elems = (size_t)batch * m * n;
+    int ksplit = 1;
+    if (blocks < 128 && k >= 128) {
+      ksplit = (int)std::min<long long>(k / 64, (256 + blocks - 1) / blocks);
+      while (ksplit > 1 && out_elems * 2 * ksplit > state().scratch_bytes) {
+        ksplit--;
+      }
+    }
+    if ((long long)batch * ksplit > 65535) {
+      ksplit = 1;
+    }
+    uint16_t *part = static_cast<uint16_t *>(state().scratch());
+    dim3 grid(n / 64, m / 64, batch * ksplit);
+    fp_matmul64_kernel<<<grid, kThreads, 0, st>>>(A, B, C, m, n, k, ksplit, part);
+    if (ksplit > 1) {
+      fp_sum_slabs_kernel<<<grid_for(out_elems), kThreads, 0, st>>>(part, C, out_elems, ksplit);
+    }
   } else if (m >= 128) {
     dim3 grid((n + 63) / 64, (m + 127) / 128, batch);
     fp_matmul_kernel<8><<<grid, kThreads, 0, st>>>(A, B, C, m, n, k);
