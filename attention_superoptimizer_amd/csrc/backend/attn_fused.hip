@@ -93,6 +93,18 @@ __device__ __forceinline__ Patch load_patch(_Float16 const *__restrict__ src, in
   return q;
 }
 
+// The same patch addressed as (wavefront-uniform base) + (32-bit lane offset): the rows
+// differ by the uniform leading dimension, so one lane offset serves all four loads.
+__device__ __forceinline__ Patch load_patch_at(_Float16 const *__restrict__ base, uint32_t lane_off,
+                                               int ld) {
+  Patch q;
+  q.x[0] = *reinterpret_cast<uint4v const *>(base + lane_off);
+  q.x[1] = *reinterpret_cast<uint4v const *>(base + ld + lane_off);
+  q.x[2] = *reinterpret_cast<uint4v const *>(base + 2 * (long long)ld + lane_off);
+  q.x[3] = *reinterpret_cast<uint4v const *>(base + 3 * (long long)ld + lane_off);
+  return q;
+}
+
 // Writes the patch transposed into a swizzled tile: dst row c + i holds source
 // rows r..r+3 as four consecutive halfs, i < 8.
 __device__ __forceinline__ void store_patch_transposed(Patch const &q, _Float16 *__restrict__ dst,
@@ -101,10 +113,11 @@ __device__ __forceinline__ void store_patch_transposed(Patch const &q, _Float16 
 #pragma unroll
   for (int w = 0; w < 4; w++) {
     uint2v even, odd;  // source columns 2w and 2w+1, rows 0..3
-    even.x = (q.x[0][w] & 0xffffu) | (q.x[1][w] << 16);
-    even.y = (q.x[2][w] & 0xffffu) | (q.x[3][w] << 16);
-    odd.x = (q.x[0][w] >> 16) | (q.x[1][w] & 0xffff0000u);
-    odd.y = (q.x[2][w] >> 16) | (q.x[3][w] & 0xffff0000u);
+    // byte permute: selector bytes 0-3 pick from the second operand, 4-7 from the first
+    even.x = __builtin_amdgcn_perm(q.x[1][w], q.x[0][w], 0x05040100u);
+    even.y = __builtin_amdgcn_perm(q.x[3][w], q.x[2][w], 0x05040100u);
+    odd.x = __builtin_amdgcn_perm(q.x[1][w], q.x[0][w], 0x07060302u);
+    odd.y = __builtin_amdgcn_perm(q.x[3][w], q.x[2][w], 0x07060302u);
     int const row = 8 * cb + 2 * w;
     *reinterpret_cast<uint2v *>(dst + swz_chunk(row, rb >> 1, LD) + (rb & 1) * 4) = even;
     *reinterpret_cast<uint2v *>(dst + swz_chunk(row + 1, rb >> 1, LD) + (rb & 1) * 4) = odd;
@@ -456,21 +469,31 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   }
 
   Patch kp[KPT], vp[VPT];
+  // lane offsets of this thread's patches inside a tile (the same every iteration)
+  uint32_t k_off[KPT], v_off[VPT];
+#pragma unroll
+  for (int i = 0; i < KPT; i++) {
+    int const p = tid + i * NT;
+    k_off[i] = (uint32_t)(4 * (p / (NK / 8)) * P.k.d_cols + 8 * (p % (NK / 8)));
+  }
+#pragma unroll
+  for (int i = 0; i < VPT; i++) {
+    int const p = tid + i * NT;
+    v_off[i] = (uint32_t)(4 * (p / (DV / 8)) * P.v.d_cols + 8 * (p % (DV / 8)));
+  }
   auto issue_loads = [&](int it) {
     _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
     _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
 #pragma unroll
     for (int i = 0; i < KPT; i++) {
-      int p = tid + i * NT;
-      if (KP % NT == 0 || p < KP) {
-        kp[i] = load_patch(kg, P.k.d_cols, NK / 8, p);
+      if (KP % NT == 0 || tid + i * NT < KP) {
+        kp[i] = load_patch_at(kg, k_off[i], P.k.d_cols);
       }
     }
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
-      int p = tid + i * NT;
-      if (VP % NT == 0 || p < VP) {
-        vp[i] = load_patch(vg, P.v.d_cols, DV / 8, p);
+      if (VP % NT == 0 || tid + i * NT < VP) {
+        vp[i] = load_patch_at(vg, v_off[i], P.v.d_cols);
       }
     }
   };
@@ -503,8 +526,13 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     _Float16 const *kt = buf + (it & 1) * STAGE;
     _Float16 const *vt = kt + NK * D;
     // ---- S^T = K^T . Q^T for RPW row groups, exp, row sums ------------------------
-    half4 e[RPW][KB];
+    // e8[rp][jj]: eight consecutive keys of this lane's query row, packed fp16: the A
+    // operand of P.V.  Roundings as the sequential program makes them: S to fp16, exp in
+    // fp32, the result to fp16; the row sum adds the rounded values in fp32.
+    uint32_t e8[RPW][KB / 2][4];
     float rs[RPW];
+    half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
+    constexpr float LOG2E = 1.44269504088896340736f;
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       rs[rp] = 0.0f;
@@ -528,11 +556,14 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          _Float16 s16 = static_cast<_Float16>(acc[rp][r]);
-          _Float16 e16 = static_cast<_Float16>(__expf(static_cast<float>(s16)));
-          e[rp][j][r] = e16;
-          rs[rp] += static_cast<float>(e16);
+        for (int h = 0; h < 2; h++) {
+          half2v const s2 = {static_cast<_Float16>(acc[rp][2 * h]),
+                             static_cast<_Float16>(acc[rp][2 * h + 1])};
+          float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
+          float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
+          half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
+          rs[rp] = __builtin_amdgcn_fdot2(e2, ones, rs[rp], false);
+          e8[rp][j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
         }
       }
     }
@@ -545,10 +576,13 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       if (HAS_DIV) {
         float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16[rp]));
 #pragma unroll
-        for (int j = 0; j < KB; j++) {
+        for (int jj = 0; jj < KB / 2; jj++) {
 #pragma unroll
-          for (int r = 0; r < 4; r++) {
-            e[rp][j][r] = static_cast<_Float16>(static_cast<float>(e[rp][j][r]) * inv);
+          for (int w = 0; w < 4; w++) {
+            half2v const e2 = __builtin_bit_cast(half2v, e8[rp][jj][w]);
+            half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
+                               static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+            e8[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
           }
         }
       } else {
@@ -573,8 +607,9 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
         half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
         for (int rp = 0; rp < RPW; rp++) {
-          half8 a = __builtin_shufflevector(e[rp][2 * jj], e[rp][2 * jj + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-          o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, o[rp], 0, 0, 0);
+          uint4v const a = {e8[rp][jj][0], e8[rp][jj][1], e8[rp][jj][2], e8[rp][jj][3]};
+          o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o[rp], 0,
+                                                         0, 0);
         }
       }
 #pragma unroll
