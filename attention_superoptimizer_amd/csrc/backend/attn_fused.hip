@@ -106,10 +106,18 @@ __device__ __forceinline__ Patch load_patch_at(_Float16 const *__restrict__ base
 }
 
 // Writes the patch transposed into a swizzled tile: dst row c + i holds source
-// rows r..r+3 as four consecutive halfs, i < 8.
+// rows r..r+3 as four consecutive halfs, i < 8.  PAIRED reorders the eight 4-half groups
+// of every 32-half block so that groups g and g + 4 sit side by side (slot 2g, 2g + 1):
+// the sixteen bytes a lane needs as the B operand of P.V (keys 4g..4g+3 and
+// 16+4g..16+4g+3, the key order the S^T accumulators leave P in) become one LDS read.
+template <bool PAIRED = false>
 __device__ __forceinline__ void store_patch_transposed(Patch const &q, _Float16 *__restrict__ dst,
                                                        int LD, int cblocks, int p) {
-  int const cb = p % cblocks, rb = p / cblocks;
+  int const cb = p % cblocks;
+  int rb = p / cblocks;
+  if (PAIRED) {
+    rb = (rb & ~7) | ((rb & 3) << 1) | ((rb >> 2) & 1);
+  }
 #pragma unroll
   for (int w = 0; w < 4; w++) {
     uint2v even, odd;  // source columns 2w and 2w+1, rows 0..3
@@ -437,7 +445,7 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   // XOR with a constant per fetch, everything else folds into the instruction offset.
   int const s0 = (c ^ (c >> 3)) & 7;
   int const k_lane = c * D, k_sg8 = (s0 ^ g) << 3;            // K^T: row c, 16-byte chunk g
-  int const v_lane = c * NK + (g & 1) * 4, v_sg8 = (s0 ^ (g >> 1)) << 3;  // V^T: 8-byte half chunks
+  int const v_lane = c * NK, v_sg8 = (s0 ^ g) << 3;           // V^T: row c, 16-byte chunk g
   int const row_base = (slice * RG + wave) * RPW * 16;
   int const F = P.forloop_range;
 
@@ -511,7 +519,7 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     for (int i = 0; i < VPT; i++) {
       int p = tid + i * NT;
       if (VP % NT == 0 || p < VP) {
-        store_patch_transposed(vp[i], vt, NK, DV / 8, p);
+        store_patch_transposed<true>(vp[i], vt, NK, DV / 8, p);
       }
     }
   };
@@ -599,12 +607,9 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       }
 #pragma unroll
       for (int jj = 0; jj < KB / 2; jj++) {
-        // row 16t + c, chunks 4jj + (g>>1) and 4jj + 2 + (g>>1)
-        half4 b0 = *reinterpret_cast<half4 const *>(
+        // row 16t + c, 16-byte chunk 4jj + g (paired key groups, see store_patch_transposed)
+        half8 b = *reinterpret_cast<half8 const *>(
             vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj) ^ ((2 * t) & 7)) << 3)));
-        half4 b1 = *reinterpret_cast<half4 const *>(
-            vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj + 2) ^ ((2 * t) & 7)) << 3)));
-        half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
         for (int rp = 0; rp < RPW; rp++) {
           uint4v const a = {e8[rp][jj][0], e8[rp][jj][1], e8[rp][jj][2], e8[rp][jj][3]};
