@@ -710,6 +710,8 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
       prog.fused = 1;
     } else if (gemm_applicable(prog)) {
       prog.fused = 2;
+    } else if (combine_applicable(prog)) {
+      prog.fused = 3;
     } else {
       rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err);
       if (rc != MI355_OK) {
@@ -745,7 +747,9 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
   if (prog.fused != 0) {
-    int rc = prog.fused == 1 ? try_launch_attention(prog) : try_launch_gemm(prog);
+    int rc = prog.fused == 1   ? try_launch_attention(prog)
+             : prog.fused == 2 ? try_launch_gemm(prog)
+                               : try_launch_combine(prog);
     if (rc == 1) {
       return MI355_OK;
     }

@@ -62,7 +62,7 @@ struct DevProgram {
   int num_ops, num_tensors;
   int forloop_range;
   int lds_bytes;  // dynamic LDS the interpreter requests (tables included)
-  int fused;      // 1 / 2: run by the fused attention / GEMM kernel instead of the interpreter
+  int fused;      // 1 / 2 / 3: run by the fused attention / GEMM / combine kernel, not the interpreter
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
@@ -90,6 +90,8 @@ int try_launch_attention(DevProgram const &prog);
 bool attention_applicable(DevProgram const &prog);
 int try_launch_gemm(DevProgram const &prog);  // gemm_fused.hip, same convention
 bool gemm_applicable(DevProgram const &prog);
+int try_launch_combine(DevProgram const &prog);  // combine_fused.hip, same convention
+bool combine_applicable(DevProgram const &prog);
 
 // Lowers `plan` for the uint16 interpreter (f16 == false: plain row-major tiles)
 // or the fp16 interpreter (f16 == true: padded rows, B operands k-contiguous).

@@ -290,7 +290,7 @@ def main() -> int:
 
     others = []
     if not args.headline_only:
-        kname = {1: "fp_interp", 2: "f16_interp", 3: "f16_attention", 4: "f16_gemm"}
+        kname = {1: "fp_interp", 2: "f16_interp", 3: "f16_attention", 4: "f16_gemm", 5: "f16_combine"}
         for name in ("C1_fused_matmul", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp"):
             g.close()
             spec2, g, vals2 = setup(name)

@@ -79,6 +79,7 @@ typedef struct mi355_launch_info {
 #define MI355_KERNEL_F16_INTERP 2
 #define MI355_KERNEL_F16_ATTENTION 3 /* fused register-resident attention family */
 #define MI355_KERNEL_F16_GEMM 4      /* fused skinny-GEMM family (split for-loop, ordered fix-up) */
+#define MI355_KERNEL_F16_COMBINE 5   /* fused fold-partials-and-divide family */
 
 /* Backend options (mi355_set_option).  FORCE_INTERPRETER = 1 sends every fp16
  * customized op through the generic LDS interpreter instead of a fused kernel

@@ -13,7 +13,7 @@ from oracle import evaluate as orc
 pytestmark = pytest.mark.gpu
 
 
-KERNEL_INTERP, KERNEL_ATTENTION, KERNEL_GEMM = 2, 3, 4
+KERNEL_INTERP, KERNEL_ATTENTION, KERNEL_GEMM, KERNEL_COMBINE = 2, 3, 4, 5
 _last_kernels = []
 
 
@@ -119,7 +119,8 @@ def test_config3_mha_prefill_small(rt, path):
     spec, ref = W.config3_mha_prefill(heads=2, seq=512, hd=128, q_split=4, kv_split=2, F=4)
     ins = _inputs(spec, 128 ** -0.5, 30)
     got = _check(rt, spec, ins, "C3 small")[-1][0]
-    assert _last_kernels[0] == (KERNEL_ATTENTION if path == "fused" else KERNEL_INTERP)
+    assert _last_kernels == ([KERNEL_ATTENTION, KERNEL_COMBINE] if path == "fused"
+                             else [KERNEL_INTERP, KERNEL_INTERP])
     # textbook special case: numerator / denominator = softmax(Q K^T) V
     Q, K, V = (ins[i].astype(np.float64) for i in range(3))
     s = Q @ K
