@@ -216,12 +216,14 @@ def config2_gqa_decode():
     return g, None
 
 
-def config3_mha_prefill(heads=32, seq=2048, hd=128, q_split=16, kv_split=4, F=8, rows2=32):
+def config3_mha_prefill(heads=32, seq=2048, hd=128, q_split=16, kv_split=1, F=32, rows2=32):
     """MHA prefill, non-causal: op1 accumulates exp(QK^T)V and rowsum(exp(QK^T))
     over a seq-tiled for-loop per (head, kv block, q block); op2 folds the kv
     blocks and divides (plan shape of cpp_examples/multi_head_attn_prefill.cc:43-98).
-    Default tiling: Q tile [128,128], K/V tiles of 64 keys; op2 works on `rows2`
-    query rows per block."""
+    Default tiling: Q tile [128,128], the whole key range walked by one block's
+    for-loop in tiles of 64 keys (no partial numerators to write and re-read; the
+    tiles also fit the LDS interpreters, so every route can run the plan); op2 works
+    on `rows2` query rows per block."""
     q, k, v = [heads, seq, hd], [heads, hd, seq], [heads, seq, hd]
     g = [
         _inp(q), _inp(k, COL), _inp(v, COL),

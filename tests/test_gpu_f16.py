@@ -129,6 +129,16 @@ def test_config3_mha_prefill_small(rt, path):
     assert_f16_close(got, att, rtol=1e-2, atol=2e-3, what="C3 vs softmax attention")
 
 
+def test_config3_single_kv_block(rt, path):
+    """the benchmark's tiling shape: one block walks the whole key range (kv_split 1),
+    so op2 folds a single partial result"""
+    from attention_superoptimizer_amd import workloads as W
+    spec, _ = W.config3_mha_prefill(heads=2, seq=512, hd=128, q_split=4, kv_split=1, F=8)
+    _check(rt, spec, _inputs(spec, 128 ** -0.5, 31), "C3 single kv block")
+    assert _last_kernels == ([KERNEL_ATTENTION, KERNEL_COMBINE] if path == "fused"
+                             else [KERNEL_INTERP, KERNEL_INTERP])
+
+
 def test_config4_lora(rt, path):
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config4_lora()
