@@ -421,8 +421,8 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
 // Throughput variant for large problems: every wavefront owns RPW row groups of 16
 // query rows (so each K^T / V^T operand fetched from LDS feeds RPW MFMAs) and walks
 // all for-loop iterations itself; K / V tiles are double-buffered in LDS and the
-// global loads of iteration i+1 are in flight (in registers) while iteration i is on
-// the matrix cores.  One barrier per iteration.
+// global loads of the next tiles are in flight (in registers) while the current ones
+// are on the matrix cores.  One barrier per iteration.
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW>
 __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
@@ -489,15 +489,17 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     int const p = tid + i * NT;
     v_off[i] = (uint32_t)(4 * (p / (DV / 8)) * P.v.d_cols + 8 * (p % (DV / 8)));
   }
-  auto issue_loads = [&](int it) {
+  auto load_k = [&](int it) {
     _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
-    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
 #pragma unroll
     for (int i = 0; i < KPT; i++) {
       if (KP % NT == 0 || tid + i * NT < KP) {
         kp[i] = load_patch_at(kg, k_off[i], P.k.d_cols);
       }
     }
+  };
+  auto load_v = [&](int it) {
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
       if (VP % NT == 0 || tid + i * NT < VP) {
@@ -505,128 +507,191 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       }
     }
   };
-  auto write_tiles = [&](int b) {
-    _Float16 *kt = buf + b * STAGE;
-    _Float16 *vt = kt + NK * D;
+  _Float16 *const kbuf = buf;               // two K^T tiles
+  _Float16 *const vbuf = buf + 2 * NK * D;  // two V^T tiles
+  auto write_k = [&](int b) {
 #pragma unroll
     for (int i = 0; i < KPT; i++) {
       int p = tid + i * NT;
       if (KP % NT == 0 || p < KP) {
-        store_patch_transposed(kp[i], kt, D, NK / 8, p);
+        store_patch_transposed(kp[i], kbuf + b * NK * D, D, NK / 8, p);
       }
     }
+  };
+  auto write_v = [&](int b) {
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
       int p = tid + i * NT;
       if (VP % NT == 0 || p < VP) {
-        store_patch_transposed<true>(vp[i], vt, NK, DV / 8, p);
+        store_patch_transposed<true>(vp[i], vbuf + b * DV * NK, NK, DV / 8, p);
       }
     }
   };
 
-  issue_loads(0);
-  write_tiles(0);
-  __syncthreads();
-  for (int it = 0; it < F; it++) {
-    if (it + 1 < F) {
-      issue_loads(it + 1);  // in flight while this iteration computes
+  // P of one iteration, packed fp16: pk[rp][jj][0..3] = eight keys of this lane's query
+  // row (keys 4g..4g+3 of key blocks 2jj and 2jj+1), the A operand of P.V.
+  // One 16-key block of S^T = K^T . Q^T for the RPW row groups, then the roundings the
+  // sequential program makes: S to fp16, exp in fp32, the result to fp16; the row sum
+  // adds the rounded values in fp32.
+  half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
+  constexpr float LOG2E = 1.44269504088896340736f;
+  auto s_block = [&](_Float16 const *kt, int j, uint32_t (&pk)[RPW][KB / 2][4], float (&rs)[RPW]) {
+    float4v acc[RPW];
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+      acc[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    _Float16 const *kt = buf + (it & 1) * STAGE;
-    _Float16 const *vt = kt + NK * D;
-    // ---- S^T = K^T . Q^T for RPW row groups, exp, row sums ------------------------
-    // e8[rp][jj]: eight consecutive keys of this lane's query row, packed fp16: the A
-    // operand of P.V.  Roundings as the sequential program makes them: S to fp16, exp in
-    // fp32, the result to fp16; the row sum adds the rounded values in fp32.
-    uint32_t e8[RPW][KB / 2][4];
+#pragma unroll
+    for (int kk = 0; kk < DK; kk++) {
+      half8 a = *reinterpret_cast<half8 const *>(
+          kt + k_lane + 16 * j * D + (k_sg8 ^ (((4 * kk) ^ ((2 * j) & 7)) << 3)));
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rp][kk], acc[rp], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        half2v const s2 = {static_cast<_Float16>(acc[rp][2 * h]),
+                           static_cast<_Float16>(acc[rp][2 * h + 1])};
+        float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
+        float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
+        half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
+        rs[rp] = __builtin_amdgcn_fdot2(e2, ones, rs[rp], false);
+        pk[rp][j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
+      }
+    }
+  };
+  // After the last key block: the row sum across the four lane groups, then either the
+  // normalisation of P (form with div) or the accumulation of the denominator.
+  auto s_finish = [&](uint32_t (&pk)[RPW][KB / 2][4], float (&rs)[RPW]) {
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+      rs[rp] += __shfl_xor(rs[rp], 16, 64);
+      rs[rp] += __shfl_xor(rs[rp], 32, 64);
+      _Float16 const r16 = static_cast<_Float16>(rs[rp]);
+      if (HAS_DIV) {
+        float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
+#pragma unroll
+        for (int jj = 0; jj < KB / 2; jj++) {
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            half2v const e2 = __builtin_bit_cast(half2v, pk[rp][jj][w]);
+            half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
+                               static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+            pk[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
+          }
+        }
+      } else {
+        racc[rp] = static_cast<_Float16>(static_cast<float>(racc[rp]) + static_cast<float>(r16));
+      }
+    }
+  };
+  // Sixteen output columns of O += P . V for the RPW row groups.
+  auto pv_block = [&](_Float16 const *vt, int t, uint32_t const (&pk)[RPW][KB / 2][4]) {
+    float4v o[RPW];
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+      o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int jj = 0; jj < KB / 2; jj++) {
+      // row 16t + c, 16-byte chunk 4jj + g (paired key groups, see store_patch_transposed)
+      half8 b = *reinterpret_cast<half8 const *>(
+          vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj) ^ ((2 * t) & 7)) << 3)));
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
+        o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o[rp], 0, 0,
+                                                       0);
+      }
+    }
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+      half2v lo = {static_cast<_Float16>(o[rp][0]), static_cast<_Float16>(o[rp][1])};
+      half2v hi = {static_cast<_Float16>(o[rp][2]), static_cast<_Float16>(o[rp][3])};
+      oacc[rp][t][0] = oacc[rp][t][0] + lo;
+      oacc[rp][t][1] = oacc[rp][t][1] + hi;
+    }
+  };
+
+  // The loop is skewed by one phase: pass `it` multiplies P(it) with V(it) while it
+  // builds P(it + 1) from K(it + 1), so every pass has two independent instruction
+  // streams (matrix-heavy P.V, conversion / exp-heavy S) to overlap.  K tiles and V
+  // tiles are double-buffered separately: pass `it` reads K(it + 1) and V(it) and, at its
+  // end, replaces K(it) by K(it + 2) and V(it - 1) by V(it + 1).
+  load_k(0);
+  load_v(0);
+  write_k(0);
+  write_v(0);
+  if (F > 1) {
+    load_k(1);
+    write_k(1);
+  }
+  __syncthreads();
+  uint32_t pcur[RPW][KB / 2][4];
+  {
     float rs[RPW];
-    half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
-    constexpr float LOG2E = 1.44269504088896340736f;
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       rs[rp] = 0.0f;
     }
 #pragma unroll
     for (int j = 0; j < KB; j++) {
-      float4v acc[RPW];
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-        acc[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
-      }
-#pragma unroll
-      for (int kk = 0; kk < DK; kk++) {
-        half8 a = *reinterpret_cast<half8 const *>(
-            kt + k_lane + 16 * j * D + (k_sg8 ^ (((4 * kk) ^ ((2 * j) & 7)) << 3)));
-#pragma unroll
-        for (int rp = 0; rp < RPW; rp++) {
-          acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rp][kk], acc[rp], 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          half2v const s2 = {static_cast<_Float16>(acc[rp][2 * h]),
-                             static_cast<_Float16>(acc[rp][2 * h + 1])};
-          float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
-          float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
-          half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
-          rs[rp] = __builtin_amdgcn_fdot2(e2, ones, rs[rp], false);
-          e8[rp][j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
-        }
-      }
+      s_block(kbuf, j, pcur, rs);
     }
-    _Float16 r16[RPW];
+    s_finish(pcur, rs);
+  }
+  __syncthreads();  // K(0) may be overwritten from here on
+  for (int it = 0; it < F; it++) {
+    bool const more = it + 1 < F;
+    if (it + 2 < F) {
+      load_k(it + 2);  // in flight while this pass computes
+    }
+    if (more) {
+      load_v(it + 1);
+    }
+    _Float16 const *vt = vbuf + (it & 1) * DV * NK;
+    if (more) {
+      _Float16 const *kt = kbuf + ((it + 1) & 1) * NK * D;
+      uint32_t pnext[RPW][KB / 2][4];
+      float rs[RPW];
 #pragma unroll
-    for (int rp = 0; rp < RPW; rp++) {
-      rs[rp] += __shfl_xor(rs[rp], 16, 64);
-      rs[rp] += __shfl_xor(rs[rp], 32, 64);
-      r16[rp] = static_cast<_Float16>(rs[rp]);
-      if (HAS_DIV) {
-        float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16[rp]));
+      for (int rp = 0; rp < RPW; rp++) {
+        rs[rp] = 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < KB; u++) {
+        s_block(kt, u, pnext, rs);
+#pragma unroll
+        for (int t = u * DB / KB; t < (u + 1) * DB / KB; t++) {
+          pv_block(vt, t, pcur);
+        }
+      }
+      s_finish(pnext, rs);
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
         for (int jj = 0; jj < KB / 2; jj++) {
 #pragma unroll
           for (int w = 0; w < 4; w++) {
-            half2v const e2 = __builtin_bit_cast(half2v, e8[rp][jj][w]);
-            half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
-                               static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
-            e8[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
+            pcur[rp][jj][w] = pnext[rp][jj][w];
           }
         }
-      } else {
-        racc[rp] = static_cast<_Float16>(static_cast<float>(racc[rp]) + static_cast<float>(r16[rp]));
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < DB; t++) {
+        pv_block(vt, t, pcur);
       }
     }
-    // ---- O = P . V ------------------------------------------------------------------
-#pragma unroll
-    for (int t = 0; t < DB; t++) {
-      float4v o[RPW];
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-        o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
-      }
-#pragma unroll
-      for (int jj = 0; jj < KB / 2; jj++) {
-        // row 16t + c, 16-byte chunk 4jj + g (paired key groups, see store_patch_transposed)
-        half8 b = *reinterpret_cast<half8 const *>(
-            vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj) ^ ((2 * t) & 7)) << 3)));
-#pragma unroll
-        for (int rp = 0; rp < RPW; rp++) {
-          uint4v const a = {e8[rp][jj][0], e8[rp][jj][1], e8[rp][jj][2], e8[rp][jj][3]};
-          o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o[rp], 0,
-                                                         0, 0);
-        }
-      }
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-        half2v lo = {static_cast<_Float16>(o[rp][0]), static_cast<_Float16>(o[rp][1])};
-        half2v hi = {static_cast<_Float16>(o[rp][2]), static_cast<_Float16>(o[rp][3])};
-        oacc[rp][t][0] = oacc[rp][t][0] + lo;
-        oacc[rp][t][1] = oacc[rp][t][1] + hi;
-      }
+    if (it + 2 < F) {
+      write_k(it & 1);  // K(it) was last read in the previous pass
     }
-    if (it + 1 < F) {
-      write_tiles((it + 1) & 1);  // that buffer was last read in iteration it - 1
+    if (more) {
+      write_v((it + 1) & 1);  // V(it - 1) was last read in the previous pass
     }
     __syncthreads();
   }
