@@ -645,53 +645,64 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     s_finish(pcur, rs);
   }
   __syncthreads();  // K(0) may be overwritten from here on
-  for (int it = 0; it < F; it++) {
-    bool const more = it + 1 < F;
-    if (it + 2 < F) {
-      load_k(it + 2);  // in flight while this pass computes
-    }
-    if (more) {
-      load_v(it + 1);
-    }
+  // One skewed pass: P(it) . V(it) interleaved with building P(it + 1) from K(it + 1).
+  auto skewed_pass = [&](int it) {
     _Float16 const *vt = vbuf + (it & 1) * DV * NK;
-    if (more) {
-      _Float16 const *kt = kbuf + ((it + 1) & 1) * NK * D;
-      uint32_t pnext[RPW][KB / 2][4];
-      float rs[RPW];
+    _Float16 const *kt = kbuf + ((it + 1) & 1) * NK * D;
+    uint32_t pnext[RPW][KB / 2][4];
+    float rs[RPW];
 #pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-        rs[rp] = 0.0f;
-      }
+    for (int rp = 0; rp < RPW; rp++) {
+      rs[rp] = 0.0f;
+    }
 #pragma unroll
-      for (int u = 0; u < KB; u++) {
-        s_block(kt, u, pnext, rs);
+    for (int u = 0; u < KB; u++) {
+      s_block(kt, u, pnext, rs);
 #pragma unroll
-        for (int t = u * DB / KB; t < (u + 1) * DB / KB; t++) {
-          pv_block(vt, t, pcur);
-        }
-      }
-      s_finish(pnext, rs);
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-#pragma unroll
-        for (int jj = 0; jj < KB / 2; jj++) {
-#pragma unroll
-          for (int w = 0; w < 4; w++) {
-            pcur[rp][jj][w] = pnext[rp][jj][w];
-          }
-        }
-      }
-    } else {
-#pragma unroll
-      for (int t = 0; t < DB; t++) {
+      for (int t = u * DB / KB; t < (u + 1) * DB / KB; t++) {
         pv_block(vt, t, pcur);
       }
     }
-    if (it + 2 < F) {
-      write_k(it & 1);  // K(it) was last read in the previous pass
+    s_finish(pnext, rs);
+#pragma unroll
+    for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+      for (int jj = 0; jj < KB / 2; jj++) {
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+          pcur[rp][jj][w] = pnext[rp][jj][w];
+        }
+      }
     }
-    if (more) {
-      write_v((it + 1) & 1);  // V(it - 1) was last read in the previous pass
+  };
+  // The steady-state loop body is branch-free (the tail passes are peeled below): with a
+  // conditional prefetch inside the loop the compiler cannot prove that the previous
+  // pass's loads were consumed and makes each new group of loads wait for the one before.
+  int it = 0;
+  for (; it + 2 < F; it++) {
+    load_k(it + 2);  // both in flight while this pass computes
+    load_v(it + 1);
+    __builtin_amdgcn_sched_barrier(0);  // keep the loads up here, a whole pass ahead of their use
+    skewed_pass(it);
+    __builtin_amdgcn_sched_barrier(0);
+    write_k(it & 1);        // K(it) was last read in the previous pass
+    write_v((it + 1) & 1);  // V(it - 1) was last read in the previous pass
+    __syncthreads();
+  }
+  if (it + 1 < F) {  // pass F - 2: no K tile left to fetch
+    load_v(it + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    skewed_pass(it);
+    __builtin_amdgcn_sched_barrier(0);
+    write_v((it + 1) & 1);
+    __syncthreads();
+    it++;
+  }
+  {  // pass F - 1: the last P . V
+    _Float16 const *vt = vbuf + (it & 1) * DV * NK;
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+      pv_block(vt, t, pcur);
     }
     __syncthreads();
   }
