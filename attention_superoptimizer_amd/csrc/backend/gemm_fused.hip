@@ -120,6 +120,52 @@ __device__ __forceinline__ void stage_weight(_Float16 const *__restrict__ src, i
   }
 }
 
+// The two halves of stage_weight for tiles that are prefetched: the global loads of the
+// next iteration's tile are issued before the current one is multiplied and the
+// register transposes / LDS writes happen an iteration later.
+template <int PPT>
+__device__ __forceinline__ void load_weight(_Float16 const *__restrict__ src, int ld, int R, int C,
+                                            uint4v (&x)[PPT][4], int tid, int nthreads) {
+  int const cblocks = C / 8, patches = (R / 4) * cblocks;
+#pragma unroll
+  for (int i = 0; i < PPT; i++) {
+    int p = tid + i * nthreads;
+    if (p < patches) {
+      int cb = p % cblocks, rb = p / cblocks;
+      _Float16 const *s = src + (long long)(4 * rb) * ld + 8 * cb;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        x[i][j] = *reinterpret_cast<uint4v const *>(s + (long long)j * ld);
+      }
+    }
+  }
+}
+
+template <int PPT>
+__device__ __forceinline__ void store_weight(uint4v const (&x)[PPT][4], int R, int C,
+                                             _Float16 *__restrict__ dst, int tid, int nthreads) {
+  int const cblocks = C / 8, patches = (R / 4) * cblocks;
+  int const mask = ((R / 8) - 1) & 7;
+#pragma unroll
+  for (int i = 0; i < PPT; i++) {
+    int p = tid + i * nthreads;
+    if (p < patches) {
+      int cb = p % cblocks, rb = p / cblocks;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        uint2v even, odd;  // byte permute: selector bytes 0-3 from the second operand
+        even.x = __builtin_amdgcn_perm(x[i][1][w], x[i][0][w], 0x05040100u);
+        even.y = __builtin_amdgcn_perm(x[i][3][w], x[i][2][w], 0x05040100u);
+        odd.x = __builtin_amdgcn_perm(x[i][1][w], x[i][0][w], 0x07060302u);
+        odd.y = __builtin_amdgcn_perm(x[i][3][w], x[i][2][w], 0x07060302u);
+        int row = 8 * cb + 2 * w;
+        *reinterpret_cast<uint2v *>(dst + sw_chunk(row, rb >> 1, R, mask) + (rb & 1) * 4) = even;
+        *reinterpret_cast<uint2v *>(dst + sw_chunk(row + 1, rb >> 1, R, mask) + (rb & 1) * 4) = odd;
+      }
+    }
+  }
+}
+
 // MT m-tiles of 16 rows, NB weight matrices, 4 wavefronts = the 4 column tiles of a
 // 64-column weight tile.  KTMAX bounds the staging register arrays.
 template <int MT, int NB, int PRO, bool LORA, int KTMAX>
@@ -165,29 +211,57 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
     }
   }
 
-  for (int it = it_begin; it < it_end; it++) {
-    if (it > it_begin) {
-      __syncthreads();  // previous iteration's tiles fully consumed
+  // Prefetch registers: the raw tiles of the next iteration.
+  constexpr int APT = (16 * MT * (KTMAX / 8) + NT - 1) / NT;  // activation chunks per thread
+  constexpr int LPPT = (KTMAX / 4) * 2 / NT + 1;             // lora A patches per thread
+  uint4v wreg[NB][WPPT][4];
+  uint4v lreg[LORA ? LPPT : 1][4];
+  half8 areg[APT], ureg[PRO == PRO_SILU_MUL ? APT : 1];
+  int const chunks_a = KT / 8;
+  auto fetch = [&](int it) {
+    _Float16 const *a0 = static_cast<_Float16 const *>(P.a0.ptr) + gtile_offset(P.a0, bx, by, bz, it);
+    _Float16 const *a1 = PRO == PRO_SILU_MUL
+                             ? static_cast<_Float16 const *>(P.a1.ptr) + gtile_offset(P.a1, bx, by, bz, it)
+                             : a0;
+#pragma unroll
+    for (int i = 0; i < APT; i++) {
+      int const e = tid + i * NT;
+      int const row = e / chunks_a, ch = e % chunks_a;
+      if (e < 16 * MT * chunks_a && row < M) {
+        areg[i] = *reinterpret_cast<half8 const *>(a0 + (long long)row * P.a0.d_cols + 8 * ch);
+        if (PRO == PRO_SILU_MUL) {
+          ureg[i] = *reinterpret_cast<half8 const *>(a1 + (long long)row * P.a1.d_cols + 8 * ch);
+        }
+      }
     }
-    // ---- stage: activation tile as it is (prologue applied), weights transposed ----
-    {
-      _Float16 const *a0 = static_cast<_Float16 const *>(P.a0.ptr) + gtile_offset(P.a0, bx, by, bz, it);
-      _Float16 const *a1 = PRO == PRO_SILU_MUL
-                               ? static_cast<_Float16 const *>(P.a1.ptr) + gtile_offset(P.a1, bx, by, bz, it)
-                               : a0;
-      int const chunks = KT / 8;
-      for (int e = tid; e < 16 * MT * chunks; e += NT) {
-        int row = e / chunks, ch = e % chunks;
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      GTile const &bt = b == 0 ? P.b0 : P.b1;
+      _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it);
+      load_weight<WPPT>(src, bt.d_cols, KT, 64, wreg[b], tid, NT);
+    }
+    if (LORA) {
+      _Float16 const *src = static_cast<_Float16 const *>(P.la.ptr) + gtile_offset(P.la, bx, by, bz, it);
+      load_weight<LORA ? LPPT : 1>(src, P.la.d_cols, KT, 16, lreg, tid, NT);
+    }
+  };
+  // registers -> LDS: activation tile as it is (prologue applied), weights transposed
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < APT; i++) {
+      int const e = tid + i * NT;
+      int const row = e / chunks_a, ch = e % chunks_a;
+      if (e < 16 * MT * chunks_a) {
         half8 v;
         if (row < M) {
-          v = *reinterpret_cast<half8 const *>(a0 + (long long)row * P.a0.d_cols + 8 * ch);
+          v = areg[i];
           if (PRO == PRO_EXP || PRO == PRO_SILU) {
 #pragma unroll
             for (int j = 0; j < 8; j++) {
               v[j] = static_cast<_Float16>(prologue(PRO, static_cast<float>(v[j])));
             }
           } else if (PRO == PRO_SILU_MUL) {
-            half8 u = *reinterpret_cast<half8 const *>(a1 + (long long)row * P.a1.d_cols + 8 * ch);
+            half8 u = ureg[i];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
               _Float16 sg = static_cast<_Float16>(prologue(PRO_SILU, static_cast<float>(v[j])));
@@ -202,18 +276,16 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
         }
         *reinterpret_cast<half8 *>(a_lds + sw_chunk(row, ch, KT, kmask)) = v;
       }
-#pragma unroll
-      for (int b = 0; b < NB; b++) {
-        GTile const &bt = b == 0 ? P.b0 : P.b1;
-        _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it);
-        stage_weight<WPPT>(src, bt.d_cols, KT, 64, b_lds + b * 64 * KT, tid, NT);
-      }
-      if (LORA) {
-        _Float16 const *src = static_cast<_Float16 const *>(P.la.ptr) + gtile_offset(P.la, bx, by, bz, it);
-        stage_weight<(KTMAX / 4) * 2 / NT + 1>(src, P.la.d_cols, KT, 16, la_lds, tid, NT);
-      }
     }
-    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      store_weight<WPPT>(wreg[b], KT, 64, b_lds + b * 64 * KT, tid, NT);
+    }
+    if (LORA) {
+      store_weight<LORA ? LPPT : 1>(lreg, KT, 16, la_lds, tid, NT);
+    }
+  };
+  auto compute = [&]() {
     // ---- lora inner product, transposed: D^T = A^T . X^T (rows past M are zero) -----
     half4 dfrag = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
     if (LORA) {
@@ -264,7 +336,24 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
         }
       }
     }
+  };
+
+  // Steady state is branch-free: the next iteration's loads are issued as soon as this
+  // iteration's tiles are in LDS and stay in flight while it is multiplied; the last
+  // iteration is peeled.
+  fetch(it_begin);
+  for (int it = it_begin; it + 1 < it_end; it++) {
+    __syncthreads();  // previous iteration's tiles fully consumed
+    stash();
+    __syncthreads();
+    fetch(it + 1);
+    __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the products
+    compute();
   }
+  __syncthreads();
+  stash();
+  __syncthreads();
+  compute();
 
   // ---- finish ---------------------------------------------------------------------------
   // The workgroup's fp16 sums go through LDS so that they leave as 16-byte row
