@@ -639,11 +639,25 @@ int try_launch_gemm(DevProgram const &P) {
   A.forloop_range = P.forloop_range;
   int const mt = (G.M + 15) / 16;
   long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
-  // aim at three workgroups per compute unit; never more ranges than iterations
-  int ksplit = (int)((3 * 256 + blocks - 1) / blocks);
-  ksplit = ksplit < 1 ? 1 : (ksplit > P.forloop_range ? P.forloop_range : ksplit);
-  int per = (P.forloop_range + ksplit - 1) / ksplit;
-  ksplit = (P.forloop_range + per - 1) / per;  // no empty ranges
+  // Ranges per block: the split that minimises (rounds of resident workgroups) x
+  // (iterations per workgroup + a fixed cost per workgroup + the combine's cost per range),
+  // with two workgroups resident per compute unit.  Never more ranges than iterations.
+  int ksplit = 1;
+  {
+    double best = 1e30;
+    for (int cand = 1; cand <= P.forloop_range; cand++) {
+      int const per = (P.forloop_range + cand - 1) / cand;
+      if ((P.forloop_range + per - 1) / per != cand) {
+        continue;  // would leave empty ranges
+      }
+      long long const rounds = (blocks * cand + 511) / 512;
+      double const cost = (double)rounds * (per + 1.5 + 0.15 * cand);
+      if (cost < best - 1e-9) {
+        best = cost;
+        ksplit = cand;
+      }
+    }
+  }
   long long const scratch_elems = blocks * ksplit * G.nb * G.M * 64;
   if (ksplit > 1 && (scratch_elems * 2 > (long long)s.scratch_bytes)) {
     ksplit = 1;
