@@ -138,6 +138,8 @@ FACADE = {
     "mirage_tensor_same_fingerprint": (_ci, [_vp, _vp]),
     "mirage_graph_fingerprint": (_ci, [_vp, _u64, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
+    "mirage_graph_from_json": (_vp, [ctypes.c_char_p]),
+    "mirage_graph_to_json": (ctypes.c_longlong, [_vp, ctypes.c_char_p, ctypes.c_longlong]),
     "mirage_set_smem_budget": (None, [_sz]),
     "mirage_get_smem_budget": (_sz, []),
     "mirage_device_ready": (_ci, []),

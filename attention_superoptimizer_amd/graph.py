@@ -128,9 +128,28 @@ def _c_plan(plan: dict) -> N.MirageCPlan:
 class KNGraph:
     """mirage::kernel::Graph."""
 
-    def __init__(self):
+    def __init__(self, _handle=None):
         self._rt = N.runtime()
-        self._g = ctypes.c_void_p(self._rt.mirage_graph_create())
+        self._g = ctypes.c_void_p(_handle if _handle is not None else self._rt.mirage_graph_create())
+
+    @classmethod
+    def from_json(cls, text) -> "KNGraph":
+        """from_json(json, Graph) of the reference (src/kernel/graph.cc:39-159): rebuilds a
+        kernel graph from its JSON wire format (a str, or an already decoded list)."""
+        import json as _json
+        if not isinstance(text, str):
+            text = _json.dumps(text)
+        h = N.runtime().mirage_graph_from_json(text.encode())
+        if not h:
+            raise ValueError("malformed mugraph JSON")
+        return cls(_handle=h)
+
+    def to_json(self) -> str:
+        """to_json(json, Graph) (src/kernel/graph.cc:33-37), one line, sorted keys."""
+        n = self._rt.mirage_graph_to_json(self._g, None, 0)
+        buf = ctypes.create_string_buffer(n + 1)
+        self._rt.mirage_graph_to_json(self._g, buf, n + 1)
+        return buf.value.decode()
 
     def close(self):
         if self._g is not None:

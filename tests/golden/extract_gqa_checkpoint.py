@@ -10,8 +10,13 @@ tensor guids), dims/layouts of inputs, and each customized op's plan.  The
 older schema has no `reduction_dimx`; the reference default 64 applies
 (include/mirage/threadblock/graph.h:40).
 
+It also keeps an excerpt of the file in its ORIGINAL schema (the computation graph
+and every ninth generated graph, verbatim JSON objects): the data the JSON wire format
+of the host API is tested against.
+
 Usage: python tests/golden/extract_gqa_checkpoint.py [reference_root]
-Writes tests/golden/gqa_spec_decode_69.json
+Writes tests/golden/gqa_spec_decode_69.json and
+tests/golden/gqa_spec_decode_checkpoint_excerpt.json
 """
 import json
 import os
@@ -78,6 +83,17 @@ def main():
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gqa_spec_decode_69.json")
     with open(dst, "w") as f:
         json.dump(doc, f, separators=(",", ":"))
+    picks = list(range(0, len(j["generated_graphs"]), 9))
+    excerpt = {
+        "source": "demo/checkpoint_group_query_attn_spec_decode.json",
+        "indices": picks,
+        "computation_graph": j["computation_graph"],
+        "generated_graphs": [j["generated_graphs"][i] for i in picks],
+    }
+    dst = os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                       "gqa_spec_decode_checkpoint_excerpt.json")
+    with open(dst, "w") as f:
+        json.dump(excerpt, f, separators=(",", ":"), sort_keys=True)
     print(dst, os.path.getsize(dst), "bytes,", len(doc["generated_graphs"]), "graphs")
 
 

@@ -99,3 +99,27 @@ def test_verify_batch_iota_inputs_and_output_count(rt):
         for g in reversed(graphs):
             g.close()
         ref_g.close()
+
+
+def test_checkpoint_graphs_loaded_from_json_verify_equal(rt):
+    """The reference's own checkpoint objects (original schema) loaded through the JSON
+    wire format: every graph its search accepted verifies equal to the computation graph
+    with the reference's `idx % 25651` inputs."""
+    import json
+    import os
+    from helpers import GOLDEN
+    with open(os.path.join(GOLDEN, "gqa_spec_decode_checkpoint_excerpt.json")) as f:
+        doc = json.load(f)
+    ref_g = rt.KNGraph.from_json(doc["computation_graph"])
+    graphs = []
+    try:
+        ref_g.fingerprint_seeded(0)
+        for ops in doc["generated_graphs"]:
+            graphs.append(rt.KNGraph.from_json(ops))
+        verdicts, stats = rt.verify_batch(graphs, ref_g, 0)
+        assert verdicts == [True] * len(graphs)
+        assert stats["customized_ops"] >= len(graphs)
+    finally:
+        for g in reversed(graphs):
+            g.close()
+        ref_g.close()
