@@ -99,6 +99,7 @@ ABI = {
     "mi355_fp_equal_enqueue": (_ci, [_vp, _vp, _sz, _ci]),
     "mi355_fp_equal_collect": (_ci, [_ci, _ci, _vp]),
     "mi355_customized_fp": (_ci, [_pplan, _pvp, _pvp]),
+    "mi355_customized_fp_batch": (_ci, [_pplan, _ci, _pvp, _pvp]),
     "mi355_plan_extents": (_ci, [_pplan, _pll, _pll, _pi, _pi]),
     "mi355_customized_run": (_ci, [_pplan, _pvp, _pvp]),
     "mi355_customized_profile": (_ci, [_pplan, _pvp, _pvp, _ci, _ci, _ci, _pf]),

@@ -842,6 +842,28 @@ extern "C" int mi355_customized_fp(mi355_plan const *plan, void const *const *in
   return launch(prog, false);
 }
 
+extern "C" int mi355_customized_fp_batch(mi355_plan const *plans, int n,
+                                         void const *const *inputs, void *const *outputs) {
+  MI355_REQUIRE_INIT();
+  if (n < 0 || (n > 0 && (plans == nullptr || inputs == nullptr || outputs == nullptr))) {
+    return fail(MI355_ERR_INVALID, "bad batch (n = %d)", n);
+  }
+  // independent operators: dealt over the queues so their (often small) grids overlap
+  int const home = tls_queue;
+  int rc = MI355_OK;
+  for (int i = 0; i < n && rc == MI355_OK; i++) {
+    tls_queue = (home + i) % MI355_NUM_QUEUES;
+    DevProgram prog;
+    rc = prepare(&plans[i], inputs + (size_t)i * MI355_MAX_DMEM_INPUTS,
+                 outputs + (size_t)i * MI355_MAX_DMEM_OUTPUTS, false, prog);
+    if (rc == MI355_OK) {
+      rc = launch(prog, false);
+    }
+  }
+  tls_queue = home;
+  return rc;
+}
+
 extern "C" int mi355_customized_run(mi355_plan const *plan, void const *const *inputs,
                                     void *const *outputs) {
   MI355_REQUIRE_INIT();

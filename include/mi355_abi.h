@@ -172,6 +172,15 @@ int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal);
 int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,
                         void *const *outputs);
 
+/* n independent customized-op fingerprints in one call (the batched form of the entry above
+ * for a verification loop that holds many candidates, src/search/search.cc:601-603):
+ * operator i reads inputs[4*i .. 4*i+3] and writes outputs[4*i .. 4*i+3]; the operators are
+ * dealt round-robin over the backend's queues starting at the caller's, so the caller must
+ * mi355_sync (or collect compares) before reading results, and must not pass operators
+ * that depend on each other. */
+int mi355_customized_fp_batch(mi355_plan const *plans, int n, void const *const *inputs,
+                              void *const *outputs);
+
 /* Host-only check of a plan (no device needed): 1 + the largest element index the
  * plan reads from each input / writes to each output, and the LDS the two
  * interpreters would request.  Callers compare the extents with their tensors'

@@ -170,3 +170,43 @@ def test_baseline_configs_fingerprint(rt):
         if ref is not None:
             got_ref = _graph_fp(rt, ref, ins)
             assert np.array_equal(got_ref[-1][0], got[-1][0]), name
+
+
+def test_customized_fp_batch_matches_single_launches(rt, abi):
+    """mi355_customized_fp_batch over several independent plans = one mi355_customized_fp
+    each, bit for bit."""
+    from attention_superoptimizer_amd import _native as N
+    from attention_superoptimizer_amd import workloads as W
+    specs = [W.tiled_matmul(128, 256, 256, (4, 2, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1))[0],
+             W.tiled_matmul(64, 64, 512, (1, 1, 1), 8, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1))[0],
+             W.config1_fused_matmul()[0], W.config2_gqa_decode()[0]]
+    built, plans, ins, outs, want = [], (N.Mi355Plan * len(specs))(), [], [], []
+    try:
+        for k, spec in enumerate(specs):
+            g, vals = rt.build_from_spec(spec)
+            built.append(g)
+            idx = len(spec) - 1
+            for i, op in enumerate(spec):
+                if op["op"] == "input":
+                    vals[i][0].write_fingerprint(uniform_fp(op["dims"], 500 + 10 * k + i))
+            g.fingerprint(idx)
+            want.append([t.read_fingerprint() for t in vals[idx]])
+            for t in vals[idx]:
+                t.write_fingerprint(np.zeros(t.dims, np.uint16))
+            plans[k] = g.lowered(idx, True)
+            row_in = [vals[a][b].device_ptr(True) for a, b in spec[idx]["in"]]
+            row_out = [t.device_ptr(True) for t in vals[idx]]
+            ins += row_in + [0] * (4 - len(row_in))
+            outs += row_out + [0] * (4 - len(row_out))
+            built[-1]._vals = vals
+        i_p = (ctypes.c_void_p * len(ins))(*ins)
+        o_p = (ctypes.c_void_p * len(outs))(*outs)
+        assert abi.mi355_customized_fp_batch(plans, len(specs), i_p, o_p) == 0, N.last_error()
+        assert abi.mi355_sync() == 0
+        for k, spec in enumerate(specs):
+            got = [t.read_fingerprint() for t in built[k]._vals[len(spec) - 1]]
+            for a, b in zip(got, want[k]):
+                assert np.array_equal(a, b), k
+    finally:
+        for g in reversed(built):
+            g.close()
