@@ -173,11 +173,14 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
   constexpr int NW = RG * IP, NT = 64 * NW;
-  // staging work per thread and per for-loop iteration, in 4x8 patches
-  constexpr int KP = (D / 4) * (NK / 8), VP = (NK / 4) * (DV / 8);
-  constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
-  // iterations whose loads are issued together (at most 8 patches = 32 x 16 B per thread)
-  constexpr int SG = (8 / (KPT + VPT)) < 1 ? 1 : ((8 / (KPT + VPT)) > 4 ? 4 : (8 / (KPT + VPT)));
+  // staging work per for-loop iteration, in 4x8 patches: K patches then V patches.  The
+  // patches of up to SG iterations form one list that ALL threads share out (a K or V
+  // tile alone may have fewer patches than the workgroup has threads)
+  constexpr int KP = (D / 4) * (NK / 8), VP = (NK / 4) * (DV / 8), PER_IT = KP + VP;
+  // iterations whose loads are issued together: at most 8 patches = 32 x 16 B per thread
+  constexpr int SG_RAW = 8 * NT / PER_IT;
+  constexpr int SG = SG_RAW < 1 ? 1 : (SG_RAW > 4 ? 4 : SG_RAW);
+  constexpr int IPT = (SG * PER_IT + NT - 1) / NT;  // patches per thread and load phase
   constexpr int SLOT_DW = DB * 2 + 1;  // one wavefront's iteration result, dwords per lane
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -224,49 +227,31 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
     }
     for (int s0 = 0; s0 < n_st; s0 += SG) {
       // phase 1: every load of up to SG iterations goes out before anything waits
-      Patch kp[SG][KPT], vp[SG][VPT];
+      Patch pt[IPT];
 #pragma unroll
-      for (int u = 0; u < SG; u++) {
-        if (s0 + u < n_st) {
-          _Float16 const *kg =
-              static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it0 + s0 + u);
-          _Float16 const *vg =
-              static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it0 + s0 + u);
-#pragma unroll
-          for (int i = 0; i < KPT; i++) {
-            int p = tid + i * NT;
-            if (KP % NT == 0 || p < KP) {
-              kp[u][i] = load_patch(kg, P.k.d_cols, NK / 8, p);
-            }
-          }
-#pragma unroll
-          for (int i = 0; i < VPT; i++) {
-            int p = tid + i * NT;
-            if (VP % NT == 0 || p < VP) {
-              vp[u][i] = load_patch(vg, P.v.d_cols, DV / 8, p);
-            }
-          }
+      for (int i = 0; i < IPT; i++) {
+        int const item = tid + i * NT;
+        int const u = item / PER_IT, r = item % PER_IT;
+        if (u < SG && s0 + u < n_st) {
+          bool const is_k = r < KP;  // uniform per wavefront: KP is a multiple of 64
+          TileAddr const &ta = is_k ? P.k : P.v;
+          _Float16 const *src =
+              static_cast<_Float16 const *>(ta.ptr) + tile_offset(ta, bx, by, bz, it0 + s0 + u);
+          pt[i] = load_patch(src, ta.d_cols, is_k ? NK / 8 : DV / 8, is_k ? r : r - KP);
         }
       }
       // phase 2: transpose in registers, write K^T [NK][D] and V^T [DV][NK]
 #pragma unroll
-      for (int u = 0; u < SG; u++) {
-        if (s0 + u < n_st) {
+      for (int i = 0; i < IPT; i++) {
+        int const item = tid + i * NT;
+        int const u = item / PER_IT, r = item % PER_IT;
+        if (u < SG && s0 + u < n_st) {
+          bool const is_k = r < KP;
           _Float16 *kt = reinterpret_cast<_Float16 *>(lds + (s0 + u) * P.lds_stage_bytes);
-          _Float16 *vt = kt + NK * D;
-#pragma unroll
-          for (int i = 0; i < KPT; i++) {
-            int p = tid + i * NT;
-            if (KP % NT == 0 || p < KP) {
-              store_patch_transposed(kp[u][i], kt, D, NK / 8, p);
-            }
-          }
-#pragma unroll
-          for (int i = 0; i < VPT; i++) {
-            int p = tid + i * NT;
-            if (VP % NT == 0 || p < VP) {
-              store_patch_transposed(vp[u][i], vt, NK, DV / 8, p);
-            }
+          if (is_k) {
+            store_patch_transposed(pt[i], kt, D, NK / 8, r);
+          } else {
+            store_patch_transposed(pt[i], kt + NK * D, NK, DV / 8, r - KP);
           }
         }
       }
