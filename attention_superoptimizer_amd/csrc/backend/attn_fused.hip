@@ -368,8 +368,8 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
           }
         }
       }
-      if (IP > 1) {
-        __syncthreads();  // slots are free again
+      if (IP > 1 && r0 + IP < n_st) {
+        __syncthreads();  // slots are free again for the next round
       }
     }
   }
