@@ -251,7 +251,7 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
           if (is_k) {
             store_patch_transposed(pt[i], kt, D, NK / 8, r);
           } else {
-            store_patch_transposed(pt[i], kt + NK * D, NK, DV / 8, r - KP);
+            store_patch_transposed<true>(pt[i], kt + NK * D, NK, DV / 8, r - KP);
           }
         }
       }
@@ -267,8 +267,14 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
         _Float16 const *kt = reinterpret_cast<_Float16 const *>(lds + s * P.lds_stage_bytes);
         _Float16 const *vt = kt + NK * D;
         // ---- S^T = K^T . Q^T, exp, row sum ----------------------------------------
-        half4 e[KB];  // e[j][r] = E[row c][key 16j + 4g + r]
+        // pk[jj][0..3]: eight keys of this lane's query row, packed fp16 (keys 4g..4g+3 of
+        // key blocks 2jj and 2jj+1): the A operand of P.V as the accumulators leave it.
+        // Roundings as the sequential program makes them: S to fp16, exp in fp32, the
+        // result to fp16; the row sum adds the rounded values in fp32.
+        uint32_t pk[KB / 2][4];
         float rs = 0.0f;
+        half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
+        constexpr float LOG2E = 1.44269504088896340736f;
 #pragma unroll
         for (int j = 0; j < KB; j++) {
           float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -278,11 +284,13 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
             acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kk], acc, 0, 0, 0);
           }
 #pragma unroll
-          for (int r = 0; r < 4; r++) {
-            _Float16 s16 = static_cast<_Float16>(acc[r]);                           // S tile
-            _Float16 e16 = static_cast<_Float16>(__expf(static_cast<float>(s16)));  // E tile
-            e[j][r] = e16;
-            rs += static_cast<float>(e16);
+          for (int h = 0; h < 2; h++) {
+            half2v const s2 = {static_cast<_Float16>(acc[2 * h]), static_cast<_Float16>(acc[2 * h + 1])};
+            float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
+            float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
+            half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
+            rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);
+            pk[j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
           }
         }
         rs += __shfl_xor(rs, 16, 64);
@@ -292,10 +300,13 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
           // one reciprocal per row, then multiplies: within an fp32 ulp of the division
           float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
 #pragma unroll
-          for (int j = 0; j < KB; j++) {
+          for (int jj = 0; jj < KB / 2; jj++) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-              e[j][r] = static_cast<_Float16>(static_cast<float>(e[j][r]) * inv);
+            for (int w = 0; w < 4; w++) {
+              half2v const e2 = __builtin_bit_cast(half2v, pk[jj][w]);
+              half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
+                                 static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+              pk[jj][w] = __builtin_bit_cast(uint32_t, p2);
             }
           }
         }
@@ -306,13 +317,10 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
           int const vrow = 16 * t + c;
 #pragma unroll
           for (int jj = 0; jj < KB / 2; jj++) {
-            half4 b0 = *reinterpret_cast<half4 const *>(vt + swz_chunk(vrow, 4 * jj + (g >> 1), NK) +
-                                                        (g & 1) * 4);
-            half4 b1 = *reinterpret_cast<half4 const *>(
-                vt + swz_chunk(vrow, 4 * jj + 2 + (g >> 1), NK) + (g & 1) * 4);
-            half8 a = __builtin_shufflevector(e[2 * jj], e[2 * jj + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-            half8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
-            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, o, 0, 0, 0);
+            // paired key groups (see store_patch_transposed): one 16-byte read per operand
+            half8 b = *reinterpret_cast<half8 const *>(vt + swz_chunk(vrow, 4 * jj + g, NK));
+            uint4v const a = {pk[jj][0], pk[jj][1], pk[jj][2], pk[jj][3]};
+            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o, 0, 0, 0);
           }
 #pragma unroll
           for (int r = 0; r < 4; r++) {
