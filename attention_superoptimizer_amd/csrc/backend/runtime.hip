@@ -10,7 +10,7 @@
 namespace mi355 {
 
 static State g_state;
-static char g_error[512] = "";
+thread_local char g_error[512] = "";  // per host thread: several may enqueue side by side
 
 State &state() { return g_state; }
 

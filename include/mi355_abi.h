@@ -98,6 +98,7 @@ typedef struct mi355_launch_info {
 int mi355_init(size_t arena_bytes, void **arena_base);
 int mi355_shutdown(void);
 int mi355_is_initialised(void);
+/* message of the calling host thread's most recent failed call */
 char const *mi355_last_error(void);
 int mi355_get_device_info(mi355_device_info *info);
 int mi355_set_option(int option, int value);
