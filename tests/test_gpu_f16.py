@@ -229,3 +229,33 @@ def test_attention_throughput_variant(rt, abi):
         assert _last_kernels[0] == KERNEL_ATTENTION
     finally:
         assert abi.mi355_set_option(2, 0) == 0
+
+
+def test_full_size_configs_routes_agree(rt, abi):
+    """Full benchmark sizes, where the scalar golden is too slow to run: the fused kernel
+    and the generic LDS interpreter (each checked against the golden at reduced size) must
+    agree within the tolerance, and C3 must be softmax attention (float64 on the host, four
+    of the 32 heads)."""
+    from attention_superoptimizer_amd import workloads as W
+    for name in ("C1_fused_matmul", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp"):
+        spec, _ = W.BASELINE_CONFIGS[name]()
+        ins = _inputs(spec, W.INPUT_STD[name], 0xC0FFEE00)
+        outs = {}
+        for route, force in (("fused", 0), ("interpreter", 1)):
+            assert abi.mi355_set_option(1, force) == 0
+            try:
+                outs[route] = _graph_f16(rt, spec, ins)[-1][0]
+                kernels = list(_last_kernels)
+            finally:
+                assert abi.mi355_set_option(1, 0) == 0
+            if route == "fused":
+                assert all(k != KERNEL_INTERP for k in kernels), (name, kernels)
+            else:
+                assert all(k == KERNEL_INTERP for k in kernels), (name, kernels)
+        assert_f16_close(outs["fused"], outs["interpreter"], what=f"{name} fused vs interpreter")
+        if name == "C3_mha_prefill":
+            Q, K, V = (ins[i][:4].astype(np.float64) for i in range(3))
+            s = Q @ K
+            p = np.exp(s - s.max(axis=-1, keepdims=True))
+            att = (p / p.sum(axis=-1, keepdims=True)) @ V
+            assert_f16_close(outs["fused"][:4], att, rtol=1e-2, atol=2e-3, what="C3 vs softmax attention")

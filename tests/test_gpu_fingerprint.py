@@ -210,3 +210,25 @@ def test_customized_fp_batch_matches_single_launches(rt, abi):
     finally:
         for g in reversed(built):
             g.close()
+
+
+def test_full_size_configs_equal_their_unfused_graphs(rt):
+    """At the benchmark's full sizes the oracle is too slow to be the checker; the
+    size-independent property is the one the reference's search relies on: a mugraph and the
+    un-fused kernel graph it rewrites have the same fingerprint.  The un-fused side runs
+    on the kernel-level fingerprint operators, code the customized-op interpreter shares
+    nothing with.  Both input conventions: uniform values and the reference's idx % 25651."""
+    from attention_superoptimizer_amd import workloads as W
+    for name in ("C1_fused_matmul", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp"):
+        spec, ref = W.BASELINE_CONFIGS[name]()
+        assert ref is not None
+        for seed in (0, 0xC0FFEE):
+            g, _ = rt.build_from_spec(spec)
+            r, _ = rt.build_from_spec(ref)
+            try:
+                r.fingerprint_seeded(seed)
+                verdicts, _ = rt.verify_batch([g], r, seed)
+                assert verdicts == [True], (name, seed)
+            finally:
+                r.close()
+                g.close()
