@@ -41,8 +41,43 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+// Two gfx950 data movers the throughput kernel is built on.
+// lds_dma16: every lane fetches 16 bytes from its own global address
+// (`gbase`, wave-uniform, plus its own byte offset); the wavefront's 64 chunks land in LDS
+// at `lds_wave_base` + 16 * lane (wave-uniform, passed in m0), without passing through
+// registers.  Completion is tracked by vmcnt.  Written as
+// inline assembly on purpose: for the builtin the compiler makes the first LDS read after
+// it wait for vmcnt(0) whenever it cannot prove the two do not alias, which serialises the
+// transfer with the compute it is meant to run under.  The caller waits (`s_waitcnt
+// vmcnt(0)`) before the barrier that publishes the data.  No other instruction of these
+// kernels reads m0.
+// lds_read_tr16: within each group of 16 lanes, lane r supplies the address of four
+// consecutive halfs X[r][0..3]; lane i receives X[i / 4 + 4 * e][i % 4] for e = 0..3, i.e.
+// the transposed operand an MFMA wants when the tile lies in LDS row-major in k.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ uint32_t lds_address(void const *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void const *)p;
+}
+__device__ __forceinline__ void lds_dma16(_Float16 const *gbase, uint32_t lane_byte_offset,
+                                          uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(lane_byte_offset),
+                 "s"(gbase)
+               : "m0", "memory");
+}
+#pragma clang diagnostic pop
+__device__ __forceinline__ half4 lds_read_tr16(_Float16 const *p) {
+  typedef short short4v __attribute__((ext_vector_type(4)));
+  short4v const v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (short4v __attribute__((address_space(3))) *)(__attribute__((address_space(3))) void *)(p));
+  return __builtin_bit_cast(half4, v);
+}
 
 struct TileAddr {
   void const *ptr;
@@ -412,33 +447,40 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
 }
 
 // Throughput variant for large problems: every wavefront owns RPW row groups of 16
-// query rows (so each K^T / V^T operand fetched from LDS feeds RPW MFMAs) and walks
-// all for-loop iterations itself; K / V tiles are double-buffered in LDS and the
-// global loads of the next tiles are in flight (in registers) while the current ones
-// are on the matrix cores.  One barrier per iteration.
+// query rows (so each K / V operand fetched from LDS feeds RPW MFMAs) and walks all
+// for-loop iterations itself.  K and V tiles are double-buffered in LDS in their global
+// (row-major) layout: the next tiles stream from global memory straight into LDS while
+// the current ones are on the matrix cores, and the MFMA operands are gathered with
+// transposing LDS reads.  One barrier per iteration.
+//
+// LDS layout of a tile with rows of CPR 16-byte chunks: chunk p of row r is stored at
+// chunk position p ^ 2 * (r & 3) of that row, which spreads the four rows a transposing
+// read touches per 16-lane group over all banks.
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW>
 __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
   constexpr int NT = 64 * RG;
-  constexpr int KP = (D / 4) * (NK / 8), VP = (NK / 4) * (DV / 8);
-  constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
-  constexpr int STAGE = (NK * D + DV * NK);  // halfs per buffer
+  constexpr int KC = D * NK / 8, VC = NK * DV / 8;  // 16-byte chunks per tile
+  constexpr int KI = KC / NT, VI = VC / NT;          // direct loads per wavefront and tile
+  static_assert(KC % NT == 0 && VC % NT == 0, "tiles must split evenly over the wavefronts");
+  static_assert(NK / 8 >= 8 && DV / 8 >= 8, "the chunk swizzle needs rows of 8 chunks");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   _Float16 *const buf = reinterpret_cast<_Float16 *>(lds);
 
   int const tid = threadIdx.x;
-  int const lane = tid % 64, wave = tid / 64;
+  int const lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
   int const g = lane / 16, c = lane % 16;
   int bx, by, bz, slice;
   decode_block(P, bx, by, bz, slice);
-  // Swizzled operand addresses = lane part + compile-time part.  For row 16j + c the
-  // swizzle key (row ^ row>>3) & 7 is s0 ^ (2j & 7) with s0 = (c ^ c>>3) & 7, and a
-  // chunk index 4kk + g is 4kk ^ g, so chunk ^ key = (s0 ^ g) ^ (4kk ^ (2j & 7)): one
-  // XOR with a constant per fetch, everything else folds into the instruction offset.
-  int const s0 = (c ^ (c >> 3)) & 7;
-  int const k_lane = c * D, k_sg8 = (s0 ^ g) << 3;            // K^T: row c, 16-byte chunk g
-  int const v_lane = c * NK, v_sg8 = (s0 ^ g) << 3;           // V^T: row c, 16-byte chunk g
+  // Transposing reads: lane (g, c) supplies row 8g + c / 4 (K, rows are d) or 4g + c / 4
+  // (V, rows are keys) and halfs 4 * (c % 4) .. + 3 of a 16-column block.  The row's
+  // swizzle key is 2 * (c / 4) whatever the block, so the swizzled chunk of column block
+  // x is 2 * (x ^ c / 4) + (c % 4) / 2: one XOR with a compile-time constant per fetch.
+  int const a4 = c >> 2, b4 = c & 3;
+  int const k_lane = (8 * g + a4) * NK + ((b4 >> 1) << 3) + (b4 & 1) * 4;
+  int const v_lane = (4 * g + a4) * DV + ((b4 >> 1) << 3) + (b4 & 1) * 4;
+  int const sw = a4 << 4;
   int const row_base = (slice * RG + wave) * RPW * 16;
   int const F = P.forloop_range;
 
@@ -469,57 +511,41 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     }
   }
 
-  Patch kp[KPT], vp[VPT];
-  // lane offsets of this thread's patches inside a tile (the same every iteration)
-  uint32_t k_off[KPT], v_off[VPT];
+  _Float16 *const kbuf = buf;               // two K tiles [D][NK]
+  _Float16 *const vbuf = buf + 2 * NK * D;  // two V tiles [NK][DV]
+  uint32_t const lds_k = lds_address(kbuf), lds_v = lds_address(vbuf);
+  // Direct load i of this wavefront fills LDS chunks 64 * (wave * KI + i) .. + 63 of the
+  // tile; this lane's chunk is (row r, position pos) and comes from global chunk
+  // pos ^ 2 * (r & 3) of row r (byte offsets from the tile's first element).
+  uint32_t k_goff[KI], v_goff[VI];
 #pragma unroll
-  for (int i = 0; i < KPT; i++) {
-    int const p = tid + i * NT;
-    k_off[i] = (uint32_t)(4 * (p / (NK / 8)) * P.k.d_cols + 8 * (p % (NK / 8)));
+  for (int i = 0; i < KI; i++) {
+    int const q = (wave * KI + i) * 64 + lane;
+    int const r = q / (NK / 8), pos = q % (NK / 8);
+    k_goff[i] = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * (r & 3))));
   }
 #pragma unroll
-  for (int i = 0; i < VPT; i++) {
-    int const p = tid + i * NT;
-    v_off[i] = (uint32_t)(4 * (p / (DV / 8)) * P.v.d_cols + 8 * (p % (DV / 8)));
+  for (int i = 0; i < VI; i++) {
+    int const q = (wave * VI + i) * 64 + lane;
+    int const r = q / (DV / 8), pos = q % (DV / 8);
+    v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * (r & 3))));
   }
-  auto load_k = [&](int it) {
+  auto fetch_k = [&](int it, int b) {
     _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
 #pragma unroll
-    for (int i = 0; i < KPT; i++) {
-      if (KP % NT == 0 || tid + i * NT < KP) {
-        kp[i] = load_patch_at(kg, k_off[i], P.k.d_cols);
-      }
+    for (int i = 0; i < KI; i++) {
+      lds_dma16(kg, k_goff[i], lds_k + 2u * (uint32_t)(b * NK * D + (wave * KI + i) * 512));
     }
   };
-  auto load_v = [&](int it) {
+  auto fetch_v = [&](int it, int b) {
     _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
 #pragma unroll
-    for (int i = 0; i < VPT; i++) {
-      if (VP % NT == 0 || tid + i * NT < VP) {
-        vp[i] = load_patch_at(vg, v_off[i], P.v.d_cols);
-      }
+    for (int i = 0; i < VI; i++) {
+      lds_dma16(vg, v_goff[i], lds_v + 2u * (uint32_t)(b * DV * NK + (wave * VI + i) * 512));
     }
   };
-  _Float16 *const kbuf = buf;               // two K^T tiles
-  _Float16 *const vbuf = buf + 2 * NK * D;  // two V^T tiles
-  auto write_k = [&](int b) {
-#pragma unroll
-    for (int i = 0; i < KPT; i++) {
-      int p = tid + i * NT;
-      if (KP % NT == 0 || p < KP) {
-        store_patch_transposed(kp[i], kbuf + b * NK * D, D, NK / 8, p);
-      }
-    }
-  };
-  auto write_v = [&](int b) {
-#pragma unroll
-    for (int i = 0; i < VPT; i++) {
-      int p = tid + i * NT;
-      if (VP % NT == 0 || p < VP) {
-        store_patch_transposed<true>(vp[i], vbuf + b * DV * NK, NK, DV / 8, p);
-      }
-    }
-  };
+  // all direct loads of this wavefront have landed; the barrier that follows publishes them
+  auto fetched = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
   // P of one iteration, packed fp16: pk[rp][jj][0..3] = eight keys of this lane's query
   // row (keys 4g..4g+3 of key blocks 2jj and 2jj+1), the A operand of P.V.
@@ -536,8 +562,10 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     }
 #pragma unroll
     for (int kk = 0; kk < DK; kk++) {
-      half8 a = *reinterpret_cast<half8 const *>(
-          kt + k_lane + 16 * j * D + (k_sg8 ^ (((4 * kk) ^ ((2 * j) & 7)) << 3)));
+      // K[32kk + 8g + 0..7][16j + c]
+      _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw ^ (j << 4));
+      half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
+      half8 const a = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
         acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rp][kk], acc[rp], 0, 0, 0);
@@ -547,8 +575,8 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
       for (int h = 0; h < 2; h++) {
-        half2v const s2 = {static_cast<_Float16>(acc[rp][2 * h]),
-                           static_cast<_Float16>(acc[rp][2 * h + 1])};
+        float2v const f2 = {acc[rp][2 * h], acc[rp][2 * h + 1]};
+        half2v const s2 = __builtin_convertvector(f2, half2v);  // one packed conversion
         float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
         float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
         half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
@@ -591,9 +619,10 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     }
 #pragma unroll
     for (int jj = 0; jj < KB / 2; jj++) {
-      // row 16t + c, 16-byte chunk 4jj + g (paired key groups, see store_patch_transposed)
-      half8 b = *reinterpret_cast<half8 const *>(
-          vt + v_lane + 16 * t * NK + (v_sg8 ^ (((4 * jj) ^ ((2 * t) & 7)) << 3)));
+      // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
+      _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw ^ (t << 4));
+      half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
+      half8 const b = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
         uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
@@ -615,16 +644,14 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   // streams (matrix-heavy P.V, conversion / exp-heavy S) to overlap.  K tiles and V
   // tiles are double-buffered separately: pass `it` reads K(it + 1) and V(it) and, at its
   // end, replaces K(it) by K(it + 2) and V(it - 1) by V(it + 1).
-  load_k(0);
-  load_v(0);
-  write_k(0);
-  write_v(0);
+  fetch_k(0, 0);
+  fetch_v(0, 0);
   if (F > 1) {
-    load_k(1);
-    write_k(1);
+    fetch_k(1, 1);
   }
+  fetched();
   __syncthreads();
-  uint32_t pcur[RPW][KB / 2][4];
+  uint32_t pa[RPW][KB / 2][4], pb[RPW][KB / 2][4];  // P(it) and P(it + 1), roles alternate
   {
     float rs[RPW];
 #pragma unroll
@@ -633,16 +660,16 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     }
 #pragma unroll
     for (int j = 0; j < KB; j++) {
-      s_block(kbuf, j, pcur, rs);
+      s_block(kbuf, j, pa, rs);
     }
-    s_finish(pcur, rs);
+    s_finish(pa, rs);
   }
   __syncthreads();  // K(0) may be overwritten from here on
   // One skewed pass: P(it) . V(it) interleaved with building P(it + 1) from K(it + 1).
-  auto skewed_pass = [&](int it) {
+  auto skewed_pass = [&](int it, uint32_t const (&pcur)[RPW][KB / 2][4],
+                         uint32_t (&pnext)[RPW][KB / 2][4]) {
     _Float16 const *vt = vbuf + (it & 1) * DV * NK;
     _Float16 const *kt = kbuf + ((it + 1) & 1) * NK * D;
-    uint32_t pnext[RPW][KB / 2][4];
     float rs[RPW];
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
@@ -657,45 +684,50 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       }
     }
     s_finish(pnext, rs);
+  };
+  // Pass `it` starts by sending K(it + 2) after K(it) and V(it + 1) after V(it - 1) (both
+  // last read in the previous pass); the transfers run under the whole pass.  Two passes
+  // per trip, so that P(it) and P(it + 1) swap roles instead of being copied.
+  int it = 0;
+  for (; it + 3 < F; it += 2) {
+    fetch_k(it + 2, 0);
+    fetch_v(it + 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    skewed_pass(0, pa, pb);
+    fetched();
+    __syncthreads();
+    fetch_k(it + 3, 1);
+    fetch_v(it + 2, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    skewed_pass(1, pb, pa);
+    fetched();
+    __syncthreads();
+  }
+  for (; it + 1 < F; it++) {  // at most two passes left before the last P . V
+    if (it + 2 < F) {
+      fetch_k(it + 2, it & 1);
+    }
+    fetch_v(it + 1, (it + 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    skewed_pass(it, pa, pb);
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
       for (int jj = 0; jj < KB / 2; jj++) {
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-          pcur[rp][jj][w] = pnext[rp][jj][w];
+          pa[rp][jj][w] = pb[rp][jj][w];
         }
       }
     }
-  };
-  // The steady-state loop body is branch-free (the tail passes are peeled below): with a
-  // conditional prefetch inside the loop the compiler cannot prove that the previous
-  // pass's loads were consumed and makes each new group of loads wait for the one before.
-  int it = 0;
-  for (; it + 2 < F; it++) {
-    load_k(it + 2);  // both in flight while this pass computes
-    load_v(it + 1);
-    __builtin_amdgcn_sched_barrier(0);  // keep the loads up here, a whole pass ahead of their use
-    skewed_pass(it);
-    __builtin_amdgcn_sched_barrier(0);
-    write_k(it & 1);        // K(it) was last read in the previous pass
-    write_v((it + 1) & 1);  // V(it - 1) was last read in the previous pass
+    fetched();
     __syncthreads();
-  }
-  if (it + 1 < F) {  // pass F - 2: no K tile left to fetch
-    load_v(it + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    skewed_pass(it);
-    __builtin_amdgcn_sched_barrier(0);
-    write_v((it + 1) & 1);
-    __syncthreads();
-    it++;
   }
   {  // pass F - 1: the last P . V
     _Float16 const *vt = vbuf + (it & 1) * DV * NK;
 #pragma unroll
     for (int t = 0; t < DB; t++) {
-      pv_block(vt, t, pcur);
+      pv_block(vt, t, pa);
     }
     __syncthreads();
   }
