@@ -453,9 +453,22 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
 // the current ones are on the matrix cores, and the MFMA operands are gathered with
 // transposing LDS reads.  One barrier per iteration.
 //
-// LDS layout of a tile with rows of CPR 16-byte chunks: chunk p of row r is stored at
-// chunk position p ^ 2 * (r & 3) of that row, which spreads the four rows a transposing
-// read touches per 16-lane group over all banks.
+// LDS layout of a tile: 16-byte chunk p of row r is stored at chunk position
+// p ^ 2 * key(r) of that row.  A transposing read is served 32 lanes at a time; those
+// lanes touch eight rows (lane groups g, g + 1 and four rows each) and 32 bytes per row,
+// and the LDS has 64 banks of 4 bytes, so the keys are chosen to send the eight 32-byte
+// pieces to eight different bank groups:
+//   rows of 256 bytes (V, DV = 128): the rows are keys 4g + c / 4 (+ multiples of 16), and
+//     key(r) = r & 7 permutes the eight chunk pairs of the row;
+//   rows of 128 bytes, two per bank line: the row's parity picks the half line, the key
+//     permutes the four chunk pairs within it.  For K the rows are 8g + c / 4 (+ multiples
+//     of 4 and 32) and key(r) = bit 1 of r | bit 3 of r << 1; for V with DV = 64 the rows
+//     are 4g + c / 4 and key(r) = (r >> 1) & 3.
+template <int RowHalfs, bool IsK>
+__device__ __forceinline__ constexpr int stream_swizzle_key(int r) {
+  return RowHalfs == 128 ? (r & 7) : (IsK ? (((r >> 1) & 1) | (((r >> 3) & 1) << 1)) : ((r >> 1) & 3));
+}
+
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW>
 __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
@@ -475,12 +488,15 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   decode_block(P, bx, by, bz, slice);
   // Transposing reads: lane (g, c) supplies row 8g + c / 4 (K, rows are d) or 4g + c / 4
   // (V, rows are keys) and halfs 4 * (c % 4) .. + 3 of a 16-column block.  The row's
-  // swizzle key is 2 * (c / 4) whatever the block, so the swizzled chunk of column block
-  // x is 2 * (x ^ c / 4) + (c % 4) / 2: one XOR with a compile-time constant per fetch.
+  // swizzle key is the same for every block the lane reads, so the swizzled chunk of
+  // column block x is 2 * (x ^ key) + (c % 4) / 2: one XOR with a compile-time constant
+  // per fetch.
+  static_assert(NK == 64, "the K swizzle assumes rows of 128 bytes");
   int const a4 = c >> 2, b4 = c & 3;
   int const k_lane = (8 * g + a4) * NK + ((b4 >> 1) << 3) + (b4 & 1) * 4;
   int const v_lane = (4 * g + a4) * DV + ((b4 >> 1) << 3) + (b4 & 1) * 4;
-  int const sw = a4 << 4;
+  int const sw_k = stream_swizzle_key<NK, true>(8 * g + a4) << 4;
+  int const sw_v = stream_swizzle_key<DV, false>(4 * g + a4) << 4;
   int const row_base = (slice * RG + wave) * RPW * 16;
   int const F = P.forloop_range;
 
@@ -516,19 +532,19 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   uint32_t const lds_k = lds_address(kbuf), lds_v = lds_address(vbuf);
   // Direct load i of this wavefront fills LDS chunks 64 * (wave * KI + i) .. + 63 of the
   // tile; this lane's chunk is (row r, position pos) and comes from global chunk
-  // pos ^ 2 * (r & 3) of row r (byte offsets from the tile's first element).
+  // pos ^ 2 * key(r) of row r (byte offsets from the tile's first element).
   uint32_t k_goff[KI], v_goff[VI];
 #pragma unroll
   for (int i = 0; i < KI; i++) {
     int const q = (wave * KI + i) * 64 + lane;
     int const r = q / (NK / 8), pos = q % (NK / 8);
-    k_goff[i] = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * (r & 3))));
+    k_goff[i] = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(r))));
   }
 #pragma unroll
   for (int i = 0; i < VI; i++) {
     int const q = (wave * VI + i) * 64 + lane;
     int const r = q / (DV / 8), pos = q % (DV / 8);
-    v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * (r & 3))));
+    v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(r))));
   }
   auto fetch_k = [&](int it, int b) {
     _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
@@ -549,28 +565,38 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
 
   // P of one iteration, packed fp16: pk[rp][jj][0..3] = eight keys of this lane's query
   // row (keys 4g..4g+3 of key blocks 2jj and 2jj+1), the A operand of P.V.
-  // One 16-key block of S^T = K^T . Q^T for the RPW row groups, then the roundings the
-  // sequential program makes: S to fp16, exp in fp32, the result to fp16; the row sum
-  // adds the rounded values in fp32.
+  // One 16-key block of S^T = K^T . Q^T for the RPW row groups is made in three steps the
+  // pipeline below places separately: operand fetch from LDS, the MFMA chain, and the
+  // roundings the sequential program makes (S to fp16, exp in fp32, the result to fp16;
+  // the row sum adds the rounded values in fp32).
   half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
   constexpr float LOG2E = 1.44269504088896340736f;
-  auto s_block = [&](_Float16 const *kt, int j, uint32_t (&pk)[RPW][KB / 2][4], float (&rs)[RPW]) {
-    float4v acc[RPW];
+  auto s_fetch = [&](_Float16 const *kt, int j, half8 (&a)[DK]) {
+#pragma unroll
+    for (int kk = 0; kk < DK; kk++) {
+      // K[32kk + 8g + 0..7][16j + c]
+      _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw_k ^ (j << 4));
+      half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
+      a[kk] = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
+  auto s_mfma = [&](half8 const (&a)[DK], float4v (&acc)[RPW]) {
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       acc[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
     }
 #pragma unroll
     for (int kk = 0; kk < DK; kk++) {
-      // K[32kk + 8g + 0..7][16j + c]
-      _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw ^ (j << 4));
-      half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
-      half8 const a = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
-        acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rp][kk], acc[rp], 0, 0, 0);
+        acc[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[kk], qf[rp][kk], acc[rp], 0, 0, 0);
       }
     }
+  };
+  // Runs at raised wave priority: this is the only long stretch without matrix work, and
+  // the other wavefronts of the SIMD have MFMAs to overlap with it.
+  auto s_post = [&](float4v const (&acc)[RPW], int j, uint32_t (&pk)[RPW][KB / 2][4], float (&rs)[RPW]) {
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
@@ -584,6 +610,14 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
         pk[rp][j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
       }
     }
+    __builtin_amdgcn_s_setprio(0);
+  };
+  auto s_block = [&](_Float16 const *kt, int j, uint32_t (&pk)[RPW][KB / 2][4], float (&rs)[RPW]) {
+    half8 a[DK];
+    float4v acc[RPW];
+    s_fetch(kt, j, a);
+    s_mfma(a, acc);
+    s_post(acc, j, pk, rs);
   };
   // After the last key block: the row sum across the four lane groups, then either the
   // normalisation of P (form with div) or the accumulation of the denominator.
@@ -610,26 +644,33 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       }
     }
   };
-  // Sixteen output columns of O += P . V for the RPW row groups.
-  auto pv_block = [&](_Float16 const *vt, int t, uint32_t const (&pk)[RPW][KB / 2][4]) {
-    float4v o[RPW];
+  // Sixteen output columns of O += P . V for the RPW row groups: operand fetch, then the
+  // MFMA chain and the fp16 accumulation.
+  auto pv_fetch = [&](_Float16 const *vt, int t, half8 (&b)[KB / 2]) {
+#pragma unroll
+    for (int jj = 0; jj < KB / 2; jj++) {
+      // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
+      _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
+      half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
+      b[jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
+  auto pv_mfma = [&](half8 const (&b)[KB / 2], uint32_t const (&pk)[RPW][KB / 2][4], float4v (&o)[RPW]) {
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
     }
 #pragma unroll
     for (int jj = 0; jj < KB / 2; jj++) {
-      // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
-      _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw ^ (t << 4));
-      half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
-      half8 const b = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
         uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
-        o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o[rp], 0, 0,
-                                                       0);
+        o[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b[jj], o[rp], 0,
+                                                       0, 0);
       }
     }
+  };
+  auto pv_post = [&](float4v const (&o)[RPW], int t) {
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       half2v lo = {static_cast<_Float16>(o[rp][0]), static_cast<_Float16>(o[rp][1])};
@@ -637,6 +678,13 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       oacc[rp][t][0] = oacc[rp][t][0] + lo;
       oacc[rp][t][1] = oacc[rp][t][1] + hi;
     }
+  };
+  auto pv_block = [&](_Float16 const *vt, int t, uint32_t const (&pk)[RPW][KB / 2][4]) {
+    half8 b[KB / 2];
+    float4v o[RPW];
+    pv_fetch(vt, t, b);
+    pv_mfma(b, pk, o);
+    pv_post(o, t);
   };
 
   // The loop is skewed by one phase: pass `it` multiplies P(it) with V(it) while it
@@ -666,6 +714,10 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   }
   __syncthreads();  // K(0) may be overwritten from here on
   // One skewed pass: P(it) . V(it) interleaved with building P(it + 1) from K(it + 1).
+  // Within the pass the LDS operands of a step are requested one step ahead (before the
+  // exp stretch or the MFMA chain that precedes their use), so their latency is covered
+  // by this wavefront's own work; the scheduling barriers keep that order.
+  constexpr int TPU = DB / KB;  // P.V column blocks per S block
   auto skewed_pass = [&](int it, uint32_t const (&pcur)[RPW][KB / 2][4],
                          uint32_t (&pnext)[RPW][KB / 2][4]) {
     _Float16 const *vt = vbuf + (it & 1) * DV * NK;
@@ -675,13 +727,33 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     for (int rp = 0; rp < RPW; rp++) {
       rs[rp] = 0.0f;
     }
+    half8 ka[DK];
+    s_fetch(kt, 0, ka);
 #pragma unroll
     for (int u = 0; u < KB; u++) {
-      s_block(kt, u, pnext, rs);
+      float4v sacc[RPW];
+      s_mfma(ka, sacc);
+      half8 vb[TPU][KB / 2];
 #pragma unroll
-      for (int t = u * DB / KB; t < (u + 1) * DB / KB; t++) {
-        pv_block(vt, t, pcur);
+      for (int x = 0; x < TPU; x++) {
+        pv_fetch(vt, u * TPU + x, vb[x]);
       }
+      __builtin_amdgcn_sched_barrier(0);
+      s_post(sacc, u, pnext, rs);
+      if (u + 1 < KB) {
+        s_fetch(kt, u + 1, ka);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      float4v o[TPU][RPW];
+#pragma unroll
+      for (int x = 0; x < TPU; x++) {
+        pv_mfma(vb[x], pcur, o[x]);
+      }
+#pragma unroll
+      for (int x = 0; x < TPU; x++) {
+        pv_post(o[x], u * TPU + x);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
     s_finish(pnext, rs);
   };
