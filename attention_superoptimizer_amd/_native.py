@@ -114,6 +114,16 @@ ABI = {
     "mi355_timer_stop": (_ci, [_pf]),
 }
 
+class MirageLayoutStats(ctypes.Structure):
+    _fields_ = [("assignments", ctypes.c_longlong), ("measurements", ctypes.c_longlong),
+                ("truncated", ctypes.c_int), ("first_ms", ctypes.c_float),
+                ("best_ms", ctypes.c_float), ("worst_ms", ctypes.c_float)]
+
+
+# float cost(void *user, int op_index, int const *loader_layouts, int n)
+LAYOUT_COST_FN = ctypes.CFUNCTYPE(ctypes.c_float, ctypes.c_void_p, ctypes.c_int,
+                                  ctypes.POINTER(ctypes.c_int), ctypes.c_int)
+
 FACADE = {
     "mirage_graph_create": (_vp, []),
     "mirage_graph_destroy": (None, [_vp]),
@@ -139,6 +149,8 @@ FACADE = {
     "mirage_tensor_same_fingerprint": (_ci, [_vp, _vp]),
     "mirage_graph_fingerprint": (_ci, [_vp, _u64, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
+    "mirage_optimize_layout": (_ci, [_vp, ctypes.c_longlong, LAYOUT_COST_FN, _vp,
+                                     ctypes.POINTER(MirageLayoutStats)]),
     "mirage_graph_from_json": (_vp, [ctypes.c_char_p]),
     "mirage_graph_to_json": (ctypes.c_longlong, [_vp, ctypes.c_char_p, ctypes.c_longlong]),
     "mirage_set_smem_budget": (None, [_sz]),

@@ -61,6 +61,7 @@ struct State {
   mi355_launch_info last_launch{};
   int force_interpreter = 0;
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
+  int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
   // fused-kernel workspace: fp16 range sums of split for-loops
   // (each queue has its own slice of scratch_base, so concurrent queues never share)
   size_t scratch_bytes = 0;  // per queue

@@ -175,6 +175,10 @@ extern "C" int mi355_set_option(int option, int value) {
     state().attention_mode = value;
     return MI355_OK;
   }
+  if (option == MI355_OPT_PLAN_SMEM_LAYOUT && (value == 0 || value == 1)) {
+    state().plan_smem_layout = value;
+    return MI355_OK;
+  }
   return fail(MI355_ERR_INVALID, "unknown option %d", option);
 }
 

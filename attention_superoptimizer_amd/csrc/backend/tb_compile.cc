@@ -18,8 +18,23 @@ struct TensorInfo {
   int def_op = 0, last_use = 0;
   bool persistent = false;
   bool as_a = false, as_b = false;
+  int declared = 299;  // loader tiles: the plan's stensor layout word (SmemUnknownLayout otherwise)
   int bytes = 0;
 };
+
+// Declared thread-block layouts (values of the reference's include/mirage/layout.h:37-47):
+// 200 / 202-204 are the row-major family, 201 / 205-207 the column-major one; the
+// TensorOpMultiplicand_Crosswise{16,32,64} members pad by 4 / 8 / 16 halfs.
+bool declared_known(int l) { return l >= 200 && l <= 207; }
+bool declared_column_major(int l) { return l == 201 || (l >= 205 && l <= 207); }
+int declared_pad(int l) {
+  switch (l) {
+    case 202: case 205: return 4;
+    case 203: case 206: return 8;
+    case 204: case 207: return 16;
+    default: return 0;
+  }
+}
 
 std::string fmt(char const *f, ...) {
   char buf[256];
@@ -35,21 +50,23 @@ int round_up(int x, int a) { return (x + a - 1) / a * a; }
 }  // namespace
 
 static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int max_lds,
-                               DevProgram &prog, PlanExtents &ext, std::string &err);
+                               DevProgram &prog, PlanExtents &ext, std::string &err,
+                               bool declared_layouts);
 
 int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,
-                 PlanExtents &ext, std::string &err) {
+                 PlanExtents &ext, std::string &err, bool declared_layouts) {
   // fp16 tiles are padded by 8 halfs per row to spread 16-byte reads over the LDS
   // banks; a graph that only fits unpadded runs unpadded
-  int rc = compile_plan_padded(plan, f16, 8, max_lds, prog, ext, err);
+  int rc = compile_plan_padded(plan, f16, 8, max_lds, prog, ext, err, declared_layouts);
   if (rc == MI355_ERR_UNSUPPORTED && f16 && prog.lds_bytes > max_lds) {
-    rc = compile_plan_padded(plan, f16, 0, max_lds, prog, ext, err);
+    rc = compile_plan_padded(plan, f16, 0, max_lds, prog, ext, err, declared_layouts);
   }
   return rc;
 }
 
 static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int max_lds,
-                               DevProgram &prog, PlanExtents &ext, std::string &err) {
+                               DevProgram &prog, PlanExtents &ext, std::string &err,
+                               bool declared_layouts) {
   memset(&prog, 0, sizeof(prog));
   memset(&ext, 0, sizeof(ext));
   if (plan.num_operators < 1 || plan.num_operators > MI355_MAX_OPERATORS ||
@@ -135,6 +152,9 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
         return MI355_ERR_INVALID;
       }
       d.dst = define(q[18], rows, cols, o);
+      if (d.dst >= 0) {
+        T[d.dst].declared = q[17];
+      }
       d.hoist = (F == 1) || (d.row_fs == 0 && d.col_fs == 0 && d.g_fs == 0);
       long long max_row = (long long)(F - 1) * d.row_fs + rows - 1;
       long long max_col = (long long)(F - 1) * d.col_fs + cols - 1;
@@ -352,15 +372,24 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       dt.rs = ti.cols;
       dt.cs = 1;
       ti.bytes = round_up(ti.rows * ti.cols * 2, 16);
-    } else if (ti.as_b && !ti.as_a) {
-      // k-contiguous for the matrix-core B operand: column-major, padded columns
-      dt.rs = 1;
-      dt.cs = ti.rows >= 8 ? round_up(ti.rows, 8) + pad : ti.rows;
-      ti.bytes = round_up(dt.cs * ti.cols * 2, 16);
     } else {
-      dt.cs = 1;
-      dt.rs = ti.cols >= 8 ? round_up(ti.cols, 8) + pad : ti.cols;
-      ti.bytes = round_up(dt.rs * ti.rows * 2, 16);
+      // k-contiguous for the matrix-core B operand: column-major, padded columns;
+      // everything else row-major, padded rows -- unless the plan's declaration rules
+      bool column_major = ti.as_b && !ti.as_a;
+      int p = pad;
+      if (declared_layouts && declared_known(ti.declared)) {
+        column_major = declared_column_major(ti.declared);
+        p = pad == 0 ? 0 : declared_pad(ti.declared);
+      }
+      if (column_major) {
+        dt.rs = 1;
+        dt.cs = ti.rows >= 8 ? round_up(ti.rows, 8) + p : ti.rows;
+        ti.bytes = round_up(dt.cs * ti.cols * 2, 16);
+      } else {
+        dt.cs = 1;
+        dt.rs = ti.cols >= 8 ? round_up(ti.cols, 8) + p : ti.cols;
+        ti.bytes = round_up(dt.rs * ti.rows * 2, 16);
+      }
     }
   }
   // persistent tiles: accumulators and hoisted loads stay live over the whole loop

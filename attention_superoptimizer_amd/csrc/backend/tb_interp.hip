@@ -692,7 +692,8 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   bool const try_fused = f16 && !state().force_interpreter;
   // a fused kernel keeps tiles in registers, so the interpreter's LDS need does not
   // bound it: lower without the limit first, and again with it if no fused kernel fits
-  int rc = compile_plan(*plan, f16, try_fused ? (1 << 30) : state().max_lds, prog, ext, err);
+  bool const declared = f16 && state().plan_smem_layout != 0;
+  int rc = compile_plan(*plan, f16, try_fused ? (1 << 30) : state().max_lds, prog, ext, err, declared);
   if (rc != MI355_OK) {
     return fail(rc, "%s", err.c_str());
   }
@@ -713,7 +714,7 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     } else if (combine_applicable(prog)) {
       prog.fused = 3;
     } else {
-      rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err);
+      rc = compile_plan(*plan, f16, state().max_lds, prog, ext, err, declared);
       if (rc != MI355_OK) {
         return fail(rc, "%s", err.c_str());
       }

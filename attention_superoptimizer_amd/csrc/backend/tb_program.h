@@ -96,7 +96,9 @@ bool combine_applicable(DevProgram const &prog);
 // Lowers `plan` for the uint16 interpreter (f16 == false: plain row-major tiles)
 // or the fp16 interpreter (f16 == true: padded rows, B operands k-contiguous).
 // Returns MI355_OK or an error code with `err` set.
+// `declared_layouts`: fp16 loader tiles take the LDS layout the plan declares for them
+// (see MI355_OPT_PLAN_SMEM_LAYOUT) instead of the one their consumers want.
 int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,
-                 PlanExtents &ext, std::string &err);
+                 PlanExtents &ext, std::string &err, bool declared_layouts = false);
 
 }  // namespace mi355

@@ -25,6 +25,7 @@ SMEM_LAYOUT = {
     "SmemColumnMajorTensorOpMultiplicand_Crosswise16": 205,
     "SmemColumnMajorTensorOpMultiplicand_Crosswise32": 206,
     "SmemColumnMajorTensorOpMultiplicand_Crosswise64": 207,
+    "SmemUnknownLayout": 299,
 }
 KN_OP = {"exp": 1007, "add": 1008, "mul": 1009, "div": 1010, "silu": 1011}
 TB_OP = {
@@ -259,6 +260,24 @@ def _stats(st) -> dict:
     return {"kernel_ops": st.kernel_ops, "customized_ops": st.customized_ops,
             "compares": st.compares, "fp_bytes": st.fp_bytes, "matmul_macs": st.matmul_macs,
             "enqueue_seconds": st.enqueue_seconds, "wait_seconds": st.wait_seconds}
+
+
+def optimize_layout(graph: "KNGraph", cost=None, max_assignments: int = 0) -> dict:
+    """KernelGraphGenerator::optimize_layout (reference src/search/search.cc:699-777):
+    enumerates the layouts of every kernel-level output tensor and of every tile inside
+    the customized operators, costs each complete assignment and leaves `graph` under the
+    cheapest one.  `cost(op_index, loader_layouts) -> ms` replaces the measurement by
+    KNOperator::profile (which needs the device)."""
+    st = N.MirageLayoutStats()
+    if cost is None:
+        cb = N.LAYOUT_COST_FN()
+    else:
+        cb = N.LAYOUT_COST_FN(lambda user, op, lay, n: float(cost(op, [lay[i] for i in range(n)])))
+    rc = N.runtime().mirage_optimize_layout(graph._g, max_assignments, cb, None, ctypes.byref(st))
+    assert rc == 0
+    return {"assignments": st.assignments, "measurements": st.measurements,
+            "truncated": bool(st.truncated), "first_ms": st.first_ms, "best_ms": st.best_ms,
+            "worst_ms": st.worst_ms}
 
 
 def verify_batch(candidates: Sequence["KNGraph"], reference: "KNGraph", input_seed: int = 0):

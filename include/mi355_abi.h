@@ -89,6 +89,18 @@ typedef struct mi355_launch_info {
  * variant of the fused attention kernel, 2 = the throughput variant whenever the
  * tile shape allows it. */
 #define MI355_OPT_ATTENTION_MODE 2
+/* PLAN_SMEM_LAYOUT: 0 = the lowering gives every fp16 tile the LDS layout its
+ * consumers want (default); 1 = a loader's tile takes the layout its plan declares
+ * (the stensor layout word of the input-loader bytecode, values of the reference's
+ * include/mirage/layout.h:37-47): the RowMajor family is stored row-major, the
+ * ColumnMajor family column-major; the plain layouts are unpadded, the
+ * TensorOpMultiplicand_Crosswise{16,32,64} ones pad every row / column by 8, 16 and
+ * 32 bytes to spread matrix-core operand fetches over the LDS banks.
+ * SmemUnknownLayout leaves the choice to the lowering.  Results do not depend on
+ * the layout; this is the knob the layout search (reference
+ * src/search/search.cc:625-763) turns with profile() as its cost.  Fused kernels
+ * keep their own staging layouts. */
+#define MI355_OPT_PLAN_SMEM_LAYOUT 3
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor

@@ -1,0 +1,59 @@
+// Layout selection for a verified kernel graph: the reference's
+// KernelGraphGenerator::{get_valid_output_layout, optimize_layout, update_best_graph}
+// (src/search/search.cc:625-777) as free functions.
+//
+// The search walks every kernel-level output tensor (row- or column-major; a matmul
+// result stays row-major) and, inside every customized operator, every tile a
+// thread-block operator defines (the layouts its operator admits), profiles each
+// complete assignment with KNOperator::profile and keeps the fastest.
+//
+// What a layout means on this backend: the LDS layout of a loader's tile while the
+// fp16 interpreter runs with MI355_OPT_PLAN_SMEM_LAYOUT = 1 (row- or column-major,
+// unpadded or padded against bank conflicts).  Device-tensor layouts and the layouts
+// of tiles that never reach the lowered program are carried as metadata, and the
+// fused kernels stage operands their own way, so many assignments cost the same; the
+// cost of an operator is therefore measured once per distinct set of loader layouts.
+#pragma once
+
+#include "mirage/kernel/graph.h"
+#include <functional>
+#include <string>
+#include <vector>
+
+namespace mirage {
+namespace search {
+
+// Layouts the `idx`-th output tile of a thread-block operator may take, given the
+// layouts of its inputs (search.cc:625-697).  Empty: the inputs' layouts rule the
+// operator out.
+std::vector<mirage::layout::SmemLayout>
+    get_valid_output_layout(mirage::threadblock::TBOperator const *op, int idx);
+
+struct LayoutSearchConfig {
+  // Assignments evaluated at most; the search stops there and reports `truncated`.
+  long long max_assignments = 1 << 22;
+  // Cost of one operator under the graph's current layouts, in milliseconds.  Must
+  // depend on nothing but the operator and, for a customized operator, the layouts
+  // of its loaders' tiles.  Empty: KNOperator::profile with the backend honouring
+  // declared loader layouts.
+  std::function<float(mirage::kernel::KNOperator *)> cost;
+};
+
+struct LayoutSearchResult {
+  long long assignments = 0;   // complete layout assignments evaluated
+  long long measurements = 0;  // operator costs actually measured (the rest were known)
+  bool truncated = false;
+  float first_run_time = 0.0f;  // total of the first assignment evaluated
+  float best_run_time = 0.0f;
+  float worst_run_time = 0.0f;
+  std::string best_graph;  // JSON of the graph under the best assignment
+};
+
+// Leaves `g` under the best assignment found (every tensor's and tile's `layout`,
+// and the copies its consumers hold).  A graph with no valid assignment is left as
+// it was and reports assignments == 0.
+void optimize_layout(mirage::kernel::Graph &g, LayoutSearchResult *result = nullptr,
+                     LayoutSearchConfig const *config = nullptr);
+
+}  // namespace search
+}  // namespace mirage
