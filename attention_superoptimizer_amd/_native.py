@@ -110,6 +110,9 @@ ABI = {
     "mi355_f16_unary": (_ci, [_ci, _vp, _vp, _sz]),
     "mi355_f16_binary": (_ci, [_ci, _vp, _pi, _vp, _pi, _vp, _pi, _ci]),
     "mi355_f16_reduce": (_ci, [_vp, _vp, _sz, _ci, _ci, _ci]),
+    "mi355_emit_hip_preamble": (ctypes.c_char_p, []),
+    "mi355_emit_hip_kernel": (ctypes.c_longlong, [_pplan, ctypes.c_char_p, _ci, ctypes.c_char_p,
+                                                  ctypes.c_longlong]),
     "mi355_timer_start": (_ci, []),
     "mi355_timer_stop": (_ci, [_pf]),
 }
@@ -151,6 +154,7 @@ FACADE = {
     "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_optimize_layout": (_ci, [_vp, ctypes.c_longlong, LAYOUT_COST_FN, _vp,
                                      ctypes.POINTER(MirageLayoutStats)]),
+    "mirage_graph_generate_hip_program": (_ci, [_vp, ctypes.c_char_p]),
     "mirage_graph_from_json": (_vp, [ctypes.c_char_p]),
     "mirage_graph_to_json": (ctypes.c_longlong, [_vp, ctypes.c_char_p, ctypes.c_longlong]),
     "mirage_set_smem_budget": (None, [_sz]),

@@ -2,6 +2,8 @@
 
   libmi355_backend.so   HIP kernels + the C ABI of include/mi355_abi.h
   libmirage_runtime.so  the mirage:: host API (C++) + its C facade for ctypes
+  generated/            HIP programs written by Graph::generate_hip_program for the example
+                        graphs of codegen.py, compiled as libraries and executables
 
 Run as `python -m attention_superoptimizer_amd.build`.
 """
@@ -59,10 +61,23 @@ def build_runtime():
          ["-L" + HERE, "-lmi355_backend", "-Wl,-rpath,$ORIGIN", "-pthread"])
 
 
+def build_generated():
+    """Generated HIP programs of the example graphs (codegen.py), in a process of their own:
+    building the graphs loads the runtime just built, in host-only mode."""
+    env = dict(os.environ, MIRAGE_HOST_ONLY="1")
+    _run_env([sys.executable, "-m", "attention_superoptimizer_amd.codegen"], env)
+
+
+def _run_env(cmd, env):
+    print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd, env=env, cwd=ROOT)
+
+
 def main():
     build_backend()
     if os.path.isdir(os.path.join(CSRC, "host")):
         build_runtime()
+        build_generated()
     return 0
 
 

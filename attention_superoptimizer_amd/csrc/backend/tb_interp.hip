@@ -529,9 +529,12 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
               int row = e / n, col = e % n;
               float acc = 0.0f;
               for (int kk = 0; kk < k; kk++) {
-                acc += static_cast<float>(A[row * ta.rs + kk * ta.cs]) *
-                       static_cast<float>(B[kk * tb.rs + col * tb.cs]);
+                acc = __builtin_fmaf(static_cast<float>(A[row * ta.rs + kk * ta.cs]),
+                                     static_cast<float>(B[kk * tb.rs + col * tb.cs]), acc);
               }
+              // rounded to fp32 first and to fp16 second: the fence keeps the last multiply-add
+              // and the conversion from merging into one instruction that rounds once
+              asm volatile("" : "+v"(acc));
               C[row * tc.rs + col * tc.cs] = static_cast<_Float16>(acc);
             }
           }

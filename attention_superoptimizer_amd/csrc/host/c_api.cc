@@ -233,6 +233,12 @@ int mirage_tensor_same_fingerprint(void *a, void *b) {
   return static_cast<DTensor *>(a)->has_same_fingerprint(*static_cast<DTensor *>(b)) ? 1 : 0;
 }
 
+// Graph::generate_hip_program
+int mirage_graph_generate_hip_program(void *g, char const *path) {
+  static_cast<kernel::Graph *>(g)->generate_hip_program(path);
+  return 0;
+}
+
 void mirage_set_smem_budget(size_t bytes) { threadblock::Graph::set_smem_budget(bytes); }
 size_t mirage_get_smem_budget(void) { return threadblock::Graph::smem_budget(); }
 

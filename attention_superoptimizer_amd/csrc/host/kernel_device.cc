@@ -10,6 +10,11 @@
 #include "mirage/utils/hip_types.h"
 
 #include <cstring>
+#include <fstream>
+#include <map>
+#include <sstream>
+#include <string>
+#include <vector>
 
 namespace mirage {
 namespace kernel {
@@ -259,6 +264,124 @@ bool KNCustomizedOp::fingerprint(void) {
   LoweredOp l = lower(*this, true);
   MI355_CALL(mi355_customized_fp(&l.plan, l.inputs, l.outputs));
   return true;
+}
+
+}  // namespace kernel
+}  // namespace mirage
+
+// ---- source emission (reference src/kernel/triton_code_gen.cc:354-450) ---------------------
+namespace mirage {
+namespace kernel {
+
+void Graph::generate_hip_program(char const *file_path) {
+  std::ofstream file(file_path);
+  MIRAGE_CHECK(file.good(), "generate_hip_program: cannot open the output file");
+  file << mi355_emit_hip_preamble();
+  // device tensors are numbered in creation order: every operator's outputs
+  std::map<int, int> index_of;  // guid -> number
+  std::vector<long long> elements;
+  std::vector<bool> is_input;
+  for (KNOperator *op : operators) {
+    for (DTensor const &t : op->output_tensors) {
+      index_of[t.guid] = (int)elements.size();
+      elements.push_back((long long)t.num_elements());
+      is_input.push_back(op->op_type == mirage::type::KN_INPUT_OP);
+    }
+  }
+  std::stringstream launcher;
+  launcher << "// Launches every customized operator of the graph in order.  dtensors[i] is device\n"
+              "// tensor i in creation order (see graphdef_tensor_elements).\n"
+              "extern \"C\" int graphdef_launch(void *const *dtensors, hipStream_t stream) {\n";
+  int kernels = 0;
+  for (KNOperator *op : operators) {
+    if (op->op_type != mirage::type::KN_CUSTOMIZED_OP) {
+      continue;  // as the reference: only customized operators are emitted
+    }
+    LoweredOp l = lower(*static_cast<KNCustomizedOp *>(op), false);
+    std::string const name = "graphdef_kernel_" + std::to_string(kernels++);
+    long long const n = mi355_emit_hip_kernel(&l.plan, name.c_str(), 0, nullptr, 0);
+    MIRAGE_CHECK(n >= 0, mi355_last_error());
+    std::vector<char> text((size_t)n + 1);
+    MIRAGE_CHECK(mi355_emit_hip_kernel(&l.plan, name.c_str(), 0, text.data(), n + 1) == n,
+                 "generate_hip_program: emission changed size");
+    file << text.data();
+    launcher << "  {\n    void const *in[] = {";
+    for (size_t i = 0; i < op->input_tensors.size(); i++) {
+      launcher << (i ? ", " : "") << "dtensors[" << index_of.at(op->input_tensors[i].guid) << "]";
+    }
+    launcher << "};\n    void *out[] = {";
+    for (size_t i = 0; i < op->output_tensors.size(); i++) {
+      launcher << (i ? ", " : "") << "dtensors[" << index_of.at(op->output_tensors[i].guid) << "]";
+    }
+    launcher << "};\n    if (int rc = " << name << "_launch(in, out, stream)) {\n      return rc;\n    }\n  }\n";
+  }
+  launcher << "  return 0;\n}\n\n";
+  file << "static long long const kTensorElements[] = {";
+  for (size_t i = 0; i < elements.size(); i++) {
+    file << (i ? ", " : "") << elements[i];
+  }
+  file << "};\nstatic int const kTensorIsInput[] = {";
+  for (size_t i = 0; i < elements.size(); i++) {
+    file << (i ? ", " : "") << (is_input[i] ? 1 : 0);
+  }
+  file << "};\n"
+          "extern \"C\" int graphdef_num_tensors(void) { return " << elements.size() << "; }\n"
+          "extern \"C\" long long graphdef_tensor_elements(int i) { return kTensorElements[i]; }\n"
+          "extern \"C\" int graphdef_sync(void) { return (int)hipDeviceSynchronize(); }\n\n";
+  file << launcher.str();
+  // the profiling main: random fp16 tensors, 1000 warm-up launches, 1000 timed
+  file << R"HIP(#ifndef GRAPHDEF_NO_MAIN
+static uint64_t mix64(uint64_t x) {
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+
+int main() {
+  int const n = graphdef_num_tensors();
+  std::vector<void *> dtensors(n);
+  for (int t = 0; t < n; t++) {
+    long long const e = kTensorElements[t];
+    GRAPHDEF_HIP(hipMalloc(&dtensors[t], (size_t)e * 2));
+    std::vector<_Float16> host((size_t)e);
+    for (long long i = 0; i < e; i++) {
+      // N(0, 1) / 8 by Box-Muller on two 24-bit uniforms
+      uint64_t const r = mix64(((uint64_t)t << 40) ^ (uint64_t)i);
+      float const u1 = ((r >> 40) + 1) * (1.0f / 16777216.0f), u2 = ((r >> 16) & 0xffffff) * (1.0f / 16777216.0f);
+      host[(size_t)i] = (_Float16)(0.125f * __builtin_sqrtf(-2.0f * __builtin_logf(u1)) * __builtin_cosf(6.2831853f * u2));
+    }
+    GRAPHDEF_HIP(hipMemcpy(dtensors[t], host.data(), (size_t)e * 2, hipMemcpyHostToDevice));
+  }
+  hipStream_t stream;
+  GRAPHDEF_HIP(hipStreamCreate(&stream));
+  hipEvent_t e0, e1;
+  GRAPHDEF_HIP(hipEventCreate(&e0));
+  GRAPHDEF_HIP(hipEventCreate(&e1));
+  for (int i = 0; i < 1000; i++) {
+    if (graphdef_launch(dtensors.data(), stream)) {
+      return 1;
+    }
+  }
+  GRAPHDEF_HIP(hipEventRecord(e0, stream));
+  for (int i = 0; i < 1000; i++) {
+    if (graphdef_launch(dtensors.data(), stream)) {
+      return 1;
+    }
+  }
+  GRAPHDEF_HIP(hipEventRecord(e1, stream));
+  GRAPHDEF_HIP(hipEventSynchronize(e1));
+  float ms = 0.0f;
+  GRAPHDEF_HIP(hipEventElapsedTime(&ms, e0, e1));
+  printf("%.6f ms per launch of the whole graph (mean of 1000)\n", ms / 1000.0f);
+  for (void *p : dtensors) {
+    GRAPHDEF_HIP(hipFree(p));
+  }
+  return 0;
+}
+#endif
+)HIP";
+  file.close();
 }
 
 }  // namespace kernel

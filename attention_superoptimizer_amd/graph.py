@@ -145,6 +145,13 @@ class KNGraph:
             raise ValueError("malformed mugraph JSON")
         return cls(_handle=h)
 
+    def generate_hip_program(self, path: str) -> None:
+        """Graph::generate_hip_program: writes a self-contained HIP program (one specialised
+        gfx950 kernel per customized operator, a launcher, a timing main) -- this backend's
+        counterpart of the reference's generate_triton_program
+        (src/kernel/triton_code_gen.cc:354-450)."""
+        assert self._rt.mirage_graph_generate_hip_program(self._g, path.encode()) == 0
+
     def to_json(self) -> str:
         """to_json(json, Graph) (src/kernel/graph.cc:33-37), one line, sorted keys."""
         n = self._rt.mirage_graph_to_json(self._g, None, 0)

@@ -238,6 +238,19 @@ int mi355_f16_reduce(void const *in, void *out, size_t n_out, int factor, int in
 int mi355_timer_start(void);
 int mi355_timer_stop(float *ms); /* blocking */
 
+/* ---- source emission -------------------------------------------------------
+ * Replaces generate_kernel_code (src/kernel/triton_code_gen.cc:84-352): the fp16
+ * lowering of one customized op printed as a specialised gfx950 kernel named `name`
+ * plus `extern "C" int <name>_launch(void const *const *in, void *const *out,
+ * hipStream_t)`.  Host code only, no device needed.  Returns the length of the text
+ * (without the terminator) and copies at most capacity - 1 bytes of it into `buf`;
+ * -1 on error (mi355_last_error).  max_lds_bytes <= 0 means gfx950's 160 KB.
+ * mi355_emit_hip_preamble: the includes, typedefs and tile helpers the kernels use,
+ * once per file. */
+char const *mi355_emit_hip_preamble(void);
+long long mi355_emit_hip_kernel(mi355_plan const *plan, char const *name, int max_lds_bytes,
+                                char *buf, long long capacity);
+
 #ifdef __cplusplus
 }
 #endif

@@ -58,6 +58,14 @@ public:
   KNOperator *create_customized_op(std::vector<DTensor> const &inputs,
                                    mirage::threadblock::Graph const &_graph);
 
+  // Writes a self-contained HIP program for gfx950: one specialised kernel per
+  // customized operator, a launcher over all of them and a main() that fills the
+  // tensors with random values and times the launcher (the role of the reference's
+  // generate_triton_program, include/mirage/kernel/graph.h:79 and
+  // src/kernel/triton_code_gen.cc:354-450; other kernel-level operators are skipped,
+  // as there).
+  void generate_hip_program(char const *filepath);
+
   // Operators in creation order.  The graph deletes them newest-first on
   // destruction (the arena is LIFO); callers that pop an operator delete it
   // themselves, as the reference's search does.
