@@ -97,6 +97,7 @@ ABI = {
     "mi355_fp_equal": (_ci, [_vp, _vp, _sz, _pi]),
     "mi355_fp_equal_reset": (_ci, [_ci, _ci]),
     "mi355_fp_equal_enqueue": (_ci, [_vp, _vp, _sz, _ci]),
+    "mi355_fp_equal_enqueue_many": (_ci, [_pvp, _pvp, ctypes.POINTER(_sz), _pi, _ci]),
     "mi355_fp_equal_collect": (_ci, [_ci, _ci, _vp]),
     "mi355_customized_fp": (_ci, [_pplan, _pvp, _pvp]),
     "mi355_customized_fp_batch": (_ci, [_pplan, _ci, _pvp, _pvp]),

@@ -58,6 +58,17 @@ struct State {
   int *cmp_host = nullptr;    // pinned mirror
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int max_lds = 65536;
+  // staging of batched launches (mi355_customized_fp_batch): per queue a small ring of
+  // pinned host / device buffer pairs that carry the program records of one call
+  static constexpr int kBatchSlots = 16;
+  static constexpr size_t kBatchSlotBytes = (size_t)256 << 10;
+  struct BatchSlot {
+    char *host = nullptr;
+    char *dev = nullptr;
+    hipEvent_t copied = nullptr;  // the host buffer may be rewritten once this has passed
+  };
+  BatchSlot batch[MI355_NUM_QUEUES][kBatchSlots];
+  int batch_next[MI355_NUM_QUEUES] = {};
   mi355_launch_info last_launch{};
   int force_interpreter = 0;
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits

@@ -715,6 +715,34 @@ __global__ void fp_differ_kernel(uint16_t const *__restrict__ a, uint16_t const 
   }
 }
 
+struct DifferMany {
+  uint16_t const *a[MI355_MAX_COMPARE_PAIRS];
+  uint16_t const *b[MI355_MAX_COMPARE_PAIRS];
+  size_t n[MI355_MAX_COMPARE_PAIRS];
+  int slot[MI355_MAX_COMPARE_PAIRS];
+};
+
+// blockIdx.y names the pair
+__global__ void fp_differ_many_kernel(DifferMany const D, int *slots) {
+  uint16_t const *a = D.a[blockIdx.y], *b = D.b[blockIdx.y];
+  size_t const n = D.n[blockIdx.y];
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  bool differ = false;
+  size_t const n8 = (((uintptr_t)a | (uintptr_t)b) & 15) == 0 ? n / 8 : 0;
+  for (size_t j = i; j < n8; j += stride) {
+    uint4v x = reinterpret_cast<uint4v const *>(a)[j];
+    uint4v y = reinterpret_cast<uint4v const *>(b)[j];
+    differ |= (x[0] != y[0]) | (x[1] != y[1]) | (x[2] != y[2]) | (x[3] != y[3]);
+  }
+  for (size_t j = n8 * 8 + i; j < n; j += stride) {
+    differ |= (a[j] != b[j]);
+  }
+  if (differ) {
+    slots[D.slot[blockIdx.y]] = 1;  // every writer stores the same value
+  }
+}
+
 extern "C" int mi355_fp_equal_reset(int first_slot, int count) {
   MI355_REQUIRE_INIT();
   State &s = state();
@@ -739,6 +767,39 @@ extern "C" int mi355_fp_equal_enqueue(uint16_t const *a, uint16_t const *b, size
   if (n > 0) {
     fp_differ_kernel<<<grid_for((n + 7) / 8, kThreads, 1024), kThreads, 0, s.stream()>>>(
         a, b, n, s.cmp_slots + slot);
+    MI355_HIP(hipGetLastError());
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_equal_enqueue_many(uint16_t const *const *a, uint16_t const *const *b,
+                                           size_t const *n, int const *slots, int count) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (count < 0 || count > MI355_MAX_COMPARE_PAIRS ||
+      (count > 0 && (a == nullptr || b == nullptr || n == nullptr || slots == nullptr))) {
+    return fail(MI355_ERR_INVALID, "bad compare list (count %d)", count);
+  }
+  DifferMany D{};
+  size_t largest = 0;
+  int pairs = 0;
+  for (int i = 0; i < count; i++) {
+    if (slots[i] < 0 || slots[i] >= MI355_COMPARE_SLOTS) {
+      return fail(MI355_ERR_INVALID, "compare slot %d out of range", slots[i]);
+    }
+    if (n[i] == 0) {
+      continue;
+    }
+    D.a[pairs] = a[i];
+    D.b[pairs] = b[i];
+    D.n[pairs] = n[i];
+    D.slot[pairs] = slots[i];
+    pairs++;
+    largest = std::max(largest, n[i]);
+  }
+  if (pairs > 0) {
+    dim3 grid(grid_for((largest + 7) / 8, kThreads, 256), pairs);
+    fp_differ_many_kernel<<<grid, kThreads, 0, s.stream()>>>(D, s.cmp_slots);
     MI355_HIP(hipGetLastError());
   }
   return MI355_OK;

@@ -114,6 +114,16 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
                           hipHostMallocDefault));
   MI355_HIP(hipEventCreate(&s.ev0));
   MI355_HIP(hipEventCreate(&s.ev1));
+  for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+    for (int b = 0; b < State::kBatchSlots; b++) {
+      State::BatchSlot &slot = s.batch[q][b];
+      MI355_HIP(hipHostMalloc(reinterpret_cast<void **>(&slot.host), State::kBatchSlotBytes,
+                              hipHostMallocDefault));
+      MI355_HIP(hipMalloc(reinterpret_cast<void **>(&slot.dev), State::kBatchSlotBytes));
+      MI355_HIP(hipEventCreateWithFlags(&slot.copied, hipEventDisableTiming));
+    }
+    s.batch_next[q] = 0;
+  }
   s.scratch_bytes = (size_t)64 << 20;  // per queue
   MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.scratch_base),
                       s.scratch_bytes * MI355_NUM_QUEUES));
@@ -141,6 +151,13 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipFree(s.cmp_slots));
   MI355_HIP(hipHostFree(s.cmp_host));
   MI355_HIP(hipFree(s.scratch_base));
+  for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+    for (int b = 0; b < State::kBatchSlots; b++) {
+      MI355_HIP(hipHostFree(s.batch[q][b].host));
+      MI355_HIP(hipFree(s.batch[q][b].dev));
+      MI355_HIP(hipEventDestroy(s.batch[q][b].copied));
+    }
+  }
   for (int i = 0; i < MI355_NUM_QUEUES; i++) {
     MI355_HIP(hipStreamDestroy(s.queues[i]));
   }

@@ -13,6 +13,8 @@
 
 #include <algorithm>
 #include <string>
+#include <vector>
+#include <cstring>
 
 namespace mi355 {
 
@@ -29,14 +31,16 @@ struct TileOrigin {
   int row0, col0;
 };
 
-__device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it, int bx) {
+__device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it, int bx, int by, int bz) {
   TileOrigin o;
-  int by = blockIdx.y, bz = blockIdx.z;
   o.row0 = bx * op.row_bs[0] + by * op.row_bs[1] + bz * op.row_bs[2] + it * op.row_fs;
   o.col0 = bx * op.col_bs[0] + by * op.col_bs[1] + bz * op.col_bs[2] + it * op.col_fs;
   o.base = (long long)bx * op.g_bs[0] + (long long)by * op.g_bs[1] + (long long)bz * op.g_bs[2] +
            (long long)it * op.g_fs;
   return o;
+}
+__device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it, int bx) {
+  return tile_origin(op, it, bx, blockIdx.y, blockIdx.z);
 }
 
 // ===========================================================================
@@ -167,23 +171,14 @@ __device__ __forceinline__ uint32_t add_mod_pair(uint32_t a, uint32_t b) {
   return lo | (hi << 16);
 }
 
-__global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
-    DevProgram const P, uint16_t const *__restrict__ g_exp, uint16_t const *__restrict__ g_divp,
-    uint16_t const *__restrict__ g_divq) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+// One workgroup of the uint16 interpreter: logical block (bx, by, bz) of program P, part
+// `split` of its for-loop.  The lookup tables are already in LDS.
+__device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned char *lds, int bx,
+                                                int by, int bz, int split) {
   uint16_t *tbl = reinterpret_cast<uint16_t *>(lds);
   int const tid = threadIdx.x;
-  for (int i = tid; i < (int)FP_Q; i += kInterpThreads) {
-    tbl[i] = static_cast<uint16_t>((g_exp[i] * FP_Q_MUL_P_MOD_1) % FP_PQ);
-    tbl[384 + i] = g_divq[i];
-  }
-  for (int i = tid; i < (int)FP_P; i += kInterpThreads) {
-    tbl[128 + i] = g_divp[i];
-  }
-  __syncthreads();
   int const F = P.forloop_range;
   // a split for-loop: this workgroup covers iterations [it_begin, it_end) of block bx
-  int const bx = blockIdx.x % P.grid[0], split = blockIdx.x / P.grid[0];
   int const it_begin = (int)((long long)F * split / P.splits);
   int const it_end = (int)((long long)F * (split + 1) / P.splits);
   for (int it = it_begin; it < it_end; it++) {
@@ -196,7 +191,7 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           }
           DevTensor const &t = P.t[op.dst];
           uint16_t *s = reinterpret_cast<uint16_t *>(lds + t.off);
-          TileOrigin org = tile_origin(op, it, bx);
+          TileOrigin org = tile_origin(op, it, bx, by, bz);
           uint16_t const *g = static_cast<uint16_t const *>(P.in[op.io]) + org.base +
                               (long long)org.row0 * op.d_cols + org.col0;
           if (op.vec8) {
@@ -352,7 +347,7 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
           uint16_t *acc = reinterpret_cast<uint16_t *>(lds + ta.off);
           int const n = ta.rows * ta.cols;
           bool const last = (it == it_end - 1), first = (it == it_begin);
-          TileOrigin org = tile_origin(op, 0, bx);
+          TileOrigin org = tile_origin(op, 0, bx, by, bz);
           uint16_t *g = (P.splits > 1 ? P.part[op.io] + (long long)split * P.part_stride[op.io]
                                       : static_cast<uint16_t *>(P.out[op.io])) +
                         org.base + (long long)org.row0 * op.d_cols + org.col0;
@@ -396,6 +391,66 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
       __syncthreads();
     }
   }
+}
+
+
+__device__ __forceinline__ void fp_load_tables(unsigned char *lds, uint16_t const *__restrict__ g_exp,
+                                               uint16_t const *__restrict__ g_divp,
+                                               uint16_t const *__restrict__ g_divq) {
+  uint16_t *tbl = reinterpret_cast<uint16_t *>(lds);
+  int const tid = threadIdx.x;
+  for (int i = tid; i < (int)FP_Q; i += kInterpThreads) {
+    tbl[i] = static_cast<uint16_t>((g_exp[i] * FP_Q_MUL_P_MOD_1) % FP_PQ);
+    tbl[384 + i] = g_divq[i];
+  }
+  for (int i = tid; i < (int)FP_P; i += kInterpThreads) {
+    tbl[128 + i] = g_divp[i];
+  }
+}
+
+__global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
+    DevProgram const P, uint16_t const *__restrict__ g_exp, uint16_t const *__restrict__ g_divp,
+    uint16_t const *__restrict__ g_divq) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  fp_load_tables(lds, g_exp, g_divp, g_divq);
+  __syncthreads();
+  fp_interp_block(P, lds, blockIdx.x % P.grid[0], blockIdx.y, blockIdx.z, blockIdx.x / P.grid[0]);
+}
+
+// Many programs in one launch (a 1-D grid): workgroup w belongs to the program i with
+// first_block[i] <= w < first_block[i + 1] and is workgroup w - first_block[i] of that
+// program's own (grid.x * splits, grid.y, grid.z) grid.  The program record is copied from
+// global memory to LDS (above every program's tiles, at `program_lds_offset`) once, so the
+// interpreter reads it as it reads a kernel argument.
+__global__ __launch_bounds__(kInterpThreads) void fp_interp_multi_kernel(
+    DevProgram const *__restrict__ progs, int const *__restrict__ first_block, int n,
+    int program_lds_offset, uint16_t const *__restrict__ g_exp,
+    uint16_t const *__restrict__ g_divp, uint16_t const *__restrict__ g_divq) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int lo = 0, hi = n;
+  int const w = blockIdx.x;
+  while (hi - lo > 1) {
+    int const mid = (lo + hi) / 2;
+    if (first_block[mid] <= w) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  static_assert(sizeof(DevProgram) % 16 == 0, "the program record is copied in 16-byte words");
+  uint4v const *src = reinterpret_cast<uint4v const *>(progs + lo);
+  uint4v *dst = reinterpret_cast<uint4v *>(lds + program_lds_offset);
+  for (int i = threadIdx.x; i < (int)(sizeof(DevProgram) / 16); i += kInterpThreads) {
+    dst[i] = src[i];
+  }
+  fp_load_tables(lds, g_exp, g_divp, g_divq);
+  __syncthreads();
+  DevProgram const &P = *reinterpret_cast<DevProgram const *>(lds + program_lds_offset);
+  int v = w - first_block[lo];
+  int const gx = P.grid[0] * P.splits;
+  int const x = v % gx;
+  v /= gx;
+  fp_interp_block(P, lds, x % P.grid[0], v % P.grid[1], v / P.grid[1], x / P.grid[0]);
 }
 
 // ===========================================================================
@@ -653,40 +708,95 @@ __global__ void fp_combine_splits_kernel(uint16_t const *__restrict__ part,
   }
 }
 
+// pinned host buffer -> device buffer, 16 bytes per lane
+__global__ void stage_records_kernel(uint4v const *__restrict__ src, uint4v *__restrict__ dst, int n16) {
+  int const i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n16) {
+    dst[i] = src[i];
+  }
+}
+
+// The same for many (partials, output) pairs in one launch; job j owns workgroups
+// [first_block[j], first_block[j + 1]).
+struct CombineJob {
+  uint16_t const *part;
+  uint16_t *out;
+  long long n, stride_elems;
+  int splits, pad;
+};
+__global__ void fp_combine_splits_multi_kernel(CombineJob const *__restrict__ jobs,
+                                               int const *__restrict__ first_block, int n_jobs) {
+  int lo = 0, hi = n_jobs;
+  int const w = blockIdx.x;
+  while (hi - lo > 1) {
+    int const mid = (lo + hi) / 2;
+    if (first_block[mid] <= w) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  CombineJob const J = jobs[lo];
+  long long const blocks = first_block[lo + 1] - first_block[lo];
+  long long i = (long long)(w - first_block[lo]) * blockDim.x + threadIdx.x;
+  long long const stride = blocks * blockDim.x;
+  for (; i < J.n; i += stride) {
+    uint32_t v = 0;
+    for (int s = 0; s < J.splits; s++) {
+      v += J.part[(long long)s * J.stride_elems + i];
+    }
+    J.out[i] = static_cast<uint16_t>(v % FP_PQ);
+  }
+}
+
 // How many workgroups share one logical block's for-loop in the uint16 interpreter.
 // The accumulating saver is a sum over iterations in a ring, so any split of the
 // iteration range gives the same value; small grids are split until the device is full.
-static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outputs) {
+// `wanted` splits at most, fewer if the partial sums do not fit what is left of this queue's
+// scratch after `used` bytes; the partials are placed there and `used` advances.
+static void set_splits(DevProgram &prog, PlanExtents const &ext, int num_outputs, int wanted,
+                       size_t &used) {
   State &s = state();
   prog.splits = 1;
-  int const blocks = prog.grid[0] * prog.grid[1] * prog.grid[2];
-  int const F = prog.forloop_range;
-  if (F < 2 || blocks >= 192 || s.scratch() == nullptr) {
+  if (wanted < 2 || s.scratch() == nullptr) {
     return;
   }
-  int splits = std::min(std::min(F, 64), (256 + blocks - 1) / blocks);
   long long elems = 0;
   for (int i = 0; i < num_outputs; i++) {
     elems += (ext.out_elems[i] + 7) / 8 * 8;
   }
-  while (splits > 1 && (size_t)(elems * splits * 2) > s.scratch_bytes) {
+  int splits = wanted;
+  while (splits > 1 && used + (size_t)(elems * splits * 2) > s.scratch_bytes) {
     splits--;
   }
   if (splits < 2) {
     return;
   }
   prog.splits = splits;
-  uint16_t *p = static_cast<uint16_t *>(s.scratch());
+  uint16_t *p = reinterpret_cast<uint16_t *>(static_cast<char *>(s.scratch()) + used);
   for (int i = 0; i < num_outputs; i++) {
     prog.part[i] = p;
     prog.part_elems[i] = ext.out_elems[i];
     prog.part_stride[i] = (ext.out_elems[i] + 7) / 8 * 8;
     p += prog.part_stride[i] * splits;
   }
+  used += (size_t)(elems * splits * 2);
 }
 
+static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outputs) {
+  prog.splits = 1;
+  int const blocks = prog.grid[0] * prog.grid[1] * prog.grid[2];
+  int const F = prog.forloop_range;
+  if (F < 2 || blocks >= 192) {
+    return;
+  }
+  size_t used = 0;
+  set_splits(prog, ext, num_outputs, std::min(std::min(F, 64), (256 + blocks - 1) / blocks), used);
+}
+
+// `ext_out` set: the caller decides about split for-loops itself (batched launches).
 static int prepare(mi355_plan const *plan, void const *const *inputs, void *const *outputs,
-                   bool f16, DevProgram &prog) {
+                   bool f16, DevProgram &prog, PlanExtents *ext_out = nullptr) {
   if (plan == nullptr || inputs == nullptr || outputs == nullptr) {
     return fail(MI355_ERR_INVALID, "null argument");
   }
@@ -735,7 +845,10 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     }
     prog.out[i] = outputs[i];
   }
-  if (!f16) {
+  if (ext_out != nullptr) {
+    *ext_out = ext;
+    prog.splits = 1;
+  } else if (!f16) {
     choose_splits(prog, ext, plan->num_dmem_outputs);
   }
   // 16-byte global accesses also need 16-byte aligned base pointers
@@ -846,26 +959,178 @@ extern "C" int mi355_customized_fp(mi355_plan const *plan, void const *const *in
   return launch(prog, false);
 }
 
+// One chunk of a batch: every program in one multi-program launch per LDS class, then one
+// launch that folds the partial sums of all split for-loops.  A program whose tiles leave
+// no room in LDS for its own record is launched by itself.
+static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExtents> const &exts,
+                           std::vector<int> const &num_outputs) {
+  State &s = state();
+  int const n = (int)progs.size();
+  // split for-loops until the chunk as a whole offers the device a few workgroups per CU
+  long long total = 0;
+  for (DevProgram const &p : progs) {
+    total += (long long)p.grid[0] * p.grid[1] * p.grid[2];
+  }
+  int const scale = (int)std::min<long long>(64, (1024 + total - 1) / total);
+  size_t used = 0;
+  for (int i = 0; i < n; i++) {
+    set_splits(progs[i], exts[i], num_outputs[i], std::min(progs[i].forloop_range, scale), used);
+  }
+  int const record = (int)sizeof(DevProgram);
+  // LDS classes: a launch requests the largest need of its members, which bounds how many
+  // workgroups share a compute unit
+  int const bounds[3] = {24 * 1024, 64 * 1024, s.max_lds - record - 16};
+  std::vector<int> order;
+  int class_begin[4] = {0, 0, 0, 0};
+  for (int c = 0; c < 3; c++) {
+    for (int i = 0; i < n; i++) {
+      int const need = progs[i].lds_bytes;
+      if (need <= bounds[c] && (c == 0 || need > bounds[c - 1])) {
+        order.push_back(i);
+      }
+    }
+    class_begin[c + 1] = (int)order.size();
+  }
+  int const members = (int)order.size();
+  std::vector<CombineJob> jobs;
+  std::vector<int> job_first(1, 0);
+  for (int i : order) {
+    DevProgram const &p = progs[i];
+    if (p.splits < 2) {
+      continue;
+    }
+    for (int o = 0; o < MI355_MAX_DMEM_OUTPUTS; o++) {
+      if (p.out[o] == nullptr || p.part_elems[o] <= 0) {
+        continue;
+      }
+      CombineJob j;
+      j.part = p.part[o];
+      j.out = static_cast<uint16_t *>(p.out[o]);
+      j.n = p.part_elems[o];
+      j.stride_elems = p.part_stride[o];
+      j.splits = p.splits;
+      j.pad = 0;
+      jobs.push_back(j);
+      job_first.push_back(job_first.back() + (int)std::min<long long>((j.n + 255) / 256, 256));
+    }
+  }
+  int launched = 0;
+  if (members > 0) {
+    // staging layout: programs | first_block per class (members + 3 ints) | jobs | job_first
+    size_t const off_first = sizeof(DevProgram) * (size_t)members;
+    size_t const off_jobs = (off_first + sizeof(int) * (size_t)(members + 3) + 15) / 16 * 16;
+    size_t const off_jfirst = off_jobs + sizeof(CombineJob) * jobs.size();
+    size_t const bytes = (off_jfirst + sizeof(int) * job_first.size() + 15) / 16 * 16;
+    if (bytes > State::kBatchSlotBytes) {
+      return fail(MI355_ERR_UNSUPPORTED, "batch chunk does not fit its staging buffer");
+    }
+    State::BatchSlot &slot = s.batch[tls_queue][s.batch_next[tls_queue]];
+    s.batch_next[tls_queue] = (s.batch_next[tls_queue] + 1) % State::kBatchSlots;
+    MI355_HIP(hipEventSynchronize(slot.copied));  // the copy that last read this buffer is done
+    DevProgram *hp = reinterpret_cast<DevProgram *>(slot.host);
+    int *hf = reinterpret_cast<int *>(slot.host + off_first);
+    int fpos = 0;
+    int first_off[3], first_cnt[3];
+    for (int c = 0; c < 3; c++) {
+      first_off[c] = fpos;
+      first_cnt[c] = class_begin[c + 1] - class_begin[c];
+      int acc = 0;
+      for (int k = class_begin[c]; k < class_begin[c + 1]; k++) {
+        DevProgram const &p = progs[order[k]];
+        hp[k] = p;
+        hf[fpos++] = acc;
+        acc += p.grid[0] * p.splits * p.grid[1] * p.grid[2];
+      }
+      hf[fpos++] = acc;  // total of the class
+    }
+    if (!jobs.empty()) {
+      memcpy(slot.host + off_jobs, jobs.data(), sizeof(CombineJob) * jobs.size());
+      memcpy(slot.host + off_jfirst, job_first.data(), sizeof(int) * job_first.size());
+    }
+    // the records travel by a copy kernel that reads the pinned buffer over the bus: a
+    // stream-ordered hipMemcpyAsync of this size costs the host ~100 us per call here
+    stage_records_kernel<<<(int)((bytes / 16 + 255) / 256), 256, 0, s.stream()>>>(
+        reinterpret_cast<uint4v const *>(slot.host), reinterpret_cast<uint4v *>(slot.dev),
+        (int)(bytes / 16));
+    MI355_HIP(hipEventRecord(slot.copied, s.stream()));
+    static bool lds_raised = false;
+    DevProgram const *dp = reinterpret_cast<DevProgram const *>(slot.dev);
+    int const *df = reinterpret_cast<int const *>(slot.dev + off_first);
+    for (int c = 0; c < 3; c++) {
+      if (first_cnt[c] == 0) {
+        continue;
+      }
+      int lds = 0;
+      for (int k = class_begin[c]; k < class_begin[c + 1]; k++) {
+        lds = std::max(lds, progs[order[k]].lds_bytes);
+      }
+      int const program_off = (lds + 15) / 16 * 16;
+      int const lds_total = program_off + record;
+      if (lds_total > 65536 && !lds_raised) {
+        MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_interp_multi_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, s.max_lds));
+        lds_raised = true;
+      }
+      int const blocks = hf[first_off[c] + first_cnt[c]];
+      fp_interp_multi_kernel<<<blocks, kInterpThreads, lds_total, s.stream()>>>(
+          dp + class_begin[c], df + first_off[c], first_cnt[c], program_off, s.exp_tbl, s.div_p,
+          s.div_q);
+      launched += blocks;
+    }
+    if (!jobs.empty()) {
+      fp_combine_splits_multi_kernel<<<job_first.back(), 256, 0, s.stream()>>>(
+          reinterpret_cast<CombineJob const *>(slot.dev + off_jobs),
+          reinterpret_cast<int const *>(slot.dev + off_jfirst), (int)jobs.size());
+    }
+    MI355_HIP(hipGetLastError());
+  }
+  // programs too large to share LDS with their own record: one launch each (launch() also
+  // folds their split for-loops)
+  for (int i = 0; i < n; i++) {
+    if (progs[i].lds_bytes > bounds[2]) {
+      int rc = launch(progs[i], false);
+      if (rc != MI355_OK) {
+        return rc;
+      }
+      launched += s.last_launch.workgroups;
+    }
+  }
+  s.last_launch.kernel_id = MI355_KERNEL_FP_INTERP;
+  s.last_launch.workgroups = launched;
+  s.last_launch.threads = kInterpThreads;
+  s.last_launch.lds_bytes = 0;
+  s.last_launch.row_split = 1;
+  return MI355_OK;
+}
+
 extern "C" int mi355_customized_fp_batch(mi355_plan const *plans, int n,
                                          void const *const *inputs, void *const *outputs) {
   MI355_REQUIRE_INIT();
   if (n < 0 || (n > 0 && (plans == nullptr || inputs == nullptr || outputs == nullptr))) {
     return fail(MI355_ERR_INVALID, "bad batch (n = %d)", n);
   }
-  // independent operators: dealt over the queues so their (often small) grids overlap
-  int const home = tls_queue;
-  int rc = MI355_OK;
-  for (int i = 0; i < n && rc == MI355_OK; i++) {
-    tls_queue = (home + i) % MI355_NUM_QUEUES;
-    DevProgram prog;
-    rc = prepare(&plans[i], inputs + (size_t)i * MI355_MAX_DMEM_INPUTS,
-                 outputs + (size_t)i * MI355_MAX_DMEM_OUTPUTS, false, prog);
-    if (rc == MI355_OK) {
-      rc = launch(prog, false);
+  // independent operators: a handful of launches for all of them, on the caller's queue
+  int const chunk_max = 64;
+  for (int begin = 0; begin < n; begin += chunk_max) {
+    int const m = std::min(chunk_max, n - begin);
+    std::vector<DevProgram> progs((size_t)m);
+    std::vector<PlanExtents> exts((size_t)m);
+    std::vector<int> nout((size_t)m);
+    for (int i = 0; i < m; i++) {
+      int rc = prepare(&plans[begin + i], inputs + (size_t)(begin + i) * MI355_MAX_DMEM_INPUTS,
+                       outputs + (size_t)(begin + i) * MI355_MAX_DMEM_OUTPUTS, false, progs[(size_t)i],
+                       &exts[(size_t)i]);
+      if (rc != MI355_OK) {
+        return rc;
+      }
+      nout[(size_t)i] = plans[begin + i].num_dmem_outputs;
+    }
+    int rc = launch_fp_chunk(progs, exts, nout);
+    if (rc != MI355_OK) {
+      return rc;
     }
   }
-  tls_queue = home;
-  return rc;
+  return MI355_OK;
 }
 
 extern "C" int mi355_customized_run(mi355_plan const *plan, void const *const *inputs,

@@ -58,7 +58,7 @@ struct DevOp {
   uint32_t mg0, mg1, mg2;
 };
 
-struct DevProgram {
+struct alignas(16) DevProgram {
   int num_ops, num_tensors;
   int forloop_range;
   int lds_bytes;  // dynamic LDS the interpreter requests (tables included)

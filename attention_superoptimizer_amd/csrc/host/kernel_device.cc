@@ -242,6 +242,15 @@ static LoweredOp lower(KNCustomizedOp const &op, bool fingerprint) {
   return l;
 }
 
+// for batched submission (verify.cc): the lowered program and its bound pointers
+void lower_customized(KNCustomizedOp const &op, bool fingerprint, mi355_plan *plan,
+                      void const **inputs, void **outputs) {
+  LoweredOp l = lower(op, fingerprint);
+  *plan = l.plan;
+  std::memcpy(inputs, l.inputs, sizeof(l.inputs));
+  std::memcpy(outputs, l.outputs, sizeof(l.outputs));
+}
+
 void KNCustomizedOp::run() {
   require_device("KNCustomizedOp::run");
   LoweredOp l = lower(*this, false);

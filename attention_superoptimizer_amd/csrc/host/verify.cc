@@ -15,6 +15,12 @@
 #include <unordered_set>
 
 namespace mirage {
+namespace kernel {
+// kernel_device.cc: the lowered program of a customized operator and its bound pointers
+void lower_customized(KNCustomizedOp const &op, bool fingerprint, mi355_plan *plan,
+                      void const **inputs, void **outputs);
+}  // namespace kernel
+
 namespace search {
 
 using kernel::DTensor;
@@ -71,39 +77,96 @@ static void account(KNOperator const *op, VerifyStats *stats) {
   }
 }
 
-void fingerprint_graph(kernel::Graph const &g, uint64_t input_seed, VerifyStats *stats) {
+// Inputs depend on nothing: the inputs of all the graphs given are filled by as few
+// launches as the backend's tensor list allows.  Input number j of every graph draws from
+// (input_seed, j).
+static void fill_inputs(std::vector<kernel::Graph const *> const &graphs, uint64_t input_seed) {
   kernel::require_device("fingerprint_graph");
-  // inputs depend on nothing: all of them in one launch (batches of MI355_MAX_FILL_TENSORS)
   uint16_t *ptrs[MI355_MAX_FILL_TENSORS];
   size_t counts[MI355_MAX_FILL_TENSORS];
   uint64_t seeds[MI355_MAX_FILL_TENSORS];
   int pending = 0;
-  uint64_t ordinal = 0;
   auto flush = [&]() {
     if (pending > 0) {
       MI355_CALL(mi355_fp_fill_many(ptrs, counts, seeds, pending, input_seed == 0 ? 1 : 0));
       pending = 0;
     }
   };
-  for (KNOperator *op : g.operators) {
-    if (op->op_type != KN_INPUT_OP) {
-      continue;
-    }
-    DTensor const &t = op->output_tensors[0];
-    ptrs[pending] = t.fp_ptr;
-    counts[pending] = t.num_elements();
-    seeds[pending] = input_seed ^ (ordinal << 40);
-    ordinal++;
-    if (++pending == MI355_MAX_FILL_TENSORS) {
-      flush();
+  for (kernel::Graph const *g : graphs) {
+    uint64_t ordinal = 0;
+    for (KNOperator *op : g->operators) {
+      if (op->op_type != KN_INPUT_OP) {
+        continue;
+      }
+      DTensor const &t = op->output_tensors[0];
+      ptrs[pending] = t.fp_ptr;
+      counts[pending] = t.num_elements();
+      seeds[pending] = input_seed ^ (ordinal << 40);
+      ordinal++;
+      if (++pending == MI355_MAX_FILL_TENSORS) {
+        flush();
+      }
     }
   }
   flush();
+}
+
+void fingerprint_graph(kernel::Graph const &g, uint64_t input_seed, VerifyStats *stats) {
+  fill_inputs({&g}, input_seed);
   for (KNOperator *op : g.operators) {
     account(op, stats);
     if (op->op_type != KN_INPUT_OP) {
       op->fingerprint();
     }
+  }
+}
+
+// Fingerprints several independent graphs on the calling thread's queue.  Kernel-level
+// operators are enqueued one by one; the customized operators the graphs reach next are
+// collected and submitted together (mi355_customized_fp_batch: a handful of launches for
+// all of them), round after round, until every graph is through.  The queue is in order,
+// so an operator's producers are always ahead of it.
+static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint64_t input_seed,
+                               VerifyStats *stats) {
+  size_t const n = graphs.size();
+  std::vector<size_t> cursor(n, 0);
+  fill_inputs(std::vector<kernel::Graph const *>(graphs.begin(), graphs.end()), input_seed);
+  for (kernel::Graph *g : graphs) {
+    for (KNOperator *op : g->operators) {
+      account(op, stats);
+    }
+  }
+  std::vector<mi355_plan> plans;
+  std::vector<void const *> ins;
+  std::vector<void *> outs;
+  for (;;) {
+    plans.clear();
+    ins.clear();
+    outs.clear();
+    for (size_t k = 0; k < n; k++) {
+      std::vector<KNOperator *> const &ops = graphs[k]->operators;
+      while (cursor[k] < ops.size()) {
+        KNOperator *op = ops[cursor[k]++];
+        if (op->op_type == KN_INPUT_OP) {
+          continue;
+        }
+        if (op->op_type != KN_CUSTOMIZED_OP) {
+          op->fingerprint();
+          continue;
+        }
+        plans.emplace_back();
+        ins.resize(ins.size() + MI355_MAX_DMEM_INPUTS, nullptr);
+        outs.resize(outs.size() + MI355_MAX_DMEM_OUTPUTS, nullptr);
+        kernel::lower_customized(*static_cast<kernel::KNCustomizedOp *>(op), true, &plans.back(),
+                                 &ins[ins.size() - MI355_MAX_DMEM_INPUTS],
+                                 &outs[outs.size() - MI355_MAX_DMEM_OUTPUTS]);
+        break;
+      }
+    }
+    if (plans.empty()) {
+      break;
+    }
+    MI355_CALL(mi355_customized_fp_batch(plans.data(), (int)plans.size(), ins.data(), outs.data()));
   }
 }
 
@@ -152,8 +215,23 @@ void verify_batch(std::vector<kernel::Graph *> const &candidates,
   std::vector<VerifyStats> local((size_t)std::max(workers, 1));
   auto work = [&](int w) {
     MI355_CALL(mi355_queue_select(w));
+    std::vector<kernel::Graph *> mine;
     for (size_t i = (size_t)w; i < n; i += (size_t)workers) {
-      fingerprint_graph(*candidates[i], input_seed, &local[w]);
+      mine.push_back(candidates[i]);
+    }
+    fingerprint_graphs(mine, input_seed, &local[w]);
+    // this worker's compares, MI355_MAX_COMPARE_PAIRS per launch
+    uint16_t const *ca[MI355_MAX_COMPARE_PAIRS], *cb[MI355_MAX_COMPARE_PAIRS];
+    size_t cn[MI355_MAX_COMPARE_PAIRS];
+    int cs[MI355_MAX_COMPARE_PAIRS];
+    int pairs = 0;
+    auto flush = [&]() {
+      if (pairs > 0) {
+        MI355_CALL(mi355_fp_equal_enqueue_many(ca, cb, cn, cs, pairs));
+        pairs = 0;
+      }
+    };
+    for (size_t i = (size_t)w; i < n; i += (size_t)workers) {
       if (pend[i].first_slot < 0) {
         continue;
       }
@@ -164,14 +242,19 @@ void verify_batch(std::vector<kernel::Graph *> const &candidates,
           }
           int const slot = pend[i].first_slot + (int)(r * no + c);
           possible[slot] = 1;
-          MI355_CALL(mi355_fp_equal_enqueue(reference_outputs[r].fp_ptr,
-                                            pend[i].outputs[c].fp_ptr,
-                                            reference_outputs[r].num_elements(), slot));
+          ca[pairs] = reference_outputs[r].fp_ptr;
+          cb[pairs] = pend[i].outputs[c].fp_ptr;
+          cn[pairs] = reference_outputs[r].num_elements();
+          cs[pairs] = slot;
+          if (++pairs == MI355_MAX_COMPARE_PAIRS) {
+            flush();
+          }
           local[w].compares++;
           local[w].fp_bytes += 2 * (long long)reference_outputs[r].fingerprint_size();
         }
       }
     }
+    flush();
   };
   {
     std::vector<std::thread> threads;

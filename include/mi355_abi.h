@@ -147,10 +147,11 @@ int mi355_fp_fill_iota(uint16_t *fp, size_t n);
 /* seeded inputs: fp[i] = splitmix64(seed + i) % 25651 (no reference counterpart;
  * the reference's FIXME at input_kernel.cu:59 asks for random inputs) */
 int mi355_fp_fill_uniform(uint16_t *fp, size_t n, uint64_t seed);
-/* Every input of one graph in a single launch (init_input_fingerprint once per tensor in
- * the reference, input_kernel.cu:56-72): tensor i gets `idx % 25651` when iota != 0, else
- * the uniform values of mi355_fp_fill_uniform with seeds[i]. */
-#define MI355_MAX_FILL_TENSORS 8
+/* Up to MI355_MAX_FILL_TENSORS input tensors (of one graph or of several) in a single
+ * launch (init_input_fingerprint once per tensor in the reference, input_kernel.cu:56-72):
+ * tensor i gets `idx % 25651` when iota != 0, else the uniform values of
+ * mi355_fp_fill_uniform with seeds[i]. */
+#define MI355_MAX_FILL_TENSORS 64
 int mi355_fp_fill_many(uint16_t *const *fp, size_t const *n, uint64_t const *seeds, int count,
                        int iota);
 /* compute_matmul_fingerprint, src/kernel/cuda/matmul_kernel.cu:145-203 */
@@ -179,6 +180,11 @@ int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, int *equal);
 #define MI355_COMPARE_SLOTS 65536
 int mi355_fp_equal_reset(int first_slot, int count);
 int mi355_fp_equal_enqueue(uint16_t const *a, uint16_t const *b, size_t n, int slot);
+/* `count` <= MI355_MAX_COMPARE_PAIRS compares in one launch: pair i is (a[i], b[i]) of n[i]
+ * elements and reports into slots[i]. */
+#define MI355_MAX_COMPARE_PAIRS 64
+int mi355_fp_equal_enqueue_many(uint16_t const *const *a, uint16_t const *const *b,
+                                size_t const *n, int const *slots, int count);
 int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal);
 /* KNCustomizedOp::fingerprint + compute_customizedop_fingerprint,
  * src/kernel/cuda/customized_kernel.cu:307-603,655-678 */
@@ -187,10 +193,10 @@ int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,
 
 /* n independent customized-op fingerprints in one call (the batched form of the entry above
  * for a verification loop that holds many candidates, src/search/search.cc:601-603):
- * operator i reads inputs[4*i .. 4*i+3] and writes outputs[4*i .. 4*i+3]; the operators are
- * dealt round-robin over the backend's queues starting at the caller's, so the caller must
- * mi355_sync (or collect compares) before reading results, and must not pass operators
- * that depend on each other. */
+ * operator i reads inputs[4*i .. 4*i+3] and writes outputs[4*i .. 4*i+3].  The operators must
+ * not depend on each other: they run as a handful of launches on the caller's queue, each
+ * covering many operators (grouped by LDS need; workgroup -> operator by a prefix table in
+ * device memory), plus one launch that folds the partial sums of every split for-loop. */
 int mi355_customized_fp_batch(mi355_plan const *plans, int n, void const *const *inputs,
                               void *const *outputs);
 

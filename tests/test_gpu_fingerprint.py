@@ -104,6 +104,87 @@ def test_uniform_fill_matches_host_generator(rt, abi):
         g.close()
 
 
+def test_many_fills_and_many_compares_in_one_launch(rt, abi):
+    """mi355_fp_fill_many over 40 tensors of ragged sizes = the single-tensor fill of each;
+    mi355_fp_equal_enqueue_many over 40 pairs = the verdict of each pair (every third pair is
+    made to differ in one element, at the very end or the very start)."""
+    sizes = [1 + 37 * i + (i % 5) * 4096 for i in range(40)]
+    spec = [{"op": "input", "dims": [n]} for n in sizes] * 2
+    g, vals = rt.build_from_spec(spec)
+    try:
+        left, right = [v[0] for v in vals[:40]], [v[0] for v in vals[40:]]
+        for side in (left, right):
+            ptrs = (ctypes.c_void_p * 40)(*[t.device_ptr(True) for t in side])
+            ns = (ctypes.c_size_t * 40)(*sizes)
+            seeds = (ctypes.c_uint64 * 40)(*[9000 + i for i in range(40)])
+            assert abi.mi355_fp_fill_many(ptrs, ns, seeds, 40, 0) == 0
+        for i, t in enumerate(left):
+            assert np.array_equal(t.read_fingerprint(), uniform_fp(t.dims, 9000 + i)), i
+        differ = [i % 3 == 1 for i in range(40)]
+        for i, t in enumerate(right):
+            if differ[i]:
+                a = t.read_fingerprint()
+                a[-1 if i % 2 else 0] ^= 1
+                t.write_fingerprint(a)
+        assert abi.mi355_fp_equal_reset(100, 40) == 0
+        pa = (ctypes.c_void_p * 40)(*[t.device_ptr(True) for t in left])
+        pb = (ctypes.c_void_p * 40)(*[t.device_ptr(True) for t in right])
+        ns = (ctypes.c_size_t * 40)(*sizes)
+        slots = (ctypes.c_int * 40)(*[100 + i for i in range(40)])
+        assert abi.mi355_fp_equal_enqueue_many(pa, pb, ns, slots, 40) == 0
+        eq = (ctypes.c_ubyte * 40)()
+        assert abi.mi355_fp_equal_collect(100, 40, eq) == 0
+        assert [bool(e) for e in eq] == [not d for d in differ]
+    finally:
+        g.close()
+
+
+def test_batched_customized_fingerprints_of_generated_candidates(rt, abi):
+    """Many small, unlike customized ops (the generator's candidates, dims <= 256) through
+    mi355_customized_fp_batch in one call = one mi355_customized_fp each, bit for bit."""
+    from attention_superoptimizer_amd import _native as N
+    from attention_superoptimizer_amd import candidates as C
+    problems = C.generate(num_problems=4, per_problem=12, seed=77, max_dim=256)
+    built, plans, ins, outs, want = [], [], [], [], []
+    try:
+        for prob in problems:
+            for cand in prob["candidates"]:
+                spec = cand["spec"]
+                # candidates whose customized op consumes only graph inputs
+                idx = [i for i, op in enumerate(spec) if op["op"] == "customized"
+                       and all(spec[a]["op"] == "input" for a, _ in op["in"])]
+                if not idx:
+                    continue
+                g, vals = rt.build_from_spec(spec)
+                built.append((g, vals, idx[0]))
+                for i, op in enumerate(spec):
+                    if op["op"] == "input":
+                        vals[i][0].write_fingerprint(uniform_fp(op["dims"], 4000 + i))
+                g.fingerprint(idx[0])
+                want.append([t.read_fingerprint() for t in vals[idx[0]]])
+                for t in vals[idx[0]]:
+                    t.write_fingerprint(np.zeros(t.dims, np.uint16))
+                plans.append(g.lowered(idx[0], True))
+                row_in = [vals[a][b].device_ptr(True) for a, b in spec[idx[0]]["in"]]
+                row_out = [t.device_ptr(True) for t in vals[idx[0]]]
+                ins += row_in + [0] * (4 - len(row_in))
+                outs += row_out + [0] * (4 - len(row_out))
+        n = len(plans)
+        assert n >= 24
+        arr = (N.Mi355Plan * n)(*plans)
+        assert abi.mi355_sync() == 0
+        print("batch of", n, "customized ops", flush=True)
+        assert abi.mi355_customized_fp_batch(arr, n, (ctypes.c_void_p * len(ins))(*ins),
+                                             (ctypes.c_void_p * len(outs))(*outs)) == 0, N.last_error()
+        assert abi.mi355_sync() == 0
+        for k, (g, vals, i) in enumerate(built):
+            for a, b in zip([t.read_fingerprint() for t in vals[i]], want[k]):
+                assert np.array_equal(a, b), k
+    finally:
+        for g, _, _ in reversed(built):
+            g.close()
+
+
 def _check_examples(rt, names, random_inputs):
     from attention_superoptimizer_amd import workloads as W
     for name in names:
