@@ -426,7 +426,21 @@ __global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
         acc[j] = (_Float16)0.0f;
       }
       int q = 0;
-      for (; q + 4 <= P.ksplit; q += 4) {  // four loads in flight, adds in order
+      for (; q + 8 <= P.ksplit; q += 8) {  // eight loads in flight, adds in order
+        half8 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          v[u] = *reinterpret_cast<half8 const *>(sp + (long long)(q + u) * slab);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            acc[j] = static_cast<_Float16>(static_cast<float>(acc[j]) + static_cast<float>(v[u][j]));
+          }
+        }
+      }
+      for (; q + 4 <= P.ksplit; q += 4) {
         half8 v[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
