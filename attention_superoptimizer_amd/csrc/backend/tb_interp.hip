@@ -806,9 +806,32 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   // a fused kernel keeps tiles in registers, so the interpreter's LDS need does not
   // bound it: lower without the limit first, and again with it if no fused kernel fits
   bool const declared = f16 && state().plan_smem_layout != 0;
-  int rc = compile_plan(*plan, f16, try_fused ? (1 << 30) : state().max_lds, prog, ext, err, declared);
+  // (only a load-load-matmul-save plan can take the fused fingerprint kernel: everything
+  // else is lowered once, with the limit)
+  bool const try_fused_fp = !f16 && !state().force_interpreter && plan->num_operators == 4 &&
+                            plan->operator_types[0] == TB_INPUT_OP &&
+                            plan->operator_types[1] == TB_INPUT_OP &&
+                            plan->operator_types[2] == TB_MATMUL_OP &&
+                            plan->operator_types[3] == TB_OUTPUT_OP;
+  int rc = compile_plan(*plan, f16, (try_fused || try_fused_fp) ? (1 << 30) : state().max_lds, prog, ext,
+                        err, declared);
   if (rc != MI355_OK) {
     return fail(rc, "%s", err.c_str());
+  }
+  if (try_fused_fp) {
+    // the fused fingerprint matmul keeps no tile in LDS either: same two-step lowering
+    for (int i = 0; i < plan->num_dmem_inputs; i++) {
+      prog.in[i] = inputs[i];
+    }
+    for (int i = 0; i < plan->num_dmem_outputs; i++) {
+      prog.out[i] = outputs[i];
+    }
+    if (!fp_gemm_applicable(prog)) {
+      rc = compile_plan(*plan, false, state().max_lds, prog, ext, err);
+      if (rc != MI355_OK) {
+        return fail(rc, "%s", err.c_str());
+      }
+    }
   }
   auto bind = [&]() {
     for (int i = 0; i < plan->num_dmem_inputs; i++) {
@@ -861,8 +884,39 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   return MI355_OK;
 }
 
+static int fold_splits(DevProgram const &prog) {
+  State &s = state();
+  for (int o = 0; o < MI355_MAX_DMEM_OUTPUTS; o++) {
+    if (prog.out[o] == nullptr || prog.part_elems[o] <= 0) {
+      continue;
+    }
+    long long const n = prog.part_elems[o];
+    int const blocks = (int)std::min<long long>((n + 255) / 256, 2048);
+    fp_combine_splits_kernel<<<blocks, 256, 0, s.stream()>>>(
+        prog.part[o], static_cast<uint16_t *>(prog.out[o]), n, prog.part_stride[o], prog.splits);
+  }
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
+  if (!f16 && prog.fused == 4) {
+    if (int rc = launch_fp_gemm(prog, s.stream())) {
+      return rc;
+    }
+    if (prog.splits > 1) {
+      if (int rc = fold_splits(prog)) {
+        return rc;
+      }
+    }
+    s.last_launch.kernel_id = MI355_KERNEL_FP_GEMM;
+    s.last_launch.workgroups = prog.grid[0] * prog.splits * prog.grid[1] * prog.grid[2];
+    s.last_launch.threads = kInterpThreads;
+    s.last_launch.lds_bytes = prog.lds_bytes;
+    s.last_launch.row_split = prog.splits;
+    return MI355_OK;
+  }
   if (prog.fused != 0) {
     int rc = prog.fused == 1   ? try_launch_attention(prog)
              : prog.fused == 2 ? try_launch_gemm(prog)
@@ -891,14 +945,8 @@ static int launch(DevProgram const &prog, bool f16) {
     fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog, s.exp_tbl,
                                                                           s.div_p, s.div_q);
     if (prog.splits > 1) {
-      for (int o = 0; o < MI355_MAX_DMEM_OUTPUTS; o++) {
-        if (prog.out[o] == nullptr || prog.part_elems[o] <= 0) {
-          continue;
-        }
-        long long const n = prog.part_elems[o];
-        int const blocks = (int)std::min<long long>((n + 255) / 256, 2048);
-        fp_combine_splits_kernel<<<blocks, 256, 0, s.stream()>>>(
-            prog.part[o], static_cast<uint16_t *>(prog.out[o]), n, prog.part_stride[o], prog.splits);
+      if (int rc = fold_splits(prog)) {
+        return rc;
       }
     }
   }
@@ -977,15 +1025,27 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
     set_splits(progs[i], exts[i], num_outputs[i], std::min(progs[i].forloop_range, scale), used);
   }
   int const record = (int)sizeof(DevProgram);
-  // LDS classes: a launch requests the largest need of its members, which bounds how many
-  // workgroups share a compute unit
+  // Launch classes.  Interpreter programs by LDS need (a launch requests the largest need of
+  // its members, which bounds how many workgroups share a compute unit); fused matmul
+  // programs by register tiles per thread (a template argument of their kernel).
+  constexpr int kClasses = 6;
   int const bounds[3] = {24 * 1024, 64 * 1024, s.max_lds - record - 16};
+  auto class_of = [&](DevProgram const &p) {
+    if (p.fused == 4) {
+      return p.fg[3] == 1 ? 3 : (p.fg[3] == 2 ? 4 : 5);
+    }
+    for (int c = 0; c < 3; c++) {
+      if (p.lds_bytes <= bounds[c]) {
+        return c;
+      }
+    }
+    return -1;  // no room for the record above its tiles: launched by itself
+  };
   std::vector<int> order;
-  int class_begin[4] = {0, 0, 0, 0};
-  for (int c = 0; c < 3; c++) {
+  int class_begin[kClasses + 1] = {};
+  for (int c = 0; c < kClasses; c++) {
     for (int i = 0; i < n; i++) {
-      int const need = progs[i].lds_bytes;
-      if (need <= bounds[c] && (c == 0 || need > bounds[c - 1])) {
+      if (class_of(progs[i]) == c) {
         order.push_back(i);
       }
     }
@@ -1016,9 +1076,9 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
   }
   int launched = 0;
   if (members > 0) {
-    // staging layout: programs | first_block per class (members + 3 ints) | jobs | job_first
+    // staging layout: programs | first_block per class (members + kClasses ints) | jobs | job_first
     size_t const off_first = sizeof(DevProgram) * (size_t)members;
-    size_t const off_jobs = (off_first + sizeof(int) * (size_t)(members + 3) + 15) / 16 * 16;
+    size_t const off_jobs = (off_first + sizeof(int) * (size_t)(members + kClasses) + 15) / 16 * 16;
     size_t const off_jfirst = off_jobs + sizeof(CombineJob) * jobs.size();
     size_t const bytes = (off_jfirst + sizeof(int) * job_first.size() + 15) / 16 * 16;
     if (bytes > State::kBatchSlotBytes) {
@@ -1030,8 +1090,8 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
     DevProgram *hp = reinterpret_cast<DevProgram *>(slot.host);
     int *hf = reinterpret_cast<int *>(slot.host + off_first);
     int fpos = 0;
-    int first_off[3], first_cnt[3];
-    for (int c = 0; c < 3; c++) {
+    int first_off[kClasses], first_cnt[kClasses];
+    for (int c = 0; c < kClasses; c++) {
       first_off[c] = fpos;
       first_cnt[c] = class_begin[c + 1] - class_begin[c];
       int acc = 0;
@@ -1056,13 +1116,22 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
     static bool lds_raised = false;
     DevProgram const *dp = reinterpret_cast<DevProgram const *>(slot.dev);
     int const *df = reinterpret_cast<int const *>(slot.dev + off_first);
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < kClasses; c++) {
       if (first_cnt[c] == 0) {
         continue;
       }
       int lds = 0;
       for (int k = class_begin[c]; k < class_begin[c + 1]; k++) {
         lds = std::max(lds, progs[order[k]].lds_bytes);
+      }
+      if (c >= 3) {
+        int const blocks = hf[first_off[c] + first_cnt[c]];
+        if (int rc = launch_fp_gemm_multi(dp + class_begin[c], df + first_off[c], first_cnt[c], blocks,
+                                          c == 3 ? 1 : (c == 4 ? 2 : 4), lds, s.stream())) {
+          return rc;
+        }
+        launched += blocks;
+        continue;
       }
       int const program_off = (lds + 15) / 16 * 16;
       int const lds_total = program_off + record;
@@ -1087,7 +1156,7 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
   // programs too large to share LDS with their own record: one launch each (launch() also
   // folds their split for-loops)
   for (int i = 0; i < n; i++) {
-    if (progs[i].lds_bytes > bounds[2]) {
+    if (class_of(progs[i]) < 0) {
       int rc = launch(progs[i], false);
       if (rc != MI355_OK) {
         return rc;

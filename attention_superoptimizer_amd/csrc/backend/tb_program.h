@@ -8,6 +8,7 @@
 #pragma once
 
 #include "mi355_abi.h"
+#include <hip/hip_runtime_api.h>
 #include <cstdint>
 #include <string>
 
@@ -62,7 +63,9 @@ struct alignas(16) DevProgram {
   int num_ops, num_tensors;
   int forloop_range;
   int lds_bytes;  // dynamic LDS the interpreter requests (tables included)
-  int fused;      // 1 / 2 / 3: run by the fused attention / GEMM / combine kernel, not the interpreter
+  int fused;      // fp16: 1 / 2 / 3 = run by the fused attention / GEMM / combine kernel; uint16:
+                  // 4 = run by the fused fingerprint matmul kernel; 0 = the interpreter
+  int fg[4];      // fused fingerprint matmul: loader of A, loader of B, k chunk, register tiles per thread
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
@@ -96,6 +99,14 @@ bool combine_applicable(DevProgram const &prog);
 // Lowers `plan` for the uint16 interpreter (f16 == false: plain row-major tiles)
 // or the fp16 interpreter (f16 == true: padded rows, B operands k-contiguous).
 // Returns MI355_OK or an error code with `err` set.
+// Fused fingerprint matmul family (fp_gemm_fused.hip): recognise (marks the program and
+// replaces its LDS need), launch one program, launch many (programs and prefix table in
+// device memory, `staging_bytes` = the largest member's LDS need).
+bool fp_gemm_applicable(DevProgram &P);
+int launch_fp_gemm(DevProgram const &P, hipStream_t stream);
+int launch_fp_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks, int tpt,
+                         int staging_bytes, hipStream_t stream);
+
 // `declared_layouts`: fp16 loader tiles take the LDS layout the plan declares for them
 // (see MI355_OPT_PLAN_SMEM_LAYOUT) instead of the one their consumers want.
 int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,

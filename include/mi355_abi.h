@@ -80,9 +80,10 @@ typedef struct mi355_launch_info {
 #define MI355_KERNEL_F16_ATTENTION 3 /* fused register-resident attention family */
 #define MI355_KERNEL_F16_GEMM 4      /* fused skinny-GEMM family (split for-loop, ordered fix-up) */
 #define MI355_KERNEL_F16_COMBINE 5   /* fused fold-partials-and-divide family */
+#define MI355_KERNEL_FP_GEMM 6       /* fused fingerprint tiled-matmul family (uint16) */
 
-/* Backend options (mi355_set_option).  FORCE_INTERPRETER = 1 sends every fp16
- * customized op through the generic LDS interpreter instead of a fused kernel
+/* Backend options (mi355_set_option).  FORCE_INTERPRETER = 1 sends every customized op,
+ * fp16 or fingerprint, through the generic LDS interpreter instead of a fused kernel
  * (both must agree with the oracle; tests run the two against each other). */
 #define MI355_OPT_FORCE_INTERPRETER 1
 /* ATTENTION_MODE: 0 = choose by problem size (default), 1 = always the latency

@@ -104,6 +104,68 @@ def test_uniform_fill_matches_host_generator(rt, abi):
         g.close()
 
 
+@pytest.mark.parametrize("m,n,k,grid,F,amap,bmap,omap", [
+    (128, 256, 256, (4, 2, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),     # 64x64 tiles, k chunk 64
+    (256, 256, 512, (2, 2, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),     # 128x128 tiles, 4 register tiles
+    (64, 64, 512, (1, 1, 1), 8, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),   # one block: for-loop split 8 ways
+    (16, 40, 96, (1, 1, 1), 4, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),    # 16x40 tile, k tile 24 -> chunk 8
+    (64, 1024, 1024, (16, 1, 1), 16, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),  # config C1
+    (96, 192, 320, (2, 3, 1), 2, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),      # 32x96 tiles, k tile 160 -> chunk 32
+])
+def test_fused_matmul_fingerprint_equals_interpreter_and_oracle(rt, abi, m, n, k, grid, F, amap, bmap, omap):
+    """A load-load-matmul-accumulate plan runs on the fused fingerprint matmul kernel; forced
+    through the interpreter it must give the same uint16 tensor, and both the oracle's."""
+    import ctypes as ct
+    from attention_superoptimizer_amd import _native as N
+    from attention_superoptimizer_amd import workloads as W
+    spec = W.tiled_matmul(m, n, k, grid, F, amap, bmap, omap)[0]
+    ins = {0: uniform_fp(spec[0]["dims"], 31), 1: uniform_fp(spec[1]["dims"], 32)}
+    ins[0].flat[:7] = 25650  # worst-case operands in one corner
+    ins[1].flat[:7] = 25650
+    want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
+    got = {}
+    for forced in (0, 1):
+        assert abi.mi355_set_option(1, forced) == 0
+        try:
+            g, vals = rt.build_from_spec(spec)
+            try:
+                vals[0][0].write_fingerprint(ins[0])
+                vals[1][0].write_fingerprint(ins[1])
+                g.fingerprint(2)
+                info = N.Mi355LaunchInfo()
+                N.backend().mi355_last_launch(ct.byref(info))
+                assert info.kernel_id == (1 if forced else 6)
+                got[forced] = vals[2][0].read_fingerprint()
+            finally:
+                g.close()
+        finally:
+            assert abi.mi355_set_option(1, 0) == 0
+    assert np.array_equal(got[0], want)
+    assert np.array_equal(got[1], want)
+
+
+def test_fused_matmul_fingerprint_takes_tiles_the_interpreter_cannot_hold(rt, abi):
+    """A [128,256] and B [256,128] tiles need 197 KB of LDS in the interpreter; the fused
+    kernel streams them in k chunks of 64 and matches the oracle."""
+    import ctypes as ct
+    from attention_superoptimizer_amd import _native as N
+    from attention_superoptimizer_amd import workloads as W
+    spec = W.tiled_matmul(512, 512, 1024, (4, 4, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1))[0]
+    ins = {0: uniform_fp(spec[0]["dims"], 41), 1: uniform_fp(spec[1]["dims"], 42)}
+    want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        vals[0][0].write_fingerprint(ins[0])
+        vals[1][0].write_fingerprint(ins[1])
+        g.fingerprint(2)
+        info = N.Mi355LaunchInfo()
+        N.backend().mi355_last_launch(ct.byref(info))
+        assert info.kernel_id == 6 and info.lds_bytes == 2 * 2 * 16 * (128 + 4 + 128) * 4
+        assert np.array_equal(vals[2][0].read_fingerprint(), want)
+    finally:
+        g.close()
+
+
 def test_many_fills_and_many_compares_in_one_launch(rt, abi):
     """mi355_fp_fill_many over 40 tensors of ragged sizes = the single-tensor fill of each;
     mi355_fp_equal_enqueue_many over 40 pairs = the verdict of each pair (every third pair is
