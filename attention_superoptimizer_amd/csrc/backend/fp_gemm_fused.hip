@@ -120,11 +120,16 @@ __device__ __forceinline__ void fp_gemm_block(DevProgram const &P, uint32_t *lds
   };
 
   int const tiles_n = n / 4, tiles = (m / 4) * tiles_n;
+  // A small output tile leaves most threads without a register tile; they form further
+  // groups of `tiles` threads that each take every kgroups-th k quad of a step, and the
+  // groups' sums are added at the end (exact in the ring).  kgroups == 1 when TPT > 1.
+  int const kgroups = TPT == 1 ? P.fg[4] : 1;
+  int const kgroup = TPT == 1 ? tid / tiles : 0;
   int r0[TPT], c0[TPT];
   uint32_t accp[TPT][4][4], accq[TPT][4][4];
 #pragma unroll
   for (int u = 0; u < TPT; u++) {
-    int const t = tid + u * kThreads;
+    int const t = TPT == 1 ? tid % tiles : tid + u * kThreads;
     int const tt = t < tiles ? t : 0;  // idle threads shadow tile 0 and store nothing
     r0[u] = (tt / tiles_n) * 4;
     c0[u] = (tt % tiles_n) * 4;
@@ -148,7 +153,7 @@ __device__ __forceinline__ void fp_gemm_block(DevProgram const &P, uint32_t *lds
       fetch(s + 1);
     }
     uint32_t const *Ap = lds + (s & 1) * buf_dwords, *Bp = Ap + 2 * kq * lda;
-    for (int q = 0; q < kq; q++) {
+    for (int q = kgroup < kgroups ? kgroup : kq; q < kq; q += kgroups) {
 #pragma unroll
       for (int u = 0; u < TPT; u++) {
         uint4v const a_p = *reinterpret_cast<uint4v const *>(Ap + q * lda + r0[u]);
@@ -185,12 +190,50 @@ __device__ __forceinline__ void fp_gemm_block(DevProgram const &P, uint32_t *lds
     __syncthreads();
   }
 
+  if (TPT == 1 && kgroups > 1) {
+    // the step loop ended with a barrier: the staging buffers are free to carry the sums
+    uint32_t *red = lds;
+    if (kgroup > 0 && kgroup < kgroups) {
+      uint32_t *mine = red + ((kgroup - 1) * tiles + tid % tiles) * 32;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        *reinterpret_cast<uint4v *>(mine + 4 * i) = uint4v{accp[0][i][0] % FP_P, accp[0][i][1] % FP_P,
+                                                           accp[0][i][2] % FP_P, accp[0][i][3] % FP_P};
+        *reinterpret_cast<uint4v *>(mine + 16 + 4 * i) =
+            uint4v{accq[0][i][0] % FP_Q, accq[0][i][1] % FP_Q, accq[0][i][2] % FP_Q, accq[0][i][3] % FP_Q};
+      }
+    }
+    __syncthreads();
+    if (kgroup == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          accp[0][i][j] %= FP_P;
+          accq[0][i][j] %= FP_Q;
+        }
+      }
+      for (int gk = 1; gk < kgroups; gk++) {
+        uint32_t const *other = red + ((gk - 1) * tiles + tid) * 32;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          uint4v const vp = *reinterpret_cast<uint4v const *>(other + 4 * i);
+          uint4v const vq = *reinterpret_cast<uint4v const *>(other + 16 + 4 * i);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            accp[0][i][j] += vp[j];
+            accq[0][i][j] += vq[j];
+          }
+        }
+      }
+    }
+  }
   uint16_t *g = (P.splits > 1 ? P.part[so.io] + (long long)split * P.part_stride[so.io]
                               : static_cast<uint16_t *>(P.out[so.io])) +
                 origin(so, 0, bx, by, bz);
 #pragma unroll
   for (int u = 0; u < TPT; u++) {
-    if (tid + u * kThreads < tiles) {
+    if (tid + u * kThreads < tiles) {  // with k groups: the threads of group 0
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         uint32_t z[4];
@@ -308,7 +351,17 @@ bool fp_gemm_applicable(DevProgram &P) {
   P.fg[1] = b;
   P.fg[2] = kc;
   P.fg[3] = tpt;
-  P.lds_bytes = 2 * (2 * (kc / 4) * (m + 4 + n)) * 4;
+  int kgroups = 1;
+  if (tpt == 1) {
+    kgroups = kThreads / tiles;
+    kgroups = kgroups > kc / 4 ? kc / 4 : kgroups;
+    kgroups = kgroups > 8 ? 8 : kgroups;
+  }
+  P.fg[4] = kgroups;
+  P.fg[5] = 0;
+  int const staging = 2 * (2 * (kc / 4) * (m + 4 + n)) * 4;
+  int const reduce = (kgroups - 1) * tiles * 32 * 4;
+  P.lds_bytes = staging > reduce ? staging : reduce;
   return true;
 }
 

@@ -65,7 +65,8 @@ struct alignas(16) DevProgram {
   int lds_bytes;  // dynamic LDS the interpreter requests (tables included)
   int fused;      // fp16: 1 / 2 / 3 = run by the fused attention / GEMM / combine kernel; uint16:
                   // 4 = run by the fused fingerprint matmul kernel; 0 = the interpreter
-  int fg[4];      // fused fingerprint matmul: loader of A, loader of B, k chunk, register tiles per thread
+  int fg[6];      // fused fingerprint matmul: loader of A, loader of B, k chunk, register tiles per
+                  // thread, thread groups sharing a tile's k range (small tiles), spare
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
