@@ -198,14 +198,15 @@ def config1_fused_matmul():
     return tiled_matmul(64, 1024, 1024, (16, 1, 1), 16, (-1, -1, -1), (1, -1, -1), (1, -1, -1))
 
 
-def config2_gqa_decode():
+def config2_gqa_decode(groups=2, rows=256, seq=4096, kv_blocks=16, F=4):
     """GQA incremental decode as ONE customized op: Q[2,256,64] K[2,64,4096]
     V[2,4096,64], grid (2,16,1), for-loop 4 over the sequence,
-    matmul -> exp -> sum-reduce -> div -> matmul, output [2,256,1024]."""
+    matmul -> exp -> sum-reduce -> div -> matmul, output [2,256,1024].
+    The arguments scale the same plan (more kv-head groups, a longer sequence)."""
     g = [
-        _inp([2, 256, 64]), _inp([2, 64, 4096], COL), _inp([2, 4096, 64], COL),
+        _inp([groups, rows, 64]), _inp([groups, 64, seq], COL), _inp([groups, seq, 64], COL),
         {"op": "customized", "in": [[0, 0], [1, 0], [2, 0]],
-         "plan": _plan((2, 16, 1), 4, [(0, -1, -1), (0, 2, -1), (0, 1, -1)], (-1, 2, 1),
+         "plan": _plan((groups, kv_blocks, 1), F, [(0, -1, -1), (0, 2, -1), (0, 1, -1)], (-1, 2, 1),
                        (0, 2, -1),
                        [("tb_matmul_op", [(0, 0), (1, 0)]),
                         ("tb_exp_op", [(3, 0)]),
@@ -214,6 +215,12 @@ def config2_gqa_decode():
                         ("tb_matmul_op", [(6, 0), (2, 0)])])},
     ]
     return g, None
+
+
+def config2_gqa_decode_long():
+    """The C2 plan at a size where a launch is no longer most of the time: 32 kv-head
+    groups, 16,384 cached keys (K and V 67 MB each), for-loop 16."""
+    return config2_gqa_decode(groups=32, seq=16384, kv_blocks=16, F=16)
 
 
 def config3_mha_prefill(heads=32, seq=2048, hd=128, q_split=16, kv_split=1, F=32, rows2=32):
@@ -305,10 +312,16 @@ BASELINE_CONFIGS = {
     "C5a_gated_mlp": config5_gated_mlp,
 }
 
+# the same plans at other sizes (reported beside the baseline configurations, not instead)
+SCALED_CONFIGS = {
+    "C2_gqa_decode_long": config2_gqa_decode_long,
+}
+
 # fp16 input distributions per config (std of N(0, std)), keyed by input op index
 INPUT_STD = {
     "C1_fused_matmul": {0: 0.1, 1: 0.1},
     "C2_gqa_decode": {0: 0.125, 1: 0.125, 2: 0.125},
+    "C2_gqa_decode_long": {0: 0.125, 1: 0.125, 2: 0.125},
     "C3_mha_prefill": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
     # the configurations leave X's distribution open; N(0, 0.25) keeps every partial
     # sum below 2, where one fp16 ulp is still under the 1e-3 absolute tolerance

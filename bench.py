@@ -191,7 +191,7 @@ def main() -> int:
         return 0
 
     def setup(name):
-        spec, _ = W.BASELINE_CONFIGS[name]()
+        spec, _ = (W.BASELINE_CONFIGS.get(name) or W.SCALED_CONFIGS[name])()
         g, vals = G.build_from_spec(spec)
         for i, op in enumerate(spec):
             if op["op"] == "input":
@@ -297,7 +297,10 @@ def main() -> int:
     others = []
     if not args.headline_only:
         kname = {1: "fp_interp", 2: "f16_interp", 3: "f16_attention", 4: "f16_gemm", 5: "f16_combine"}
-        for name in ("C1_fused_matmul", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp"):
+        # the four other baseline configurations, then the headline plan at a size where the
+        # launch floor no longer dominates (32 groups x 16,384 keys)
+        for name in ("C1_fused_matmul", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp",
+                     "C2_gqa_decode_long"):
             g.close()
             spec2, g, vals2 = setup(name)
             rec = {"config": name, "ops": []}
