@@ -111,6 +111,9 @@ def test_uniform_fill_matches_host_generator(rt, abi):
     (16, 40, 96, (1, 1, 1), 4, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),    # 16x40 tile, k tile 24 -> chunk 8
     (64, 1024, 1024, (16, 1, 1), 16, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),  # config C1
     (96, 192, 320, (2, 3, 1), 2, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),      # 32x96 tiles, k tile 160 -> chunk 32
+    # 40,000 iterations of an 8-deep k tile: 625 steps per workgroup after the 64-way split, so
+    # the running sums are folded mid-way
+    (16, 32, 320000, (1, 1, 1), 40000, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),
 ])
 def test_fused_matmul_fingerprint_equals_interpreter_and_oracle(rt, abi, m, n, k, grid, F, amap, bmap, omap):
     """A load-load-matmul-accumulate plan runs on the fused fingerprint matmul kernel; forced
