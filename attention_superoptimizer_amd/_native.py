@@ -93,6 +93,7 @@ ABI = {
     "mi355_fp_matmul": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci]),
     "mi355_fp_unary": (_ci, [_ci, _vp, _vp, _sz]),
     "mi355_fp_binary": (_ci, [_ci, _vp, _pi, _vp, _pi, _vp, _pi, _ci]),
+    "mi355_fp_binary_many": (_ci, [_pi, _pvp, _pi, _pvp, _pi, _pvp, _pi, _pi, _ci]),
     "mi355_fp_reduce": (_ci, [_vp, _vp, _sz, _ci, _ci, _ci]),
     "mi355_fp_equal": (_ci, [_vp, _vp, _sz, _pi]),
     "mi355_fp_equal_reset": (_ci, [_ci, _ci]),

@@ -420,6 +420,47 @@ __global__ void fp_binary_kernel(int op, FpTables t, uint16_t const *__restrict_
   }
 }
 
+// Several independent element-wise binary operators in one launch: blockIdx.y names the entry.
+struct BinaryMany {
+  uint16_t const *in1[MI355_MAX_BINARY_OPS];
+  uint16_t const *in2[MI355_MAX_BINARY_OPS];
+  uint16_t *out[MI355_MAX_BINARY_OPS];
+  unsigned int n[MI355_MAX_BINARY_OPS];
+  int op[MI355_MAX_BINARY_OPS];
+  int nd[MI355_MAX_BINARY_OPS];
+  unsigned short d1[MI355_MAX_BINARY_OPS][4], d2[MI355_MAX_BINARY_OPS][4], od[MI355_MAX_BINARY_OPS][4];
+};
+
+__global__ void fp_binary_many_kernel(BinaryMany const B, FpTables t) {
+  int const e = blockIdx.y;
+  uint16_t const *in1 = B.in1[e], *in2 = B.in2[e];
+  uint16_t *out = B.out[e];
+  unsigned int const n = B.n[e];
+  int const op = B.op[e], nd = B.nd[e];
+  unsigned int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned int const stride = gridDim.x * blockDim.x;
+  for (; gid < n; gid += stride) {
+    // reference element_binary_kernel.cu:108-116
+    unsigned int i = gid, s1 = 1, i1 = 0, s2 = 1, i2 = 0;
+    for (int d = nd - 1; d >= 0; d--) {
+      i1 += (i % B.d1[e][d]) * s1;
+      i2 += (i % B.d2[e][d]) * s2;
+      s1 *= B.d1[e][d];
+      s2 *= B.d2[e][d];
+      i /= B.od[e][d];
+    }
+    uint32_t x = in1[i1], y = in2[i2], z;
+    if (op == KN_ADD_OP) {
+      z = (x + y) % FP_PQ;
+    } else if (op == KN_MUL_OP) {
+      z = (x * y) % FP_PQ;
+    } else {
+      z = fp_div_value(t, x, y);
+    }
+    out[gid] = static_cast<uint16_t>(z);
+  }
+}
+
 // ---- reduction (reference src/kernel/cuda/reduction_kernel.cu:80-108) ----------
 // out[i] = sum_k in[(i / os) * is + i % os + k * os]; sums of uint16 are folded
 // every 32768 terms so the 32-bit accumulator cannot wrap.
@@ -642,6 +683,59 @@ extern "C" int mi355_fp_binary(int op, uint16_t const *in1, int const *dims1,
   }
   fp_binary_kernel<<<grid_for(n), kThreads, 0, state().stream()>>>(op, tables(), in1, in2, out, D,
                                                                n);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_binary_many(int const *ops, uint16_t const *const *in1, int const *dims1,
+                                    uint16_t const *const *in2, int const *dims2,
+                                    uint16_t *const *out, int const *dims_out, int const *num_dims,
+                                    int count) {
+  MI355_REQUIRE_INIT();
+  if (count < 0 || count > MI355_MAX_BINARY_OPS ||
+      (count > 0 && (ops == nullptr || in1 == nullptr || dims1 == nullptr || in2 == nullptr ||
+                     dims2 == nullptr || out == nullptr || dims_out == nullptr || num_dims == nullptr))) {
+    return fail(MI355_ERR_INVALID, "bad operator list (count %d)", count);
+  }
+  if (count == 0) {
+    return MI355_OK;
+  }
+  BinaryMany B{};
+  size_t largest = 0;
+  for (int e = 0; e < count; e++) {
+    if (ops[e] != KN_ADD_OP && ops[e] != KN_MUL_OP && ops[e] != KN_DIV_OP) {
+      return fail(MI355_ERR_UNSUPPORTED, "binary fingerprint op %d", ops[e]);
+    }
+    if (num_dims[e] < 1 || num_dims[e] > 4) {
+      return fail(MI355_ERR_INVALID, "num_dims %d out of range", num_dims[e]);
+    }
+    if (in1[e] == nullptr || in2[e] == nullptr || out[e] == nullptr) {
+      return fail(MI355_ERR_INVALID, "operator %d: null tensor", e);
+    }
+    size_t n = 1;
+    for (int d = 0; d < num_dims[e]; d++) {
+      int const a = dims1[4 * e + d], b = dims2[4 * e + d], o = dims_out[4 * e + d];
+      if (a <= 0 || b <= 0 || o <= 0 || o > 65535 || (a != o && a != 1) || (b != o && b != 1)) {
+        return fail(MI355_ERR_INVALID, "operator %d: dim %d is not broadcastable (or above 65535)", e, d);
+      }
+      B.d1[e][d] = (unsigned short)a;
+      B.d2[e][d] = (unsigned short)b;
+      B.od[e][d] = (unsigned short)o;
+      n *= (size_t)o;
+    }
+    if (n > 0xffffffffu) {
+      return fail(MI355_ERR_UNSUPPORTED, "operator %d: more than 2^32 elements", e);
+    }
+    B.in1[e] = in1[e];
+    B.in2[e] = in2[e];
+    B.out[e] = out[e];
+    B.n[e] = (unsigned int)n;
+    B.op[e] = ops[e];
+    B.nd[e] = num_dims[e];
+    largest = std::max(largest, n);
+  }
+  dim3 grid(grid_for(largest, kThreads, 512), count);
+  fp_binary_many_kernel<<<grid, kThreads, 0, state().stream()>>>(B, tables());
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }

@@ -121,11 +121,12 @@ void fingerprint_graph(kernel::Graph const &g, uint64_t input_seed, VerifyStats 
   }
 }
 
-// Fingerprints several independent graphs on the calling thread's queue.  Kernel-level
-// operators are enqueued one by one; the customized operators the graphs reach next are
-// collected and submitted together (mi355_customized_fp_batch: a handful of launches for
-// all of them), round after round, until every graph is through.  The queue is in order,
-// so an operator's producers are always ahead of it.
+// Fingerprints several independent graphs on the calling thread's queue, round by round.
+// In a round every graph advances through its kernel-level matmuls, unary operators and
+// reductions (enqueued one by one) up to its next element-wise binary or customized
+// operator; those are collected and submitted together (mi355_fp_binary_many,
+// mi355_customized_fp_batch: a handful of launches for all of them).  The queue is in
+// order, so an operator's producers are always ahead of it.
 static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint64_t input_seed,
                                VerifyStats *stats) {
   size_t const n = graphs.size();
@@ -139,16 +140,55 @@ static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint6
   std::vector<mi355_plan> plans;
   std::vector<void const *> ins;
   std::vector<void *> outs;
+  int b_op[MI355_MAX_BINARY_OPS], b_nd[MI355_MAX_BINARY_OPS];
+  uint16_t const *b_in1[MI355_MAX_BINARY_OPS], *b_in2[MI355_MAX_BINARY_OPS];
+  uint16_t *b_out[MI355_MAX_BINARY_OPS];
+  int b_d1[4 * MI355_MAX_BINARY_OPS], b_d2[4 * MI355_MAX_BINARY_OPS], b_od[4 * MI355_MAX_BINARY_OPS];
+  int binaries = 0;
+  auto flush_binaries = [&]() {
+    if (binaries > 0) {
+      MI355_CALL(mi355_fp_binary_many(b_op, b_in1, b_d1, b_in2, b_d2, b_out, b_od, b_nd, binaries));
+      binaries = 0;
+    }
+  };
   for (;;) {
     plans.clear();
     ins.clear();
     outs.clear();
+    bool any = false;
     for (size_t k = 0; k < n; k++) {
       std::vector<KNOperator *> const &ops = graphs[k]->operators;
       while (cursor[k] < ops.size()) {
         KNOperator *op = ops[cursor[k]++];
         if (op->op_type == KN_INPUT_OP) {
           continue;
+        }
+        any = true;
+        if (op->op_type == KN_ADD_OP || op->op_type == KN_MUL_OP || op->op_type == KN_DIV_OP) {
+          DTensor const &a = op->input_tensors[0], &b = op->input_tensors[1],
+                        &o = op->output_tensors[0];
+          bool small = true;
+          for (int d = 0; d < o.num_dims; d++) {
+            small = small && o.dim[d] <= 65535;
+          }
+          if (!small || o.num_elements() > 0xffffffffull) {
+            op->fingerprint();  // beyond the batched form's index range
+            continue;
+          }
+          b_op[binaries] = op->op_type;
+          b_nd[binaries] = o.num_dims;
+          b_in1[binaries] = a.fp_ptr;
+          b_in2[binaries] = b.fp_ptr;
+          b_out[binaries] = o.fp_ptr;
+          for (int d = 0; d < 4; d++) {
+            b_d1[4 * binaries + d] = d < o.num_dims ? a.dim[d] : 1;
+            b_d2[4 * binaries + d] = d < o.num_dims ? b.dim[d] : 1;
+            b_od[4 * binaries + d] = d < o.num_dims ? o.dim[d] : 1;
+          }
+          if (++binaries == MI355_MAX_BINARY_OPS) {
+            flush_binaries();
+          }
+          break;
         }
         if (op->op_type != KN_CUSTOMIZED_OP) {
           op->fingerprint();
@@ -163,10 +203,13 @@ static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint6
         break;
       }
     }
-    if (plans.empty()) {
+    flush_binaries();
+    if (!plans.empty()) {
+      MI355_CALL(mi355_customized_fp_batch(plans.data(), (int)plans.size(), ins.data(), outs.data()));
+    }
+    if (!any) {
       break;
     }
-    MI355_CALL(mi355_customized_fp_batch(plans.data(), (int)plans.size(), ins.data(), outs.data()));
   }
 }
 

@@ -165,6 +165,13 @@ int mi355_fp_unary(int op, uint16_t const *in, uint16_t *out, size_t n);
  * op = KN_ADD_OP / KN_MUL_OP / KN_DIV_OP (1008 / 1009 / 1010) */
 int mi355_fp_binary(int op, uint16_t const *in1, int const *dims1, uint16_t const *in2,
                     int const *dims2, uint16_t *out, int const *dims_out, int num_dims);
+/* `count` <= MI355_MAX_BINARY_OPS independent operators of the kind above in one launch (a
+ * verification batch holds one per candidate): operator e uses ops[e], in1[e], in2[e], out[e],
+ * num_dims[e] and the dims at dims1 / dims2 / dims_out + 4 * e.  Every dim <= 65535. */
+#define MI355_MAX_BINARY_OPS 32
+int mi355_fp_binary_many(int const *ops, uint16_t const *const *in1, int const *dims1,
+                         uint16_t const *const *in2, int const *dims2, uint16_t *const *out,
+                         int const *dims_out, int const *num_dims, int count);
 /* compute_reduction_fingerprint, src/kernel/cuda/reduction_kernel.cu:80-133 */
 int mi355_fp_reduce(uint16_t const *in, uint16_t *out, size_t n_out, int factor,
                     int in_stride, int out_stride);

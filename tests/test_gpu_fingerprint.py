@@ -204,6 +204,49 @@ def test_many_fills_and_many_compares_in_one_launch(rt, abi):
         g.close()
 
 
+def test_many_binary_operators_in_one_launch(rt, abi):
+    """mi355_fp_binary_many over 30 add / mul / div operators of unlike shapes, with operands
+    broadcast along any axis, = the oracle's element-wise result of each."""
+    shapes = [((3, 70, 33), (3, 70, 33)), ((2, 64, 96), (2, 64, 1)), ((2, 64, 96), (2, 1, 96)),
+              ((1, 1, 257), (4, 5, 257)), ((1000,), (1000,)), ((16, 1), (16, 4096)),
+              ((2, 3, 5, 7), (2, 1, 5, 1)), ((1, 512, 512), (1, 512, 512)), ((7, 1), (1, 9)),
+              ((1,), (1,))]
+    names, codes = ["add", "mul", "div"], [1008, 1009, 1010]
+    cases = [(shapes[i % len(shapes)], i % 3) for i in range(30)]
+    spec = []
+    for (sa, sb), _ in cases:
+        so = list(np.broadcast_shapes(sa, sb))
+        spec += [{"op": "input", "dims": list(sa)}, {"op": "input", "dims": list(sb)},
+                 {"op": "input", "dims": so}]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        n = len(cases)
+        want = []
+        for i, ((sa, sb), which) in enumerate(cases):
+            A, B = uniform_fp(sa, 500 + i), uniform_fp(sb, 700 + i)
+            vals[3 * i][0].write_fingerprint(A)
+            vals[3 * i + 1][0].write_fingerprint(B)
+            want.append(orc.fp_binary(names[which], A, B))
+        pad = lambda d: list(d) + [1] * (4 - len(d))
+        ops = (ctypes.c_int * n)(*[codes[w] for _, w in cases])
+        in1 = (ctypes.c_void_p * n)(*[vals[3 * i][0].device_ptr(True) for i in range(n)])
+        in2 = (ctypes.c_void_p * n)(*[vals[3 * i + 1][0].device_ptr(True) for i in range(n)])
+        out = (ctypes.c_void_p * n)(*[vals[3 * i + 2][0].device_ptr(True) for i in range(n)])
+        d1 = (ctypes.c_int * (4 * n))(*sum([pad(sa) for (sa, _), _ in cases], []))
+        d2 = (ctypes.c_int * (4 * n))(*sum([pad(sb) for (_, sb), _ in cases], []))
+        do = (ctypes.c_int * (4 * n))(*sum([pad(np.broadcast_shapes(sa, sb)) for (sa, sb), _ in cases], []))
+        nd = (ctypes.c_int * n)(*[len(sa) for (sa, _), _ in cases])
+        assert abi.mi355_fp_binary_many(ops, in1, d1, in2, d2, out, do, nd, n) == 0
+        for i in range(n):
+            assert np.array_equal(vals[3 * i + 2][0].read_fingerprint(), want[i]), cases[i]
+        # more operators than one launch takes, or a shape that does not broadcast: refused
+        assert abi.mi355_fp_binary_many(ops, in1, d1, in2, d2, out, do, nd, 33) != 0
+        d2[1] = 5
+        assert abi.mi355_fp_binary_many(ops, in1, d1, in2, d2, out, do, nd, n) != 0
+    finally:
+        g.close()
+
+
 def test_batched_customized_fingerprints_of_generated_candidates(rt, abi):
     """Many small, unlike customized ops (the generator's candidates, dims <= 256) through
     mi355_customized_fp_batch in one call = one mi355_customized_fp each, bit for bit."""
