@@ -92,6 +92,7 @@ ABI = {
     "mi355_fp_fill_many": (_ci, [_pvp, ctypes.POINTER(_sz), ctypes.POINTER(_u64), _ci, _ci]),
     "mi355_fp_matmul": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci]),
     "mi355_fp_unary": (_ci, [_ci, _vp, _vp, _sz]),
+    "mi355_fp_matmul_many": (_ci, [_pvp, _pvp, _pvp, _pi, _pi, _pi, _pi, _ci]),
     "mi355_fp_binary": (_ci, [_ci, _vp, _pi, _vp, _pi, _vp, _pi, _ci]),
     "mi355_fp_binary_many": (_ci, [_pi, _pvp, _pi, _pvp, _pi, _pvp, _pi, _pi, _ci]),
     "mi355_fp_reduce": (_ci, [_vp, _vp, _sz, _ci, _ci, _ci]),

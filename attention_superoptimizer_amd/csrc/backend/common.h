@@ -80,6 +80,12 @@ struct State {
   void *scratch() const {
     return scratch_base == nullptr ? nullptr : scratch_base + (size_t)tls_queue * scratch_bytes;
   }
+  // residue planes of the matrix-core fingerprint matmul (per queue, like scratch)
+  size_t planes_bytes = 0;
+  char *planes_base = nullptr;
+  char *planes() const {
+    return planes_base == nullptr ? nullptr : planes_base + (size_t)tls_queue * planes_bytes;
+  }
 };
 
 State &state();

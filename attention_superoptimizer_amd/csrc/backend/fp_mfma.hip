@@ -1,0 +1,476 @@
+// Fingerprint matmul on the matrix cores (reference src/kernel/cuda/matmul_kernel.cu:145-173
+// computes `r = (r + a*b) % 25651` per multiply-accumulate in one thread per output).
+//
+// (sum a*b) mod 25651 is fixed by its residues mod 227 and mod 113.  Every operand is first
+// split, once per matrix, into two planes of signed bytes: the residue mod 227 recentred to
+// [-113, 113] and the residue mod 113; A keeps its orientation [rows][k], B is transposed
+// to [columns][k], k padded with zeros to a multiple of 64.  Both operands of
+// v_mfma_i32_16x16x64_i8 then want the same thing: 16 consecutive k of one row per lane,
+// one 16-byte load.  Planes are stored in blocks of 16 rows x 16 k (plane[row / 16][k / 16]
+// [row % 16][16 bytes]), so the 64 loads of a wavefront's operand fetch are one contiguous
+// kilobyte and a strip of 16 rows is one stream along k.  A 16 x 16 x 64 step per residue is one matrix instruction; the int32
+// sums are exact (|sum| <= 113^2 * k, folded every 131072 k) and are recombined once per
+// output with the reference's CRT multipliers, so results are bit-identical.
+//
+// One submission takes many independent matmuls (the kernel-level matmuls of a batch of
+// candidate graphs): one launch splits all operands, one launch multiplies.  A workgroup
+// owns a 64 x 64 output tile (each wavefront a 32 x 32 quadrant over all of k) when its
+// matmul has enough tiles to matter, otherwise a 32 x 32 tile whose k range the four
+// wavefronts share, added up through LDS.
+#include "common.h"
+
+#include <algorithm>
+#include <vector>
+
+namespace mi355 {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxJobs = MI355_MAX_MATMULS;
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+// residue mod 227 as a signed byte congruent to it, residue mod 113 as it is
+__device__ __forceinline__ uint32_t byte_p(uint32_t x) {
+  uint32_t const r = x % FP_P;
+  return (r > 113u ? r + 29u : r) & 0xffu;  // r - 227 = r + 29 (mod 256)
+}
+__device__ __forceinline__ uint32_t byte_q(uint32_t x) { return x % FP_Q; }
+
+struct SplitJob {
+  uint16_t const *src;   // [slabs][rows][cols], row-major
+  int8_t *plane_p, *plane_q;
+  int slabs, rows, cols;
+  int kp;                // padded k of the planes
+  int rp;                // plane rows per slab (a multiple of 16)
+  int transpose;         // 0: plane rows = source rows, k = cols; 1: plane rows = source columns, k = rows
+  int vec;               // source rows may be read 8 (plain) / 4 (transposed) values at a time
+  unsigned first_block, blocks;
+};
+struct SplitMany {
+  SplitJob job[2 * kMaxJobs];
+  int count;
+};
+
+__global__ __launch_bounds__(kThreads) void fp_split_planes_kernel(SplitMany const S) {
+  __shared__ uint32_t tile[2][64][17];
+  int j = 0;
+  while (j + 1 < S.count && blockIdx.x >= S.job[j + 1].first_block) {
+    j++;
+  }
+  SplitJob const &J = S.job[j];
+  unsigned const block = blockIdx.x - J.first_block;
+  int const tid = threadIdx.x;
+  if (!J.transpose) {
+    // unit = 16 consecutive k of one plane row; the 16 rows of a block go to 16 neighbouring
+    // threads, which write one contiguous 256-byte block
+    int const chunks = J.kp / 16;
+    size_t const units = (size_t)J.slabs * J.rp * chunks;
+    for (size_t u = (size_t)block * kThreads + tid; u < units; u += (size_t)J.blocks * kThreads) {
+      int const r = (int)(u % 16);
+      size_t const blk = u / 16;                 // (slab, strip, chunk)
+      int const c = (int)(blk % chunks);
+      size_t const strip = blk / chunks;         // over slabs * rp / 16
+      int const slab = (int)(strip / (J.rp / 16));
+      int const row = (int)(strip % (J.rp / 16)) * 16 + r;
+      int const k0 = c * 16;
+      uint32_t v[16];
+      if (row < J.rows) {
+        uint16_t const *src = J.src + ((size_t)slab * J.rows + row) * J.cols + k0;
+        if (J.vec && k0 + 16 <= J.cols) {
+          uint4v const lo = *reinterpret_cast<uint4v const *>(src);
+          uint4v const hi = *reinterpret_cast<uint4v const *>(src + 8);
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            v[2 * i] = lo[i] & 0xffffu;
+            v[2 * i + 1] = lo[i] >> 16;
+            v[8 + 2 * i] = hi[i] & 0xffffu;
+            v[8 + 2 * i + 1] = hi[i] >> 16;
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            v[i] = k0 + i < J.cols ? src[i] : 0u;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          v[i] = 0u;
+        }
+      }
+      uint4v p, q;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        p[w] = byte_p(v[4 * w]) | (byte_p(v[4 * w + 1]) << 8) | (byte_p(v[4 * w + 2]) << 16) |
+               (byte_p(v[4 * w + 3]) << 24);
+        q[w] = byte_q(v[4 * w]) | (byte_q(v[4 * w + 1]) << 8) | (byte_q(v[4 * w + 2]) << 16) |
+               (byte_q(v[4 * w + 3]) << 24);
+      }
+      *reinterpret_cast<uint4v *>(J.plane_p + u * 16) = p;  // u = ((strip * chunks + c) * 16 + r)
+      *reinterpret_cast<uint4v *>(J.plane_q + u * 16) = q;
+    }
+    return;
+  }
+  // transposed: tiles of 64 k (source rows) x 64 n (source columns) through LDS
+  int const tiles_k = J.kp / 64, tiles_n = (J.cols + 63) / 64;
+  int const tiles = J.slabs * tiles_k * tiles_n;
+  int const kq = tid / 16, ng = tid % 16;      // patch read: k = 4 kq .. +3, n = 4 ng .. +3
+  int const out_n = tid % 64, out_c = tid / 64;  // chunk written: row out_n, k = 16 out_c .. +15
+  for (int t = block; t < tiles; t += J.blocks) {
+    int const slab = t / (tiles_k * tiles_n);
+    int const k0 = (t / tiles_n) % tiles_k * 64, n0 = (t % tiles_n) * 64;
+    uint16_t const *src = J.src + (size_t)slab * J.rows * J.cols;
+    uint32_t v[4][4];  // [k][n]
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      int const k = k0 + 4 * kq + r, n = n0 + 4 * ng;
+      if (J.vec && k < J.rows && n + 4 <= J.cols) {
+        uint2 const w = *reinterpret_cast<uint2 const *>(src + (size_t)k * J.cols + n);
+        v[r][0] = w.x & 0xffffu;
+        v[r][1] = w.x >> 16;
+        v[r][2] = w.y & 0xffffu;
+        v[r][3] = w.y >> 16;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          v[r][c] = (k < J.rows && n + c < J.cols) ? src[(size_t)k * J.cols + n + c] : 0u;
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      tile[0][4 * ng + c][kq] = byte_p(v[0][c]) | (byte_p(v[1][c]) << 8) | (byte_p(v[2][c]) << 16) |
+                                (byte_p(v[3][c]) << 24);
+      tile[1][4 * ng + c][kq] = byte_q(v[0][c]) | (byte_q(v[1][c]) << 8) | (byte_q(v[2][c]) << 16) |
+                                (byte_q(v[3][c]) << 24);
+    }
+    __syncthreads();
+    if (n0 + out_n < J.rp) {  // rows past the last column hold zeros
+      size_t const strip = (size_t)slab * (J.rp / 16) + (n0 + out_n) / 16;
+      size_t const at = ((strip * (J.kp / 16) + k0 / 16 + out_c) * 16 + out_n % 16) * 16;
+      uint4v p, q;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        p[w] = tile[0][out_n][4 * out_c + w];
+        q[w] = tile[1][out_n][4 * out_c + w];
+      }
+      *reinterpret_cast<uint4v *>(J.plane_p + at) = p;
+      *reinterpret_cast<uint4v *>(J.plane_q + at) = q;
+    }
+    __syncthreads();
+  }
+}
+
+struct GemmJob {
+  int8_t const *a_p, *a_q;    // blocked planes, mp rows per batch
+  int8_t const *bt_p, *bt_q;  // blocked planes, np rows per batch
+  uint16_t *out;              // [batch][m][n]
+  int batch, m, n, kp;
+  int mp, np;                 // m, n rounded up to 16
+  int shared_k;               // 1: 32 x 32 tile per workgroup, wavefronts share k
+  int tiles_m, tiles_n;
+  unsigned first_block;
+};
+struct GemmMany {
+  GemmJob job[kMaxJobs];
+  int count;
+};
+
+__device__ __forceinline__ int fold_signed(int v, int mod) { return v % mod; }
+
+__global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const G) {
+  __shared__ int part[4][32][64];  // shared-k reduction: [wavefront][register][lane]
+  int j = 0;
+  while (j + 1 < G.count && blockIdx.x >= G.job[j + 1].first_block) {
+    j++;
+  }
+  GemmJob const &J = G.job[j];
+  int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
+  unsigned t = blockIdx.x - J.first_block;
+  int const per_batch = J.tiles_m * J.tiles_n;
+  int const b = (int)(t / per_batch);
+  t %= per_batch;
+  int const steps = J.kp / 64;
+  int row0, col0, s_begin, s_end;
+  if (J.shared_k) {
+    row0 = (int)(t / J.tiles_n) * 32;
+    col0 = (int)(t % J.tiles_n) * 32;
+    s_begin = (int)((long long)steps * wave / 4);
+    s_end = (int)((long long)steps * (wave + 1) / 4);
+  } else {
+    row0 = (int)(t / J.tiles_n) * 64 + (wave / 2) * 32;
+    col0 = (int)(t % J.tiles_n) * 64 + (wave % 2) * 32;
+    s_begin = 0;
+    s_end = steps;
+  }
+  // a strip past the edge reads the last strip; its results are not stored
+  size_t a_off[2], b_off[2];
+  size_t const strip_bytes = (size_t)J.kp * 16;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    size_t const sa = ((size_t)b * J.mp + min(row0 + 16 * i, J.mp - 16)) / 16;
+    size_t const sb = ((size_t)b * J.np + min(col0 + 16 * i, J.np - 16)) / 16;
+    a_off[i] = sa * strip_bytes + g * 256 + r * 16;
+    b_off[i] = sb * strip_bytes + g * 256 + r * 16;
+  }
+  // acc[res][i][jn]: rows of the MFMA result are columns of C (B^T is the first operand), so a
+  // lane ends up with four consecutive columns of one row of C
+  v4i acc[2][2][2];
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
+  }
+  v4i ap[2], aq[2], bp[2], bq[2];
+  auto fetch = [&](int s) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      ap[i] = *reinterpret_cast<v4i const *>(J.a_p + a_off[i] + (size_t)s * 1024);
+      aq[i] = *reinterpret_cast<v4i const *>(J.a_q + a_off[i] + (size_t)s * 1024);
+      bp[i] = *reinterpret_cast<v4i const *>(J.bt_p + b_off[i] + (size_t)s * 1024);
+      bq[i] = *reinterpret_cast<v4i const *>(J.bt_q + b_off[i] + (size_t)s * 1024);
+    }
+  };
+  if (s_begin < s_end) {
+    fetch(s_begin);
+  }
+  for (int s = s_begin; s < s_end; s++) {
+    v4i cap[2] = {ap[0], ap[1]}, caq[2] = {aq[0], aq[1]}, cbp[2] = {bp[0], bp[1]}, cbq[2] = {bq[0], bq[1]};
+    if (s + 1 < s_end) {
+      fetch(s + 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+      for (int jn = 0; jn < 2; jn++) {
+        acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbp[jn], cap[i], acc[0][i][jn], 0, 0, 0);
+        acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbq[jn], caq[i], acc[1][i][jn], 0, 0, 0);
+      }
+    }
+    if (((s - s_begin) & 2047) == 2047) {  // 2048 steps x 64 k x 113^2 < 2^31
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int jn = 0; jn < 2; jn++) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            acc[0][i][jn][e] = fold_signed(acc[0][i][jn][e], (int)FP_P);
+            acc[1][i][jn][e] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
+          }
+        }
+      }
+    }
+  }
+  uint16_t *out = J.out + (size_t)b * J.m * J.n;
+  bool const whole4 = J.n % 4 == 0;
+  auto store = [&](int i, int jn, v4i const &sp, v4i const &sq) {
+    int const row = row0 + 16 * i + r, col = col0 + 16 * jn + 4 * g;
+    if (row >= J.m || col >= J.n) {
+      return;
+    }
+    uint32_t z[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      int const rp = (sp[e] % (int)FP_P + (int)FP_P) % (int)FP_P;
+      int const rq = (sq[e] % (int)FP_Q + (int)FP_Q) % (int)FP_Q;
+      z[e] = ((uint32_t)rp * FP_Q_MUL_P_MOD_1 + (uint32_t)rq * FP_P_MUL_Q_MOD_1) % FP_PQ;
+    }
+    uint16_t *dst = out + (size_t)row * J.n + col;
+    if (whole4 && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+      uint2 w;
+      w.x = z[0] | (z[1] << 16);
+      w.y = z[2] | (z[3] << 16);
+      *reinterpret_cast<uint2 *>(dst) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (col + e < J.n) {
+          dst[e] = (uint16_t)z[e];
+        }
+      }
+    }
+  };
+  if (!J.shared_k) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+      for (int jn = 0; jn < 2; jn++) {
+        store(i, jn, acc[0][i][jn], acc[1][i][jn]);
+      }
+    }
+    return;
+  }
+  // shared k: every wavefront leaves its folded sums, wavefront w finishes sub-tile w
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+#pragma unroll
+    for (int jn = 0; jn < 2; jn++) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        part[wave][(i * 2 + jn) * 8 + e][lane] = fold_signed(acc[0][i][jn][e], (int)FP_P);
+        part[wave][(i * 2 + jn) * 8 + 4 + e][lane] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
+      }
+    }
+  }
+  __syncthreads();
+  v4i sp = {0, 0, 0, 0}, sq = {0, 0, 0, 0};
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      sp[e] += part[w][wave * 8 + e][lane];
+      sq[e] += part[w][wave * 8 + 4 + e][lane];
+    }
+  }
+  store(wave / 2, wave % 2, sp, sq);
+}
+
+inline size_t round_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
+
+}  // namespace
+
+// Whether one matmul can take the matrix-core path, and the bytes of planes it needs.
+static bool mfma_matmul_fits(int batch, int m, int n, int k, size_t *plane_bytes) {
+  if (batch <= 0 || m <= 0 || n <= 0 || k <= 0) {
+    return false;
+  }
+  size_t const kp = round_up((size_t)k, 64);
+  size_t const rows = (size_t)batch * (round_up((size_t)m, 16) + round_up((size_t)n, 16));
+  if (rows * kp > ((size_t)1 << 31)) {
+    return false;
+  }
+  *plane_bytes = 2 * rows * kp;  // two residues; every plane is a multiple of 64 bytes
+  return true;
+}
+
+// Enqueues matmuls [0, count) whose planes fit the queue's plane memory together.
+static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B, uint16_t *const *C,
+                             int const *batch, int const *m, int const *n, int const *k, int count) {
+  SplitMany S{};
+  GemmMany G{};
+  char *planes = state().planes();
+  size_t used = 0;
+  unsigned split_blocks = 0, gemm_blocks = 0;
+  for (int e = 0; e < count; e++) {
+    int const kp = (int)round_up((size_t)k[e], 64);
+    int const mp = (int)round_up((size_t)m[e], 16), np = (int)round_up((size_t)n[e], 16);
+    size_t const a_plane = (size_t)batch[e] * mp * kp, b_plane = (size_t)batch[e] * np * kp;
+    int8_t *a_p = reinterpret_cast<int8_t *>(planes + used);
+    int8_t *a_q = a_p + a_plane;
+    int8_t *bt_p = a_q + a_plane;
+    int8_t *bt_q = bt_p + b_plane;
+    used += 2 * (a_plane + b_plane);
+    SplitJob &sa = S.job[2 * e], &sb = S.job[2 * e + 1];
+    sa.src = A[e];
+    sa.plane_p = a_p;
+    sa.plane_q = a_q;
+    sa.slabs = batch[e];
+    sa.rows = m[e];
+    sa.cols = k[e];
+    sa.kp = kp;
+    sa.rp = mp;
+    sa.transpose = 0;
+    sa.vec = k[e] % 8 == 0 && (reinterpret_cast<uintptr_t>(A[e]) & 15) == 0;
+    size_t const a_units = (size_t)batch[e] * mp * (kp / 16);
+    sa.blocks = (unsigned)std::min<size_t>((a_units + kThreads - 1) / kThreads, 1024);
+    sa.first_block = split_blocks;
+    split_blocks += sa.blocks;
+    sb.src = B[e];
+    sb.plane_p = bt_p;
+    sb.plane_q = bt_q;
+    sb.slabs = batch[e];
+    sb.rows = k[e];
+    sb.cols = n[e];
+    sb.kp = kp;
+    sb.rp = np;
+    sb.transpose = 1;
+    sb.vec = n[e] % 4 == 0 && (reinterpret_cast<uintptr_t>(B[e]) & 7) == 0;
+    size_t const b_tiles = (size_t)batch[e] * (kp / 64) * ((n[e] + 63) / 64);
+    sb.blocks = (unsigned)std::min<size_t>(b_tiles, 1024);
+    sb.first_block = split_blocks;
+    split_blocks += sb.blocks;
+    GemmJob &g = G.job[e];
+    g.a_p = a_p;
+    g.a_q = a_q;
+    g.bt_p = bt_p;
+    g.bt_q = bt_q;
+    g.out = C[e];
+    g.batch = batch[e];
+    g.m = m[e];
+    g.n = n[e];
+    g.kp = kp;
+    g.mp = mp;
+    g.np = np;
+    long long const big_tiles = (long long)((m[e] + 63) / 64) * ((n[e] + 63) / 64) * batch[e];
+    g.shared_k = big_tiles < 64;
+    int const edge = g.shared_k ? 32 : 64;
+    g.tiles_m = (m[e] + edge - 1) / edge;
+    g.tiles_n = (n[e] + edge - 1) / edge;
+    g.first_block = gemm_blocks;
+    gemm_blocks += (unsigned)((long long)g.tiles_m * g.tiles_n * batch[e]);
+  }
+  S.count = 2 * count;
+  G.count = count;
+  hipStream_t st = state().stream();
+  fp_split_planes_kernel<<<split_blocks, kThreads, 0, st>>>(S);
+  MI355_HIP(hipGetLastError());
+  fp_mfma_matmul_kernel<<<gemm_blocks, kThreads, 0, st>>>(G);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m,
+                               int n, int k);
+
+extern "C" int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *const *B,
+                                    uint16_t *const *C, int const *batch, int const *m,
+                                    int const *n, int const *k, int count) {
+  MI355_REQUIRE_INIT();
+  if (count < 0 || (count > 0 && (A == nullptr || B == nullptr || C == nullptr || batch == nullptr ||
+                                  m == nullptr || n == nullptr || k == nullptr))) {
+    return fail(MI355_ERR_INVALID, "bad matmul list (count %d)", count);
+  }
+  for (int e = 0; e < count; e++) {
+    if (batch[e] < 0 || m[e] < 0 || n[e] < 0 || k[e] < 0) {
+      return fail(MI355_ERR_INVALID, "matmul %d: negative extent", e);
+    }
+    bool const any_output = (long long)batch[e] * m[e] * n[e] > 0;
+    if (any_output && (C[e] == nullptr || (k[e] > 0 && (A[e] == nullptr || B[e] == nullptr)))) {
+      return fail(MI355_ERR_INVALID, "matmul %d: null matrix", e);
+    }
+  }
+  // consecutive matmuls whose planes fit the queue's plane memory go out together; one that
+  // cannot take this path at all (no k, planes too large) goes through the single entry point
+  int begin = 0;
+  while (begin < count) {
+    size_t need = 0;
+    if (!mfma_matmul_fits(batch[begin], m[begin], n[begin], k[begin], &need) ||
+        need > state().planes_bytes) {
+      if (int rc = mi355_fp_matmul(A[begin], B[begin], C[begin], batch[begin], m[begin], n[begin], k[begin])) {
+        return rc;
+      }
+      begin++;
+      continue;
+    }
+    int end = begin + 1;
+    size_t total = need;
+    while (end < count && end - begin < kMaxJobs) {
+      size_t more = 0;
+      if (!mfma_matmul_fits(batch[end], m[end], n[end], k[end], &more) ||
+          total + more > state().planes_bytes) {
+        break;
+      }
+      total += more;
+      end++;
+    }
+    if (int rc = launch_mfma_group(A + begin, B + begin, C + begin, batch + begin, m + begin,
+                                   n + begin, k + begin, end - begin)) {
+      return rc;
+    }
+    begin = end;
+  }
+  return MI355_OK;
+}
+
+}  // namespace mi355

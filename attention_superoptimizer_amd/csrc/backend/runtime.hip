@@ -127,6 +127,9 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
   s.scratch_bytes = (size_t)64 << 20;  // per queue
   MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.scratch_base),
                       s.scratch_bytes * MI355_NUM_QUEUES));
+  s.planes_bytes = (size_t)128 << 20;  // per queue
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.planes_base),
+                      s.planes_bytes * MI355_NUM_QUEUES));
   s.ready = true;
   if (arena_base != nullptr) {
     *arena_base = s.arena;
@@ -151,6 +154,8 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipFree(s.cmp_slots));
   MI355_HIP(hipHostFree(s.cmp_host));
   MI355_HIP(hipFree(s.scratch_base));
+  MI355_HIP(hipFree(s.planes_base));
+  s.planes_base = nullptr;
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     for (int b = 0; b < State::kBatchSlots; b++) {
       MI355_HIP(hipHostFree(s.batch[q][b].host));

@@ -122,9 +122,9 @@ void fingerprint_graph(kernel::Graph const &g, uint64_t input_seed, VerifyStats 
 }
 
 // Fingerprints several independent graphs on the calling thread's queue, round by round.
-// In a round every graph advances through its kernel-level matmuls, unary operators and
-// reductions (enqueued one by one) up to its next element-wise binary or customized
-// operator; those are collected and submitted together (mi355_fp_binary_many,
+// In a round every graph advances through its unary operators and reductions (enqueued
+// one by one) up to its next matmul, element-wise binary or customized operator; those
+// are collected and submitted together (mi355_fp_matmul_many, mi355_fp_binary_many,
 // mi355_customized_fp_batch: a handful of launches for all of them).  The queue is in
 // order, so an operator's producers are always ahead of it.
 static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint64_t input_seed,
@@ -144,6 +144,16 @@ static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint6
   uint16_t const *b_in1[MI355_MAX_BINARY_OPS], *b_in2[MI355_MAX_BINARY_OPS];
   uint16_t *b_out[MI355_MAX_BINARY_OPS];
   int b_d1[4 * MI355_MAX_BINARY_OPS], b_d2[4 * MI355_MAX_BINARY_OPS], b_od[4 * MI355_MAX_BINARY_OPS];
+  uint16_t const *m_a[MI355_MAX_MATMULS], *m_b[MI355_MAX_MATMULS];
+  uint16_t *m_c[MI355_MAX_MATMULS];
+  int m_batch[MI355_MAX_MATMULS], m_m[MI355_MAX_MATMULS], m_n[MI355_MAX_MATMULS], m_k[MI355_MAX_MATMULS];
+  int matmuls = 0;
+  auto flush_matmuls = [&]() {
+    if (matmuls > 0) {
+      MI355_CALL(mi355_fp_matmul_many(m_a, m_b, m_c, m_batch, m_m, m_n, m_k, matmuls));
+      matmuls = 0;
+    }
+  };
   int binaries = 0;
   auto flush_binaries = [&]() {
     if (binaries > 0) {
@@ -164,6 +174,25 @@ static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint6
           continue;
         }
         any = true;
+        if (op->op_type == KN_MATMUL_OP) {
+          DTensor const &a = op->input_tensors[0], &b = op->input_tensors[1];
+          int const nd = a.num_dims;
+          int batch = 1;
+          for (int d = 0; d < nd - 2; d++) {
+            batch *= a.dim[d];
+          }
+          m_a[matmuls] = a.fp_ptr;
+          m_b[matmuls] = b.fp_ptr;
+          m_c[matmuls] = op->output_tensors[0].fp_ptr;
+          m_batch[matmuls] = batch;
+          m_m[matmuls] = a.dim[nd - 2];
+          m_k[matmuls] = a.dim[nd - 1];
+          m_n[matmuls] = b.dim[nd - 1];
+          if (++matmuls == MI355_MAX_MATMULS) {
+            flush_matmuls();
+          }
+          break;
+        }
         if (op->op_type == KN_ADD_OP || op->op_type == KN_MUL_OP || op->op_type == KN_DIV_OP) {
           DTensor const &a = op->input_tensors[0], &b = op->input_tensors[1],
                         &o = op->output_tensors[0];
@@ -203,6 +232,7 @@ static void fingerprint_graphs(std::vector<kernel::Graph *> const &graphs, uint6
         break;
       }
     }
+    flush_matmuls();
     flush_binaries();
     if (!plans.empty()) {
       MI355_CALL(mi355_customized_fp_batch(plans.data(), (int)plans.size(), ins.data(), outs.data()));

@@ -158,6 +158,15 @@ int mi355_fp_fill_many(uint16_t *const *fp, size_t const *n, uint64_t const *see
 /* compute_matmul_fingerprint, src/kernel/cuda/matmul_kernel.cu:145-203 */
 int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m,
                     int n, int k);
+/* Several independent matmuls in one submission (compute_matmul_fingerprint once per
+ * operator in the reference, matmul_kernel.cu:175-203): C[i] = A[i] . B[i] with extents
+ * batch[i], m[i], n[i], k[i], bit-identical to mi355_fp_matmul of each.  Operands are split
+ * once into signed-byte residue planes (mod 227 recentred, mod 113) in backend memory and
+ * multiplied with int8 matrix instructions; up to MI355_MAX_MATMULS go out as two launches,
+ * longer lists in groups.  Outputs must not alias inputs of the same call. */
+#define MI355_MAX_MATMULS 32
+int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *const *B, uint16_t *const *C,
+                         int const *batch, int const *m, int const *n, int const *k, int count);
 /* compute_elementunary_fingerprint, src/kernel/cuda/element_unary_kernel.cu:77-112;
  * op = KN_EXP_OP (1007) or the silu extension (1011) */
 int mi355_fp_unary(int op, uint16_t const *in, uint16_t *out, size_t n);

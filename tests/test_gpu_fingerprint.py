@@ -204,6 +204,60 @@ def test_many_fills_and_many_compares_in_one_launch(rt, abi):
         g.close()
 
 
+def _matmul_many(abi, rt, shapes, fill):
+    """Runs mi355_fp_matmul_many over (batch, m, n, k) shapes; returns inputs and outputs."""
+    spec = []
+    for b, m, n, k in shapes:
+        spec += [{"op": "input", "dims": [b, m, k]}, {"op": "input", "dims": [b, k, n]},
+                 {"op": "input", "dims": [b, m, n]}]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        cnt = len(shapes)
+        ins = []
+        for i, (b, m, n, k) in enumerate(shapes):
+            A, B = fill(i, (b, m, k)), fill(100 + i, (b, k, n))
+            vals[3 * i][0].write_fingerprint(A)
+            vals[3 * i + 1][0].write_fingerprint(B)
+            vals[3 * i + 2][0].write_fingerprint(np.full((b, m, n), 7, np.uint16))
+            ins.append((A, B))
+        pa = (ctypes.c_void_p * cnt)(*[vals[3 * i][0].device_ptr(True) for i in range(cnt)])
+        pb = (ctypes.c_void_p * cnt)(*[vals[3 * i + 1][0].device_ptr(True) for i in range(cnt)])
+        pc = (ctypes.c_void_p * cnt)(*[vals[3 * i + 2][0].device_ptr(True) for i in range(cnt)])
+        arr = lambda j: (ctypes.c_int * cnt)(*[s[j] for s in shapes])
+        assert abi.mi355_fp_matmul_many(pa, pb, pc, arr(0), arr(1), arr(2), arr(3), cnt) == 0
+        return ins, [vals[3 * i + 2][0].read_fingerprint() for i in range(cnt)]
+    finally:
+        g.close()
+
+
+def test_many_matmuls_on_the_matrix_cores_match_oracle(rt, abi):
+    """mi355_fp_matmul_many (signed-byte residue planes, int8 matrix instructions) over ragged,
+    batched, tiny and large shapes = the oracle's `(r + a*b) % 25651` chains, bit for bit; more
+    matmuls than one group takes; both workgroup shapes (64x64 tiles, and 32x32 tiles whose
+    wavefronts share k)."""
+    shapes = [(1, 16, 64, 48), (3, 70, 33, 129), (2, 256, 64, 4096), (1, 5, 7, 3), (1, 130, 200, 72),
+              (3, 64, 128, 64), (1, 192, 320, 448), (1, 1024, 1024, 256), (1, 1, 1, 1),
+              (4, 512, 512, 64), (1, 64, 1024, 1024), (1, 33, 65, 4100)]
+    shapes = shapes + [(1, 16 + 16 * (i % 5), 32 + 8 * i, 64 + 24 * i) for i in range(28)]
+    ins, got = _matmul_many(abi, rt, shapes, lambda i, d: uniform_fp(d, 60 + i))
+    for (A, B), C, s in zip(ins, got, shapes):
+        assert np.array_equal(C, orc.fp_matmul(A, B)), s
+
+
+def test_matrix_core_matmul_extreme_values_and_long_k(rt, abi):
+    """Operands whose residues are the largest in magnitude the planes hold (-113 mod 227,
+    112 mod 113), k long enough that a wavefront's int32 sums must be folded on the way."""
+    x = (114 * 25425 + 112 * 227) % FP_PQ       # = -113 (mod 227), 112 (mod 113)
+    y = (113 * 25425 + 112 * 227) % FP_PQ       # = +113 (mod 227)
+    assert x % 227 == 114 and y % 227 == 113 and x % 113 == 112
+    shapes = [(1, 16, 16, 800000), (1, 48, 32, 70000), (2, 128, 192, 1024)]
+    for a, b in ((x, x), (x, y), (FP_PQ - 1, FP_PQ - 1)):
+        fill = lambda i, d: np.full(d, a if i < 100 else b, np.uint16)
+        _, got = _matmul_many(abi, rt, shapes, fill)
+        for C, (_, m, n, k) in zip(got, shapes):
+            assert np.all(C == (k * a * b) % FP_PQ), (a, b, k)
+
+
 def test_many_binary_operators_in_one_launch(rt, abi):
     """mi355_fp_binary_many over 30 add / mul / div operators of unlike shapes, with operands
     broadcast along any axis, = the oracle's element-wise result of each."""
