@@ -72,6 +72,7 @@ struct State {
   mi355_launch_info last_launch{};
   int force_interpreter = 0;
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
+  int fp_vector_dot_only = 0;  // 1: fingerprint matmuls never take the matrix-core kernels
   int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
   // fused-kernel workspace: fp16 range sums of split for-loops
   // (each queue has its own slice of scratch_base, so concurrent queues never share)
@@ -89,6 +90,12 @@ struct State {
 };
 
 State &state();
+
+// Matrix-core fingerprint matmul (fp_mfma.hip): whether a single matmul is large enough to
+// repay the extra launch that splits its operands into residue planes, and its launch.
+bool mfma_matmul_pays(int batch, int m, int n, int k);
+int launch_mfma_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m, int n,
+                       int k);
 int sync_all_queues();
 int fail(int code, char const *fmt, ...);
 

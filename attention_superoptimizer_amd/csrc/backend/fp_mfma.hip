@@ -18,6 +18,7 @@
 // matmul has enough tiles to matter, otherwise a 32 x 32 tile whose k range the four
 // wavefronts share, added up through LDS.
 #include "common.h"
+#include "tb_program.h"
 
 #include <algorithm>
 #include <vector>
@@ -326,6 +327,211 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
   store(wave / 2, wave % 2, sp, sq);
 }
 
+// ---- fused tiled-matmul plans (load A tile, load B tile, matmul, accumulate, store) -------
+// One workgroup: logical block (bx, by, bz), part `split` of the for-loop.  The for-loop's
+// k tiles, 16 k at a time, form one sequence of chunks; a matrix instruction takes four
+// of them (one per 16-lane group), so tiles of 16 or 32 k pair up across iterations.  Tile
+// origins come from the plan's own strides, as byte strides into the blocked planes.  A
+// wavefront owns 32 x 32 outputs at a time; a tile with fewer than three such pieces shares
+// its chunk sequence between wavefronts and adds their sums through `part`.
+__device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *part, int bx, int by,
+                                                   int bz, int split) {
+  DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]], &so = P.ops[3];
+  int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
+  int const cpi = kt / 16;  // chunks per iteration
+  int const F = P.forloop_range;
+  int const it_begin = (int)((long long)F * split / P.splits);
+  int const it_end = (int)((long long)F * (split + 1) / P.splits);
+  int const Q = (it_end - it_begin) * cpi, steps = (Q + 3) / 4;
+  int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
+  int const a0 = bx * P.pl_a[0] + by * P.pl_a[1] + bz * P.pl_a[2] + it_begin * P.pl_a[3];
+  int const b0 = bx * P.pl_b[0] + by * P.pl_b[1] + bz * P.pl_b[2] + it_begin * P.pl_b[3];
+  int const a_it = P.pl_a[3], b_it = P.pl_b[3];
+  int const dq_it = 4 / cpi, dq_c = 4 % cpi;
+  int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
+  int const ways = mt >= 3 ? 1 : (mt == 2 ? 2 : 4);  // wavefronts sharing one piece's chunks
+  uint16_t *gout = (P.splits > 1 ? P.part[so.io] + (long long)split * P.part_stride[so.io]
+                                 : static_cast<uint16_t *>(P.out[so.io]));
+  {
+    int const row0 = bx * so.row_bs[0] + by * so.row_bs[1] + bz * so.row_bs[2];
+    int const col0 = bx * so.col_bs[0] + by * so.col_bs[1] + bz * so.col_bs[2];
+    long long const base = (long long)bx * so.g_bs[0] + (long long)by * so.g_bs[1] +
+                           (long long)bz * so.g_bs[2];
+    gout += base + (long long)row0 * so.d_cols + col0;
+  }
+  int8_t const *const pa = P.pl[0], *const qa = P.pl[1], *const pb = P.pl[2], *const qb = P.pl[3];
+  for (int t = ways == 1 ? wave : wave / ways; t < mt; t += 4) {
+    int const ks = ways == 1 ? 0 : wave % ways;
+    int const s_begin = (int)((long long)steps * ks / ways);
+    int const s_end = (int)((long long)steps * (ks + 1) / ways);
+    int const row_m = (t / mt_n) * 32, col_n = (t % mt_n) * 32;
+    int const i1 = row_m + 16 < m ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
+    int a_base[2], b_base[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      a_base[i] = a0 + (row_m / 16 + (i ? i1 : 0)) * P.pl_a[4] + r * 16;
+      b_base[i] = b0 + (col_n / 16 + (i ? j1 : 0)) * P.pl_b[4] + r * 16;
+    }
+    // this lane's chunk of step s: number 4 s + g of the sequence
+    int q = 4 * s_begin + g;
+    int itr = q / cpi, c = q - itr * cpi;
+    v4i ap[2], aq[2], bp[2], bq[2];
+    auto fetch = [&]() {
+      bool const valid = q < Q;
+      int const oa = itr * a_it + c * 256, ob = itr * b_it + c * 256;
+      v4i const zero = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        ap[i] = valid ? *reinterpret_cast<v4i const *>(pa + a_base[i] + oa) : zero;
+        aq[i] = valid ? *reinterpret_cast<v4i const *>(qa + a_base[i] + oa) : zero;
+        bp[i] = valid ? *reinterpret_cast<v4i const *>(pb + b_base[i] + ob) : zero;
+        bq[i] = valid ? *reinterpret_cast<v4i const *>(qb + b_base[i] + ob) : zero;
+      }
+      q += 4;
+      itr += dq_it;
+      c += dq_c;
+      if (c >= cpi) {
+        c -= cpi;
+        itr++;
+      }
+    };
+    v4i acc[2][2][2];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
+    }
+    if (s_begin < s_end) {
+      fetch();
+    }
+    for (int s = s_begin; s < s_end; s++) {
+      v4i cap[2] = {ap[0], ap[1]}, caq[2] = {aq[0], aq[1]}, cbp[2] = {bp[0], bp[1]}, cbq[2] = {bq[0], bq[1]};
+      if (s + 1 < s_end) {
+        fetch();
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int jn = 0; jn < 2; jn++) {
+          acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbp[jn], cap[i], acc[0][i][jn], 0, 0, 0);
+          acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbq[jn], caq[i], acc[1][i][jn], 0, 0, 0);
+        }
+      }
+      if (((s - s_begin) & 2047) == 2047) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+          for (int jn = 0; jn < 2; jn++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              acc[0][i][jn][e] = fold_signed(acc[0][i][jn][e], (int)FP_P);
+              acc[1][i][jn][e] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
+            }
+          }
+        }
+      }
+    }
+    auto store = [&](int i, int jn, v4i const &sp, v4i const &sq) {
+      if (i > i1 || jn > j1) {
+        return;
+      }
+      uint32_t z[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        int const rp = (sp[e] % (int)FP_P + (int)FP_P) % (int)FP_P;
+        int const rq = (sq[e] % (int)FP_Q + (int)FP_Q) % (int)FP_Q;
+        z[e] = ((uint32_t)rp * FP_Q_MUL_P_MOD_1 + (uint32_t)rq * FP_P_MUL_Q_MOD_1) % FP_PQ;
+      }
+      uint2 w;
+      w.x = z[0] | (z[1] << 16);
+      w.y = z[2] | (z[3] << 16);
+      *reinterpret_cast<uint2 *>(gout + (long long)(row_m + 16 * i + r) * so.d_cols + col_n + 16 * jn +
+                                 4 * g) = w;
+    };
+    if (ways == 1) {
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int jn = 0; jn < 2; jn++) {
+          store(i, jn, acc[0][i][jn], acc[1][i][jn]);
+        }
+      }
+      continue;
+    }
+    // shared chunk sequence: every wavefront but the piece's first leaves its folded sums
+    if (ks != 0) {
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int jn = 0; jn < 2; jn++) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            part[(wave * 32 + (i * 2 + jn) * 8 + e) * 64 + lane] = fold_signed(acc[0][i][jn][e], (int)FP_P);
+            part[(wave * 32 + (i * 2 + jn) * 8 + 4 + e) * 64 + lane] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (ks == 0) {
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int jn = 0; jn < 2; jn++) {
+          v4i sp, sq;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            sp[e] = fold_signed(acc[0][i][jn][e], (int)FP_P);
+            sq[e] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
+          }
+          for (int w = 1; w < ways; w++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              sp[e] += part[((wave + w) * 32 + (i * 2 + jn) * 8 + e) * 64 + lane];
+              sq[e] += part[((wave + w) * 32 + (i * 2 + jn) * 8 + 4 + e) * 64 + lane];
+            }
+          }
+          store(i, jn, sp, sq);
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void fp_mfma_gemm_kernel(DevProgram const P) {
+  __shared__ int part[kFpMfmaLdsBytes / 4];
+  fp_mfma_gemm_block(P, part, blockIdx.x % P.grid[0], blockIdx.y, blockIdx.z, blockIdx.x / P.grid[0]);
+}
+
+// Many programs in one launch: workgroup -> program by a prefix table, the program record
+// copied to LDS above the wavefront sums.
+__global__ __launch_bounds__(kThreads) void fp_mfma_gemm_multi_kernel(
+    DevProgram const *__restrict__ progs, int const *__restrict__ first_block, int n) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int lo = 0, hi = n;
+  int const w = blockIdx.x;
+  while (hi - lo > 1) {
+    int const mid = (lo + hi) / 2;
+    if (first_block[mid] <= w) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  uint4v const *src = reinterpret_cast<uint4v const *>(progs + lo);
+  uint4v *dst = reinterpret_cast<uint4v *>(lds + kFpMfmaLdsBytes);
+  for (int i = threadIdx.x; i < (int)(sizeof(DevProgram) / 16); i += kThreads) {
+    dst[i] = src[i];
+  }
+  __syncthreads();
+  DevProgram const &P = *reinterpret_cast<DevProgram const *>(lds + kFpMfmaLdsBytes);
+  int v = w - first_block[lo];
+  int const gx = P.grid[0] * P.splits;
+  int const x = v % gx;
+  v /= gx;
+  fp_mfma_gemm_block(P, reinterpret_cast<int *>(lds), x % P.grid[0], v % P.grid[1], v / P.grid[1],
+                     x / P.grid[0]);
+}
+
 inline size_t round_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
 
 }  // namespace
@@ -423,6 +629,17 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
 extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m,
                                int n, int k);
 
+bool mfma_matmul_pays(int batch, int m, int n, int k) {
+  size_t need = 0;
+  return mfma_matmul_fits(batch, m, n, k, &need) && need <= state().planes_bytes &&
+         (double)batch * m * n * k >= (double)(1 << 27);
+}
+
+int launch_mfma_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m, int n,
+                       int k) {
+  return launch_mfma_group(&A, &B, &C, &batch, &m, &n, &k, 1);
+}
+
 extern "C" int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *const *B,
                                     uint16_t *const *C, int const *batch, int const *m,
                                     int const *n, int const *k, int count) {
@@ -470,6 +687,151 @@ extern "C" int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *co
     }
     begin = end;
   }
+  return MI355_OK;
+}
+
+// ---- fused tiled-matmul plans, host side ---------------------------------------------------
+static bool multiple_of_16(int const *v, int count) {
+  for (int i = 0; i < count; i++) {
+    if (v[i] % 16 != 0) {
+      return false;
+    }
+  }
+  return true;
+}
+
+bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_bytes) {
+  if (P.fused != 4 || state().fp_vector_dot_only || state().planes() == nullptr) {
+    return false;
+  }
+  DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]];
+  int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
+  if (m % 16 != 0 || n % 16 != 0 || kt % 16 != 0) {
+    return false;
+  }
+  size_t total = 0;
+  DevOp const *ops[2] = {&la, &lb};
+  for (int which = 0; which < 2; which++) {
+    DevOp const &op = *ops[which];
+    long long const matrix = (long long)op.d_rows * op.d_cols;
+    long long const elems = ext.in_elems[op.io];
+    if (!multiple_of_16(op.row_bs, 3) || !multiple_of_16(op.col_bs, 3) || op.row_fs % 16 != 0 ||
+        op.col_fs % 16 != 0 || matrix <= 0 || elems <= 0 || elems % matrix != 0 || op.g_fs % matrix != 0 ||
+        op.g_bs[0] % matrix != 0 || op.g_bs[1] % matrix != 0 || op.g_bs[2] % matrix != 0) {
+      return false;
+    }
+    long long const slabs = elems / matrix;
+    // plane rows: A keeps its rows, B^T has one row per column of B; k the other extent
+    long long const rows = which == 0 ? op.d_rows : op.d_cols, k = which == 0 ? op.d_cols : op.d_rows;
+    long long const rp = (rows + 15) / 16 * 16, kp = (k + 63) / 64 * 64;
+    if (slabs * rp * kp > ((long long)1 << 26)) {  // a plane stays addressable by a 32-bit offset
+      return false;
+    }
+    P.pl_geo[3 * which] = (int)slabs;
+    P.pl_geo[3 * which + 1] = (int)rp;
+    P.pl_geo[3 * which + 2] = (int)kp;
+    total += (size_t)(2 * slabs * rp * kp);
+  }
+  *plane_bytes = total;
+  return true;
+}
+
+void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
+  DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]];
+  size_t const a_plane = (size_t)P.pl_geo[0] * P.pl_geo[1] * P.pl_geo[2];
+  size_t const b_plane = (size_t)P.pl_geo[3] * P.pl_geo[4] * P.pl_geo[5];
+  P.pl[0] = reinterpret_cast<int8_t *>(planes);
+  P.pl[1] = P.pl[0] + a_plane;
+  P.pl[2] = P.pl[1] + a_plane;
+  P.pl[3] = P.pl[2] + b_plane;
+  // A: strips follow rows, chunks follow columns
+  {
+    long long const matrix = (long long)la.d_rows * la.d_cols;
+    int const strip = P.pl_geo[2] * 16, per_slab = P.pl_geo[1] / 16;
+    auto stride = [&](int g, int row, int col) {
+      return (int)(((long long)(g / matrix) * per_slab + row / 16) * strip + (col / 16) * 256);
+    };
+    for (int d = 0; d < 3; d++) {
+      P.pl_a[d] = stride(la.g_bs[d], la.row_bs[d], la.col_bs[d]);
+    }
+    P.pl_a[3] = stride(la.g_fs, la.row_fs, la.col_fs);
+    P.pl_a[4] = strip;
+  }
+  // B^T: strips follow columns of B, chunks follow its rows
+  {
+    long long const matrix = (long long)lb.d_rows * lb.d_cols;
+    int const strip = P.pl_geo[5] * 16, per_slab = P.pl_geo[4] / 16;
+    auto stride = [&](int g, int row, int col) {
+      return (int)(((long long)(g / matrix) * per_slab + col / 16) * strip + (row / 16) * 256);
+    };
+    for (int d = 0; d < 3; d++) {
+      P.pl_b[d] = stride(lb.g_bs[d], lb.row_bs[d], lb.col_bs[d]);
+    }
+    P.pl_b[3] = stride(lb.g_fs, lb.row_fs, lb.col_fs);
+    P.pl_b[4] = strip;
+  }
+  P.fg[5] = 1;
+  P.lds_bytes = kFpMfmaLdsBytes;
+}
+
+int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream) {
+  int done = 0;
+  while (done < n) {
+    int const group = std::min(n - done, kMaxJobs);
+    SplitMany S{};
+    unsigned blocks = 0;
+    for (int e = 0; e < group; e++) {
+      DevProgram const &P = *progs[done + e];
+      DevOp const *ops[2] = {&P.ops[P.fg[0]], &P.ops[P.fg[1]]};
+      for (int which = 0; which < 2; which++) {
+        DevOp const &op = *ops[which];
+        SplitJob &j = S.job[2 * e + which];
+        j.src = static_cast<uint16_t const *>(P.in[op.io]);
+        j.plane_p = P.pl[2 * which];
+        j.plane_q = P.pl[2 * which + 1];
+        j.slabs = P.pl_geo[3 * which];
+        j.rows = op.d_rows;
+        j.cols = op.d_cols;
+        j.rp = P.pl_geo[3 * which + 1];
+        j.kp = P.pl_geo[3 * which + 2];
+        j.transpose = which;
+        size_t work;
+        if (which == 0) {
+          j.vec = op.d_cols % 8 == 0 && (reinterpret_cast<uintptr_t>(j.src) & 15) == 0;
+          work = ((size_t)j.slabs * j.rp * (j.kp / 16) + kThreads - 1) / kThreads;
+        } else {
+          j.vec = op.d_cols % 4 == 0 && (reinterpret_cast<uintptr_t>(j.src) & 7) == 0;
+          work = (size_t)j.slabs * (j.kp / 64) * ((op.d_cols + 63) / 64);
+        }
+        j.blocks = (unsigned)std::min<size_t>(work, 1024);
+        j.first_block = blocks;
+        blocks += j.blocks;
+      }
+    }
+    S.count = 2 * group;
+    fp_split_planes_kernel<<<blocks, kThreads, 0, stream>>>(S);
+    MI355_HIP(hipGetLastError());
+    done += group;
+  }
+  return MI355_OK;
+}
+
+int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream) {
+  DevProgram const *one = &P;
+  if (int rc = fp_mfma_split_programs(&one, 1, stream)) {
+    return rc;
+  }
+  dim3 grid(P.grid[0] * P.splits, P.grid[1], P.grid[2]);
+  fp_mfma_gemm_kernel<<<grid, kThreads, 0, stream>>>(P);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,
+                              hipStream_t stream) {
+  int const lds_total = kFpMfmaLdsBytes + (int)sizeof(DevProgram);
+  fp_mfma_gemm_multi_kernel<<<blocks, kThreads, lds_total, stream>>>(progs, first_block, n);
+  MI355_HIP(hipGetLastError());
   return MI355_OK;
 }
 

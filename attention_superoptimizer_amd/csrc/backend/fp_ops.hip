@@ -1,6 +1,7 @@
 // Kernel-level fingerprint operators over Z_25651 = Z_227 x Z_113 (uint16 storage).
 //
-// Integer only, no matrix cores.  The matmul does not repeat the reference's
+// Integer vector instructions (large matmuls go to the matrix-core kernel of fp_mfma.hip).
+// The matmul does not repeat the reference's
 // `(r + a*b) % 25651` per multiply-accumulate: it splits every operand into its
 // residues modulo 227 and 113 (both fit a byte), packs four consecutive k into
 // one dword, accumulates with the packed 4x8-bit dot instruction in each
@@ -604,6 +605,9 @@ extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C
   }
   if (batch > 65535) {
     return fail(MI355_ERR_UNSUPPORTED, "batch %d exceeds grid.z", batch);
+  }
+  if (mfma_matmul_pays(batch, m, n, k)) {
+    return launch_mfma_matmul(A, B, C, batch, m, n, k);
   }
   hipStream_t st = state().stream();
   bool const aligned = m % 64 == 0 && n % 64 == 0 && k % 64 == 0 && k > 0 &&

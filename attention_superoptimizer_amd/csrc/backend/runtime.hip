@@ -201,6 +201,10 @@ extern "C" int mi355_set_option(int option, int value) {
     state().plan_smem_layout = value;
     return MI355_OK;
   }
+  if (option == MI355_OPT_FP_MATMUL_ROUTE && (value == 0 || value == 1)) {
+    state().fp_vector_dot_only = value;
+    return MI355_OK;
+  }
   return fail(MI355_ERR_INVALID, "unknown option %d", option);
 }
 

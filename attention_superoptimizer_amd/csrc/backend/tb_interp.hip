@@ -881,6 +881,14 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
       d.vec8 = 0;
     }
   }
+  // a fused matmul plan launched by itself takes the matrix cores when its operand tensors'
+  // residue planes fit this queue's plane memory (a batch places the planes of its members)
+  if (!f16 && prog.fused == 4 && ext_out == nullptr) {
+    size_t need = 0;
+    if (fp_mfma_gemm_fits(prog, ext, &need) && need <= state().planes_bytes) {
+      fp_mfma_gemm_bind(prog, state().planes());
+    }
+  }
   return MI355_OK;
 }
 
@@ -902,7 +910,7 @@ static int fold_splits(DevProgram const &prog) {
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
   if (!f16 && prog.fused == 4) {
-    if (int rc = launch_fp_gemm(prog, s.stream())) {
+    if (int rc = prog.fg[5] ? launch_fp_mfma_gemm(prog, s.stream()) : launch_fp_gemm(prog, s.stream())) {
       return rc;
     }
     if (prog.splits > 1) {
@@ -1024,15 +1032,29 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
   for (int i = 0; i < n; i++) {
     set_splits(progs[i], exts[i], num_outputs[i], std::min(progs[i].forloop_range, scale), used);
   }
+  // fused matmul plans take the matrix cores while the residue planes of their operand
+  // tensors fit what is left of this queue's plane memory
+  std::vector<DevProgram const *> on_matrix_cores;
+  size_t planes_used = 0;
+  for (int i = 0; i < n; i++) {
+    size_t need = 0;
+    if (progs[i].fused == 4 && fp_mfma_gemm_fits(progs[i], exts[i], &need) &&
+        planes_used + need <= s.planes_bytes) {
+      fp_mfma_gemm_bind(progs[i], s.planes() + planes_used);
+      planes_used += (need + 255) / 256 * 256;
+      on_matrix_cores.push_back(&progs[i]);
+    }
+  }
   int const record = (int)sizeof(DevProgram);
   // Launch classes.  Interpreter programs by LDS need (a launch requests the largest need of
   // its members, which bounds how many workgroups share a compute unit); fused matmul
-  // programs by register tiles per thread (a template argument of their kernel).
-  constexpr int kClasses = 6;
+  // programs by register tiles per thread (a template argument of their kernel), those on
+  // the matrix cores in a class of their own.
+  constexpr int kClasses = 7;
   int const bounds[3] = {24 * 1024, 64 * 1024, s.max_lds - record - 16};
   auto class_of = [&](DevProgram const &p) {
     if (p.fused == 4) {
-      return p.fg[3] == 1 ? 3 : (p.fg[3] == 2 ? 4 : 5);
+      return p.fg[5] ? 6 : (p.fg[3] == 1 ? 3 : (p.fg[3] == 2 ? 4 : 5));
     }
     for (int c = 0; c < 3; c++) {
       if (p.lds_bytes <= bounds[c]) {
@@ -1113,6 +1135,11 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
         reinterpret_cast<uint4v const *>(slot.host), reinterpret_cast<uint4v *>(slot.dev),
         (int)(bytes / 16));
     MI355_HIP(hipEventRecord(slot.copied, s.stream()));
+    if (!on_matrix_cores.empty()) {
+      if (int rc = fp_mfma_split_programs(on_matrix_cores.data(), (int)on_matrix_cores.size(), s.stream())) {
+        return rc;
+      }
+    }
     static bool lds_raised = false;
     DevProgram const *dp = reinterpret_cast<DevProgram const *>(slot.dev);
     int const *df = reinterpret_cast<int const *>(slot.dev + off_first);
@@ -1123,6 +1150,15 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
       int lds = 0;
       for (int k = class_begin[c]; k < class_begin[c + 1]; k++) {
         lds = std::max(lds, progs[order[k]].lds_bytes);
+      }
+      if (c == 6) {
+        int const blocks = hf[first_off[c] + first_cnt[c]];
+        if (int rc = launch_fp_mfma_gemm_multi(dp + class_begin[c], df + first_off[c], first_cnt[c], blocks,
+                                               s.stream())) {
+          return rc;
+        }
+        launched += blocks;
+        continue;
       }
       if (c >= 3) {
         int const blocks = hf[first_off[c] + first_cnt[c]];

@@ -66,7 +66,16 @@ struct alignas(16) DevProgram {
   int fused;      // fp16: 1 / 2 / 3 = run by the fused attention / GEMM / combine kernel; uint16:
                   // 4 = run by the fused fingerprint matmul kernel; 0 = the interpreter
   int fg[6];      // fused fingerprint matmul: loader of A, loader of B, k chunk, register tiles per
-                  // thread, thread groups sharing a tile's k range (small tiles), spare
+                  // thread, thread groups sharing a tile's k range (small tiles), 1 = matrix-core
+                  // route (the operand tensors are read from residue planes, see pl / pl_geo)
+  // matrix-core route: signed-byte residue planes of the two operand tensors in 16 x 16 blocks
+  // (A mod 227, A mod 113, B^T mod 227, B^T mod 113) and their geometry: A slabs, A plane rows
+  // per slab, A padded k; B slabs, B^T plane rows per slab, B padded k
+  int8_t *pl[4];
+  int pl_geo[6];
+  // byte offset of a tile's first block in the A / B^T planes = bx * [0] + by * [1] + bz * [2] +
+  // iteration * [3]; [4] = bytes of one strip of 16 plane rows
+  int pl_a[5], pl_b[5];
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
@@ -107,6 +116,18 @@ bool fp_gemm_applicable(DevProgram &P);
 int launch_fp_gemm(DevProgram const &P, hipStream_t stream);
 int launch_fp_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks, int tpt,
                          int staging_bytes, hipStream_t stream);
+
+// Matrix-core route of the same family (fp_mfma.hip).  fp_mfma_gemm_fits: whether a program
+// already marked fused = 4 can take it, and the bytes of residue planes it needs;
+// fp_mfma_gemm_bind: places the planes at `planes` and marks the program; the launches split
+// the operand tensors of the bound programs into their planes first (fp_mfma_split_programs).
+bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_bytes);
+void fp_mfma_gemm_bind(DevProgram &P, char *planes);
+int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream);
+int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream);
+int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,
+                              hipStream_t stream);
+constexpr int kFpMfmaLdsBytes = 32768;  // wavefront sums of a tile whose k range is shared
 
 // `declared_layouts`: fp16 loader tiles take the LDS layout the plan declares for them
 // (see MI355_OPT_PLAN_SMEM_LAYOUT) instead of the one their consumers want.

@@ -102,6 +102,10 @@ typedef struct mi355_launch_info {
  * src/search/search.cc:625-763) turns with profile() as its cost.  Fused kernels
  * keep their own staging layouts. */
 #define MI355_OPT_PLAN_SMEM_LAYOUT 3
+/* FP_MATMUL_ROUTE: 0 = fingerprint matmuls (kernel-level and the fused tiled-matmul plans)
+ * take the int8 matrix-core kernels whenever their shapes allow (default); 1 = always the
+ * packed 4 x 8-bit vector-dot kernels.  Results are bit-identical; tests run both. */
+#define MI355_OPT_FP_MATMUL_ROUTE 4
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor

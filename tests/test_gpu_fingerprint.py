@@ -104,8 +104,41 @@ def test_uniform_fill_matches_host_generator(rt, abi):
         g.close()
 
 
+def _fused_matmul_routes(rt, abi, spec, ins, op_index=2):
+    """Fingerprints the customized op of `spec` three ways: matrix cores where the plan allows
+    them, vector-dot kernel only, interpreter.  Returns {route: (kernel id, LDS bytes, output)}."""
+    import ctypes as ct
+    from attention_superoptimizer_amd import _native as N
+    got = {}
+    for route, (forced, vector_only) in {"auto": (0, 0), "vector-dot": (0, 1), "interpreter": (1, 0)}.items():
+        assert abi.mi355_set_option(1, forced) == 0 and abi.mi355_set_option(4, vector_only) == 0
+        try:
+            g, vals = rt.build_from_spec(spec)
+            try:
+                for i, a in ins.items():
+                    vals[i][0].write_fingerprint(a)
+                g.fingerprint(op_index)
+                info = N.Mi355LaunchInfo()
+                N.backend().mi355_last_launch(ct.byref(info))
+                got[route] = (info.kernel_id, info.lds_bytes, vals[op_index][0].read_fingerprint())
+            finally:
+                g.close()
+        finally:
+            assert abi.mi355_set_option(1, 0) == 0 and abi.mi355_set_option(4, 0) == 0
+    return got
+
+
 @pytest.mark.parametrize("m,n,k,grid,F,amap,bmap,omap", [
     (128, 256, 256, (4, 2, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),     # 64x64 tiles, k chunk 64
+    # matrix-core route: k tiles of 16 / 48 / 80 (chunks of several iterations share a matrix
+    # instruction, the last one partly empty), tiles of 16 / 48 rows or columns, one / two /
+    # many 32 x 32 pieces per tile, for-loops split over workgroups
+    (16, 16, 16 * 7, (1, 1, 1), 7, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),
+    (48, 32, 48 * 5, (1, 1, 1), 5, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),
+    (32, 64, 80 * 3, (1, 1, 1), 3, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),
+    (96, 240, 32 * 9, (3, 2, 1), 9, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),    # 48 x 80 tiles
+    (256, 128, 2048, (2, 1, 1), 128, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),  # 256 x 64 tiles, k 16
+    (64, 64, 16 * 1001, (1, 1, 1), 1001, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),
     (256, 256, 512, (2, 2, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),     # 128x128 tiles, 4 register tiles
     (64, 64, 512, (1, 1, 1), 8, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),   # one block: for-loop split 8 ways
     (16, 40, 96, (1, 1, 1), 4, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),    # 16x40 tile, k tile 24 -> chunk 8
@@ -118,55 +151,74 @@ def test_uniform_fill_matches_host_generator(rt, abi):
 def test_fused_matmul_fingerprint_equals_interpreter_and_oracle(rt, abi, m, n, k, grid, F, amap, bmap, omap):
     """A load-load-matmul-accumulate plan runs on the fused fingerprint matmul kernel; forced
     through the interpreter it must give the same uint16 tensor, and both the oracle's."""
-    import ctypes as ct
-    from attention_superoptimizer_amd import _native as N
     from attention_superoptimizer_amd import workloads as W
     spec = W.tiled_matmul(m, n, k, grid, F, amap, bmap, omap)[0]
     ins = {0: uniform_fp(spec[0]["dims"], 31), 1: uniform_fp(spec[1]["dims"], 32)}
     ins[0].flat[:7] = 25650  # worst-case operands in one corner
     ins[1].flat[:7] = 25650
     want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
-    got = {}
-    for forced in (0, 1):
-        assert abi.mi355_set_option(1, forced) == 0
+    got = _fused_matmul_routes(rt, abi, spec, ins)
+    for route, (kernel_id, _, out) in got.items():
+        assert kernel_id == (1 if route == "interpreter" else 6), route
+        assert np.array_equal(out, want), route
+
+
+def test_fused_matmul_fingerprint_takes_tiles_the_interpreter_cannot_hold(rt, abi):
+    """A [128,256] and B [256,128] tiles need 197 KB of LDS in the interpreter; the fused
+    kernels keep no tile there (the matrix-core one reads residue planes, the vector-dot one
+    streams k chunks of 64 through LDS) and match the oracle."""
+    from attention_superoptimizer_amd import workloads as W
+    spec = W.tiled_matmul(512, 512, 1024, (4, 4, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1))[0]
+    ins = {0: uniform_fp(spec[0]["dims"], 41), 1: uniform_fp(spec[1]["dims"], 42)}
+    want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
+    for vector_only, lds in ((0, 32768), (1, 2 * 2 * 16 * (128 + 4 + 128) * 4)):
+        assert abi.mi355_set_option(4, vector_only) == 0
         try:
             g, vals = rt.build_from_spec(spec)
             try:
                 vals[0][0].write_fingerprint(ins[0])
                 vals[1][0].write_fingerprint(ins[1])
                 g.fingerprint(2)
-                info = N.Mi355LaunchInfo()
-                N.backend().mi355_last_launch(ct.byref(info))
-                assert info.kernel_id == (1 if forced else 6)
-                got[forced] = vals[2][0].read_fingerprint()
+                info = N_launch_info()
+                assert info.kernel_id == 6 and info.lds_bytes == lds
+                assert np.array_equal(vals[2][0].read_fingerprint(), want)
             finally:
                 g.close()
         finally:
-            assert abi.mi355_set_option(1, 0) == 0
-    assert np.array_equal(got[0], want)
-    assert np.array_equal(got[1], want)
+            assert abi.mi355_set_option(4, 0) == 0
 
 
-def test_fused_matmul_fingerprint_takes_tiles_the_interpreter_cannot_hold(rt, abi):
-    """A [128,256] and B [256,128] tiles need 197 KB of LDS in the interpreter; the fused
-    kernel streams them in k chunks of 64 and matches the oracle."""
+def N_launch_info():
     import ctypes as ct
     from attention_superoptimizer_amd import _native as N
+    info = N.Mi355LaunchInfo()
+    N.backend().mi355_last_launch(ct.byref(info))
+    return info
+
+
+def test_fused_matmul_fingerprint_batched_operands_and_mismatched_maps(rt, abi):
+    """Matrix-core route over 3-D operands (grid z walks the batch dim), and over plans whose
+    maps do not describe A.B (the for-loop walks A's rows; both loaders take the same block
+    column): every route must give what the plan says, i.e. the oracle's answer."""
     from attention_superoptimizer_amd import workloads as W
-    spec = W.tiled_matmul(512, 512, 1024, (4, 4, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1))[0]
-    ins = {0: uniform_fp(spec[0]["dims"], 41), 1: uniform_fp(spec[1]["dims"], 42)}
-    want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
-    g, vals = rt.build_from_spec(spec)
-    try:
-        vals[0][0].write_fingerprint(ins[0])
-        vals[1][0].write_fingerprint(ins[1])
-        g.fingerprint(2)
-        info = N.Mi355LaunchInfo()
-        N.backend().mi355_last_launch(ct.byref(info))
-        assert info.kernel_id == 6 and info.lds_bytes == 2 * 2 * 16 * (128 + 4 + 128) * 4
-        assert np.array_equal(vals[2][0].read_fingerprint(), want)
-    finally:
-        g.close()
+    cases = []
+    b, m, n, k = 3, 64, 96, 128
+    cases.append(([W._inp([b, m, k]), W._inp([b, k, n]),
+                   {"op": "customized", "in": [[0, 0], [1, 0]],
+                    "plan": W._plan((2, 3, b), 4, [(1, -1, 0), (-1, 2, 0)], (2, 1), (1, 2, 0),
+                                    [("tb_matmul_op", [(0, 0), (1, 0)])])}], 51))
+    # for-loop over A's rows and B's rows: sum over i of A[32 i : 32 i + 32, :64] . B[64 i : 64 i + 64, :]
+    cases.append(([W._inp([128, 64]), W._inp([256, 48]),
+                   {"op": "customized", "in": [[0, 0], [1, 0]],
+                    "plan": W._plan((1, 1, 1), 4, [(-1, -1, -1), (-1, -1, -1)], (0, 0), (-1, -1, -1),
+                                    [("tb_matmul_op", [(0, 0), (1, 0)])])}], 52))
+    for spec, seed in cases:
+        ins = {0: uniform_fp(spec[0]["dims"], seed), 1: uniform_fp(spec[1]["dims"], seed + 100)}
+        want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
+        got = _fused_matmul_routes(rt, abi, spec, ins)
+        for route, (kernel_id, lds, out) in got.items():
+            assert np.array_equal(out, want), (route, spec[2]["plan"])
+        assert got["auto"][0] == 6 and got["auto"][1] == 32768
 
 
 def test_many_fills_and_many_compares_in_one_launch(rt, abi):
