@@ -61,17 +61,21 @@ __global__ void fp_fill_uniform_kernel(uint16_t *fp, size_t n, uint64_t seed) {
   }
 }
 
-// All inputs of one graph in a single launch: blockIdx.y names the tensor.
+// Many input tensors in a single launch.  Tensors that get the same values (same length,
+// same seed: the same input of several candidate graphs) form a group; blockIdx.y names the
+// group, its values are computed once and stored to every member.
 struct FillMany {
-  uint16_t *ptr[MI355_MAX_FILL_TENSORS];
-  size_t n[MI355_MAX_FILL_TENSORS];
-  uint64_t seed[MI355_MAX_FILL_TENSORS];
+  uint16_t *ptr[MI355_MAX_FILL_TENSORS];  // members of a group are neighbours
+  size_t n[MI355_MAX_FILL_TENSORS];       // per group
+  uint64_t seed[MI355_MAX_FILL_TENSORS];  // per group
+  int first[MI355_MAX_FILL_TENSORS], members[MI355_MAX_FILL_TENSORS];
 };
 
 __global__ void fp_fill_many_kernel(FillMany const F, int iota) {
-  uint16_t *fp = F.ptr[blockIdx.y];
-  size_t const n = F.n[blockIdx.y];
-  uint64_t const seed = F.seed[blockIdx.y];
+  int const group = blockIdx.y;
+  size_t const n = F.n[group];
+  uint64_t const seed = F.seed[group];
+  int const first = F.first[group], members = F.members[group];
   size_t i = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) * 8;
   size_t const stride = (size_t)gridDim.x * blockDim.x * 8;
   for (; i < n; i += stride) {
@@ -82,10 +86,14 @@ __global__ void fp_fill_many_kernel(FillMany const F, int iota) {
     }
     if (end == i + 8) {
       uint4v w = {v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
-      *reinterpret_cast<uint4v *>(fp + i) = w;
+      for (int t = 0; t < members; t++) {
+        *reinterpret_cast<uint4v *>(F.ptr[first + t] + i) = w;
+      }
     } else {
-      for (size_t j = i; j < end; j++) {
-        fp[j] = static_cast<uint16_t>(v[j - i]);
+      for (int t = 0; t < members; t++) {
+        for (size_t j = i; j < end; j++) {
+          F.ptr[first + t][j] = static_cast<uint16_t>(v[j - i]);
+        }
       }
     }
   }
@@ -580,15 +588,40 @@ extern "C" int mi355_fp_fill_many(uint16_t *const *fp, size_t const *n, uint64_t
     if ((reinterpret_cast<uintptr_t>(fp[i]) & 15) != 0) {
       return fail(MI355_ERR_INVALID, "fingerprint buffers are 16-byte aligned");
     }
-    F.ptr[i] = fp[i];
-    F.n[i] = n[i];
-    F.seed[i] = iota ? 0 : seeds[i];
     largest = std::max(largest, n[i]);
   }
   if (count == 0 || largest == 0) {
     return MI355_OK;
   }
-  dim3 grid(grid_for((largest + 7) / 8, kThreads, 2048), count);
+  // group tensors that receive the same values
+  int group_of[MI355_MAX_FILL_TENSORS];
+  int groups = 0;
+  for (int i = 0; i < count; i++) {
+    uint64_t const seed = iota ? 0 : seeds[i];
+    int g = 0;
+    while (g < groups && (F.n[g] != n[i] || F.seed[g] != seed)) {
+      g++;
+    }
+    if (g == groups) {
+      F.n[g] = n[i];
+      F.seed[g] = seed;
+      F.members[g] = 0;
+      groups++;
+    }
+    F.members[g]++;
+    group_of[i] = g;
+  }
+  int at = 0;
+  for (int g = 0; g < groups; g++) {
+    F.first[g] = at;
+    at += F.members[g];
+    F.members[g] = 0;
+  }
+  for (int i = 0; i < count; i++) {
+    int const g = group_of[i];
+    F.ptr[F.first[g] + F.members[g]++] = fp[i];
+  }
+  dim3 grid(grid_for((largest + 7) / 8, kThreads, 2048), groups);
   fp_fill_many_kernel<<<grid, kThreads, 0, state().stream()>>>(F, iota);
   MI355_HIP(hipGetLastError());
   return MI355_OK;

@@ -480,6 +480,7 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
     // a k chunk of kc.  Each matmul takes the largest chunk that still fits; one that
     // cannot get even 16 keeps the scalar path.
     int const device_lds = max_lds;
+    int const vector_dot_only = state().fp_vector_dot_only;
     int scratch = 0;
     for (int o = 0; o < prog.num_ops; o++) {
       DevOp &d = prog.ops[o];
@@ -490,13 +491,18 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       if (m % 4 != 0 || n % 4 != 0 || k % 4 != 0) {
         continue;
       }
+      // matrix-core variant (signed-byte residues, rows padded by 16 bytes): tiles whose m
+      // and n are multiples of 16, k chunks that are multiples of 64; `sub` = 1 selects it
+      d.sub = 0;
       for (int kc = k; kc >= 16 || kc == k; kc /= 2) {
         if (kc % 4 != 0 || k % kc != 0) {
           break;
         }
-        int const need = 2 * kc * (m + 4 + n);
+        bool const mfma = vector_dot_only == 0 && m % 16 == 0 && n % 16 == 0 && kc % 64 == 0;
+        int const need = mfma ? 2 * (kc + 16) * (m + n) : 2 * kc * (m + 4 + n);
         if (peak + need <= device_lds) {
           d.mm_kc = kc;
+          d.sub = mfma ? 1 : 0;
           scratch = std::max(scratch, need);
           break;
         }

@@ -164,6 +164,122 @@ __device__ void fp_matmul_packed(uint16_t const *A, uint16_t const *B, uint16_t 
   }
 }
 
+// The same product on the int8 matrix cores, for tiles whose m and n are multiples of 16
+// and a k chunk that is a multiple of 64.  Residues are packed as signed bytes (mod 227
+// recentred to [-113, 113], mod 113 as it is), A as Ab[field][m][kc + 16], B transposed as
+// Bb[field][n][kc + 16] (the 16 bytes of padding spread a 16-lane group's 16-byte operand
+// reads over all banks); a wavefront owns 32 x 32 outputs at a time and issues
+// v_mfma_i32_16x16x64_i8 per field; B^T is the first operand, so a lane ends up with four
+// consecutive columns of one row of C.  One CRT recombination per output and k chunk.
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t signed_residues_p(uint32_t v0, uint32_t v1, uint32_t v2, uint32_t v3) {
+  auto one = [](uint32_t x) {
+    uint32_t const r = x % FP_P;
+    return (r > 113u ? r + 29u : r) & 0xffu;  // r - 227 = r + 29 (mod 256)
+  };
+  return one(v0) | (one(v1) << 8) | (one(v2) << 16) | (one(v3) << 24);
+}
+
+__device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C, int m, int n, int k,
+                               DevOp const &op, unsigned char *scratch, int tid) {
+  int const kc = op.mm_kc, kq = kc / 4, pitch = kc + 16;
+  unsigned char *Ab = scratch, *Bb = scratch + 2 * m * pitch;
+  int const n2 = n / 2;
+  int const wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
+  int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
+  for (int k0 = 0; k0 < k; k0 += kc) {
+    if (k0 > 0) {
+      __syncthreads();  // the previous chunk's residues are still being read
+    }
+    for (int e = tid; e < m * kq; e += kInterpThreads) {
+      int const row = fdiv(e, op.mg0), q = e - row * kq;
+      uint2 v = *reinterpret_cast<uint2 const *>(A + row * k + k0 + 4 * q);
+      uint32_t v0 = v.x & 0xffffu, v1 = v.x >> 16, v2 = v.y & 0xffffu, v3 = v.y >> 16;
+      *reinterpret_cast<uint32_t *>(Ab + row * pitch + 4 * q) = signed_residues_p(v0, v1, v2, v3);
+      *reinterpret_cast<uint32_t *>(Ab + (m + row) * pitch + 4 * q) = pack_residues(v0, v1, v2, v3, FP_Q);
+    }
+    for (int e = tid; e < kq * n2; e += kInterpThreads) {
+      int const q = fdiv(e, op.mg1), c2 = (e - q * n2) * 2;
+      uint16_t const *bp = B + (k0 + 4 * q) * n + c2;
+      uint32_t w0 = *reinterpret_cast<uint32_t const *>(bp);
+      uint32_t w1 = *reinterpret_cast<uint32_t const *>(bp + n);
+      uint32_t w2 = *reinterpret_cast<uint32_t const *>(bp + 2 * n);
+      uint32_t w3 = *reinterpret_cast<uint32_t const *>(bp + 3 * n);
+      *reinterpret_cast<uint32_t *>(Bb + c2 * pitch + 4 * q) =
+          signed_residues_p(w0 & 0xffffu, w1 & 0xffffu, w2 & 0xffffu, w3 & 0xffffu);
+      *reinterpret_cast<uint32_t *>(Bb + (c2 + 1) * pitch + 4 * q) =
+          signed_residues_p(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16);
+      *reinterpret_cast<uint32_t *>(Bb + (n + c2) * pitch + 4 * q) =
+          pack_residues(w0 & 0xffffu, w1 & 0xffffu, w2 & 0xffffu, w3 & 0xffffu, FP_Q);
+      *reinterpret_cast<uint32_t *>(Bb + (n + c2 + 1) * pitch + 4 * q) =
+          pack_residues(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16, FP_Q);
+    }
+    __syncthreads();
+    for (int t = wave; t < mt; t += kInterpThreads / 64) {
+      int const row_m = (t / mt_n) * 32, col_n = (t - (t / mt_n) * mt_n) * 32;
+      int const i1 = row_m + 16 < m ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
+      unsigned char const *a_at[2], *b_at[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        a_at[i] = Ab + (row_m + 16 * (i ? i1 : 0) + r) * pitch + 16 * g;
+        b_at[i] = Bb + (col_n + 16 * (i ? j1 : 0) + r) * pitch + 16 * g;
+      }
+      v4i acc[2][2][2];
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
+      }
+      for (int ks = 0; ks < kc; ks += 64) {
+        v4i ap[2], aq[2], bp[2], bq[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+          ap[i] = *reinterpret_cast<v4i const *>(a_at[i] + ks);
+          aq[i] = *reinterpret_cast<v4i const *>(a_at[i] + m * pitch + ks);
+          bp[i] = *reinterpret_cast<v4i const *>(b_at[i] + ks);
+          bq[i] = *reinterpret_cast<v4i const *>(b_at[i] + n * pitch + ks);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+          for (int jn = 0; jn < 2; jn++) {
+            acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bp[jn], ap[i], acc[0][i][jn], 0, 0, 0);
+            acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[jn], aq[i], acc[1][i][jn], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int jn = 0; jn < 2; jn++) {
+          if (i > i1 || jn > j1) {
+            continue;
+          }
+          uint16_t *cp = C + (row_m + 16 * i + r) * n + col_n + 16 * jn + 4 * g;
+          uint32_t z[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            int const rp = (acc[0][i][jn][e] % (int)FP_P + (int)FP_P) % (int)FP_P;
+            int const rq = acc[1][i][jn][e] % (int)FP_Q;  // both operands non-negative
+            z[e] = ((uint32_t)rp * FP_Q_MUL_P_MOD_1 + (uint32_t)rq * FP_P_MUL_Q_MOD_1) % FP_PQ;
+          }
+          if (k0 > 0) {
+            uint2 old = *reinterpret_cast<uint2 const *>(cp);
+            z[0] = (z[0] + (old.x & 0xffffu)) % FP_PQ;
+            z[1] = (z[1] + (old.x >> 16)) % FP_PQ;
+            z[2] = (z[2] + (old.y & 0xffffu)) % FP_PQ;
+            z[3] = (z[3] + (old.y >> 16)) % FP_PQ;
+          }
+          uint2 out;
+          out.x = z[0] | (z[1] << 16);
+          out.y = z[2] | (z[3] << 16);
+          *reinterpret_cast<uint2 *>(cp) = out;
+        }
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ uint32_t add_mod_pair(uint32_t a, uint32_t b) {
   // two uint16 lanes: (a + b) mod 25651 in each
   uint32_t lo = ((a & 0xffffu) + (b & 0xffffu)) % FP_PQ;
@@ -217,7 +333,9 @@ __device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned ch
           uint16_t const *B = reinterpret_cast<uint16_t const *>(lds + tb.off);
           uint16_t *C = reinterpret_cast<uint16_t *>(lds + tc.off);
           int const m = ta.rows, k = ta.cols, n = tb.cols;
-          if (op.mm_kc > 0) {
+          if (op.mm_kc > 0 && op.sub == 1) {
+            fp_matmul_mfma(A, B, C, m, n, k, op, lds + P.mm_off, tid);
+          } else if (op.mm_kc > 0) {
             fp_matmul_packed(A, B, C, m, n, k, op, reinterpret_cast<uint32_t *>(lds + P.mm_off),
                              tid);
           } else {

@@ -105,12 +105,14 @@ def test_uniform_fill_matches_host_generator(rt, abi):
 
 
 def _fused_matmul_routes(rt, abi, spec, ins, op_index=2):
-    """Fingerprints the customized op of `spec` three ways: matrix cores where the plan allows
-    them, vector-dot kernel only, interpreter.  Returns {route: (kernel id, LDS bytes, output)}."""
+    """Fingerprints the customized op of `spec` four ways: fused kernel and interpreter, each on
+    the matrix cores where the shapes allow and with the vector-dot path only.  Returns
+    {route: (kernel id, LDS bytes, output)}."""
     import ctypes as ct
     from attention_superoptimizer_amd import _native as N
     got = {}
-    for route, (forced, vector_only) in {"auto": (0, 0), "vector-dot": (0, 1), "interpreter": (1, 0)}.items():
+    routes = {"auto": (0, 0), "vector-dot": (0, 1), "interpreter": (1, 0), "interpreter, vector-dot": (1, 1)}
+    for route, (forced, vector_only) in routes.items():
         assert abi.mi355_set_option(1, forced) == 0 and abi.mi355_set_option(4, vector_only) == 0
         try:
             g, vals = rt.build_from_spec(spec)
@@ -159,7 +161,7 @@ def test_fused_matmul_fingerprint_equals_interpreter_and_oracle(rt, abi, m, n, k
     want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
     got = _fused_matmul_routes(rt, abi, spec, ins)
     for route, (kernel_id, _, out) in got.items():
-        assert kernel_id == (1 if route == "interpreter" else 6), route
+        assert kernel_id == (1 if route.startswith("interpreter") else 6), route
         assert np.array_equal(out, want), route
 
 
@@ -237,6 +239,22 @@ def test_many_fills_and_many_compares_in_one_launch(rt, abi):
             assert abi.mi355_fp_fill_many(ptrs, ns, seeds, 40, 0) == 0
         for i, t in enumerate(left):
             assert np.array_equal(t.read_fingerprint(), uniform_fp(t.dims, 9000 + i)), i
+        # tensors of equal length and seed (the same input of several candidates) are computed
+        # once and stored to each: every one of them must still hold the sequence
+        same = list(range(0, 40, 5))  # sizes 1, 186, 371, ... with i % 5 == 0
+        rep = [left[i] for i in same] + [right[i] for i in same]
+        ptrs = (ctypes.c_void_p * 16)(*[t.device_ptr(True) for t in rep])
+        ns = (ctypes.c_size_t * 16)(*([sizes[i] for i in same] * 2))
+        seeds = (ctypes.c_uint64 * 16)(*([77 + (i % 10) for i in same] * 2))
+        assert abi.mi355_fp_fill_many(ptrs, ns, seeds, 16, 0) == 0
+        for j, t in enumerate(rep):
+            i = same[j % 8]
+            assert np.array_equal(t.read_fingerprint(), uniform_fp(t.dims, 77 + (i % 10))), j
+        for side in (left, right):  # back to the values the compares below expect
+            ptrs = (ctypes.c_void_p * 40)(*[t.device_ptr(True) for t in side])
+            ns = (ctypes.c_size_t * 40)(*sizes)
+            seeds = (ctypes.c_uint64 * 40)(*[9000 + i for i in range(40)])
+            assert abi.mi355_fp_fill_many(ptrs, ns, seeds, 40, 0) == 0
         differ = [i % 3 == 1 for i in range(40)]
         for i, t in enumerate(right):
             if differ[i]:
