@@ -491,15 +491,16 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       if (m % 4 != 0 || n % 4 != 0 || k % 4 != 0) {
         continue;
       }
-      // matrix-core variant (signed-byte residues, rows padded by 16 bytes): tiles whose m
-      // and n are multiples of 16, k chunks that are multiples of 64; `sub` = 1 selects it
+      // matrix-core variant (signed-byte residues, swizzled rows, no padding): tiles whose m
+      // and n are multiples of 16, k chunks that are powers of two from 64; `sub` = 1 selects it
       d.sub = 0;
       for (int kc = k; kc >= 16 || kc == k; kc /= 2) {
         if (kc % 4 != 0 || k % kc != 0) {
           break;
         }
-        bool const mfma = vector_dot_only == 0 && m % 16 == 0 && n % 16 == 0 && kc % 64 == 0;
-        int const need = mfma ? 2 * (kc + 16) * (m + n) : 2 * kc * (m + 4 + n);
+        bool const mfma = vector_dot_only == 0 && m % 16 == 0 && n % 16 == 0 && kc >= 64 &&
+                          (kc & (kc - 1)) == 0;
+        int const need = mfma ? 2 * kc * (m + n) : 2 * kc * (m + 4 + n);
         if (peak + need <= device_lds) {
           d.mm_kc = kc;
           d.sub = mfma ? 1 : 0;

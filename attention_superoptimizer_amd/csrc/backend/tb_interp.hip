@@ -166,9 +166,10 @@ __device__ void fp_matmul_packed(uint16_t const *A, uint16_t const *B, uint16_t 
 
 // The same product on the int8 matrix cores, for tiles whose m and n are multiples of 16
 // and a k chunk that is a multiple of 64.  Residues are packed as signed bytes (mod 227
-// recentred to [-113, 113], mod 113 as it is), A as Ab[field][m][kc + 16], B transposed as
-// Bb[field][n][kc + 16] (the 16 bytes of padding spread a 16-lane group's 16-byte operand
-// reads over all banks); a wavefront owns 32 x 32 outputs at a time and issues
+// recentred to [-113, 113], mod 113 as it is), A as Ab[field][m][kc], B transposed as
+// Bb[field][n][kc]; kc is a power of two and the 16-byte chunks of a row are XOR-swizzled by
+// a key of the row so that the 16 rows a 16-lane group reads fall on all banks without any
+// padding (the scratch is no larger than the dot4 path's); a wavefront owns 32 x 32 outputs at a time and issues
 // v_mfma_i32_16x16x64_i8 per field; B^T is the first operand, so a lane ends up with four
 // consecutive columns of one row of C.  One CRT recombination per output and k chunk.
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -183,8 +184,15 @@ __device__ __forceinline__ uint32_t signed_residues_p(uint32_t v0, uint32_t v1, 
 
 __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C, int m, int n, int k,
                                DevOp const &op, unsigned char *scratch, int tid) {
-  int const kc = op.mm_kc, kq = kc / 4, pitch = kc + 16;
+  int const kc = op.mm_kc, kq = kc / 4, pitch = kc;
   unsigned char *Ab = scratch, *Bb = scratch + 2 * m * pitch;
+  // chunk c of row `row` lives at chunk c ^ key(row): rows that share a 256-byte bank line
+  // (4 rows of 64 bytes, 2 of 128) and rows a multiple of that apart get different keys
+  int const key_shift = kc >= 256 ? 0 : (kc == 128 ? 1 : 2);
+  int const key_mask = (kc / 16 < 16 ? kc / 16 : 16) - 1;
+  auto swz = [&](int row, int byte) {  // byte offset within the row -> swizzled byte offset
+    return (((byte >> 4) ^ ((row >> key_shift) & key_mask)) << 4) | (byte & 15);
+  };
   int const n2 = n / 2;
   int const wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
   int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
@@ -196,8 +204,9 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
       int const row = fdiv(e, op.mg0), q = e - row * kq;
       uint2 v = *reinterpret_cast<uint2 const *>(A + row * k + k0 + 4 * q);
       uint32_t v0 = v.x & 0xffffu, v1 = v.x >> 16, v2 = v.y & 0xffffu, v3 = v.y >> 16;
-      *reinterpret_cast<uint32_t *>(Ab + row * pitch + 4 * q) = signed_residues_p(v0, v1, v2, v3);
-      *reinterpret_cast<uint32_t *>(Ab + (m + row) * pitch + 4 * q) = pack_residues(v0, v1, v2, v3, FP_Q);
+      int const at = row * pitch + swz(row, 4 * q);
+      *reinterpret_cast<uint32_t *>(Ab + at) = signed_residues_p(v0, v1, v2, v3);
+      *reinterpret_cast<uint32_t *>(Ab + m * pitch + at) = pack_residues(v0, v1, v2, v3, FP_Q);
     }
     for (int e = tid; e < kq * n2; e += kInterpThreads) {
       int const q = fdiv(e, op.mg1), c2 = (e - q * n2) * 2;
@@ -206,13 +215,13 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
       uint32_t w1 = *reinterpret_cast<uint32_t const *>(bp + n);
       uint32_t w2 = *reinterpret_cast<uint32_t const *>(bp + 2 * n);
       uint32_t w3 = *reinterpret_cast<uint32_t const *>(bp + 3 * n);
-      *reinterpret_cast<uint32_t *>(Bb + c2 * pitch + 4 * q) =
+      int const at0 = c2 * pitch + swz(c2, 4 * q), at1 = (c2 + 1) * pitch + swz(c2 + 1, 4 * q);
+      *reinterpret_cast<uint32_t *>(Bb + at0) =
           signed_residues_p(w0 & 0xffffu, w1 & 0xffffu, w2 & 0xffffu, w3 & 0xffffu);
-      *reinterpret_cast<uint32_t *>(Bb + (c2 + 1) * pitch + 4 * q) =
-          signed_residues_p(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16);
-      *reinterpret_cast<uint32_t *>(Bb + (n + c2) * pitch + 4 * q) =
+      *reinterpret_cast<uint32_t *>(Bb + at1) = signed_residues_p(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16);
+      *reinterpret_cast<uint32_t *>(Bb + n * pitch + at0) =
           pack_residues(w0 & 0xffffu, w1 & 0xffffu, w2 & 0xffffu, w3 & 0xffffu, FP_Q);
-      *reinterpret_cast<uint32_t *>(Bb + (n + c2 + 1) * pitch + 4 * q) =
+      *reinterpret_cast<uint32_t *>(Bb + n * pitch + at1) =
           pack_residues(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16, FP_Q);
     }
     __syncthreads();
@@ -220,10 +229,14 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
       int const row_m = (t / mt_n) * 32, col_n = (t - (t / mt_n) * mt_n) * 32;
       int const i1 = row_m + 16 < m ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
       unsigned char const *a_at[2], *b_at[2];
+      int a_key[2], b_key[2];
 #pragma unroll
       for (int i = 0; i < 2; i++) {
-        a_at[i] = Ab + (row_m + 16 * (i ? i1 : 0) + r) * pitch + 16 * g;
-        b_at[i] = Bb + (col_n + 16 * (i ? j1 : 0) + r) * pitch + 16 * g;
+        int const ar = row_m + 16 * (i ? i1 : 0) + r, br = col_n + 16 * (i ? j1 : 0) + r;
+        a_at[i] = Ab + ar * pitch;
+        b_at[i] = Bb + br * pitch;
+        a_key[i] = (ar >> key_shift) & key_mask;
+        b_key[i] = (br >> key_shift) & key_mask;
       }
       v4i acc[2][2][2];
 #pragma unroll
@@ -234,10 +247,11 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
         v4i ap[2], aq[2], bp[2], bq[2];
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-          ap[i] = *reinterpret_cast<v4i const *>(a_at[i] + ks);
-          aq[i] = *reinterpret_cast<v4i const *>(a_at[i] + m * pitch + ks);
-          bp[i] = *reinterpret_cast<v4i const *>(b_at[i] + ks);
-          bq[i] = *reinterpret_cast<v4i const *>(b_at[i] + n * pitch + ks);
+          int const ca = (((ks >> 4) + g) ^ a_key[i]) << 4, cb = (((ks >> 4) + g) ^ b_key[i]) << 4;
+          ap[i] = *reinterpret_cast<v4i const *>(a_at[i] + ca);
+          aq[i] = *reinterpret_cast<v4i const *>(a_at[i] + m * pitch + ca);
+          bp[i] = *reinterpret_cast<v4i const *>(b_at[i] + cb);
+          bq[i] = *reinterpret_cast<v4i const *>(b_at[i] + n * pitch + cb);
         }
 #pragma unroll
         for (int i = 0; i < 2; i++) {
