@@ -101,6 +101,11 @@ ABI = {
     "mi355_fp_equal_enqueue": (_ci, [_vp, _vp, _sz, _ci]),
     "mi355_fp_equal_enqueue_many": (_ci, [_pvp, _pvp, ctypes.POINTER(_sz), _pi, _ci]),
     "mi355_fp_equal_collect": (_ci, [_ci, _ci, _vp]),
+    "mi355_fp_equal_read": (_ci, [_ci, _ci, _vp]),
+    "mi355_queue_current": (_ci, []),
+    "mi355_mark_record": (_ci, [_ci]),
+    "mi355_mark_wait_queue": (_ci, [_ci, _ci]),
+    "mi355_mark_wait_host": (_ci, [_ci]),
     "mi355_customized_fp": (_ci, [_pplan, _pvp, _pvp]),
     "mi355_customized_fp_batch": (_ci, [_pplan, _ci, _pvp, _pvp]),
     "mi355_plan_extents": (_ci, [_pplan, _pll, _pll, _pi, _pi]),
@@ -155,6 +160,8 @@ FACADE = {
     "mirage_tensor_same_fingerprint": (_ci, [_vp, _vp]),
     "mirage_graph_fingerprint": (_ci, [_vp, _u64, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
+    "mirage_verify_batch_begin": (_vp, [_pvp, _ci, _vp, _u64, _ci]),
+    "mirage_verify_batch_end": (_ci, [_vp, _ci, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_optimize_layout": (_ci, [_vp, ctypes.c_longlong, LAYOUT_COST_FN, _vp,
                                      ctypes.POINTER(MirageLayoutStats)]),
     "mirage_graph_generate_hip_program": (_ci, [_vp, ctypes.c_char_p]),

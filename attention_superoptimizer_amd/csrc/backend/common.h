@@ -54,8 +54,10 @@ struct State {
   uint16_t *exp_tbl = nullptr, *div_p = nullptr, *div_q = nullptr;
   int *flag = nullptr;        // 4-byte device scratch for mi355_fp_equal
   int *flag_host = nullptr;   // pinned mirror
-  int *cmp_slots = nullptr;   // MI355_COMPARE_SLOTS mismatch flags of deferred compares
-  int *cmp_host = nullptr;    // pinned mirror
+  int *cmp_host = nullptr;    // MI355_COMPARE_SLOTS mismatch flags of deferred compares, in
+                              // pinned host memory
+  int *cmp_slots = nullptr;   // the same memory as the device addresses it
+  hipEvent_t marks[MI355_NUM_MARKS][MI355_NUM_QUEUES] = {};
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int max_lds = 65536;
   // staging of batched launches (mi355_customized_fp_batch): per queue a small ring of

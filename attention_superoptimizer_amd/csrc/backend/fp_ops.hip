@@ -11,6 +11,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cstring>
 
 namespace mi355 {
 
@@ -818,14 +819,10 @@ extern "C" int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, in
 }
 
 // ---- deferred compares: many candidates, one synchronisation ----------------------------
-// Slot i of the device array holds "a mismatch was seen"; nothing comes back to the host
-// until the caller collects a range of slots.
-__global__ void clear_slots_kernel(int *slots, int count) {
-  int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < count) {
-    slots[i] = 0;
-  }
-}
+// Slot i holds "a mismatch was seen".  The slots are pinned host memory that the compare
+// kernels write directly (a store only where a mismatch is found), so resetting and reading
+// them needs no launch and no copy; the caller reads a range once it has waited for the
+// compares that target it.
 
 __global__ void fp_differ_kernel(uint16_t const *__restrict__ a, uint16_t const *__restrict__ b,
                                  size_t n, int *slot) {
@@ -882,9 +879,7 @@ extern "C" int mi355_fp_equal_reset(int first_slot, int count) {
                 first_slot + count);
   }
   if (count > 0) {
-    clear_slots_kernel<<<(count + kThreads - 1) / kThreads, kThreads, 0, s.stream()>>>(
-        s.cmp_slots + first_slot, count);
-    MI355_HIP(hipGetLastError());
+    memset(s.cmp_host + first_slot, 0, sizeof(int) * (size_t)count);  // host memory, see common.h
   }
   return MI355_OK;
 }
@@ -950,11 +945,20 @@ extern "C" int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal)
   if (int rc = sync_all_queues()) {  // compares may sit on any queue
     return rc;
   }
-  MI355_HIP(hipMemcpyAsync(s.cmp_host + first_slot, s.cmp_slots + first_slot,
-                           sizeof(int) * (size_t)count, hipMemcpyDeviceToHost, s.stream()));
-  MI355_HIP(hipStreamSynchronize(s.stream()));
+  return mi355_fp_equal_read(first_slot, count, equal);
+}
+
+extern "C" int mi355_fp_equal_read(int first_slot, int count, uint8_t *equal) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (first_slot < 0 || count < 0 || first_slot + count > MI355_COMPARE_SLOTS ||
+      (count > 0 && equal == nullptr)) {
+    return fail(MI355_ERR_INVALID, "compare slots [%d, %d) out of range", first_slot,
+                first_slot + count);
+  }
+  int const volatile *slots = s.cmp_host;
   for (int i = 0; i < count; i++) {
-    equal[i] = s.cmp_host[first_slot + i] == 0 ? 1 : 0;
+    equal[i] = slots[first_slot + i] == 0 ? 1 : 0;
   }
   return MI355_OK;
 }

@@ -4,12 +4,15 @@
 // (src/kernel/device_memory_manager.cu:26-96): one arena allocation, the three
 // fingerprint lookup tables, and the event pairs every profile() uses.
 #include "common.h"
+#include <atomic>
 #include <cstring>
 #include <vector>
 
 namespace mi355 {
 
 static State g_state;
+// which queues have recorded under each mark since its last host wait
+static std::atomic<unsigned> g_mark_bits[MI355_NUM_MARKS];
 thread_local char g_error[512] = "";  // per host thread: several may enqueue side by side
 
 State &state() { return g_state; }
@@ -109,9 +112,16 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
   MI355_HIP(hipMemcpy(s.div_q, divq_h, sizeof(divq_h), hipMemcpyHostToDevice));
   MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.flag), 256));
   MI355_HIP(hipHostMalloc(reinterpret_cast<void **>(&s.flag_host), 256, hipHostMallocDefault));
-  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.cmp_slots), sizeof(int) * MI355_COMPARE_SLOTS));
   MI355_HIP(hipHostMalloc(reinterpret_cast<void **>(&s.cmp_host), sizeof(int) * MI355_COMPARE_SLOTS,
                           hipHostMallocDefault));
+  memset(s.cmp_host, 0, sizeof(int) * MI355_COMPARE_SLOTS);
+  MI355_HIP(hipHostGetDevicePointer(reinterpret_cast<void **>(&s.cmp_slots), s.cmp_host, 0));
+  for (int m = 0; m < MI355_NUM_MARKS; m++) {
+    for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+      MI355_HIP(hipEventCreateWithFlags(&s.marks[m][q], hipEventDisableTiming));
+    }
+    g_mark_bits[m].store(0);
+  }
   MI355_HIP(hipEventCreate(&s.ev0));
   MI355_HIP(hipEventCreate(&s.ev1));
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
@@ -151,8 +161,12 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipFree(s.exp_tbl));
   MI355_HIP(hipFree(s.flag));
   MI355_HIP(hipHostFree(s.flag_host));
-  MI355_HIP(hipFree(s.cmp_slots));
   MI355_HIP(hipHostFree(s.cmp_host));
+  for (int m = 0; m < MI355_NUM_MARKS; m++) {
+    for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+      MI355_HIP(hipEventDestroy(s.marks[m][q]));
+    }
+  }
   MI355_HIP(hipFree(s.scratch_base));
   MI355_HIP(hipFree(s.planes_base));
   s.planes_base = nullptr;
@@ -185,6 +199,41 @@ extern "C" int mi355_get_device_info(mi355_device_info *info) {
   info->memory_clock_mhz = prop.memoryClockRate / 1000;
   info->lds_bytes_per_block = state().max_lds;
   info->total_memory = prop.totalGlobalMem;
+  return MI355_OK;
+}
+
+extern "C" int mi355_mark_record(int mark) {
+  MI355_REQUIRE_INIT();
+  if (mark < 0 || mark >= MI355_NUM_MARKS) {
+    return fail(MI355_ERR_INVALID, "mark %d out of range", mark);
+  }
+  MI355_HIP(hipEventRecord(state().marks[mark][tls_queue], state().stream()));
+  g_mark_bits[mark].fetch_or(1u << tls_queue);
+  return MI355_OK;
+}
+
+extern "C" int mi355_mark_wait_queue(int mark, int queue) {
+  MI355_REQUIRE_INIT();
+  if (mark < 0 || mark >= MI355_NUM_MARKS || queue < 0 || queue >= MI355_NUM_QUEUES) {
+    return fail(MI355_ERR_INVALID, "mark %d / queue %d out of range", mark, queue);
+  }
+  if (queue != tls_queue && (g_mark_bits[mark].load() & (1u << queue)) != 0) {
+    MI355_HIP(hipStreamWaitEvent(state().stream(), state().marks[mark][queue], 0));
+  }
+  return MI355_OK;
+}
+
+extern "C" int mi355_mark_wait_host(int mark) {
+  MI355_REQUIRE_INIT();
+  if (mark < 0 || mark >= MI355_NUM_MARKS) {
+    return fail(MI355_ERR_INVALID, "mark %d out of range", mark);
+  }
+  unsigned const bits = g_mark_bits[mark].exchange(0);
+  for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+    if (bits & (1u << q)) {
+      MI355_HIP(hipEventSynchronize(state().marks[mark][q]));
+    }
+  }
   return MI355_OK;
 }
 
@@ -304,6 +353,8 @@ extern "C" int mi355_queue_select(int queue) {
   tls_queue = queue;
   return MI355_OK;
 }
+
+extern "C" int mi355_queue_current(void) { return tls_queue; }
 
 extern "C" int mi355_memset(void *dst, int value, size_t bytes) {
   MI355_REQUIRE_INIT();

@@ -10,6 +10,11 @@
 
 #include <algorithm>
 #include <chrono>
+#include <condition_variable>
+#include <deque>
+#include <functional>
+#include <memory>
+#include <mutex>
 #include <numeric>
 #include <thread>
 #include <unordered_set>
@@ -255,121 +260,261 @@ static bool comparable(DTensor const &a, DTensor const &b) {
   return true;
 }
 
-void verify_batch(std::vector<kernel::Graph *> const &candidates,
-                  std::vector<DTensor> const &reference_outputs, uint64_t input_seed,
-                  std::vector<uint8_t> &equal, VerifyStats *stats) {
-  kernel::require_device("verify_batch");
-  size_t const n = candidates.size(), no = reference_outputs.size();
-  equal.assign(n, 0);
-  struct Pending {
-    std::vector<DTensor> outputs;
-    int first_slot = -1;  // no*no slots, row = reference output, column = candidate output
+// ---- worker threads ----------------------------------------------------------------
+// One host thread per backend queue, started on first use and kept: candidate i of a batch
+// is lowered and enqueued by thread i % queues.  A queue is only ever driven by its own
+// thread (and by the caller's thread for queue 0 while no batch is being enqueued), which is
+// what the backend's per-queue staging memory needs.
+namespace {
+
+class WorkerPool {
+public:
+  static WorkerPool &get() {
+    static WorkerPool pool;
+    return pool;
+  }
+  void post(int worker, std::function<void()> job) {
+    Worker &w = *workers_[(size_t)worker];
+    {
+      std::lock_guard<std::mutex> lock(w.m);
+      w.jobs.push_back(std::move(job));
+    }
+    w.cv.notify_one();
+  }
+  int size() const { return (int)workers_.size(); }
+
+private:
+  struct Worker {
+    std::thread th;
+    std::mutex m;
+    std::condition_variable cv;
+    std::deque<std::function<void()>> jobs;
+    bool stop = false;
   };
-  std::vector<Pending> pend(n);
-  int slots = 0;
-  for (size_t i = 0; i < n; i++) {
-    pend[i].outputs = graph_outputs(*candidates[i]);
-    if (pend[i].outputs.size() == no) {
-      pend[i].first_slot = slots;
-      slots += (int)(no * no);
+  std::vector<std::unique_ptr<Worker>> workers_;
+
+  WorkerPool() {
+    for (int i = 0; i < MI355_NUM_QUEUES; i++) {
+      workers_.emplace_back(new Worker);
+      Worker *w = workers_.back().get();
+      w->th = std::thread([w, i]() {
+        MI355_CALL(mi355_queue_select(i));
+        for (;;) {
+          std::function<void()> job;
+          {
+            std::unique_lock<std::mutex> lock(w->m);
+            w->cv.wait(lock, [w]() { return w->stop || !w->jobs.empty(); });
+            if (w->jobs.empty()) {
+              return;
+            }
+            job = std::move(w->jobs.front());
+            w->jobs.pop_front();
+          }
+          job();
+        }
+      });
     }
   }
-  MIRAGE_CHECK(slots <= MI355_COMPARE_SLOTS, "too many compares for one verify_batch call");
-  auto const t0 = std::chrono::steady_clock::now();
-  MI355_CALL(mi355_fp_equal_reset(0, slots));
-  // Candidates are independent: deal them over the backend's queues so their small
-  // kernels overlap.  Everything enqueued so far (the reference's fingerprints, the slot
-  // reset) must be complete before another queue may depend on it.
-  MI355_CALL(mi355_sync());
-  // which (reference, candidate) output pairs can be equal at all
-  std::vector<uint8_t> possible((size_t)slots, 0);
-  // one host thread per queue: candidate i is lowered and enqueued by thread i % queues
-  int const workers = (int)std::min<size_t>(MI355_NUM_QUEUES, n);
-  std::vector<VerifyStats> local((size_t)std::max(workers, 1));
-  auto work = [&](int w) {
-    MI355_CALL(mi355_queue_select(w));
-    std::vector<kernel::Graph *> mine;
-    for (size_t i = (size_t)w; i < n; i += (size_t)workers) {
-      mine.push_back(candidates[i]);
+  ~WorkerPool() {
+    for (auto &w : workers_) {
+      {
+        std::lock_guard<std::mutex> lock(w->m);
+        w->stop = true;
+      }
+      w->cv.notify_one();
+      w->th.join();
     }
-    fingerprint_graphs(mine, input_seed, &local[w]);
-    // this worker's compares, MI355_MAX_COMPARE_PAIRS per launch
-    uint16_t const *ca[MI355_MAX_COMPARE_PAIRS], *cb[MI355_MAX_COMPARE_PAIRS];
-    size_t cn[MI355_MAX_COMPARE_PAIRS];
-    int cs[MI355_MAX_COMPARE_PAIRS];
-    int pairs = 0;
-    auto flush = [&]() {
-      if (pairs > 0) {
-        MI355_CALL(mi355_fp_equal_enqueue_many(ca, cb, cn, cs, pairs));
-        pairs = 0;
+  }
+};
+
+struct Pending {
+  std::vector<DTensor> outputs;
+  int first_slot = -1;  // no*no slots, row = reference output, column = candidate output
+};
+
+}  // namespace
+
+struct VerifyTicket {
+  std::vector<kernel::Graph *> candidates;
+  std::vector<DTensor> reference_outputs;
+  kernel::Graph *reference = nullptr;  // fingerprinted by worker 0 when set
+  uint64_t input_seed = 0;
+  std::vector<Pending> pend;
+  std::vector<uint8_t> possible;  // which (reference, candidate) output pairs can be equal at all
+  int first_slot = 0, slots = 0;
+  int mark_reference = 0, mark_done = 0;
+  int reference_queue = 0;
+  int workers = 0;
+  std::vector<VerifyStats> local;
+  std::mutex m;
+  std::condition_variable cv;
+  bool reference_recorded = false;
+  int enqueueing = 0;
+  std::chrono::steady_clock::time_point t_begin, t_enqueued;
+};
+
+// Slot ranges and marks of the batches in flight come from rings: a range or a mark is reused
+// only MI355_COMPARE_SLOTS compares / 32 batches later.
+static std::mutex g_ring_mutex;
+static int g_next_slot = 0;
+static int g_next_ticket = 0;
+
+VerifyTicket *verify_batch_begin(std::vector<kernel::Graph *> const &candidates,
+                                 std::vector<DTensor> const &reference_outputs,
+                                 uint64_t input_seed, kernel::Graph *reference_to_fingerprint) {
+  kernel::require_device("verify_batch");
+  std::unique_ptr<VerifyTicket> t(new VerifyTicket);
+  t->t_begin = std::chrono::steady_clock::now();
+  t->candidates = candidates;
+  t->reference_outputs = reference_outputs;
+  t->reference = reference_to_fingerprint;
+  t->input_seed = input_seed;
+  size_t const n = candidates.size(), no = reference_outputs.size();
+  t->pend.resize(n);
+  for (size_t i = 0; i < n; i++) {
+    t->pend[i].outputs = graph_outputs(*candidates[i]);
+    if (t->pend[i].outputs.size() == no) {
+      t->pend[i].first_slot = t->slots;
+      t->slots += (int)(no * no);
+    }
+  }
+  MIRAGE_CHECK(t->slots <= MI355_COMPARE_SLOTS, "too many compares for one verify_batch call");
+  {
+    std::lock_guard<std::mutex> lock(g_ring_mutex);
+    if (g_next_slot + t->slots > MI355_COMPARE_SLOTS) {
+      g_next_slot = 0;
+    }
+    t->first_slot = g_next_slot;
+    g_next_slot += t->slots;
+    int const ticket = g_next_ticket;
+    g_next_ticket = (g_next_ticket + 1) % (MI355_NUM_MARKS / 2);
+    t->mark_reference = 2 * ticket;
+    t->mark_done = 2 * ticket + 1;
+  }
+  for (Pending &p : t->pend) {
+    if (p.first_slot >= 0) {
+      p.first_slot += t->first_slot;
+    }
+  }
+  t->possible.assign((size_t)t->slots, 0);
+  MI355_CALL(mi355_fp_equal_reset(t->first_slot, t->slots));
+  WorkerPool &pool = WorkerPool::get();
+  t->workers = (int)std::min<size_t>((size_t)pool.size(), std::max<size_t>(n, 1));
+  t->local.resize((size_t)t->workers);
+  t->enqueueing = t->workers;
+  if (t->reference == nullptr) {
+    // the caller has enqueued the reference graph's fingerprints on its own queue: the
+    // compares of the other queues start after them
+    t->reference_queue = mi355_queue_current();
+    MI355_CALL(mi355_mark_record(t->mark_reference));
+    t->reference_recorded = true;
+  }
+  VerifyTicket *const T = t.get();
+  for (int w = 0; w < T->workers; w++) {
+    pool.post(w, [T, w]() {
+      size_t const n = T->candidates.size(), no = T->reference_outputs.size();
+      if (w == 0 && T->reference != nullptr) {
+        fingerprint_graphs({T->reference}, T->input_seed, &T->local[0]);
+        MI355_CALL(mi355_mark_record(T->mark_reference));
+        {
+          std::lock_guard<std::mutex> lock(T->m);
+          T->reference_recorded = true;
+        }
+        T->cv.notify_all();
       }
-    };
-    for (size_t i = (size_t)w; i < n; i += (size_t)workers) {
-      if (pend[i].first_slot < 0) {
-        continue;
+      std::vector<kernel::Graph *> mine;
+      for (size_t i = (size_t)w; i < n; i += (size_t)T->workers) {
+        mine.push_back(T->candidates[i]);
       }
-      for (size_t r = 0; r < no; r++) {
-        for (size_t c = 0; c < no; c++) {
-          if (!comparable(reference_outputs[r], pend[i].outputs[c])) {
-            continue;
+      fingerprint_graphs(mine, T->input_seed, &T->local[(size_t)w]);
+      {
+        std::unique_lock<std::mutex> lock(T->m);
+        T->cv.wait(lock, [T]() { return T->reference_recorded; });
+      }
+      MI355_CALL(mi355_mark_wait_queue(T->mark_reference, T->reference_queue));
+      // this worker's compares, MI355_MAX_COMPARE_PAIRS per launch
+      uint16_t const *ca[MI355_MAX_COMPARE_PAIRS], *cb[MI355_MAX_COMPARE_PAIRS];
+      size_t cn[MI355_MAX_COMPARE_PAIRS];
+      int cs[MI355_MAX_COMPARE_PAIRS];
+      int pairs = 0;
+      auto flush = [&]() {
+        if (pairs > 0) {
+          MI355_CALL(mi355_fp_equal_enqueue_many(ca, cb, cn, cs, pairs));
+          pairs = 0;
+        }
+      };
+      for (size_t i = (size_t)w; i < n; i += (size_t)T->workers) {
+        if (T->pend[i].first_slot < 0) {
+          continue;
+        }
+        for (size_t r = 0; r < no; r++) {
+          for (size_t c = 0; c < no; c++) {
+            if (!comparable(T->reference_outputs[r], T->pend[i].outputs[c])) {
+              continue;
+            }
+            int const slot = T->pend[i].first_slot + (int)(r * no + c);
+            T->possible[(size_t)(slot - T->first_slot)] = 1;
+            ca[pairs] = T->reference_outputs[r].fp_ptr;
+            cb[pairs] = T->pend[i].outputs[c].fp_ptr;
+            cn[pairs] = T->reference_outputs[r].num_elements();
+            cs[pairs] = slot;
+            if (++pairs == MI355_MAX_COMPARE_PAIRS) {
+              flush();
+            }
+            T->local[(size_t)w].compares++;
+            T->local[(size_t)w].fp_bytes += 2 * (long long)T->reference_outputs[r].fingerprint_size();
           }
-          int const slot = pend[i].first_slot + (int)(r * no + c);
-          possible[slot] = 1;
-          ca[pairs] = reference_outputs[r].fp_ptr;
-          cb[pairs] = pend[i].outputs[c].fp_ptr;
-          cn[pairs] = reference_outputs[r].num_elements();
-          cs[pairs] = slot;
-          if (++pairs == MI355_MAX_COMPARE_PAIRS) {
-            flush();
-          }
-          local[w].compares++;
-          local[w].fp_bytes += 2 * (long long)reference_outputs[r].fingerprint_size();
         }
       }
-    }
-    flush();
-  };
-  {
-    std::vector<std::thread> threads;
-    for (int w = 1; w < workers; w++) {
-      threads.emplace_back(work, w);
-    }
-    if (workers > 0) {
-      work(0);
-    }
-    for (std::thread &t : threads) {
-      t.join();
-    }
+      flush();
+      MI355_CALL(mi355_mark_record(T->mark_done));
+      {
+        std::lock_guard<std::mutex> lock(T->m);
+        if (--T->enqueueing == 0) {
+          T->t_enqueued = std::chrono::steady_clock::now();
+        }
+      }
+      T->cv.notify_all();
+    });
   }
+  return t.release();
+}
+
+void verify_batch_end(VerifyTicket *ticket, std::vector<uint8_t> &equal, VerifyStats *stats) {
+  std::unique_ptr<VerifyTicket> t(ticket);
+  size_t const n = t->candidates.size(), no = t->reference_outputs.size();
+  equal.assign(n, 0);
+  auto const t_wait = std::chrono::steady_clock::now();
+  {
+    std::unique_lock<std::mutex> lock(t->m);
+    t->cv.wait(lock, [&]() { return t->enqueueing == 0; });
+  }
+  MI355_CALL(mi355_mark_wait_host(t->mark_done));
+  std::vector<uint8_t> same((size_t)t->slots, 0);
+  MI355_CALL(mi355_fp_equal_read(t->first_slot, t->slots, same.data()));
   if (stats != nullptr) {
-    for (VerifyStats const &l : local) {
+    auto const t_done = std::chrono::steady_clock::now();
+    for (VerifyStats const &l : t->local) {
       stats->kernel_ops += l.kernel_ops;
       stats->customized_ops += l.customized_ops;
       stats->compares += l.compares;
       stats->fp_bytes += l.fp_bytes;
       stats->matmul_macs += l.matmul_macs;
     }
-  }
-  MI355_CALL(mi355_queue_select(0));
-  auto const t1 = std::chrono::steady_clock::now();
-  std::vector<uint8_t> same((size_t)slots, 0);
-  MI355_CALL(mi355_fp_equal_collect(0, slots, same.data()));
-  if (stats != nullptr) {
-    auto const t2 = std::chrono::steady_clock::now();
-    stats->enqueue_seconds += std::chrono::duration<double>(t1 - t0).count();
-    stats->wait_seconds += std::chrono::duration<double>(t2 - t1).count();
+    stats->enqueue_seconds += std::chrono::duration<double>(t->t_enqueued - t->t_begin).count();
+    stats->wait_seconds += std::chrono::duration<double>(t_done - std::max(t_wait, t->t_enqueued)).count();
   }
   std::vector<int> perm(no);
   for (size_t i = 0; i < n; i++) {
-    if (pend[i].first_slot < 0) {
+    if (t->pend[i].first_slot < 0) {
       continue;
     }
     std::iota(perm.begin(), perm.end(), 0);
     do {  // search.cc:605-609: any output permutation may match
       bool ok = true;
       for (size_t r = 0; r < no && ok; r++) {
-        int const slot = pend[i].first_slot + (int)(r * no + perm[r]);
-        ok = possible[slot] && same[slot];
+        int const slot = t->pend[i].first_slot + (int)(r * no + perm[r]);
+        ok = t->possible[(size_t)(slot - t->first_slot)] && same[(size_t)(slot - t->first_slot)];
       }
       if (ok) {
         equal[i] = 1;
@@ -377,6 +522,12 @@ void verify_batch(std::vector<kernel::Graph *> const &candidates,
       }
     } while (std::next_permutation(perm.begin(), perm.end()));
   }
+}
+
+void verify_batch(std::vector<kernel::Graph *> const &candidates,
+                  std::vector<DTensor> const &reference_outputs, uint64_t input_seed,
+                  std::vector<uint8_t> &equal, VerifyStats *stats) {
+  verify_batch_end(verify_batch_begin(candidates, reference_outputs, input_seed, nullptr), equal, stats);
 }
 
 }  // namespace search
@@ -413,6 +564,32 @@ int mirage_graph_fingerprint(void *graph, unsigned long long input_seed,
 
 // Candidates are compared with the outputs of `reference` (which must already be
 // fingerprinted, e.g. by mirage_graph_fingerprint with the same seed).
+// Two-call form: several batches may be in flight.  `fingerprint_reference` != 0: the
+// reference graph is fingerprinted as part of the batch (on a worker's queue); otherwise it
+// must already have been, on the calling thread's queue.  The candidates, the reference and
+// their tensors stay alive until the matching mirage_verify_batch_end returns.
+void *mirage_verify_batch_begin(void *const *candidates, int n, void *reference,
+                                unsigned long long input_seed, int fingerprint_reference) {
+  std::vector<mirage::kernel::Graph *> c(n);
+  for (int i = 0; i < n; i++) {
+    c[i] = static_cast<mirage::kernel::Graph *>(candidates[i]);
+  }
+  mirage::kernel::Graph *ref = static_cast<mirage::kernel::Graph *>(reference);
+  return mirage::search::verify_batch_begin(c, mirage::search::graph_outputs(*ref), input_seed,
+                                            fingerprint_reference ? ref : nullptr);
+}
+
+int mirage_verify_batch_end(void *ticket, int n, unsigned char *equal, mirage_verify_stats *stats) {
+  std::vector<uint8_t> eq;
+  mirage::search::VerifyStats s;
+  mirage::search::verify_batch_end(static_cast<mirage::search::VerifyTicket *>(ticket), eq, &s);
+  for (int i = 0; i < n && i < (int)eq.size(); i++) {
+    equal[i] = eq[i];
+  }
+  export_stats(s, stats);
+  return 0;
+}
+
 int mirage_verify_batch(void *const *candidates, int n, void *reference,
                         unsigned long long input_seed, unsigned char *equal,
                         mirage_verify_stats *stats) {

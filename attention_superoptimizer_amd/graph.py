@@ -301,6 +301,31 @@ def verify_batch(candidates: Sequence["KNGraph"], reference: "KNGraph", input_se
     return [bool(eq[i]) for i in range(n)], _stats(st)
 
 
+def verify_batch_begin(candidates: Sequence["KNGraph"], reference: "KNGraph", input_seed: int = 0,
+                       fingerprint_reference: bool = True):
+    """First half of verify_batch: lowers and enqueues everything from the runtime's worker
+    threads and returns a ticket at once, so that the caller can build and submit the next
+    batch while the device works on this one.  With `fingerprint_reference` the reference
+    graph is fingerprinted as part of the batch.  The graphs must stay open until
+    verify_batch_end(ticket) has returned."""
+    n = len(candidates)
+    arr = (ctypes.c_void_p * n)(*[c._g for c in candidates])
+    handle = N.runtime().mirage_verify_batch_begin(arr, n, reference._g, input_seed,
+                                                   1 if fingerprint_reference else 0)
+    assert handle
+    return (handle, n)
+
+
+def verify_batch_end(ticket):
+    """Second half: waits for this batch's compares only.  Returns (list of bool, stats)."""
+    handle, n = ticket
+    eq = (ctypes.c_ubyte * n)()
+    st = N.MirageVerifyStats()
+    rc = N.runtime().mirage_verify_batch_end(handle, n, eq, ctypes.byref(st))
+    assert rc == 0
+    return [bool(eq[i]) for i in range(n)], _stats(st)
+
+
 def build_from_spec(spec: List[dict], graph: Optional[KNGraph] = None):
     """Builds a graph spec (see workloads.py) through the host API.
     Returns (graph, per-operator lists of output tensors)."""

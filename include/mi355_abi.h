@@ -142,9 +142,24 @@ int mi355_sync(void);
  * fills the chip with its many small kernels (the reference has one stream and a
  * cudaDeviceSynchronize after every fingerprint launch, customized_kernel.cu:676).
  * mi355_sync, the memcpy calls and mi355_fp_equal_collect wait for all queues.  The
- * caller orders dependent work itself: same queue, or a mi355_sync in between. */
+ * caller orders dependent work itself: same queue, a mi355_sync in between, or a mark.
+ * A queue is driven by one host thread at a time (several entry points enqueue more than
+ * one launch and keep per-queue staging memory between them). */
 #define MI355_NUM_QUEUES 4
 int mi355_queue_select(int queue);
+int mi355_queue_current(void); /* the calling thread's queue */
+/* Marks order work across queues and let the host wait for part of the work only (the
+ * reference has one stream and device-wide syncs, so no counterpart).  mi355_mark_record:
+ * everything enqueued so far on the calling thread's queue is "before" (mark, that queue).
+ * mi355_mark_wait_queue: work enqueued from now on the calling thread's queue starts after
+ * what `queue` recorded under `mark` (a device-side wait; the host does not block; a no-op
+ * if nothing was recorded).  mi355_mark_wait_host: blocks until everything recorded under
+ * `mark`, on any queue, since the last host wait on it has completed.  A mark is reusable
+ * after its host wait. */
+#define MI355_NUM_MARKS 64
+int mi355_mark_record(int mark);
+int mi355_mark_wait_queue(int mark, int queue);
+int mi355_mark_wait_host(int mark);
 
 /* ---- fingerprint path (uint16 over Z_25651, integer only) ------------------ */
 /* init_input_fingerprint, src/kernel/cuda/input_kernel.cu:56-72: fp[i] = i % 25651 */
@@ -194,7 +209,7 @@ int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, int *equal);
 /* The same compare without the round trip, for verifying many candidates
  * (the verify loop of src/search/search.cc:569-623 calls has_same_fingerprint once per
  * candidate output and blocks each time).  The backend keeps MI355_COMPARE_SLOTS result
- * slots on the device: reset a range, enqueue one compare per slot behind the
+ * slots: reset a range, enqueue one compare per slot behind the
  * fingerprint kernels on the backend stream, then collect the range with a single
  * synchronisation; equal[i] = 1/0 for slot first_slot + i.  A slot that several
  * compares target reports their conjunction. */
@@ -207,6 +222,12 @@ int mi355_fp_equal_enqueue(uint16_t const *a, uint16_t const *b, size_t n, int s
 int mi355_fp_equal_enqueue_many(uint16_t const *const *a, uint16_t const *const *b,
                                 size_t const *n, int const *slots, int count);
 int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal);
+/* The slots live in host memory that the device writes directly: mi355_fp_equal_reset
+ * clears a range at once, on the host (the range must not be the target of compares still
+ * in flight), and mi355_fp_equal_read reports a range WITHOUT waiting for anything: for
+ * callers that have waited for exactly the compares they care about (mi355_mark_wait_host)
+ * while other batches are still running. */
+int mi355_fp_equal_read(int first_slot, int count, uint8_t *equal);
 /* KNCustomizedOp::fingerprint + compute_customizedop_fingerprint,
  * src/kernel/cuda/customized_kernel.cu:307-603,655-678 */
 int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,

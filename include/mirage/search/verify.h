@@ -44,6 +44,22 @@ void verify_batch(std::vector<mirage::kernel::Graph *> const &candidates,
                   uint64_t input_seed, std::vector<uint8_t> &equal,
                   VerifyStats *stats = nullptr);
 
+// The same in two calls, so that several batches can be in flight: while the device works
+// on one, the caller builds and submits the next.  verify_batch_begin lowers and enqueues
+// everything from worker threads (one per backend queue) and returns at once;
+// verify_batch_end waits for exactly this batch's compares and fills `equal`.
+// `reference_to_fingerprint` != nullptr: that graph (whose outputs `reference_outputs` are)
+// is fingerprinted as part of the batch; nullptr: the caller has already enqueued its
+// fingerprints on its own queue.  Between the two calls the caller must not enqueue device
+// work on the worker queues itself, and the candidates, the reference and their tensors
+// must stay alive.  At most 32 batches, MI355_COMPARE_SLOTS compares in all, in flight.
+struct VerifyTicket;
+VerifyTicket *verify_batch_begin(std::vector<mirage::kernel::Graph *> const &candidates,
+                                 std::vector<mirage::kernel::DTensor> const &reference_outputs,
+                                 uint64_t input_seed,
+                                 mirage::kernel::Graph *reference_to_fingerprint = nullptr);
+void verify_batch_end(VerifyTicket *ticket, std::vector<uint8_t> &equal, VerifyStats *stats = nullptr);
+
 // fingerprint() of every operator of one graph with the same input convention.
 void fingerprint_graph(mirage::kernel::Graph const &g, uint64_t input_seed,
                        VerifyStats *stats = nullptr);
