@@ -80,6 +80,84 @@ def test_verify_batch_full_size_verdicts(rt):
         assert verdicts == [c["expect_equal"] for c in prob["candidates"]], prob["family"]
 
 
+def test_verify_batches_in_flight_match_one_at_a_time(rt):
+    """Four submissions in flight (verify_batch_begin x 4, then verify_batch_end x 4, the
+    reference graphs fingerprinted as part of their batches): same verdicts and the same
+    candidate outputs as one blocking verify_batch per problem; repeated so that marks and
+    compare-slot ranges are reused."""
+    probs = C.generate(num_problems=8, per_problem=12, seed=0xF11E, max_dim=256)
+    want = {}
+    for k, prob in enumerate(probs):
+        verdicts, outs, ref_out = _verify_problem(rt, prob)
+        assert verdicts == [c["expect_equal"] for c in prob["candidates"]]
+        want[k] = (verdicts, outs, ref_out)
+    for _ in range(5):
+        for first in range(0, len(probs), 4):
+            built = []
+            try:
+                for prob in probs[first:first + 4]:
+                    ref_g, ref_vals = rt.build_from_spec(prob["reference"])
+                    cands = [rt.build_from_spec(c["spec"]) for c in prob["candidates"]]
+                    built.append((prob, ref_g, ref_vals, cands))
+                tickets = [rt.verify_batch_begin([g for g, _ in cands], ref_g, prob["input_seed"])
+                           for prob, ref_g, _, cands in built]
+                for k, (ticket, (prob, ref_g, ref_vals, cands)) in enumerate(zip(tickets, built)):
+                    verdicts, stats = rt.verify_batch_end(ticket)
+                    w_verdicts, w_outs, w_ref = want[first + k]
+                    assert verdicts == w_verdicts
+                    assert stats["compares"] == len(cands)
+                    ref_out = [t.read_fingerprint() for t in _outputs(prob["reference"], ref_vals)]
+                    assert all(np.array_equal(a, b) for a, b in zip(ref_out, w_ref))
+                    for c, (_, vals), w in zip(prob["candidates"], cands, w_outs):
+                        got = [t.read_fingerprint() for t in _outputs(c["spec"], vals)]
+                        assert all(np.array_equal(a, b) for a, b in zip(got, w))
+            finally:
+                for prob, ref_g, _, cands in reversed(built):
+                    for g, _ in reversed(cands):
+                        g.close()
+                    ref_g.close()
+
+
+def test_marks_order_queues_and_report_only_their_work(rt, abi):
+    """A compare enqueued on queue 1 behind a mark that queue 0 recorded after filling its
+    operand sees the filled values; waiting for the mark queue 1 recorded is enough to read
+    the slot."""
+    import ctypes
+    n = 1 << 20
+    spec = [{"op": "input", "dims": [n]}, {"op": "input", "dims": [n]}]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        a, b = vals[0][0], vals[1][0]
+        a.write_fingerprint(np.zeros(n, np.uint16))
+        b.write_fingerprint(np.ones(n, np.uint16))
+        assert abi.mi355_sync() == 0
+        assert abi.mi355_queue_current() == 0
+        for rep in range(3):
+            slot = 60000 + rep
+            assert abi.mi355_fp_equal_reset(slot, 1) == 0
+            seed = 31 + rep
+            for t in (a, b):  # queue 0: both tensors get the same sequence
+                assert abi.mi355_fp_fill_uniform(ctypes.c_void_p(t.device_ptr(True)), n, seed) == 0
+            assert abi.mi355_mark_record(10) == 0
+            assert abi.mi355_queue_select(1) == 0
+            try:
+                assert abi.mi355_mark_wait_queue(10, 0) == 0
+                assert abi.mi355_fp_equal_enqueue(ctypes.c_void_p(a.device_ptr(True)),
+                                                  ctypes.c_void_p(b.device_ptr(True)), n, slot) == 0
+                assert abi.mi355_mark_record(11) == 0
+            finally:
+                assert abi.mi355_queue_select(0) == 0
+            assert abi.mi355_mark_wait_host(11) == 0
+            eq = (ctypes.c_ubyte * 1)()
+            assert abi.mi355_fp_equal_read(slot, 1, eq) == 0
+            assert eq[0] == 1
+            assert abi.mi355_mark_wait_host(10) == 0
+        assert abi.mi355_mark_record(64) != 0 and abi.mi355_mark_wait_queue(0, 4) != 0
+    finally:
+        assert abi.mi355_sync() == 0
+        g.close()
+
+
 def test_verify_batch_iota_inputs_and_output_count(rt):
     """input_seed 0 = the reference's `idx % 25651` inputs; a candidate with a different
     number of outputs is rejected without a compare."""
