@@ -333,11 +333,15 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
 // of them (one per 16-lane group), so tiles of 16 or 32 k pair up across iterations.  Tile
 // origins come from the plan's own strides, as byte strides into the blocked planes.  A
 // wavefront owns 32 x 32 outputs at a time; a tile with fewer than three such pieces shares
-// its chunk sequence between wavefronts and adds their sums through `part`.
+// its chunk sequence between wavefronts and adds their sums through `part`.  (bx, by) is the
+// first of pl_group[0] x pl_group[1] logical blocks whose tiles the workgroup treats as one
+// tile of gy * m rows and gx * n columns: strip s of its rows belongs to block by + s / (m / 16).
 __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *part, int bx, int by,
                                                    int bz, int split) {
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]], &so = P.ops[3];
-  int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
+  int const bm = P.t[la.dst].rows, kt = P.t[la.dst].cols, bn = P.t[lb.dst].cols;
+  int const m = bm * P.pl_group[1], n = bn * P.pl_group[0];  // the grouped tile
+  int const spb_m = bm / 16, spb_n = bn / 16;                // strips per block
   int const cpi = kt / 16;  // chunks per iteration
   int const F = P.forloop_range;
   int const it_begin = (int)((long long)F * split / P.splits);
@@ -350,15 +354,17 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
   int const dq_it = 4 / cpi, dq_c = 4 % cpi;
   int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
   int const ways = mt >= 3 ? 1 : (mt == 2 ? 2 : 4);  // wavefronts sharing one piece's chunks
-  uint16_t *gout = (P.splits > 1 ? P.part[so.io] + (long long)split * P.part_stride[so.io]
-                                 : static_cast<uint16_t *>(P.out[so.io]));
-  {
-    int const row0 = bx * so.row_bs[0] + by * so.row_bs[1] + bz * so.row_bs[2];
-    int const col0 = bx * so.col_bs[0] + by * so.col_bs[1] + bz * so.col_bs[2];
-    long long const base = (long long)bx * so.g_bs[0] + (long long)by * so.g_bs[1] +
+  uint16_t *const gout = (P.splits > 1 ? P.part[so.io] + (long long)split * P.part_stride[so.io]
+                                       : static_cast<uint16_t *>(P.out[so.io]));
+  // element offset of the output tile of logical block (bx + dx, by + dy, bz)
+  auto out_origin = [&](int dx, int dy) {
+    int const x = bx + dx, y = by + dy;
+    int const row0 = x * so.row_bs[0] + y * so.row_bs[1] + bz * so.row_bs[2];
+    int const col0 = x * so.col_bs[0] + y * so.col_bs[1] + bz * so.col_bs[2];
+    long long const base = (long long)x * so.g_bs[0] + (long long)y * so.g_bs[1] +
                            (long long)bz * so.g_bs[2];
-    gout += base + (long long)row0 * so.d_cols + col0;
-  }
+    return base + (long long)row0 * so.d_cols + col0;
+  };
   int8_t const *const pa = P.pl[0], *const qa = P.pl[1], *const pb = P.pl[2], *const qb = P.pl[3];
   for (int t = ways == 1 ? wave : wave / ways; t < mt; t += 4) {
     int const ks = ways == 1 ? 0 : wave % ways;
@@ -369,8 +375,9 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
     int a_base[2], b_base[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      a_base[i] = a0 + (row_m / 16 + (i ? i1 : 0)) * P.pl_a[4] + r * 16;
-      b_base[i] = b0 + (col_n / 16 + (i ? j1 : 0)) * P.pl_b[4] + r * 16;
+      int const sa = row_m / 16 + (i ? i1 : 0), sb = col_n / 16 + (i ? j1 : 0);
+      a_base[i] = a0 + (sa / spb_m) * P.pl_a[1] + (sa % spb_m) * P.pl_a[4] + r * 16;
+      b_base[i] = b0 + (sb / spb_n) * P.pl_b[0] + (sb % spb_n) * P.pl_b[4] + r * 16;
     }
     // this lane's chunk of step s: number 4 s + g of the sequence
     int q = 4 * s_begin + g;
@@ -444,8 +451,10 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
       uint2 w;
       w.x = z[0] | (z[1] << 16);
       w.y = z[2] | (z[3] << 16);
-      *reinterpret_cast<uint2 *>(gout + (long long)(row_m + 16 * i + r) * so.d_cols + col_n + 16 * jn +
-                                 4 * g) = w;
+      int const row = row_m + 16 * i + r, col = col_n + 16 * jn + 4 * g;  // in the grouped tile
+      int const dy = row / bm, dx = col / bn;
+      *reinterpret_cast<uint2 *>(gout + out_origin(dx, dy) + (long long)(row - dy * bm) * so.d_cols +
+                                 (col - dx * bn)) = w;
     };
     if (ways == 1) {
 #pragma unroll
@@ -499,7 +508,9 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
 
 __global__ __launch_bounds__(kThreads) void fp_mfma_gemm_kernel(DevProgram const P) {
   __shared__ int part[kFpMfmaLdsBytes / 4];
-  fp_mfma_gemm_block(P, part, blockIdx.x % P.grid[0], blockIdx.y, blockIdx.z, blockIdx.x / P.grid[0]);
+  int const gx = P.grid[0] / P.pl_group[0];
+  fp_mfma_gemm_block(P, part, (blockIdx.x % gx) * P.pl_group[0], blockIdx.y * P.pl_group[1], blockIdx.z,
+                     blockIdx.x / gx);
 }
 
 // Many programs in one launch: workgroup -> program by a prefix table, the program record
@@ -525,11 +536,11 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_gemm_multi_kernel(
   __syncthreads();
   DevProgram const &P = *reinterpret_cast<DevProgram const *>(lds + kFpMfmaLdsBytes);
   int v = w - first_block[lo];
-  int const gx = P.grid[0] * P.splits;
-  int const x = v % gx;
-  v /= gx;
-  fp_mfma_gemm_block(P, reinterpret_cast<int *>(lds), x % P.grid[0], v % P.grid[1], v / P.grid[1],
-                     x / P.grid[0]);
+  int const gx = P.grid[0] / P.pl_group[0], gy = P.grid[1] / P.pl_group[1];
+  int const x = v % (gx * P.splits);
+  v /= gx * P.splits;
+  fp_mfma_gemm_block(P, reinterpret_cast<int *>(lds), (x % gx) * P.pl_group[0], (v % gy) * P.pl_group[1],
+                     v / gy, x / gx);
 }
 
 inline size_t round_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
@@ -772,6 +783,22 @@ void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
   }
   P.fg[5] = 1;
   P.lds_bytes = kFpMfmaLdsBytes;
+  // group neighbouring blocks of small tiles up to 64 x 64 outputs per workgroup, as long as
+  // the program keeps a few hundred workgroups
+  P.pl_group[0] = P.pl_group[1] = 1;
+  int const m = P.t[la.dst].rows, n = P.t[lb.dst].cols;
+  if (P.pl_a[0] == 0 && P.pl_b[1] == 0) {
+    long long blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
+    auto grow = [&](int which, int tile) {
+      int &g = P.pl_group[which];
+      while (tile * g * 2 <= 64 && P.grid[which] % (g * 2) == 0 && blocks / 2 >= 256) {
+        g *= 2;
+        blocks /= 2;
+      }
+    };
+    grow(1, m);
+    grow(0, n);
+  }
 }
 
 int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream) {
@@ -821,7 +848,7 @@ int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream) {
   if (int rc = fp_mfma_split_programs(&one, 1, stream)) {
     return rc;
   }
-  dim3 grid(P.grid[0] * P.splits, P.grid[1], P.grid[2]);
+  dim3 grid(P.grid[0] / P.pl_group[0] * P.splits, P.grid[1] / P.pl_group[1], P.grid[2]);
   fp_mfma_gemm_kernel<<<grid, kThreads, 0, stream>>>(P);
   MI355_HIP(hipGetLastError());
   return MI355_OK;

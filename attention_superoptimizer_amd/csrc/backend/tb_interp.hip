@@ -917,7 +917,7 @@ static void set_splits(DevProgram &prog, PlanExtents const &ext, int num_outputs
 
 static void choose_splits(DevProgram &prog, PlanExtents const &ext, int num_outputs) {
   prog.splits = 1;
-  int const blocks = prog.grid[0] * prog.grid[1] * prog.grid[2];
+  int const blocks = (int)fp_program_blocks(prog);
   int const F = prog.forloop_range;
   if (F < 2 || blocks >= 192) {
     return;
@@ -1000,6 +1000,14 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     }
     prog.out[i] = outputs[i];
   }
+  // a fused matmul plan launched by itself takes the matrix cores when its operand tensors'
+  // residue planes fit this queue's plane memory (a batch places the planes of its members)
+  if (!f16 && prog.fused == 4 && ext_out == nullptr) {
+    size_t need = 0;
+    if (fp_mfma_gemm_fits(prog, ext, &need) && need <= state().planes_bytes) {
+      fp_mfma_gemm_bind(prog, state().planes());
+    }
+  }
   if (ext_out != nullptr) {
     *ext_out = ext;
     prog.splits = 1;
@@ -1011,14 +1019,6 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     DevOp &d = prog.ops[o];
     if (d.kind == DOP_LOAD && d.vec8 && (reinterpret_cast<uintptr_t>(prog.in[d.io]) & 15) != 0) {
       d.vec8 = 0;
-    }
-  }
-  // a fused matmul plan launched by itself takes the matrix cores when its operand tensors'
-  // residue planes fit this queue's plane memory (a batch places the planes of its members)
-  if (!f16 && prog.fused == 4 && ext_out == nullptr) {
-    size_t need = 0;
-    if (fp_mfma_gemm_fits(prog, ext, &need) && need <= state().planes_bytes) {
-      fp_mfma_gemm_bind(prog, state().planes());
     }
   }
   return MI355_OK;
@@ -1051,7 +1051,7 @@ static int launch(DevProgram const &prog, bool f16) {
       }
     }
     s.last_launch.kernel_id = MI355_KERNEL_FP_GEMM;
-    s.last_launch.workgroups = prog.grid[0] * prog.splits * prog.grid[1] * prog.grid[2];
+    s.last_launch.workgroups = (int)fp_program_blocks(prog);
     s.last_launch.threads = kInterpThreads;
     s.last_launch.lds_bytes = prog.lds_bytes;
     s.last_launch.row_split = prog.splits;
@@ -1154,16 +1154,6 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
                            std::vector<int> const &num_outputs) {
   State &s = state();
   int const n = (int)progs.size();
-  // split for-loops until the chunk as a whole offers the device a few workgroups per CU
-  long long total = 0;
-  for (DevProgram const &p : progs) {
-    total += (long long)p.grid[0] * p.grid[1] * p.grid[2];
-  }
-  int const scale = (int)std::min<long long>(64, (1024 + total - 1) / total);
-  size_t used = 0;
-  for (int i = 0; i < n; i++) {
-    set_splits(progs[i], exts[i], num_outputs[i], std::min(progs[i].forloop_range, scale), used);
-  }
   // fused matmul plans take the matrix cores while the residue planes of their operand
   // tensors fit what is left of this queue's plane memory
   std::vector<DevProgram const *> on_matrix_cores;
@@ -1177,6 +1167,17 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
       on_matrix_cores.push_back(&progs[i]);
     }
   }
+  // split for-loops until the chunk as a whole offers the device a few workgroups per CU
+  long long total = 0;
+  for (DevProgram &p : progs) {
+    p.splits = 1;
+    total += fp_program_blocks(p);
+  }
+  int const scale = (int)std::min<long long>(64, (1024 + total - 1) / total);
+  size_t used = 0;
+  for (int i = 0; i < n; i++) {
+    set_splits(progs[i], exts[i], num_outputs[i], std::min(progs[i].forloop_range, scale), used);
+  }
   int const record = (int)sizeof(DevProgram);
   // Launch classes.  Interpreter programs by LDS need (a launch requests the largest need of
   // its members, which bounds how many workgroups share a compute unit); fused matmul
@@ -1184,13 +1185,22 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
   // the matrix cores in a class of their own.
   constexpr int kClasses = 7;
   int const bounds[3] = {24 * 1024, 64 * 1024, s.max_lds - record - 16};
+  // (with fewer than three interpreter workgroups per compute unit in the whole chunk nobody's
+  // occupancy is at stake, and one launch is a third of the latency of three in a row)
+  long long interp_blocks = 0;
+  for (DevProgram const &p : progs) {
+    if (p.fused != 4 && p.lds_bytes <= bounds[2]) {
+      interp_blocks += (long long)p.grid[0] * p.splits * p.grid[1] * p.grid[2];
+    }
+  }
+  bool const one_interp_class = interp_blocks <= 768;
   auto class_of = [&](DevProgram const &p) {
     if (p.fused == 4) {
       return p.fg[5] ? 6 : (p.fg[3] == 1 ? 3 : (p.fg[3] == 2 ? 4 : 5));
     }
     for (int c = 0; c < 3; c++) {
       if (p.lds_bytes <= bounds[c]) {
-        return c;
+        return one_interp_class ? 2 : c;
       }
     }
     return -1;  // no room for the record above its tiles: launched by itself
@@ -1253,7 +1263,7 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
         DevProgram const &p = progs[order[k]];
         hp[k] = p;
         hf[fpos++] = acc;
-        acc += p.grid[0] * p.splits * p.grid[1] * p.grid[2];
+        acc += (int)fp_program_blocks(p);
       }
       hf[fpos++] = acc;  // total of the class
     }

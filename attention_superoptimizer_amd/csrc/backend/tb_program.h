@@ -76,6 +76,11 @@ struct alignas(16) DevProgram {
   // byte offset of a tile's first block in the A / B^T planes = bx * [0] + by * [1] + bz * [2] +
   // iteration * [3]; [4] = bytes of one strip of 16 plane rows
   int pl_a[5], pl_b[5];
+  // a workgroup of the matrix-core route takes pl_group[0] x pl_group[1] neighbouring logical
+  // blocks (along grid x / y) when A does not move with x and B not with y: their tiles form
+  // one larger tile whose operand strips are fetched once
+  int pl_group[2];
+  int pl_pad2[2];
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
@@ -128,6 +133,11 @@ int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream);
 int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,
                               hipStream_t stream);
 constexpr int kFpMfmaLdsBytes = 32768;  // wavefront sums of a tile whose k range is shared
+// Workgroups a fused matmul program is launched with (grouped blocks count once).
+inline long long fp_program_blocks(DevProgram const &p) {
+  long long const gx = p.fused == 4 && p.fg[5] ? p.pl_group[0] : 1, gy = p.fused == 4 && p.fg[5] ? p.pl_group[1] : 1;
+  return (long long)(p.grid[0] / gx) * p.splits * (p.grid[1] / gy) * p.grid[2];
+}
 
 // `declared_layouts`: fp16 loader tiles take the LDS layout the plan declares for them
 // (see MI355_OPT_PLAN_SMEM_LAYOUT) instead of the one their consumers want.

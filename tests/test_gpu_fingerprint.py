@@ -141,6 +141,10 @@ def _fused_matmul_routes(rt, abi, spec, ins, op_index=2):
     (96, 240, 32 * 9, (3, 2, 1), 9, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),    # 48 x 80 tiles
     (256, 128, 2048, (2, 1, 1), 128, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),  # 256 x 64 tiles, k 16
     (64, 64, 16 * 1001, (1, 1, 1), 1001, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),
+    # 2048 blocks of 16 x 32 outputs: a workgroup takes 4 x 2 neighbouring blocks as one tile
+    (1024, 1024, 256, (32, 64, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),
+    # 128 x 16 tiles, 512 blocks: two neighbours along x share their A strips
+    (512, 2048, 128, (128, 4, 1), 8, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),
     (256, 256, 512, (2, 2, 1), 4, (-1, 0, -1), (1, -1, -1), (1, 0, -1)),     # 128x128 tiles, 4 register tiles
     (64, 64, 512, (1, 1, 1), 8, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),   # one block: for-loop split 8 ways
     (16, 40, 96, (1, 1, 1), 4, (-1, -1, -1), (-1, -1, -1), (-1, -1, -1)),    # 16x40 tile, k tile 24 -> chunk 8
