@@ -223,30 +223,26 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
   for (int e = 0; e < 8; e++) {
     acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
   }
-  v4i ap[2], aq[2], bp[2], bq[2];
-  auto fetch = [&](int s) {
+  // operands of two steps are in flight while a third is multiplied
+  struct Operands {
+    v4i ap[2], aq[2], bp[2], bq[2];
+  } o0, o1;
+  auto fetch = [&](Operands &o, int s) {
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      ap[i] = *reinterpret_cast<v4i const *>(J.a_p + a_off[i] + (size_t)s * 1024);
-      aq[i] = *reinterpret_cast<v4i const *>(J.a_q + a_off[i] + (size_t)s * 1024);
-      bp[i] = *reinterpret_cast<v4i const *>(J.bt_p + b_off[i] + (size_t)s * 1024);
-      bq[i] = *reinterpret_cast<v4i const *>(J.bt_q + b_off[i] + (size_t)s * 1024);
+      o.ap[i] = *reinterpret_cast<v4i const *>(J.a_p + a_off[i] + (size_t)s * 1024);
+      o.aq[i] = *reinterpret_cast<v4i const *>(J.a_q + a_off[i] + (size_t)s * 1024);
+      o.bp[i] = *reinterpret_cast<v4i const *>(J.bt_p + b_off[i] + (size_t)s * 1024);
+      o.bq[i] = *reinterpret_cast<v4i const *>(J.bt_q + b_off[i] + (size_t)s * 1024);
     }
   };
-  if (s_begin < s_end) {
-    fetch(s_begin);
-  }
-  for (int s = s_begin; s < s_end; s++) {
-    v4i cap[2] = {ap[0], ap[1]}, caq[2] = {aq[0], aq[1]}, cbp[2] = {bp[0], bp[1]}, cbq[2] = {bq[0], bq[1]};
-    if (s + 1 < s_end) {
-      fetch(s + 1);
-    }
+  auto multiply = [&](Operands const &o, int s) {
 #pragma unroll
     for (int i = 0; i < 2; i++) {
 #pragma unroll
       for (int jn = 0; jn < 2; jn++) {
-        acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbp[jn], cap[i], acc[0][i][jn], 0, 0, 0);
-        acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbq[jn], caq[i], acc[1][i][jn], 0, 0, 0);
+        acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bp[jn], o.ap[i], acc[0][i][jn], 0, 0, 0);
+        acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bq[jn], o.aq[i], acc[1][i][jn], 0, 0, 0);
       }
     }
     if (((s - s_begin) & 2047) == 2047) {  // 2048 steps x 64 k x 113^2 < 2^31
@@ -260,6 +256,24 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
             acc[1][i][jn][e] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
           }
         }
+      }
+    }
+  };
+  if (s_begin < s_end) {
+    fetch(o0, s_begin);
+  }
+  if (s_begin + 1 < s_end) {
+    fetch(o1, s_begin + 1);
+  }
+  for (int s = s_begin; s < s_end; s += 2) {
+    multiply(o0, s);
+    if (s + 2 < s_end) {
+      fetch(o0, s + 2);
+    }
+    if (s + 1 < s_end) {
+      multiply(o1, s + 1);
+      if (s + 3 < s_end) {
+        fetch(o1, s + 3);
       }
     }
   }
@@ -382,17 +396,20 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
     // this lane's chunk of step s: number 4 s + g of the sequence
     int q = 4 * s_begin + g;
     int itr = q / cpi, c = q - itr * cpi;
-    v4i ap[2], aq[2], bp[2], bq[2];
-    auto fetch = [&]() {
+    // operands of two steps are in flight while a third is multiplied
+    struct Operands {
+      v4i ap[2], aq[2], bp[2], bq[2];
+    } o0, o1;
+    auto fetch = [&](Operands &o) {
       bool const valid = q < Q;
       int const oa = itr * a_it + c * 256, ob = itr * b_it + c * 256;
       v4i const zero = {0, 0, 0, 0};
 #pragma unroll
       for (int i = 0; i < 2; i++) {
-        ap[i] = valid ? *reinterpret_cast<v4i const *>(pa + a_base[i] + oa) : zero;
-        aq[i] = valid ? *reinterpret_cast<v4i const *>(qa + a_base[i] + oa) : zero;
-        bp[i] = valid ? *reinterpret_cast<v4i const *>(pb + b_base[i] + ob) : zero;
-        bq[i] = valid ? *reinterpret_cast<v4i const *>(qb + b_base[i] + ob) : zero;
+        o.ap[i] = valid ? *reinterpret_cast<v4i const *>(pa + a_base[i] + oa) : zero;
+        o.aq[i] = valid ? *reinterpret_cast<v4i const *>(qa + a_base[i] + oa) : zero;
+        o.bp[i] = valid ? *reinterpret_cast<v4i const *>(pb + b_base[i] + ob) : zero;
+        o.bq[i] = valid ? *reinterpret_cast<v4i const *>(qb + b_base[i] + ob) : zero;
       }
       q += 4;
       itr += dq_it;
@@ -407,20 +424,13 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
     for (int e = 0; e < 8; e++) {
       acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
     }
-    if (s_begin < s_end) {
-      fetch();
-    }
-    for (int s = s_begin; s < s_end; s++) {
-      v4i cap[2] = {ap[0], ap[1]}, caq[2] = {aq[0], aq[1]}, cbp[2] = {bp[0], bp[1]}, cbq[2] = {bq[0], bq[1]};
-      if (s + 1 < s_end) {
-        fetch();
-      }
+    auto multiply = [&](Operands const &o, int s) {
 #pragma unroll
       for (int i = 0; i < 2; i++) {
 #pragma unroll
         for (int jn = 0; jn < 2; jn++) {
-          acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbp[jn], cap[i], acc[0][i][jn], 0, 0, 0);
-          acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cbq[jn], caq[i], acc[1][i][jn], 0, 0, 0);
+          acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bp[jn], o.ap[i], acc[0][i][jn], 0, 0, 0);
+          acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bq[jn], o.aq[i], acc[1][i][jn], 0, 0, 0);
         }
       }
       if (((s - s_begin) & 2047) == 2047) {
@@ -434,6 +444,24 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
               acc[1][i][jn][e] = fold_signed(acc[1][i][jn][e], (int)FP_Q);
             }
           }
+        }
+      }
+    };
+    if (s_begin < s_end) {
+      fetch(o0);
+    }
+    if (s_begin + 1 < s_end) {
+      fetch(o1);
+    }
+    for (int s = s_begin; s < s_end; s += 2) {
+      multiply(o0, s);
+      if (s + 2 < s_end) {
+        fetch(o0);
+      }
+      if (s + 1 < s_end) {
+        multiply(o1, s + 1);
+        if (s + 3 < s_end) {
+          fetch(o1);
         }
       }
     }

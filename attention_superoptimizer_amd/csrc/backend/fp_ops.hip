@@ -439,6 +439,7 @@ struct BinaryMany {
   int op[MI355_MAX_BINARY_OPS];
   int nd[MI355_MAX_BINARY_OPS];
   unsigned short d1[MI355_MAX_BINARY_OPS][4], d2[MI355_MAX_BINARY_OPS][4], od[MI355_MAX_BINARY_OPS][4];
+  unsigned char plain[MI355_MAX_BINARY_OPS];  // no broadcast, 16-byte aligned, n a multiple of 8
 };
 
 __global__ void fp_binary_many_kernel(BinaryMany const B, FpTables t) {
@@ -449,6 +450,26 @@ __global__ void fp_binary_many_kernel(BinaryMany const B, FpTables t) {
   int const op = B.op[e], nd = B.nd[e];
   unsigned int gid = blockIdx.x * blockDim.x + threadIdx.x;
   unsigned int const stride = gridDim.x * blockDim.x;
+  if (B.plain[e]) {
+    // same shape on both sides: eight elements per lane and step, no index arithmetic
+    for (unsigned int v = gid; v < n / 8; v += stride) {
+      uint4v const a = reinterpret_cast<uint4v const *>(in1)[v];
+      uint4v const b = reinterpret_cast<uint4v const *>(in2)[v];
+      uint4v c;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        uint32_t z[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          uint32_t const x = h ? a[w] >> 16 : a[w] & 0xffffu, y = h ? b[w] >> 16 : b[w] & 0xffffu;
+          z[h] = op == KN_ADD_OP ? (x + y) % FP_PQ : (op == KN_MUL_OP ? (x * y) % FP_PQ : fp_div_value(t, x, y));
+        }
+        c[w] = z[0] | (z[1] << 16);
+      }
+      reinterpret_cast<uint4v *>(out)[v] = c;
+    }
+    return;
+  }
   for (; gid < n; gid += stride) {
     // reference element_binary_kernel.cu:108-116
     unsigned int i = gid, s1 = 1, i1 = 0, s2 = 1, i2 = 0;
@@ -739,7 +760,7 @@ extern "C" int mi355_fp_binary_many(int const *ops, uint16_t const *const *in1, 
     return MI355_OK;
   }
   BinaryMany B{};
-  size_t largest = 0;
+  size_t largest = 0, work = 1;
   for (int e = 0; e < count; e++) {
     if (ops[e] != KN_ADD_OP && ops[e] != KN_MUL_OP && ops[e] != KN_DIV_OP) {
       return fail(MI355_ERR_UNSUPPORTED, "binary fingerprint op %d", ops[e]);
@@ -767,12 +788,19 @@ extern "C" int mi355_fp_binary_many(int const *ops, uint16_t const *const *in1, 
     B.in1[e] = in1[e];
     B.in2[e] = in2[e];
     B.out[e] = out[e];
+    bool plain = n % 8 == 0 && ((reinterpret_cast<uintptr_t>(in1[e]) | reinterpret_cast<uintptr_t>(in2[e]) |
+                                 reinterpret_cast<uintptr_t>(out[e])) & 15) == 0;
+    for (int d = 0; d < num_dims[e]; d++) {
+      plain = plain && dims1[4 * e + d] == dims_out[4 * e + d] && dims2[4 * e + d] == dims_out[4 * e + d];
+    }
+    B.plain[e] = plain ? 1 : 0;
+    work = std::max(work, plain ? n / 8 : n);
     B.n[e] = (unsigned int)n;
     B.op[e] = ops[e];
     B.nd[e] = num_dims[e];
     largest = std::max(largest, n);
   }
-  dim3 grid(grid_for(largest, kThreads, 512), count);
+  dim3 grid(grid_for(work, kThreads, 512), count);
   fp_binary_many_kernel<<<grid, kThreads, 0, state().stream()>>>(B, tables());
   MI355_HIP(hipGetLastError());
   return MI355_OK;
