@@ -123,4 +123,34 @@ __device__ __forceinline__ uint32_t mod_pq(uint32_t x) { return x % FP_PQ; }
 __device__ __forceinline__ uint32_t mod_p(uint32_t x) { return x % FP_P; }
 __device__ __forceinline__ uint32_t mod_q(uint32_t x) { return x % FP_Q; }
 
+// The fingerprint lookup tables in device memory and the ring operations built on them
+// (kernel-level operators, and the operand prologue of the matrix-core matmul).
+struct FpTables {
+  uint16_t const *exp_tbl, *div_p, *div_q;
+};
+
+__device__ __forceinline__ uint32_t fp_exp_value(FpTables t, uint32_t x) {
+  // reference element_unary_kernel.cu:85-89
+  return (t.exp_tbl[x % FP_Q] * FP_Q_MUL_P_MOD_1) % FP_PQ;
+}
+
+__device__ __forceinline__ uint32_t fp_div_value(FpTables t, uint32_t x, uint32_t y) {
+  // reference element_binary_kernel.cu:155-160
+  uint32_t z = (x % FP_P) * t.div_p[y % FP_P] * FP_Q_MUL_P_MOD_1 +
+               (x % FP_Q) * t.div_q[y % FP_Q] * FP_P_MUL_Q_MOD_1;
+  return z % FP_PQ;
+}
+
+__device__ __forceinline__ uint32_t fp_silu_value(FpTables t, uint32_t x) {
+  // extension: x / (1 + exp(-x)) from the ring primitives above
+  uint32_t neg = (FP_PQ - x) % FP_PQ;
+  uint32_t den = (1u + fp_exp_value(t, neg)) % FP_PQ;
+  return fp_div_value(t, x, den);
+}
+
+inline FpTables tables() {
+  State &s = state();
+  return FpTables{s.exp_tbl, s.div_p, s.div_q};
+}
+
 }  // namespace mi355

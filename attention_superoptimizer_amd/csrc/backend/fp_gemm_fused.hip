@@ -310,24 +310,46 @@ int raise_lds(int lds_total) {
 // records which loader feeds which operand, the k chunk and the register tiles per thread,
 // and replaces the LDS need by the staging buffers'.
 bool fp_gemm_applicable(DevProgram &P) {
-  if (P.num_ops != 4 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
-      P.ops[2].kind != DOP_MATMUL || P.ops[3].kind != DOP_OUTPUT || P.ops[3].src0 != P.ops[2].dst) {
+  // load, load, [exp / silu of a loaded tile, in place]*, matmul, save
+  int const last = P.num_ops - 1, mm = P.num_ops - 2;
+  if (P.num_ops < 4 || P.num_ops > 6 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
+      P.ops[mm].kind != DOP_MATMUL || P.ops[last].kind != DOP_OUTPUT ||
+      P.ops[last].src0 != P.ops[mm].dst) {
     return false;
   }
   int a = -1, b = -1;
   for (int i = 0; i < 2; i++) {
-    if (P.ops[i].dst == P.ops[2].src0) {
+    if (P.ops[i].dst == P.ops[mm].src0) {
       a = i;
     }
-    if (P.ops[i].dst == P.ops[2].src1) {
+    if (P.ops[i].dst == P.ops[mm].src1) {
       b = i;
     }
   }
   if (a < 0 || b < 0 || a == b) {
     return false;
   }
-  DevOp const &la = P.ops[a], &lb = P.ops[b], &so = P.ops[3];
+  P.fp_unary[0] = P.fp_unary[1] = P.fp_unary[2] = 0;
+  for (int o = 2; o < mm; o++) {
+    DevOp const &u = P.ops[o];
+    int const which = u.dst == P.ops[a].dst ? 0 : (u.dst == P.ops[b].dst ? 1 : -1);
+    if (u.kind != DOP_UNARY || which < 0 || u.src0 != u.dst || P.fp_unary[which] != 0) {
+      return false;
+    }
+    P.fp_unary[which] = u.sub;
+    P.fp_unary[2] = 1;
+  }
+  DevOp const &la = P.ops[a], &lb = P.ops[b], &so = P.ops[last];
   int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
+  if (P.fp_unary[2]) {
+    // only the matrix-core route applies operand prologues; whether it fits (shapes, plane
+    // memory) is for the caller to ask fp_mfma_gemm_fits before it relies on this mark
+    P.fused = 4;
+    P.fg[0] = a;
+    P.fg[1] = b;
+    P.fg[2] = P.fg[3] = P.fg[4] = P.fg[5] = 0;
+    return true;
+  }
   if (!la.vec8 || !lb.vec8 || !so.vec8 || m % 4 != 0 || n % 8 != 0 || kt % 8 != 0 ||
       (reinterpret_cast<uintptr_t>(P.out[so.io]) & 15) != 0 ||
       (reinterpret_cast<uintptr_t>(P.in[la.io]) & 15) != 0 ||

@@ -47,12 +47,19 @@ struct SplitJob {
   int rp;                // plane rows per slab (a multiple of 16)
   int transpose;         // 0: plane rows = source rows, k = cols; 1: plane rows = source columns, k = rows
   int vec;               // source rows may be read 8 (plain) / 4 (transposed) values at a time
+  int unary;             // TB_EXP_OP / TB_SILU_OP applied to every value first, 0: none
   unsigned first_block, blocks;
 };
+constexpr int kSplitPrograms = 24;  // matmuls / programs per splitting launch (3 KB of arguments)
 struct SplitMany {
-  SplitJob job[2 * kMaxJobs];
+  SplitJob job[2 * kSplitPrograms];
   int count;
+  FpTables tables;
 };
+
+__device__ __forceinline__ uint32_t prologue(FpTables const &t, int unary, uint32_t x) {
+  return unary == 0 ? x : (unary == TB_EXP_OP ? fp_exp_value(t, x) : fp_silu_value(t, x));
+}
 
 __global__ __launch_bounds__(kThreads) void fp_split_planes_kernel(SplitMany const S) {
   __shared__ uint32_t tile[2][64][17];
@@ -101,6 +108,12 @@ __global__ __launch_bounds__(kThreads) void fp_split_planes_kernel(SplitMany con
           v[i] = 0u;
         }
       }
+      if (J.unary != 0 && row < J.rows) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          v[i] = k0 + i < J.cols ? prologue(S.tables, J.unary, v[i]) : 0u;  // the padding stays zero
+        }
+      }
       uint4v p, q;
 #pragma unroll
       for (int w = 0; w < 4; w++) {
@@ -137,6 +150,16 @@ __global__ __launch_bounds__(kThreads) void fp_split_planes_kernel(SplitMany con
 #pragma unroll
         for (int c = 0; c < 4; c++) {
           v[r][c] = (k < J.rows && n + c < J.cols) ? src[(size_t)k * J.cols + n + c] : 0u;
+        }
+      }
+    }
+    if (J.unary != 0) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          bool const inside = k0 + 4 * kq + r < J.rows && n0 + 4 * ng + c < J.cols;
+          v[r][c] = inside ? prologue(S.tables, J.unary, v[r][c]) : 0u;
         }
       }
     }
@@ -352,7 +375,7 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
 // tile of gy * m rows and gx * n columns: strip s of its rows belongs to block by + s / (m / 16).
 __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *part, int bx, int by,
                                                    int bz, int split) {
-  DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]], &so = P.ops[3];
+  DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]], &so = P.ops[P.num_ops - 1];
   int const bm = P.t[la.dst].rows, kt = P.t[la.dst].cols, bn = P.t[lb.dst].cols;
   int const m = bm * P.pl_group[1], n = bn * P.pl_group[0];  // the grouped tile
   int const spb_m = bm / 16, spb_n = bn / 16;                // strips per block
@@ -575,6 +598,25 @@ inline size_t round_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
 
 }  // namespace
 
+// Splitting launches for `count` jobs (their first_block fields are filled in here).
+static int launch_split_jobs(SplitJob *jobs, int count, hipStream_t stream) {
+  for (int done = 0; done < count; done += 2 * kSplitPrograms) {
+    int const group = std::min(count - done, 2 * kSplitPrograms);
+    SplitMany S{};
+    unsigned blocks = 0;
+    for (int j = 0; j < group; j++) {
+      jobs[done + j].first_block = blocks;
+      blocks += jobs[done + j].blocks;
+      S.job[j] = jobs[done + j];
+    }
+    S.count = group;
+    S.tables = tables();
+    fp_split_planes_kernel<<<blocks, kThreads, 0, stream>>>(S);
+    MI355_HIP(hipGetLastError());
+  }
+  return MI355_OK;
+}
+
 // Whether one matmul can take the matrix-core path, and the bytes of planes it needs.
 static bool mfma_matmul_fits(int batch, int m, int n, int k, size_t *plane_bytes) {
   if (batch <= 0 || m <= 0 || n <= 0 || k <= 0) {
@@ -592,11 +634,11 @@ static bool mfma_matmul_fits(int batch, int m, int n, int k, size_t *plane_bytes
 // Enqueues matmuls [0, count) whose planes fit the queue's plane memory together.
 static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B, uint16_t *const *C,
                              int const *batch, int const *m, int const *n, int const *k, int count) {
-  SplitMany S{};
+  std::vector<SplitJob> jobs((size_t)(2 * count));
   GemmMany G{};
   char *planes = state().planes();
   size_t used = 0;
-  unsigned split_blocks = 0, gemm_blocks = 0;
+  unsigned gemm_blocks = 0;
   for (int e = 0; e < count; e++) {
     int const kp = (int)round_up((size_t)k[e], 64);
     int const mp = (int)round_up((size_t)m[e], 16), np = (int)round_up((size_t)n[e], 16);
@@ -606,7 +648,9 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     int8_t *bt_p = a_q + a_plane;
     int8_t *bt_q = bt_p + b_plane;
     used += 2 * (a_plane + b_plane);
-    SplitJob &sa = S.job[2 * e], &sb = S.job[2 * e + 1];
+    SplitJob &sa = jobs[(size_t)(2 * e)], &sb = jobs[(size_t)(2 * e + 1)];
+    sa = SplitJob{};
+    sb = SplitJob{};
     sa.src = A[e];
     sa.plane_p = a_p;
     sa.plane_q = a_q;
@@ -619,8 +663,6 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     sa.vec = k[e] % 8 == 0 && (reinterpret_cast<uintptr_t>(A[e]) & 15) == 0;
     size_t const a_units = (size_t)batch[e] * mp * (kp / 16);
     sa.blocks = (unsigned)std::min<size_t>((a_units + kThreads - 1) / kThreads, 1024);
-    sa.first_block = split_blocks;
-    split_blocks += sa.blocks;
     sb.src = B[e];
     sb.plane_p = bt_p;
     sb.plane_q = bt_q;
@@ -633,8 +675,6 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     sb.vec = n[e] % 4 == 0 && (reinterpret_cast<uintptr_t>(B[e]) & 7) == 0;
     size_t const b_tiles = (size_t)batch[e] * (kp / 64) * ((n[e] + 63) / 64);
     sb.blocks = (unsigned)std::min<size_t>(b_tiles, 1024);
-    sb.first_block = split_blocks;
-    split_blocks += sb.blocks;
     GemmJob &g = G.job[e];
     g.a_p = a_p;
     g.a_q = a_q;
@@ -655,11 +695,11 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     g.first_block = gemm_blocks;
     gemm_blocks += (unsigned)((long long)g.tiles_m * g.tiles_n * batch[e]);
   }
-  S.count = 2 * count;
   G.count = count;
   hipStream_t st = state().stream();
-  fp_split_planes_kernel<<<split_blocks, kThreads, 0, st>>>(S);
-  MI355_HIP(hipGetLastError());
+  if (int rc = launch_split_jobs(jobs.data(), 2 * count, st)) {
+    return rc;
+  }
   fp_mfma_matmul_kernel<<<gemm_blocks, kThreads, 0, st>>>(G);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
@@ -830,45 +870,36 @@ void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
 }
 
 int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream) {
-  int done = 0;
-  while (done < n) {
-    int const group = std::min(n - done, kMaxJobs);
-    SplitMany S{};
-    unsigned blocks = 0;
-    for (int e = 0; e < group; e++) {
-      DevProgram const &P = *progs[done + e];
-      DevOp const *ops[2] = {&P.ops[P.fg[0]], &P.ops[P.fg[1]]};
-      for (int which = 0; which < 2; which++) {
-        DevOp const &op = *ops[which];
-        SplitJob &j = S.job[2 * e + which];
-        j.src = static_cast<uint16_t const *>(P.in[op.io]);
-        j.plane_p = P.pl[2 * which];
-        j.plane_q = P.pl[2 * which + 1];
-        j.slabs = P.pl_geo[3 * which];
-        j.rows = op.d_rows;
-        j.cols = op.d_cols;
-        j.rp = P.pl_geo[3 * which + 1];
-        j.kp = P.pl_geo[3 * which + 2];
-        j.transpose = which;
-        size_t work;
-        if (which == 0) {
-          j.vec = op.d_cols % 8 == 0 && (reinterpret_cast<uintptr_t>(j.src) & 15) == 0;
-          work = ((size_t)j.slabs * j.rp * (j.kp / 16) + kThreads - 1) / kThreads;
-        } else {
-          j.vec = op.d_cols % 4 == 0 && (reinterpret_cast<uintptr_t>(j.src) & 7) == 0;
-          work = (size_t)j.slabs * (j.kp / 64) * ((op.d_cols + 63) / 64);
-        }
-        j.blocks = (unsigned)std::min<size_t>(work, 1024);
-        j.first_block = blocks;
-        blocks += j.blocks;
+  std::vector<SplitJob> jobs((size_t)(2 * n));
+  for (int e = 0; e < n; e++) {
+    DevProgram const &P = *progs[e];
+    DevOp const *ops[2] = {&P.ops[P.fg[0]], &P.ops[P.fg[1]]};
+    for (int which = 0; which < 2; which++) {
+      DevOp const &op = *ops[which];
+      SplitJob &j = jobs[(size_t)(2 * e + which)];
+      j = SplitJob{};
+      j.src = static_cast<uint16_t const *>(P.in[op.io]);
+      j.plane_p = P.pl[2 * which];
+      j.plane_q = P.pl[2 * which + 1];
+      j.slabs = P.pl_geo[3 * which];
+      j.rows = op.d_rows;
+      j.cols = op.d_cols;
+      j.rp = P.pl_geo[3 * which + 1];
+      j.kp = P.pl_geo[3 * which + 2];
+      j.transpose = which;
+      j.unary = P.fp_unary[which];
+      size_t work;
+      if (which == 0) {
+        j.vec = op.d_cols % 8 == 0 && (reinterpret_cast<uintptr_t>(j.src) & 15) == 0;
+        work = ((size_t)j.slabs * j.rp * (j.kp / 16) + kThreads - 1) / kThreads;
+      } else {
+        j.vec = op.d_cols % 4 == 0 && (reinterpret_cast<uintptr_t>(j.src) & 7) == 0;
+        work = (size_t)j.slabs * (j.kp / 64) * ((op.d_cols + 63) / 64);
       }
+      j.blocks = (unsigned)std::min<size_t>(work, 1024);
     }
-    S.count = 2 * group;
-    fp_split_planes_kernel<<<blocks, kThreads, 0, stream>>>(S);
-    MI355_HIP(hipGetLastError());
-    done += group;
   }
-  return MI355_OK;
+  return launch_split_jobs(jobs.data(), 2 * n, stream);
 }
 
 int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream) {

@@ -365,29 +365,6 @@ __global__ __launch_bounds__(kThreads) void fp_matmul64_kernel(uint16_t const *_
 }
 
 // ---- element-wise ---------------------------------------------------------------
-struct FpTables {
-  uint16_t const *exp_tbl, *div_p, *div_q;
-};
-
-__device__ __forceinline__ uint32_t fp_exp_value(FpTables t, uint32_t x) {
-  // reference element_unary_kernel.cu:85-89
-  return (t.exp_tbl[x % FP_Q] * FP_Q_MUL_P_MOD_1) % FP_PQ;
-}
-
-__device__ __forceinline__ uint32_t fp_div_value(FpTables t, uint32_t x, uint32_t y) {
-  // reference element_binary_kernel.cu:155-160
-  uint32_t z = (x % FP_P) * t.div_p[y % FP_P] * FP_Q_MUL_P_MOD_1 +
-               (x % FP_Q) * t.div_q[y % FP_Q] * FP_P_MUL_Q_MOD_1;
-  return z % FP_PQ;
-}
-
-__device__ __forceinline__ uint32_t fp_silu_value(FpTables t, uint32_t x) {
-  // extension: x / (1 + exp(-x)) from the ring primitives above
-  uint32_t neg = (FP_PQ - x) % FP_PQ;
-  uint32_t den = (1u + fp_exp_value(t, neg)) % FP_PQ;
-  return fp_div_value(t, x, den);
-}
-
 __global__ void fp_unary_kernel(int op, FpTables t, uint16_t const *__restrict__ in,
                                 uint16_t *__restrict__ out, size_t n) {
   size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
@@ -565,10 +542,6 @@ static inline int grid_for(size_t n, int per_block = kThreads, int cap = 8192) {
   return static_cast<int>(g);
 }
 
-static inline FpTables tables() {
-  State &s = state();
-  return FpTables{s.exp_tbl, s.div_p, s.div_q};
-}
 
 }  // namespace mi355
 

@@ -940,11 +940,15 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   bool const declared = f16 && state().plan_smem_layout != 0;
   // (only a load-load-matmul-save plan can take the fused fingerprint kernel: everything
   // else is lowered once, with the limit)
-  bool const try_fused_fp = !f16 && !state().force_interpreter && plan->num_operators == 4 &&
-                            plan->operator_types[0] == TB_INPUT_OP &&
-                            plan->operator_types[1] == TB_INPUT_OP &&
-                            plan->operator_types[2] == TB_MATMUL_OP &&
-                            plan->operator_types[3] == TB_OUTPUT_OP;
+  // (load, load, [exp / silu]*, matmul, save)
+  bool try_fused_fp = !f16 && !state().force_interpreter && plan->num_operators >= 4 &&
+                      plan->num_operators <= 6 && plan->operator_types[0] == TB_INPUT_OP &&
+                      plan->operator_types[1] == TB_INPUT_OP &&
+                      plan->operator_types[plan->num_operators - 2] == TB_MATMUL_OP &&
+                      plan->operator_types[plan->num_operators - 1] == TB_OUTPUT_OP;
+  for (int o = 2; try_fused_fp && o < plan->num_operators - 2; o++) {
+    try_fused_fp = plan->operator_types[o] == TB_EXP_OP || plan->operator_types[o] == TB_SILU_OP;
+  }
   int rc = compile_plan(*plan, f16, (try_fused || try_fused_fp) ? (1 << 30) : state().max_lds, prog, ext,
                         err, declared);
   if (rc != MI355_OK) {
@@ -958,7 +962,14 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     for (int i = 0; i < plan->num_dmem_outputs; i++) {
       prog.out[i] = outputs[i];
     }
-    if (!fp_gemm_applicable(prog)) {
+    // a plan with an operand prologue can only run on the matrix-core route: it must fit
+    size_t need = 0;
+    bool fused = fp_gemm_applicable(prog);
+    if (fused && prog.fp_unary[2] &&
+        !(fp_mfma_gemm_fits(prog, ext, &need) && need <= state().planes_bytes)) {
+      fused = false;
+    }
+    if (!fused) {
       rc = compile_plan(*plan, false, state().max_lds, prog, ext, err);
       if (rc != MI355_OK) {
         return fail(rc, "%s", err.c_str());
@@ -1042,6 +1053,9 @@ static int fold_splits(DevProgram const &prog) {
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
   if (!f16 && prog.fused == 4) {
+    if (!prog.fg[5] && prog.fp_unary[2]) {
+      return fail(MI355_ERR_UNSUPPORTED, "operand prologue without the matrix-core route");
+    }
     if (int rc = prog.fg[5] ? launch_fp_mfma_gemm(prog, s.stream()) : launch_fp_gemm(prog, s.stream())) {
       return rc;
     }
@@ -1165,6 +1179,9 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
       fp_mfma_gemm_bind(progs[i], s.planes() + planes_used);
       planes_used += (need + 255) / 256 * 256;
       on_matrix_cores.push_back(&progs[i]);
+    } else if (progs[i].fused == 4 && progs[i].fp_unary[2]) {
+      // (the caller cuts chunks so that the planes of their members fit together)
+      return fail(MI355_ERR_UNSUPPORTED, "operand prologue without the matrix-core route");
     }
   }
   // split for-loops until the chunk as a whole offers the device a few workgroups per CU
@@ -1356,28 +1373,50 @@ extern "C" int mi355_customized_fp_batch(mi355_plan const *plans, int n,
   if (n < 0 || (n > 0 && (plans == nullptr || inputs == nullptr || outputs == nullptr))) {
     return fail(MI355_ERR_INVALID, "bad batch (n = %d)", n);
   }
-  // independent operators: a handful of launches for all of them, on the caller's queue
+  // independent operators: a handful of launches for all of them, on the caller's queue.  A
+  // chunk ends after 64 operators, or where the residue planes of its fused matmul plans
+  // would no longer fit this queue's plane memory together.
   int const chunk_max = 64;
-  for (int begin = 0; begin < n; begin += chunk_max) {
-    int const m = std::min(chunk_max, n - begin);
-    std::vector<DevProgram> progs((size_t)m);
-    std::vector<PlanExtents> exts((size_t)m);
-    std::vector<int> nout((size_t)m);
-    for (int i = 0; i < m; i++) {
-      int rc = prepare(&plans[begin + i], inputs + (size_t)(begin + i) * MI355_MAX_DMEM_INPUTS,
-                       outputs + (size_t)(begin + i) * MI355_MAX_DMEM_OUTPUTS, false, progs[(size_t)i],
-                       &exts[(size_t)i]);
-      if (rc != MI355_OK) {
-        return rc;
-      }
-      nout[(size_t)i] = plans[begin + i].num_dmem_outputs;
-    }
-    int rc = launch_fp_chunk(progs, exts, nout);
+  std::vector<DevProgram> progs;
+  std::vector<PlanExtents> exts;
+  std::vector<int> nout;
+  size_t planes_wanted = 0;
+  auto flush = [&]() {
+    int rc = progs.empty() ? MI355_OK : launch_fp_chunk(progs, exts, nout);
+    progs.clear();
+    exts.clear();
+    nout.clear();
+    planes_wanted = 0;
+    return rc;
+  };
+  for (int i = 0; i < n; i++) {
+    DevProgram prog;
+    PlanExtents ext;
+    int rc = prepare(&plans[i], inputs + (size_t)i * MI355_MAX_DMEM_INPUTS,
+                     outputs + (size_t)i * MI355_MAX_DMEM_OUTPUTS, false, prog, &ext);
     if (rc != MI355_OK) {
       return rc;
     }
+    size_t need = 0;
+    if (prog.fused == 4 && fp_mfma_gemm_fits(prog, ext, &need)) {
+      need = (need + 255) / 256 * 256;
+      if (planes_wanted + need > state().planes_bytes) {
+        if (int rc2 = flush()) {
+          return rc2;
+        }
+      }
+      planes_wanted += need;
+    }
+    progs.push_back(prog);
+    exts.push_back(ext);
+    nout.push_back(plans[i].num_dmem_outputs);
+    if ((int)progs.size() == chunk_max) {
+      if (int rc2 = flush()) {
+        return rc2;
+      }
+    }
   }
-  return MI355_OK;
+  return flush();
 }
 
 extern "C" int mi355_customized_run(mi355_plan const *plan, void const *const *inputs,

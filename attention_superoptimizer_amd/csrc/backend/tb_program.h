@@ -80,7 +80,12 @@ struct alignas(16) DevProgram {
   // blocks (along grid x / y) when A does not move with x and B not with y: their tiles form
   // one larger tile whose operand strips are fetched once
   int pl_group[2];
-  int pl_pad2[2];
+  // element-wise operator the plan applies to the A tile / the B tile before the matmul
+  // (TB_EXP_OP, TB_SILU_OP or 0): on the matrix-core route it is applied once per element
+  // while the operand tensor is split into planes; [2] != 0 marks a program that only that
+  // route can run
+  int fp_unary[3];
+  int pl_pad2[3];
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations

@@ -227,6 +227,35 @@ def test_fused_matmul_fingerprint_batched_operands_and_mismatched_maps(rt, abi):
         assert got["auto"][0] == 6 and got["auto"][1] == 32768
 
 
+@pytest.mark.parametrize("pro", [("exp", None), (None, "silu"), ("silu", "exp")])
+def test_fused_matmul_fingerprint_with_operand_prologues(rt, abi, pro):
+    """exp / silu of a loaded tile before the matmul (the second op of the MLP plans): on the
+    matrix-core route the operator is applied once per element while the operand tensor is
+    split into planes; the other routes run the plan in the interpreter.  All equal the oracle."""
+    from attention_superoptimizer_amd import workloads as W
+    m, n, k, F = 64, 256, 512, 4
+    ops, a_ref, b_ref, nxt = [], (0, 0), (1, 0), 2
+    for which, name in enumerate(pro):
+        if name is not None:
+            ops.append((f"tb_{name}_op", [(which, 0)]))
+            if which == 0:
+                a_ref = (nxt, 0)
+            else:
+                b_ref = (nxt, 0)
+            nxt += 1
+    ops.append(("tb_matmul_op", [a_ref, b_ref]))
+    spec = [W._inp([m, k]), W._inp([k, n]),
+            {"op": "customized", "in": [[0, 0], [1, 0]],
+             "plan": W._plan((4, 1, 1), F, [(-1, -1, -1), (1, -1, -1)], (1, 0), (1, -1, -1), ops)}]
+    ins = {0: uniform_fp(spec[0]["dims"], 71), 1: uniform_fp(spec[1]["dims"], 72)}
+    ins[0].flat[:5] = [0, 1, 112, 113, 25650]
+    want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
+    got = _fused_matmul_routes(rt, abi, spec, ins)
+    for route, (kernel_id, lds, out) in got.items():
+        assert kernel_id == (6 if route == "auto" else 1), route
+        assert np.array_equal(out, want), route
+
+
 def test_many_fills_and_many_compares_in_one_launch(rt, abi):
     """mi355_fp_fill_many over 40 tensors of ragged sizes = the single-tensor fill of each;
     mi355_fp_equal_enqueue_many over 40 pairs = the verdict of each pair (every third pair is

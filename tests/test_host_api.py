@@ -146,6 +146,13 @@ def test_device_work_fails_loudly_without_a_gpu():
             "g=G.KNGraph(); A=g.new_input((4,4)); g.fingerprint(0)\n")
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
     assert r.returncode != 0 and "host-only" in r.stderr
+    # the two-call verification hands work to threads: it must refuse before starting any
+    code = ("import os; os.environ['MIRAGE_HOST_ONLY']='1'\n"
+            "from attention_superoptimizer_amd import graph as G\n"
+            "g=G.KNGraph(); A=g.new_input((4,4)); r=G.KNGraph(); r.new_input((4,4))\n"
+            "G.verify_batch_begin([g], r, 1)\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
+    assert r.returncode != 0 and "host-only" in r.stderr
     code = ("import os; os.environ.pop('MIRAGE_HOST_ONLY', None)\n"
             "from attention_superoptimizer_amd import graph as G\n"
             "g=G.KNGraph(); g.new_input((4,4))\n")
