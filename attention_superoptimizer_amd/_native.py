@@ -161,6 +161,7 @@ FACADE = {
     "mirage_graph_fingerprint": (_ci, [_vp, _u64, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_verify_batch_begin": (_vp, [_pvp, _ci, _vp, _u64, _ci]),
+    "mirage_verify_set_queues_per_batch": (None, [_ci]),
     "mirage_verify_batch_end": (_ci, [_vp, _ci, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_optimize_layout": (_ci, [_vp, ctypes.c_longlong, LAYOUT_COST_FN, _vp,
                                      ctypes.POINTER(MirageLayoutStats)]),

@@ -344,7 +344,7 @@ struct VerifyTicket {
   int first_slot = 0, slots = 0;
   int mark_reference = 0, mark_done = 0;
   int reference_queue = 0;
-  int workers = 0;
+  int workers = 0, first_worker = 0;  // worker w of the batch is pool thread (first_worker + w) % queues
   std::vector<VerifyStats> local;
   std::mutex m;
   std::condition_variable cv;
@@ -358,6 +358,13 @@ struct VerifyTicket {
 static std::mutex g_ring_mutex;
 static int g_next_slot = 0;
 static int g_next_ticket = 0;
+static int g_queues_per_batch = MI355_NUM_QUEUES;
+static int g_next_queue = 0;
+
+void set_verify_queues_per_batch(int queues) {
+  std::lock_guard<std::mutex> lock(g_ring_mutex);
+  g_queues_per_batch = std::max(1, std::min(queues, (int)MI355_NUM_QUEUES));
+}
 
 VerifyTicket *verify_batch_begin(std::vector<kernel::Graph *> const &candidates,
                                  std::vector<DTensor> const &reference_outputs,
@@ -390,6 +397,9 @@ VerifyTicket *verify_batch_begin(std::vector<kernel::Graph *> const &candidates,
     g_next_ticket = (g_next_ticket + 1) % (MI355_NUM_MARKS / 2);
     t->mark_reference = 2 * ticket;
     t->mark_done = 2 * ticket + 1;
+    t->workers = g_queues_per_batch;
+    t->first_worker = g_next_queue;
+    g_next_queue = (g_next_queue + g_queues_per_batch) % MI355_NUM_QUEUES;
   }
   for (Pending &p : t->pend) {
     if (p.first_slot >= 0) {
@@ -399,7 +409,7 @@ VerifyTicket *verify_batch_begin(std::vector<kernel::Graph *> const &candidates,
   t->possible.assign((size_t)t->slots, 0);
   MI355_CALL(mi355_fp_equal_reset(t->first_slot, t->slots));
   WorkerPool &pool = WorkerPool::get();
-  t->workers = (int)std::min<size_t>((size_t)pool.size(), std::max<size_t>(n, 1));
+  t->workers = (int)std::min<size_t>((size_t)t->workers, std::max<size_t>(n, 1));
   t->local.resize((size_t)t->workers);
   t->enqueueing = t->workers;
   if (t->reference == nullptr) {
@@ -411,9 +421,10 @@ VerifyTicket *verify_batch_begin(std::vector<kernel::Graph *> const &candidates,
   }
   VerifyTicket *const T = t.get();
   for (int w = 0; w < T->workers; w++) {
-    pool.post(w, [T, w]() {
+    pool.post((T->first_worker + w) % pool.size(), [T, w]() {
       size_t const n = T->candidates.size(), no = T->reference_outputs.size();
       if (w == 0 && T->reference != nullptr) {
+        T->reference_queue = mi355_queue_current();
         fingerprint_graphs({T->reference}, T->input_seed, &T->local[0]);
         MI355_CALL(mi355_mark_record(T->mark_reference));
         {
@@ -577,6 +588,10 @@ void *mirage_verify_batch_begin(void *const *candidates, int n, void *reference,
   mirage::kernel::Graph *ref = static_cast<mirage::kernel::Graph *>(reference);
   return mirage::search::verify_batch_begin(c, mirage::search::graph_outputs(*ref), input_seed,
                                             fingerprint_reference ? ref : nullptr);
+}
+
+void mirage_verify_set_queues_per_batch(int queues) {
+  mirage::search::set_verify_queues_per_batch(queues);
 }
 
 int mirage_verify_batch_end(void *ticket, int n, unsigned char *equal, mirage_verify_stats *stats) {

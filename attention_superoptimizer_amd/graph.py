@@ -316,6 +316,12 @@ def verify_batch_begin(candidates: Sequence["KNGraph"], reference: "KNGraph", in
     return (handle, n)
 
 
+def set_verify_queues_per_batch(queues: int) -> None:
+    """How many backend queues a verification batch is dealt over (default: all four).  With
+    several batches in flight, fewer queues per batch put more candidates into every launch."""
+    N.runtime().mirage_verify_set_queues_per_batch(queues)
+
+
 def verify_batch_end(ticket):
     """Second half: waits for this batch's compares only.  Returns (list of bool, stats)."""
     handle, n = ticket

@@ -69,15 +69,19 @@ def _spec_inputs(spec, seed):
 
 
 def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_problem: int = 64,
-                           in_flight: int = 2):
+                           in_flight: int = 4, queues_per_submission: int = 2):
     """Batched verification of 4096 generated candidate mugraphs (8-12 operators, dims in
     [64, 1024]).  Per problem ONE verify_batch submission fingerprints the reference graph and
-    its 64 candidates and compares their outputs; `in_flight` submissions overlap (the graphs
+    its 64 candidates and compares their outputs; `in_flight` submissions overlap, each dealt
+    over `queues_per_submission` of the backend's queues (the graphs
     of that many problems are built through the host API first, untimed; timed, host wall
     clock: begin of each, then end of each = lowering, enqueue of every fingerprint kernel
     and compare, and waiting for the verdicts)."""
     from attention_superoptimizer_amd import candidates as C
     probs = C.generate(num_problems=num_problems, per_problem=per_problem)
+    # a submission is dealt over this many of the backend's four queues; successive submissions
+    # take successive groups of queues
+    G.set_verify_queues_per_batch(queues_per_submission)
     # submissions that overlap are problems of one family, so the per-family rates stay clean
     order = sorted(range(len(probs)), key=lambda i: (probs[i]["family"], i))
     # untimed warm-up: one problem of every family (first use of a kernel loads its code
@@ -135,11 +139,13 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
         "fingerprint_GBps": round(tot["fp_bytes"] / t_verify / 1e9, 2),
         "int_TMACps": round(tot["matmul_macs"] / t_verify / 1e12, 3),
         "verdicts_as_constructed": wrong == 0, "submissions_in_flight": in_flight,
+        "queues_per_submission": queues_per_submission,
         "candidates_per_s_by_family": {k: round(v[0] / v[1], 1) for k, v in sorted(fam.items())},
         "inputs": "uniform [0, 25651) from (seed, input index)",
     }
     if in_flight > 1:
-        one = fingerprint_throughput(G, False, num_problems, per_problem, 1)
+        one = fingerprint_throughput(G, False, num_problems, per_problem, 1, 4)
+        G.set_verify_queues_per_batch(4)
         rec["one_submission_in_flight"] = {k: one[k] for k in (
             "candidates_per_s", "verify_s", "host_enqueue_s", "final_wait_s",
             "candidates_per_s_by_family")}

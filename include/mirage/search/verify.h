@@ -53,6 +53,12 @@ void verify_batch(std::vector<mirage::kernel::Graph *> const &candidates,
 // fingerprints on its own queue.  Between the two calls the caller must not enqueue device
 // work on the worker queues itself, and the candidates, the reference and their tensors
 // must stay alive.  At most 32 batches, MI355_COMPARE_SLOTS compares in all, in flight.
+// How many backend queues (and worker threads) a batch is dealt over, MI355_NUM_QUEUES by
+// default.  Successive batches take successive groups of queues, so with two batches in
+// flight and 2 queues per batch each batch has half of the queues to itself: twice as many
+// candidates share every launch and the batches' chains of dependent launches run side by
+// side instead of one after the other.
+void set_verify_queues_per_batch(int queues);
 struct VerifyTicket;
 VerifyTicket *verify_batch_begin(std::vector<mirage::kernel::Graph *> const &candidates,
                                  std::vector<mirage::kernel::DTensor> const &reference_outputs,

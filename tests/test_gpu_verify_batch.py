@@ -91,7 +91,8 @@ def test_verify_batches_in_flight_match_one_at_a_time(rt):
         verdicts, outs, ref_out = _verify_problem(rt, prob)
         assert verdicts == [c["expect_equal"] for c in prob["candidates"]]
         want[k] = (verdicts, outs, ref_out)
-    for _ in range(5):
+    for queues in (4, 2, 1, 2, 4):  # queues a submission is dealt over; groups of queues rotate
+        rt.set_verify_queues_per_batch(queues)
         for first in range(0, len(probs), 4):
             built = []
             try:
@@ -116,6 +117,7 @@ def test_verify_batches_in_flight_match_one_at_a_time(rt):
                     for g, _ in reversed(cands):
                         g.close()
                     ref_g.close()
+    rt.set_verify_queues_per_batch(4)
 
 
 def test_marks_order_queues_and_report_only_their_work(rt, abi):
