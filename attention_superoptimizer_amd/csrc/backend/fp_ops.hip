@@ -934,7 +934,6 @@ extern "C" int mi355_fp_equal_enqueue_many(uint16_t const *const *a, uint16_t co
 
 extern "C" int mi355_fp_equal_collect(int first_slot, int count, uint8_t *equal) {
   MI355_REQUIRE_INIT();
-  State &s = state();
   if (first_slot < 0 || count < 0 || first_slot + count > MI355_COMPARE_SLOTS ||
       (count > 0 && equal == nullptr)) {
     return fail(MI355_ERR_INVALID, "compare slots [%d, %d) out of range", first_slot,
