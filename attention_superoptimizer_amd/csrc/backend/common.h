@@ -123,6 +123,18 @@ __device__ __forceinline__ uint32_t mod_pq(uint32_t x) { return x % FP_PQ; }
 __device__ __forceinline__ uint32_t mod_p(uint32_t x) { return x % FP_P; }
 __device__ __forceinline__ uint32_t mod_q(uint32_t x) { return x % FP_Q; }
 
+// Fingerprint value of a matmul output from its two residue sums (matrix-core kernels).
+// u * 25425 + v * 227 has residue u modulo 227 and v modulo 113 whatever the integers u and v
+// are (25425 = 113 * 225 = 1 mod 227, 227 = 1 mod 113), so the sums need not be reduced modulo
+// their own primes first: each is brought below 25651 and one more reduction finishes.
+// sum_p may be negative (operands recentred to [-113, 113]), |sum_p| < 2^31 - 2^17; adding
+// 83715 * 25651 makes it non-negative without changing a residue.  sum_q >= 0.
+__device__ __forceinline__ uint32_t fp_from_residue_sums(int sum_p, int sum_q) {
+  uint32_t const a = static_cast<uint32_t>(sum_p + 2147373465) % FP_PQ;
+  uint32_t const b = static_cast<uint32_t>(sum_q) % FP_PQ;
+  return (a * FP_Q_MUL_P_MOD_1 + b * FP_P_MUL_Q_MOD_1) % FP_PQ;
+}
+
 // The fingerprint lookup tables in device memory and the ring operations built on them
 // (kernel-level operators, and the operand prologue of the matrix-core matmul).
 struct FpTables {

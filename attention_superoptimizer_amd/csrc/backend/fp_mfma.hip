@@ -310,9 +310,7 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
     uint32_t z[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-      int const rp = (sp[e] % (int)FP_P + (int)FP_P) % (int)FP_P;
-      int const rq = (sq[e] % (int)FP_Q + (int)FP_Q) % (int)FP_Q;
-      z[e] = ((uint32_t)rp * FP_Q_MUL_P_MOD_1 + (uint32_t)rq * FP_P_MUL_Q_MOD_1) % FP_PQ;
+      z[e] = fp_from_residue_sums(sp[e], sq[e]);
     }
     uint16_t *dst = out + (size_t)row * J.n + col;
     if (whole4 && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
@@ -495,17 +493,17 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
       uint32_t z[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        int const rp = (sp[e] % (int)FP_P + (int)FP_P) % (int)FP_P;
-        int const rq = (sq[e] % (int)FP_Q + (int)FP_Q) % (int)FP_Q;
-        z[e] = ((uint32_t)rp * FP_Q_MUL_P_MOD_1 + (uint32_t)rq * FP_P_MUL_Q_MOD_1) % FP_PQ;
+        z[e] = fp_from_residue_sums(sp[e], sq[e]);
       }
       uint2 w;
       w.x = z[0] | (z[1] << 16);
       w.y = z[2] | (z[3] << 16);
-      int const row = row_m + 16 * i + r, col = col_n + 16 * jn + 4 * g;  // in the grouped tile
-      int const dy = row / bm, dx = col / bn;
-      *reinterpret_cast<uint2 *>(gout + out_origin(dx, dy) + (long long)(row - dy * bm) * so.d_cols +
-                                 (col - dx * bn)) = w;
+      // strip -> logical block of the grouped tile by multiply-high (magics from the host)
+      int const srow = row_m / 16 + i, scol = col_n / 16 + jn;
+      int const dy = P.pl_magic[0] ? (int)__umulhi((uint32_t)srow, P.pl_magic[0]) : srow;
+      int const dx = P.pl_magic[1] ? (int)__umulhi((uint32_t)scol, P.pl_magic[1]) : scol;
+      int const row = (srow - dy * spb_m) * 16 + r, col = (scol - dx * spb_n) * 16 + 4 * g;
+      *reinterpret_cast<uint2 *>(gout + out_origin(dx, dy) + (long long)row * so.d_cols + col) = w;
     };
     if (ways == 1) {
 #pragma unroll
@@ -710,7 +708,7 @@ extern "C" int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C
 
 bool mfma_matmul_pays(int batch, int m, int n, int k) {
   size_t need = 0;
-  return mfma_matmul_fits(batch, m, n, k, &need) && need <= state().planes_bytes &&
+  return !state().fp_vector_dot_only && mfma_matmul_fits(batch, m, n, k, &need) && need <= state().planes_bytes &&
          (double)batch * m * n * k >= (double)(1 << 27);
 }
 
@@ -741,7 +739,8 @@ extern "C" int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *co
   int begin = 0;
   while (begin < count) {
     size_t need = 0;
-    if (!mfma_matmul_fits(batch[begin], m[begin], n[begin], k[begin], &need) ||
+    if (state().fp_vector_dot_only ||
+        !mfma_matmul_fits(batch[begin], m[begin], n[begin], k[begin], &need) ||
         need > state().planes_bytes) {
       if (int rc = mi355_fp_matmul(A[begin], B[begin], C[begin], batch[begin], m[begin], n[begin], k[begin])) {
         return rc;
@@ -855,6 +854,8 @@ void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
   // the program keeps a few hundred workgroups
   P.pl_group[0] = P.pl_group[1] = 1;
   int const m = P.t[la.dst].rows, n = P.t[lb.dst].cols;
+  P.pl_magic[0] = fast_div_magic(m / 16);
+  P.pl_magic[1] = fast_div_magic(n / 16);
   if (P.pl_a[0] == 0 && P.pl_b[1] == 0) {
     long long blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
     auto grow = [&](int which, int tile) {

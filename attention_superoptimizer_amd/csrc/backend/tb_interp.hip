@@ -273,9 +273,7 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
           uint32_t z[4];
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            int const rp = (acc[0][i][jn][e] % (int)FP_P + (int)FP_P) % (int)FP_P;
-            int const rq = acc[1][i][jn][e] % (int)FP_Q;  // both operands non-negative
-            z[e] = ((uint32_t)rp * FP_Q_MUL_P_MOD_1 + (uint32_t)rq * FP_P_MUL_Q_MOD_1) % FP_PQ;
+            z[e] = fp_from_residue_sums(acc[0][i][jn][e], acc[1][i][jn][e]);
           }
           if (k0 > 0) {
             uint2 old = *reinterpret_cast<uint2 const *>(cp);

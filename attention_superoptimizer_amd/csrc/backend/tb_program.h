@@ -85,7 +85,8 @@ struct alignas(16) DevProgram {
   // while the operand tensor is split into planes; [2] != 0 marks a program that only that
   // route can run
   int fp_unary[3];
-  int pl_pad2[3];
+  uint32_t pl_magic[2];  // division magics of m / 16 and n / 16 (strips per logical block)
+  int pl_pad2[1];
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations

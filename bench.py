@@ -189,6 +189,9 @@ def main() -> int:
     ap.add_argument("--only", default="", metavar="CONFIG",
                     help="launch every customized op of one configuration --steps times and "
                          "exit (for use under the profiler), e.g. C3_mha_prefill")
+    ap.add_argument("--fp-matmul", default="", metavar="B,M,N,K",
+                    help="time the kernel-level fingerprint matmul of that shape on the matrix-core "
+                         "route and on the vector-dot route and print both (used under the profiler)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run 16 plain device copies of MIB MiB and exit: the known-size "
                          "traffic that hardware byte counters are scaled against")
@@ -212,6 +215,31 @@ def main() -> int:
 
     if args.fingerprints_only:
         print(json.dumps(fingerprint_throughput(G, False)), flush=True)
+        return 0
+
+    if args.fp_matmul:
+        b, m, n, k = (int(x) for x in args.fp_matmul.split(","))
+        g = G.KNGraph()
+        A, B = g.new_input((b, m, k)), g.new_input((b, k, n))
+        g.matmul(A, B)
+        g.fingerprint(0)
+        g.fingerprint(1)
+        rec = {"shape": [b, m, n, k], "macs": b * m * n * k}
+        for route, name in ((0, "matrix_cores"), (1, "vector_dot")):
+            assert abi.mi355_set_option(4, route) == 0
+            for _ in range(max(1, args.warmup // 64)):
+                g.fingerprint(2)
+            assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
+            iters = max(1, args.steps // 16)
+            for _ in range(iters):
+                g.fingerprint(2)
+            ms = ctypes.c_float()
+            assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
+            us = ms.value * 1e3 / iters
+            rec[name] = {"us": round(us, 2), "T_MACps": round(b * m * n * k / us / 1e6, 2)}
+        assert abi.mi355_set_option(4, 0) == 0
+        print(json.dumps(rec), flush=True)
+        g.close()
         return 0
 
     if args.calibrate_copy:
