@@ -310,10 +310,17 @@ int raise_lds(int lds_total) {
 // records which loader feeds which operand, the k chunk and the register tiles per thread,
 // and replaces the LDS need by the staging buffers'.
 bool fp_gemm_applicable(DevProgram &P) {
-  // load, load, [exp / silu of a loaded tile, in place]*, matmul, save
-  int const last = P.num_ops - 1, mm = P.num_ops - 2;
-  if (P.num_ops < 4 || P.num_ops > 6 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
-      P.ops[mm].kind != DOP_MATMUL || P.ops[last].kind != DOP_OUTPUT ||
+  // load, load, [exp / silu of a loaded tile, in place]*, matmul, [exp / silu of the product,
+  // in place], save
+  int const last = P.num_ops - 1;
+  int mm = -1;
+  for (int o = 2; o < last; o++) {
+    if (P.ops[o].kind == DOP_MATMUL) {
+      mm = mm < 0 ? o : P.num_ops;  // exactly one
+    }
+  }
+  if (P.num_ops < 4 || P.num_ops > 7 || mm < 0 || mm >= last || mm < last - 2 ||
+      P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD || P.ops[last].kind != DOP_OUTPUT ||
       P.ops[last].src0 != P.ops[mm].dst) {
     return false;
   }
@@ -337,12 +344,18 @@ bool fp_gemm_applicable(DevProgram &P) {
       return false;
     }
     P.fp_unary[which] = u.sub;
-    P.fp_unary[2] = 1;
+  }
+  if (mm == last - 2) {
+    DevOp const &u = P.ops[last - 1];
+    if (u.kind != DOP_UNARY || u.dst != P.ops[mm].dst || u.src0 != u.dst) {
+      return false;
+    }
+    P.fp_unary[2] = u.sub;
   }
   DevOp const &la = P.ops[a], &lb = P.ops[b], &so = P.ops[last];
   int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
-  if (P.fp_unary[2]) {
-    // only the matrix-core route applies operand prologues; whether it fits (shapes, plane
+  if (fp_needs_matrix_cores(P)) {
+    // only the matrix-core route applies these operators; whether it fits (shapes, plane
     // memory) is for the caller to ask fp_mfma_gemm_fits before it relies on this mark
     P.fused = 4;
     P.fg[0] = a;

@@ -371,8 +371,9 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
 // its chunk sequence between wavefronts and adds their sums through `part`.  (bx, by) is the
 // first of pl_group[0] x pl_group[1] logical blocks whose tiles the workgroup treats as one
 // tile of gy * m rows and gx * n columns: strip s of its rows belongs to block by + s / (m / 16).
-__device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *part, int bx, int by,
-                                                   int bz, int split) {
+__device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables const &tbl, int *part,
+                                                   uint16_t const *exp_lds, int bx, int by, int bz,
+                                                   int split) {
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]], &so = P.ops[P.num_ops - 1];
   int const bm = P.t[la.dst].rows, kt = P.t[la.dst].cols, bn = P.t[lb.dst].cols;
   int const m = bm * P.pl_group[1], n = bn * P.pl_group[0];  // the grouped tile
@@ -382,6 +383,10 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
   int const it_begin = (int)((long long)F * split / P.splits);
   int const it_end = (int)((long long)F * (split + 1) / P.splits);
   int const Q = (it_end - it_begin) * cpi, steps = (Q + 3) / 4;
+  // An operator applied to every iteration's product (k tiles are multiples of 64 then, so an
+  // iteration is a whole number of steps): after its last step the two sums become a
+  // fingerprint value, the operator is applied and the result added to a running sum.
+  int const epi = P.fp_unary[2], spi = cpi / 4;
   int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
   int const a0 = bx * P.pl_a[0] + by * P.pl_a[1] + bz * P.pl_a[2] + it_begin * P.pl_a[3];
   int const b0 = bx * P.pl_b[0] + by * P.pl_b[1] + bz * P.pl_b[2] + it_begin * P.pl_b[3];
@@ -403,8 +408,11 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
   int8_t const *const pa = P.pl[0], *const qa = P.pl[1], *const pb = P.pl[2], *const qb = P.pl[3];
   for (int t = ways == 1 ? wave : wave / ways; t < mt; t += 4) {
     int const ks = ways == 1 ? 0 : wave % ways;
-    int const s_begin = (int)((long long)steps * ks / ways);
-    int const s_end = (int)((long long)steps * (ks + 1) / ways);
+    // wavefronts that share a piece split its steps, by whole iterations if there is an
+    // operator on the products
+    int const units = epi ? it_end - it_begin : steps, per_unit = epi ? spi : 1;
+    int const s_begin = (int)((long long)units * ks / ways) * per_unit;
+    int const s_end = (int)((long long)units * (ks + 1) / ways) * per_unit;
     int const row_m = (t / mt_n) * 32, col_n = (t % mt_n) * 32;
     int const i1 = row_m + 16 < m ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
     int a_base[2], b_base[2];
@@ -445,6 +453,12 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
     for (int e = 0; e < 8; e++) {
       acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
     }
+    uint32_t run[4][4];  // running sums of the operator's results, [2 i + jn][e]
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      run[e / 4][e % 4] = 0;
+    }
+    int until = spi, folds = 0;
     auto multiply = [&](Operands const &o, int s) {
 #pragma unroll
       for (int i = 0; i < 2; i++) {
@@ -453,6 +467,32 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
           acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bp[jn], o.ap[i], acc[0][i][jn], 0, 0, 0);
           acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bq[jn], o.aq[i], acc[1][i][jn], 0, 0, 0);
         }
+      }
+      if (epi != 0) {
+        if (--until == 0) {  // the iteration's product is complete
+          until = spi;
+          bool const fold = (++folds & 32767) == 0;  // 32768 values below 25651 fit 32 bits
+#pragma unroll
+          for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int jn = 0; jn < 2; jn++) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                uint32_t &sum = run[2 * i + jn][e];
+                if (epi == TB_EXP_OP) {
+                  // exp reads only the value's residue modulo 113, which is the second sum's
+                  sum += exp_lds[static_cast<uint32_t>(acc[1][i][jn][e]) % FP_Q];
+                } else {
+                  sum += fp_silu_value(tbl, fp_from_residue_sums(acc[0][i][jn][e], acc[1][i][jn][e]));
+                }
+                sum = fold ? sum % FP_PQ : sum;
+                acc[0][i][jn][e] = 0;
+                acc[1][i][jn][e] = 0;
+              }
+            }
+          }
+        }
+        return;
       }
       if (((s - s_begin) & 2047) == 2047) {
 #pragma unroll
@@ -486,14 +526,9 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
         }
       }
     }
-    auto store = [&](int i, int jn, v4i const &sp, v4i const &sq) {
+    auto store_values = [&](int i, int jn, uint32_t const (&z)[4]) {
       if (i > i1 || jn > j1) {
         return;
-      }
-      uint32_t z[4];
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        z[e] = fp_from_residue_sums(sp[e], sq[e]);
       }
       uint2 w;
       w.x = z[0] | (z[1] << 16);
@@ -505,6 +540,51 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
       int const row = (srow - dy * spb_m) * 16 + r, col = (scol - dx * spb_n) * 16 + 4 * g;
       *reinterpret_cast<uint2 *>(gout + out_origin(dx, dy) + (long long)row * so.d_cols + col) = w;
     };
+    auto store = [&](int i, int jn, v4i const &sp, v4i const &sq) {
+      uint32_t z[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        z[e] = fp_from_residue_sums(sp[e], sq[e]);
+      }
+      store_values(i, jn, z);
+    };
+    if (epi != 0) {
+      // the running sums are fingerprint values already
+      if (ways > 1 && ks != 0) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          part[(wave * 32 + e) * 64 + lane] = (int)(run[e / 4][e % 4] % FP_PQ);
+        }
+      }
+      if (ways > 1) {
+        __syncthreads();
+      }
+      if (ks == 0) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+          for (int jn = 0; jn < 2; jn++) {
+            uint32_t z[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              z[e] = run[2 * i + jn][e] % FP_PQ;
+            }
+            for (int w = 1; w < ways; w++) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                z[e] += (uint32_t)part[((wave + w) * 32 + (2 * i + jn) * 4 + e) * 64 + lane];
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              z[e] %= FP_PQ;
+            }
+            store_values(i, jn, z);
+          }
+        }
+      }
+      continue;
+    }
     if (ways == 1) {
 #pragma unroll
       for (int i = 0; i < 2; i++) {
@@ -555,17 +635,30 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, int *par
   }
 }
 
-__global__ __launch_bounds__(kThreads) void fp_mfma_gemm_kernel(DevProgram const P) {
+// exp table premultiplied by the CRT lift, as exp_fp(x) = (3^(x mod 113) * 25425) mod 25651
+__device__ __forceinline__ void load_exp_table(FpTables const &tbl, uint16_t *exp_lds) {
+  if (threadIdx.x < FP_Q) {
+    exp_lds[threadIdx.x] = static_cast<uint16_t>((tbl.exp_tbl[threadIdx.x] * FP_Q_MUL_P_MOD_1) % FP_PQ);
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(kThreads) void fp_mfma_gemm_kernel(DevProgram const P, FpTables const tbl) {
   __shared__ int part[kFpMfmaLdsBytes / 4];
+  __shared__ uint16_t exp_lds[128];
+  if (P.fp_unary[2] == TB_EXP_OP) {
+    load_exp_table(tbl, exp_lds);
+  }
   int const gx = P.grid[0] / P.pl_group[0];
-  fp_mfma_gemm_block(P, part, (blockIdx.x % gx) * P.pl_group[0], blockIdx.y * P.pl_group[1], blockIdx.z,
+  fp_mfma_gemm_block(P, tbl, part, exp_lds, (blockIdx.x % gx) * P.pl_group[0], blockIdx.y * P.pl_group[1], blockIdx.z,
                      blockIdx.x / gx);
 }
 
 // Many programs in one launch: workgroup -> program by a prefix table, the program record
 // copied to LDS above the wavefront sums.
 __global__ __launch_bounds__(kThreads) void fp_mfma_gemm_multi_kernel(
-    DevProgram const *__restrict__ progs, int const *__restrict__ first_block, int n) {
+    DevProgram const *__restrict__ progs, int const *__restrict__ first_block, int n,
+    FpTables const tbl) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   int lo = 0, hi = n;
   int const w = blockIdx.x;
@@ -584,11 +677,15 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_gemm_multi_kernel(
   }
   __syncthreads();
   DevProgram const &P = *reinterpret_cast<DevProgram const *>(lds + kFpMfmaLdsBytes);
+  uint16_t *exp_lds = reinterpret_cast<uint16_t *>(lds + kFpMfmaLdsBytes + sizeof(DevProgram));
+  if (P.fp_unary[2] == TB_EXP_OP) {
+    load_exp_table(tbl, exp_lds);
+  }
   int v = w - first_block[lo];
   int const gx = P.grid[0] / P.pl_group[0], gy = P.grid[1] / P.pl_group[1];
   int const x = v % (gx * P.splits);
   v /= gx * P.splits;
-  fp_mfma_gemm_block(P, reinterpret_cast<int *>(lds), (x % gx) * P.pl_group[0], (v % gy) * P.pl_group[1],
+  fp_mfma_gemm_block(P, tbl, reinterpret_cast<int *>(lds), exp_lds, (x % gx) * P.pl_group[0], (v % gy) * P.pl_group[1],
                      v / gy, x / gx);
 }
 
@@ -784,7 +881,7 @@ bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_byte
   }
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]];
   int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
-  if (m % 16 != 0 || n % 16 != 0 || kt % 16 != 0) {
+  if (m % 16 != 0 || n % 16 != 0 || kt % 16 != 0 || (P.fp_unary[2] != 0 && kt % 64 != 0)) {
     return false;
   }
   size_t total = 0;
@@ -909,15 +1006,15 @@ int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream) {
     return rc;
   }
   dim3 grid(P.grid[0] / P.pl_group[0] * P.splits, P.grid[1] / P.pl_group[1], P.grid[2]);
-  fp_mfma_gemm_kernel<<<grid, kThreads, 0, stream>>>(P);
+  fp_mfma_gemm_kernel<<<grid, kThreads, 0, stream>>>(P, tables());
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }
 
 int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,
                               hipStream_t stream) {
-  int const lds_total = kFpMfmaLdsBytes + (int)sizeof(DevProgram);
-  fp_mfma_gemm_multi_kernel<<<blocks, kThreads, lds_total, stream>>>(progs, first_block, n);
+  int const lds_total = kFpMfmaLdsBytes + (int)sizeof(DevProgram) + 256;  // sums, record, exp table
+  fp_mfma_gemm_multi_kernel<<<blocks, kThreads, lds_total, stream>>>(progs, first_block, n, tables());
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }

@@ -938,15 +938,18 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   bool const declared = f16 && state().plan_smem_layout != 0;
   // (only a load-load-matmul-save plan can take the fused fingerprint kernel: everything
   // else is lowered once, with the limit)
-  // (load, load, [exp / silu]*, matmul, save)
+  // (load, load, [exp / silu]*, matmul, [exp / silu], save)
   bool try_fused_fp = !f16 && !state().force_interpreter && plan->num_operators >= 4 &&
-                      plan->num_operators <= 6 && plan->operator_types[0] == TB_INPUT_OP &&
+                      plan->num_operators <= 7 && plan->operator_types[0] == TB_INPUT_OP &&
                       plan->operator_types[1] == TB_INPUT_OP &&
-                      plan->operator_types[plan->num_operators - 2] == TB_MATMUL_OP &&
                       plan->operator_types[plan->num_operators - 1] == TB_OUTPUT_OP;
-  for (int o = 2; try_fused_fp && o < plan->num_operators - 2; o++) {
-    try_fused_fp = plan->operator_types[o] == TB_EXP_OP || plan->operator_types[o] == TB_SILU_OP;
+  int matmuls = 0;
+  for (int o = 2; try_fused_fp && o < plan->num_operators - 1; o++) {
+    int const t = plan->operator_types[o];
+    matmuls += t == TB_MATMUL_OP ? 1 : 0;
+    try_fused_fp = t == TB_MATMUL_OP || t == TB_EXP_OP || t == TB_SILU_OP;
   }
+  try_fused_fp = try_fused_fp && matmuls == 1;
   int rc = compile_plan(*plan, f16, (try_fused || try_fused_fp) ? (1 << 30) : state().max_lds, prog, ext,
                         err, declared);
   if (rc != MI355_OK) {
@@ -963,7 +966,7 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
     // a plan with an operand prologue can only run on the matrix-core route: it must fit
     size_t need = 0;
     bool fused = fp_gemm_applicable(prog);
-    if (fused && prog.fp_unary[2] &&
+    if (fused && fp_needs_matrix_cores(prog) &&
         !(fp_mfma_gemm_fits(prog, ext, &need) && need <= state().planes_bytes)) {
       fused = false;
     }
@@ -1051,7 +1054,7 @@ static int fold_splits(DevProgram const &prog) {
 static int launch(DevProgram const &prog, bool f16) {
   State &s = state();
   if (!f16 && prog.fused == 4) {
-    if (!prog.fg[5] && prog.fp_unary[2]) {
+    if (!prog.fg[5] && fp_needs_matrix_cores(prog)) {
       return fail(MI355_ERR_UNSUPPORTED, "operand prologue without the matrix-core route");
     }
     if (int rc = prog.fg[5] ? launch_fp_mfma_gemm(prog, s.stream()) : launch_fp_gemm(prog, s.stream())) {
@@ -1177,7 +1180,7 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
       fp_mfma_gemm_bind(progs[i], s.planes() + planes_used);
       planes_used += (need + 255) / 256 * 256;
       on_matrix_cores.push_back(&progs[i]);
-    } else if (progs[i].fused == 4 && progs[i].fp_unary[2]) {
+    } else if (progs[i].fused == 4 && fp_needs_matrix_cores(progs[i])) {
       // (the caller cuts chunks so that the planes of their members fit together)
       return fail(MI355_ERR_UNSUPPORTED, "operand prologue without the matrix-core route");
     }

@@ -80,10 +80,10 @@ struct alignas(16) DevProgram {
   // blocks (along grid x / y) when A does not move with x and B not with y: their tiles form
   // one larger tile whose operand strips are fetched once
   int pl_group[2];
-  // element-wise operator the plan applies to the A tile / the B tile before the matmul
-  // (TB_EXP_OP, TB_SILU_OP or 0): on the matrix-core route it is applied once per element
-  // while the operand tensor is split into planes; [2] != 0 marks a program that only that
-  // route can run
+  // element-wise operators around the matmul (TB_EXP_OP, TB_SILU_OP or 0): [0] / [1] applied
+  // to the A / B tile before it (on the matrix-core route once per element, while the operand
+  // tensor is split into planes), [2] applied to every iteration's product before the saver
+  // adds it up.  Only the matrix-core route runs a program that has any of them.
   int fp_unary[3];
   uint32_t pl_magic[2];  // division magics of m / 16 and n / 16 (strips per logical block)
   int pl_pad2[1];
@@ -139,6 +139,9 @@ int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream);
 int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,
                               hipStream_t stream);
 constexpr int kFpMfmaLdsBytes = 32768;  // wavefront sums of a tile whose k range is shared
+inline bool fp_needs_matrix_cores(DevProgram const &p) {
+  return (p.fp_unary[0] | p.fp_unary[1] | p.fp_unary[2]) != 0;
+}
 // Workgroups a fused matmul program is launched with (grouped blocks count once).
 inline long long fp_program_blocks(DevProgram const &p) {
   long long const gx = p.fused == 4 && p.fg[5] ? p.pl_group[0] : 1, gy = p.fused == 4 && p.fg[5] ? p.pl_group[1] : 1;

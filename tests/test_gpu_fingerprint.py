@@ -256,6 +256,37 @@ def test_fused_matmul_fingerprint_with_operand_prologues(rt, abi, pro):
         assert np.array_equal(out, want), route
 
 
+@pytest.mark.parametrize("m,n,k,grid,F,epi,pro,fused", [
+    (64, 256, 512, (4, 1, 1), 8, "exp", None, True),      # k tile 64: one step per iteration
+    (64, 256, 512, (4, 1, 1), 4, "silu", "exp", True),    # k tile 128, exp(A) before, silu after
+    (32, 32, 1024, (1, 1, 1), 16, "exp", None, True),     # one 32 x 32 piece: wavefronts share iterations
+    (64, 32, 64 * 37, (1, 1, 1), 37, "exp", None, True),  # two pieces, 37 iterations: uneven shares, split for-loop
+    (64, 256, 512, (4, 1, 1), 16, "exp", None, False),    # k tile 32: not whole steps, interpreter
+])
+def test_fused_matmul_fingerprint_with_operator_on_the_products(rt, abi, m, n, k, grid, F, epi, pro, fused):
+    """exp / silu of every iteration's product before the saver adds it up (sum over
+    iterations of f(A_it . B_it)): on the matrix-core route each iteration's residue sums are
+    recombined, the operator applied and the result added to a running sum."""
+    from attention_superoptimizer_amd import workloads as W
+    ops, a_ref, nxt = [], (0, 0), 2
+    if pro is not None:
+        ops.append((f"tb_{pro}_op", [(0, 0)]))
+        a_ref, nxt = (nxt, 0), nxt + 1
+    ops.append(("tb_matmul_op", [a_ref, (1, 0)]))
+    ops.append((f"tb_{epi}_op", [(nxt, 0)]))
+    b_imap = (1, -1, -1) if grid[0] > 1 else (-1, -1, -1)
+    omap = (1, -1, -1) if grid[0] > 1 else (-1, -1, -1)
+    spec = [W._inp([m, k]), W._inp([k, n]),
+            {"op": "customized", "in": [[0, 0], [1, 0]],
+             "plan": W._plan(grid, F, [(-1, -1, -1), b_imap], (1, 0), omap, ops)}]
+    ins = {0: uniform_fp(spec[0]["dims"], 81), 1: uniform_fp(spec[1]["dims"], 82)}
+    want = orc.eval_graph(spec, "fp", ins, threads=8)[2][0]
+    got = _fused_matmul_routes(rt, abi, spec, ins)
+    for route, (kernel_id, lds, out) in got.items():
+        assert kernel_id == (6 if route == "auto" and fused else 1), route
+        assert np.array_equal(out, want), route
+
+
 def test_many_fills_and_many_compares_in_one_launch(rt, abi):
     """mi355_fp_fill_many over 40 tensors of ragged sizes = the single-tensor fill of each;
     mi355_fp_equal_enqueue_many over 40 pairs = the verdict of each pair (every third pair is
