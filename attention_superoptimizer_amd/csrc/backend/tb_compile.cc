@@ -491,19 +491,41 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       if (m % 4 != 0 || n % 4 != 0 || k % 4 != 0) {
         continue;
       }
-      // matrix-core variant (signed-byte residues, swizzled rows, no padding): tiles whose m
-      // and n are multiples of 16, k chunks that are powers of two from 64; `sub` = 1 selects it
+      // Matrix-core variant (signed-byte residues, swizzled rows, no padding): tiles whose m
+      // and n are multiples of 16, k chunks that are powers of two from 64; A may be packed in
+      // row blocks (a power-of-two fraction of m, at least 16 rows) when the whole tile does
+      // not fit beside B^T.  `sub` = 1 selects it; preferred over the vector-dot path, which
+      // takes whatever chunk still fits otherwise.
       d.sub = 0;
-      for (int kc = k; kc >= 16 || kc == k; kc /= 2) {
+      d.mm_mb = 0;
+      if (vector_dot_only == 0 && m % 16 == 0 && n % 16 == 0) {
+        int top = 64;
+        while (top * 2 <= k) {
+          top *= 2;
+        }
+        for (int kc = top; kc >= 64 && kc <= k && d.sub == 0; kc /= 2) {
+          if (k % kc != 0) {
+            continue;
+          }
+          for (int mb = m; mb >= 16 && mb % 16 == 0 && m % mb == 0; mb /= 2) {
+            int const need = 2 * kc * (mb + n);
+            if (peak + need <= device_lds) {
+              d.mm_kc = kc;
+              d.mm_mb = mb;
+              d.sub = 1;
+              scratch = std::max(scratch, need);
+              break;
+            }
+          }
+        }
+      }
+      for (int kc = k; d.sub == 0 && (kc >= 16 || kc == k); kc /= 2) {
         if (kc % 4 != 0 || k % kc != 0) {
           break;
         }
-        bool const mfma = vector_dot_only == 0 && m % 16 == 0 && n % 16 == 0 && kc >= 64 &&
-                          (kc & (kc - 1)) == 0;
-        int const need = mfma ? 2 * kc * (m + n) : 2 * kc * (m + 4 + n);
+        int const need = 2 * kc * (m + 4 + n);
         if (peak + need <= device_lds) {
           d.mm_kc = kc;
-          d.sub = mfma ? 1 : 0;
           scratch = std::max(scratch, need);
           break;
         }

@@ -184,8 +184,10 @@ __device__ __forceinline__ uint32_t signed_residues_p(uint32_t v0, uint32_t v1, 
 
 __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C, int m, int n, int k,
                                DevOp const &op, unsigned char *scratch, int tid) {
-  int const kc = op.mm_kc, kq = kc / 4, pitch = kc;
-  unsigned char *Ab = scratch, *Bb = scratch + 2 * m * pitch;
+  // A is packed `mb` rows at a time (op.mm_mb, a multiple of 16 that divides m; the whole
+  // tile when the scratch allows), B^T once per k chunk
+  int const kc = op.mm_kc, kq = kc / 4, pitch = kc, mb = op.mm_mb;
+  unsigned char *Ab = scratch, *Bb = scratch + 2 * mb * pitch;
   // chunk c of row `row` lives at chunk c ^ key(row): rows that share a 256-byte bank line
   // (4 rows of 64 bytes, 2 of 128) and rows a multiple of that apart get different keys
   int const key_shift = kc >= 256 ? 0 : (kc == 128 ? 1 : 2);
@@ -195,18 +197,10 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
   };
   int const n2 = n / 2;
   int const wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
-  int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
+  int const mt_n = (n + 31) / 32, mt = ((mb + 31) / 32) * mt_n;  // 32 x 32 pieces of a row block
   for (int k0 = 0; k0 < k; k0 += kc) {
     if (k0 > 0) {
       __syncthreads();  // the previous chunk's residues are still being read
-    }
-    for (int e = tid; e < m * kq; e += kInterpThreads) {
-      int const row = fdiv(e, op.mg0), q = e - row * kq;
-      uint2 v = *reinterpret_cast<uint2 const *>(A + row * k + k0 + 4 * q);
-      uint32_t v0 = v.x & 0xffffu, v1 = v.x >> 16, v2 = v.y & 0xffffu, v3 = v.y >> 16;
-      int const at = row * pitch + swz(row, 4 * q);
-      *reinterpret_cast<uint32_t *>(Ab + at) = signed_residues_p(v0, v1, v2, v3);
-      *reinterpret_cast<uint32_t *>(Ab + m * pitch + at) = pack_residues(v0, v1, v2, v3, FP_Q);
     }
     for (int e = tid; e < kq * n2; e += kInterpThreads) {
       int const q = fdiv(e, op.mg1), c2 = (e - q * n2) * 2;
@@ -224,68 +218,81 @@ __device__ void fp_matmul_mfma(uint16_t const *A, uint16_t const *B, uint16_t *C
       *reinterpret_cast<uint32_t *>(Bb + n * pitch + at1) =
           pack_residues(w0 >> 16, w1 >> 16, w2 >> 16, w3 >> 16, FP_Q);
     }
-    __syncthreads();
-    for (int t = wave; t < mt; t += kInterpThreads / 64) {
-      int const row_m = (t / mt_n) * 32, col_n = (t - (t / mt_n) * mt_n) * 32;
-      int const i1 = row_m + 16 < m ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
-      unsigned char const *a_at[2], *b_at[2];
-      int a_key[2], b_key[2];
-#pragma unroll
-      for (int i = 0; i < 2; i++) {
-        int const ar = row_m + 16 * (i ? i1 : 0) + r, br = col_n + 16 * (i ? j1 : 0) + r;
-        a_at[i] = Ab + ar * pitch;
-        b_at[i] = Bb + br * pitch;
-        a_key[i] = (ar >> key_shift) & key_mask;
-        b_key[i] = (br >> key_shift) & key_mask;
+    for (int m0 = 0; m0 < m; m0 += mb) {
+      if (m0 > 0) {
+        __syncthreads();  // the previous row block's residues are still being read
       }
-      v4i acc[2][2][2];
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
+      for (int e = tid; e < mb * kq; e += kInterpThreads) {
+        int const row = fdiv(e, op.mg0), q = e - row * kq;
+        uint2 v = *reinterpret_cast<uint2 const *>(A + (m0 + row) * k + k0 + 4 * q);
+        uint32_t v0 = v.x & 0xffffu, v1 = v.x >> 16, v2 = v.y & 0xffffu, v3 = v.y >> 16;
+        int const at = row * pitch + swz(row, 4 * q);
+        *reinterpret_cast<uint32_t *>(Ab + at) = signed_residues_p(v0, v1, v2, v3);
+        *reinterpret_cast<uint32_t *>(Ab + mb * pitch + at) = pack_residues(v0, v1, v2, v3, FP_Q);
       }
-      for (int ks = 0; ks < kc; ks += 64) {
-        v4i ap[2], aq[2], bp[2], bq[2];
+      __syncthreads();
+      for (int t = wave; t < mt; t += kInterpThreads / 64) {
+        int const row_m = (t / mt_n) * 32, col_n = (t - (t / mt_n) * mt_n) * 32;
+        int const i1 = row_m + 16 < mb ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
+        unsigned char const *a_at[2], *b_at[2];
+        int a_key[2], b_key[2];
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-          int const ca = (((ks >> 4) + g) ^ a_key[i]) << 4, cb = (((ks >> 4) + g) ^ b_key[i]) << 4;
-          ap[i] = *reinterpret_cast<v4i const *>(a_at[i] + ca);
-          aq[i] = *reinterpret_cast<v4i const *>(a_at[i] + m * pitch + ca);
-          bp[i] = *reinterpret_cast<v4i const *>(b_at[i] + cb);
-          bq[i] = *reinterpret_cast<v4i const *>(b_at[i] + n * pitch + cb);
+          int const ar = row_m + 16 * (i ? i1 : 0) + r, br = col_n + 16 * (i ? j1 : 0) + r;
+          a_at[i] = Ab + ar * pitch;
+          b_at[i] = Bb + br * pitch;
+          a_key[i] = (ar >> key_shift) & key_mask;
+          b_key[i] = (br >> key_shift) & key_mask;
+        }
+        v4i acc[2][2][2];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          acc[e / 4][(e / 2) % 2][e % 2] = v4i{0, 0, 0, 0};
+        }
+        for (int ks = 0; ks < kc; ks += 64) {
+          v4i ap[2], aq[2], bp[2], bq[2];
+#pragma unroll
+          for (int i = 0; i < 2; i++) {
+            int const ca = (((ks >> 4) + g) ^ a_key[i]) << 4, cb = (((ks >> 4) + g) ^ b_key[i]) << 4;
+            ap[i] = *reinterpret_cast<v4i const *>(a_at[i] + ca);
+            aq[i] = *reinterpret_cast<v4i const *>(a_at[i] + mb * pitch + ca);
+            bp[i] = *reinterpret_cast<v4i const *>(b_at[i] + cb);
+            bq[i] = *reinterpret_cast<v4i const *>(b_at[i] + n * pitch + cb);
+          }
+#pragma unroll
+          for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int jn = 0; jn < 2; jn++) {
+              acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bp[jn], ap[i], acc[0][i][jn], 0, 0, 0);
+              acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[jn], aq[i], acc[1][i][jn], 0, 0, 0);
+            }
+          }
         }
 #pragma unroll
         for (int i = 0; i < 2; i++) {
 #pragma unroll
           for (int jn = 0; jn < 2; jn++) {
-            acc[0][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bp[jn], ap[i], acc[0][i][jn], 0, 0, 0);
-            acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[jn], aq[i], acc[1][i][jn], 0, 0, 0);
-          }
-        }
-      }
+            if (i > i1 || jn > j1) {
+              continue;
+            }
+            uint16_t *cp = C + (m0 + row_m + 16 * i + r) * n + col_n + 16 * jn + 4 * g;
+            uint32_t z[4];
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-#pragma unroll
-        for (int jn = 0; jn < 2; jn++) {
-          if (i > i1 || jn > j1) {
-            continue;
+            for (int e = 0; e < 4; e++) {
+              z[e] = fp_from_residue_sums(acc[0][i][jn][e], acc[1][i][jn][e]);
+            }
+            if (k0 > 0) {
+              uint2 old = *reinterpret_cast<uint2 const *>(cp);
+              z[0] = (z[0] + (old.x & 0xffffu)) % FP_PQ;
+              z[1] = (z[1] + (old.x >> 16)) % FP_PQ;
+              z[2] = (z[2] + (old.y & 0xffffu)) % FP_PQ;
+              z[3] = (z[3] + (old.y >> 16)) % FP_PQ;
+            }
+            uint2 out;
+            out.x = z[0] | (z[1] << 16);
+            out.y = z[2] | (z[3] << 16);
+            *reinterpret_cast<uint2 *>(cp) = out;
           }
-          uint16_t *cp = C + (row_m + 16 * i + r) * n + col_n + 16 * jn + 4 * g;
-          uint32_t z[4];
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            z[e] = fp_from_residue_sums(acc[0][i][jn][e], acc[1][i][jn][e]);
-          }
-          if (k0 > 0) {
-            uint2 old = *reinterpret_cast<uint2 const *>(cp);
-            z[0] = (z[0] + (old.x & 0xffffu)) % FP_PQ;
-            z[1] = (z[1] + (old.x >> 16)) % FP_PQ;
-            z[2] = (z[2] + (old.y & 0xffffu)) % FP_PQ;
-            z[3] = (z[3] + (old.y >> 16)) % FP_PQ;
-          }
-          uint2 out;
-          out.x = z[0] | (z[1] << 16);
-          out.y = z[2] | (z[3] << 16);
-          *reinterpret_cast<uint2 *>(cp) = out;
         }
       }
     }

@@ -55,6 +55,7 @@ struct DevOp {
   int red_deg, red_inner;                    // REDUCE (flat row-major rule of the reference)
   int cat_a, cat_b, cat_inner;               // CONCAT
   int mm_kc;  // MATMUL, uint16 interpreter: k chunk of the packed-residue path, 0 = scalar path
+  int mm_mb;  // MATMUL, matrix-core variant (sub == 1): rows of A packed at a time
   // division magics.  MATMUL: kc / 4, n / 2, n / 4.  REDUCE: inner.  CONCAT: inner, a + b.
   uint32_t mg0, mg1, mg2;
 };
