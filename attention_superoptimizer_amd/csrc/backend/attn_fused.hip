@@ -956,6 +956,253 @@ bool match(DevProgram const &P, Match &M) {
   return true;
 }
 
+// Latency variant for short for-loops (every iteration has a wavefront of its own: F <= IP)
+// with the staging of the throughput variant: each wavefront streams the K and V tile of ITS
+// iteration from global memory straight into its own 16 KB of LDS, in their row-major layout
+// (sixteen direct loads, no registers, no transposing stores, and no workgroup barrier before
+// the arithmetic: a wavefront only waits for its own loads), and gathers the MFMA operands
+// with transposing LDS reads under the same chunk swizzle.  Arithmetic, rounding points, the
+// ordered hand-over of the iterations' results and the store are those of attn_fused_kernel.
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
+__global__ __launch_bounds__(64 * RG * IP) void attn_direct_kernel(AttnParams const P) {
+  static_assert(NK == 64 && DV == 64, "the chunk swizzles assume rows of 128 bytes");
+  constexpr int LDO = DV + 8;
+  constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
+  constexpr int NW = RG * IP;
+  constexpr int KI = D * NK / 8 / 64, VI = NK * DV / 8 / 64;  // direct loads per tile
+  constexpr int WAVE_HALFS = D * NK + NK * DV;
+  constexpr int SLOT_DW = DB * 2 + 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+  int const tid = threadIdx.x;
+  int const lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  int const rg = wave / IP, ip = wave % IP;
+  int const g = lane / 16, c = lane % 16;
+  int bx, by, bz, slice;
+  decode_block(P, bx, by, bz, slice);
+  int const row_base = (slice * RG + rg) * 16;
+  bool const active = ip < P.forloop_range;
+
+  _Float16 *const kt = reinterpret_cast<_Float16 *>(lds) + wave * WAVE_HALFS;
+  _Float16 *const vt = kt + D * NK;
+  if (active) {
+    // this lane's chunk of direct load i is (row r, position pos) of the tile and comes from
+    // global chunk pos ^ 2 * key(r) of row r
+    uint32_t const lds_k = lds_address(kt), lds_v = lds_address(vt);
+    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, ip);
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, ip);
+#pragma unroll
+    for (int i = 0; i < KI; i++) {
+      int const q = i * 64 + lane, r = q / (NK / 8), pos = q % (NK / 8);
+      uint32_t const off = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(r))));
+      lds_dma16(kg, off, lds_k + 1024u * (uint32_t)i);
+    }
+#pragma unroll
+    for (int i = 0; i < VI; i++) {
+      int const q = i * 64 + lane, r = q / (DV / 8), pos = q % (DV / 8);
+      uint32_t const off = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(r))));
+      lds_dma16(vg, off, lds_v + 1024u * (uint32_t)i);
+    }
+  }
+  // Q fragments (B operand of S^T): Q[row c][32kk + 8g .. +7]
+  half8 qf[DK];
+  {
+    _Float16 const *q = static_cast<_Float16 const *>(P.q.ptr) + tile_offset(P.q, bx, by, bz, 0) +
+                        (long long)(row_base + c) * P.q.d_cols + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < DK; kk++) {
+      qf[kk] = *reinterpret_cast<half8 const *>(q + 32 * kk);
+    }
+  }
+  int const a4 = c >> 2, b4 = c & 3;
+  int const k_lane = (8 * g + a4) * NK + ((b4 >> 1) << 3) + (b4 & 1) * 4;
+  int const v_lane = (4 * g + a4) * DV + ((b4 >> 1) << 3) + (b4 & 1) * 4;
+  int const sw_k = stream_swizzle_key<NK, true>(8 * g + a4) << 4;
+  int const sw_v = stream_swizzle_key<DV, false>(4 * g + a4) << 4;
+
+  unsigned char *const tail = lds + NW * WAVE_HALFS * 2;
+  _Float16 *const o_stage = reinterpret_cast<_Float16 *>(tail);
+  uint32_t *const slots = reinterpret_cast<uint32_t *>(tail + RG * 16 * LDO * 2);
+
+  _Float16 o16[DB][4];
+  _Float16 r16 = (_Float16)0.0f;
+#pragma unroll
+  for (int t = 0; t < DB; t++) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      o16[t][r] = (_Float16)0.0f;
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's own tiles have landed
+  if (active) {
+    uint32_t pk[KB / 2][4];
+    float rs = 0.0f;
+    half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
+    constexpr float LOG2E = 1.44269504088896340736f;
+#pragma unroll
+    for (int j = 0; j < KB; j++) {
+      float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int kk = 0; kk < DK; kk++) {
+        // K[32kk + 8g + 0..7][16j + c]
+        _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw_k ^ (j << 4));
+        half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
+        half8 const a = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kk], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        half2v const s2 = {static_cast<_Float16>(acc[2 * h]), static_cast<_Float16>(acc[2 * h + 1])};
+        float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
+        float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
+        half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
+        rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);
+        pk[j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
+      }
+    }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    r16 = static_cast<_Float16>(rs);
+    if (HAS_DIV) {
+      float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
+#pragma unroll
+      for (int jj = 0; jj < KB / 2; jj++) {
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+          half2v const e2 = __builtin_bit_cast(half2v, pk[jj][w]);
+          half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
+                             static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+          pk[jj][w] = __builtin_bit_cast(uint32_t, p2);
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+      float4v o = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int jj = 0; jj < KB / 2; jj++) {
+        // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
+        _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
+        half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
+        half8 const b = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        uint4v const a = {pk[jj][0], pk[jj][1], pk[jj][2], pk[jj][3]};
+        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        o16[t][r] = static_cast<_Float16>(o[r]);
+      }
+    }
+  }
+  // hand the iteration's result to the row group's first wavefront, which adds the
+  // iterations in order, rounding to fp16 after each add as the sequential loop would
+  _Float16 oacc[DB][4];
+  _Float16 racc = (_Float16)0.0f;
+  if (IP > 1) {
+    if (ip > 0 && active) {
+      uint32_t *slot = slots + ((rg * (IP - 1) + (ip - 1)) * SLOT_DW) * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < DB; t++) {
+        half2v lo = {o16[t][0], o16[t][1]}, hi = {o16[t][2], o16[t][3]};
+        slot[(2 * t) * 64] = __builtin_bit_cast(uint32_t, lo);
+        slot[(2 * t + 1) * 64] = __builtin_bit_cast(uint32_t, hi);
+      }
+      half2v rr = {r16, (_Float16)0.0f};
+      slot[(2 * DB) * 64] = __builtin_bit_cast(uint32_t, rr);
+    }
+    __syncthreads();
+  }
+  _Float16 *ow = o_stage + rg * 16 * LDO;
+  if (ip == 0) {
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        oacc[t][r] = (_Float16)0.0f;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < IP; q++) {
+      if (q < P.forloop_range) {
+        if (q > 0) {
+          uint32_t const *slot = slots + ((rg * (IP - 1) + (q - 1)) * SLOT_DW) * 64 + lane;
+#pragma unroll
+          for (int t = 0; t < DB; t++) {
+            half2v lo = __builtin_bit_cast(half2v, slot[(2 * t) * 64]);
+            half2v hi = __builtin_bit_cast(half2v, slot[(2 * t + 1) * 64]);
+            o16[t][0] = lo[0];
+            o16[t][1] = lo[1];
+            o16[t][2] = hi[0];
+            o16[t][3] = hi[1];
+          }
+          r16 = __builtin_bit_cast(half2v, slot[(2 * DB) * 64])[0];
+        }
+#pragma unroll
+        for (int t = 0; t < DB; t++) {
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            oacc[t][r] = static_cast<_Float16>(static_cast<float>(oacc[t][r]) + static_cast<float>(o16[t][r]));
+          }
+        }
+        if (!HAS_DIV) {
+          racc = static_cast<_Float16>(static_cast<float>(racc) + static_cast<float>(r16));
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < DB; t++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        ow[(4 * g + r) * LDO + 16 * t + c] = oacc[t][r];
+      }
+    }
+  }
+  __syncthreads();
+  if (ip == 0) {
+    _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
+                   tile_offset(P.o, bx, by, bz, 0) + (long long)row_base * P.o.d_cols;
+    constexpr int CH = DV / 8;
+    for (int e = lane; e < 16 * CH; e += 64) {
+      int rr = e / CH, cc = (e % CH) * 8;
+      *reinterpret_cast<uint4v *>(og + (long long)rr * P.o.d_cols + cc) =
+          *reinterpret_cast<uint4v const *>(ow + rr * LDO + cc);
+    }
+    if (!HAS_DIV && g == 0) {
+      _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
+                      tile_offset(P.r, bx, by, bz, 0);
+      rgp[(long long)(row_base + c) * P.r.d_cols] = racc;
+    }
+  }
+}
+
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
+int launch_direct_one(AttnParams const &A, dim3 grid, int lds) {
+  auto *fn = attn_direct_kernel<D, NK, DV, HAS_DIV, RG, IP>;
+  static int granted = 0;  // per instantiation
+  if (lds > 65536 && lds > granted) {
+    MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
+    granted = state().max_lds;
+  }
+  fn<<<grid, 64 * RG * IP, lds, state().stream()>>>(A);
+  MI355_HIP(hipGetLastError());
+  return 1;
+}
+
+// 64 / 64 / 64 tiles only; 0: no instantiation for these wavefront counts
+template <bool HAS_DIV>
+int launch_direct(AttnParams const &A, dim3 grid, int rg, int ip, int lds) {
+  switch (rg * 16 + ip) {
+    case 1 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 2>(A, grid, lds);
+    case 1 * 16 + 4: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 4>(A, grid, lds);
+    case 1 * 16 + 8: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 8>(A, grid, lds);
+    case 2 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 2, 2>(A, grid, lds);
+    case 2 * 16 + 4: return launch_direct_one<64, 64, 64, HAS_DIV, 2, 4>(A, grid, lds);
+    case 4 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 4, 2>(A, grid, lds);
+    default: return 0;
+  }
+}
+
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
 int launch_one(AttnParams const &A, dim3 grid, int lds) {
   auto *fn = attn_fused_kernel<D, NK, DV, HAS_DIV, RG, IP>;
@@ -1066,7 +1313,7 @@ int try_launch_attention(DevProgram const &P) {
     int rgs = (M.m % 128 == 0) ? 4 : ((M.m % 64 == 0) ? 2 : 0);
     bool const shape = (M.D == 64 && M.NK == 64 && M.DV == 64) || (M.D == 128 && M.NK == 64 && M.DV == 128);
     bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512;
-    if (s.attention_mode == 1) {
+    if (s.attention_mode == 1 || s.attention_mode == 3) {
       want = false;
     } else if (s.attention_mode == 2) {
       want = rgs != 0 && shape;
@@ -1126,14 +1373,26 @@ int try_launch_attention(DevProgram const &P) {
   }
   A.stages = stages;
   A.lds_stage_bytes = stage_bytes;
-  int const lds = stages * stage_bytes + tail_bytes;
+  int lds = stages * stage_bytes + tail_bytes;
   if (lds > s.max_lds) {
     return 0;
   }
   dim3 grid(P.grid[0] * A.split, P.grid[1], P.grid[2]);
   int const nw = rg * ip;
-  int rc;
-  if (M.D == 64 && M.NK == 64) {
+  int rc = 0;
+  // every iteration on a wavefront of its own and tiles of 64 x 64: the variant that streams
+  // the tiles straight into LDS (attention mode 3 keeps the register-transposed staging)
+  int const direct_lds = nw * stage_bytes + tail_bytes;
+  if (M.D == 64 && M.NK == 64 && M.DV == 64 && P.forloop_range <= ip && ip > 1 &&
+      direct_lds <= s.max_lds && s.attention_mode != 3) {
+    rc = M.has_div ? launch_direct<true>(A, grid, rg, ip, direct_lds)
+                   : launch_direct<false>(A, grid, rg, ip, direct_lds);
+    if (rc == 1) {
+      lds = direct_lds;
+    }
+  }
+  if (rc == 1) {
+  } else if (M.D == 64 && M.NK == 64) {
     rc = launch_shape<64, 64, 64>(A, M.has_div, grid, rg, ip, lds);
   } else if (M.D == 64 && M.NK == 128) {
     rc = launch_shape<64, 128, 64>(A, M.has_div, grid, rg, ip, lds);

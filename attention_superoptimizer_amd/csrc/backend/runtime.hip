@@ -242,7 +242,7 @@ extern "C" int mi355_set_option(int option, int value) {
     state().force_interpreter = value;
     return MI355_OK;
   }
-  if (option == MI355_OPT_ATTENTION_MODE && value >= 0 && value <= 2) {
+  if (option == MI355_OPT_ATTENTION_MODE && value >= 0 && value <= 3) {
     state().attention_mode = value;
     return MI355_OK;
   }

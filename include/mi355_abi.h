@@ -86,9 +86,10 @@ typedef struct mi355_launch_info {
  * fp16 or fingerprint, through the generic LDS interpreter instead of a fused kernel
  * (both must agree with the oracle; tests run the two against each other). */
 #define MI355_OPT_FORCE_INTERPRETER 1
-/* ATTENTION_MODE: 0 = choose by problem size (default), 1 = always the latency
+/* ATTENTION_MODE: 0 = choose by problem size (default), 1 = always a latency
  * variant of the fused attention kernel, 2 = the throughput variant whenever the
- * tile shape allows it. */
+ * tile shape allows it, 3 = the latency variant with register-transposed staging
+ * only (not the one that streams tiles straight into LDS). */
 #define MI355_OPT_ATTENTION_MODE 2
 /* PLAN_SMEM_LAYOUT: 0 = the lowering gives every fp16 tile the LDS layout its
  * consumers want (default); 1 = a loader's tile takes the layout its plan declares

@@ -231,6 +231,32 @@ def test_attention_throughput_variant(rt, abi):
         assert abi.mi355_set_option(2, 0) == 0
 
 
+def test_attention_latency_variants_agree(rt, abi):
+    """The two latency variants of the fused attention kernel (tiles streamed straight into
+    LDS and gathered with transposing reads / tiles transposed in registers while staged)
+    make the same roundings in the same order: identical fp16 outputs, each within the
+    tolerance of the golden.  C2 and the reference's decode examples with one iteration per
+    wavefront, both forms (with and without the division)."""
+    from attention_superoptimizer_amd import workloads as W
+    cases = [(W.config2_gqa_decode()[0], W.INPUT_STD["C2_gqa_decode"], "C2"),
+             (W.REFERENCE_EXAMPLES["dnn"][0], 0.05, "dnn"),                       # 8 iterations, 8 wavefronts
+             (W.REFERENCE_EXAMPLES["multi_head_attn_inc_decode"][0], 0.05, "mha inc decode")]
+    for spec, stds, what in cases:
+        ins = _inputs(spec, stds, 95)
+        outs = {}
+        for mode in (0, 3):
+            assert abi.mi355_set_option(2, mode) == 0
+            try:
+                got = _check(rt, spec, ins, f"{what} mode {mode}")
+                assert _last_kernels[0] == KERNEL_ATTENTION
+                outs[mode] = [got[i] for i in range(len(spec)) if spec[i]["op"] == "customized"]
+            finally:
+                assert abi.mi355_set_option(2, 0) == 0
+        for a, b in zip(outs[0], outs[3]):
+            for x, y in zip(a, b):
+                assert np.array_equal(x, y), what
+
+
 def test_full_size_configs_routes_agree(rt, abi):
     """Full benchmark sizes, where the scalar golden is too slow to run: the fused kernel
     and the generic LDS interpreter (each checked against the golden at reduced size) must
