@@ -1196,9 +1196,6 @@ int launch_direct(AttnParams const &A, dim3 grid, int rg, int ip, int lds) {
     case 1 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 2>(A, grid, lds);
     case 1 * 16 + 4: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 4>(A, grid, lds);
     case 1 * 16 + 8: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 8>(A, grid, lds);
-    case 2 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 2, 2>(A, grid, lds);
-    case 2 * 16 + 4: return launch_direct_one<64, 64, 64, HAS_DIV, 2, 4>(A, grid, lds);
-    case 4 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 4, 2>(A, grid, lds);
     default: return 0;
   }
 }
@@ -1382,13 +1379,24 @@ int try_launch_attention(DevProgram const &P) {
   int rc = 0;
   // every iteration on a wavefront of its own and tiles of 64 x 64: the variant that streams
   // the tiles straight into LDS (attention mode 3 keeps the register-transposed staging)
-  int const direct_lds = nw * stage_bytes + tail_bytes;
+  // (one row group per workgroup there: nothing is shared between row groups, and smaller
+  // workgroups start sooner; C2: 5.28 us against 5.38 with two)
+  int const direct_lds = ip * stage_bytes + 16 * (M.DV + 8) * 2 + (ip - 1) * (M.DV / 8 + 1) * 64 * 4;
   if (M.D == 64 && M.NK == 64 && M.DV == 64 && P.forloop_range <= ip && ip > 1 &&
-      direct_lds <= s.max_lds && s.attention_mode != 3) {
-    rc = M.has_div ? launch_direct<true>(A, grid, rg, ip, direct_lds)
-                   : launch_direct<false>(A, grid, rg, ip, direct_lds);
+      direct_lds <= s.max_lds && s.attention_mode != 3 &&
+      (long long)P.grid[0] * groups <= 2147483647LL) {
+    AttnParams B = A;
+    B.split = groups;
+    dim3 const direct_grid(P.grid[0] * B.split, P.grid[1], P.grid[2]);
+    rc = M.has_div ? launch_direct<true>(B, direct_grid, 1, ip, direct_lds)
+                   : launch_direct<false>(B, direct_grid, 1, ip, direct_lds);
     if (rc == 1) {
-      lds = direct_lds;
+      s.last_launch.kernel_id = MI355_KERNEL_F16_ATTENTION;
+      s.last_launch.workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
+      s.last_launch.threads = ip * 64;
+      s.last_launch.lds_bytes = direct_lds;
+      s.last_launch.row_split = B.split;
+      return rc;
     }
   }
   if (rc == 1) {
