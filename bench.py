@@ -32,11 +32,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_FP16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the headline kernel from hardware counters: rocprofv3 --pmc
-# FETCH_SIZE (1340.5 KiB per dispatch) and WRITE_SIZE (1024.0 KiB), each scaled by what the
+# FETCH_SIZE (1329.5 KiB per dispatch) and WRITE_SIZE (1024.0 KiB), each scaled by what the
 # same counter reads for a plain 256 MiB device copy (`--calibrate-copy 256`: FETCH_SIZE
 # counts half the bytes, factor 2.0; WRITE_SIZE factor 1.0).  A profiler cannot run inside
 # the timed process, so the figure is carried here; profiles/ holds the runs it comes from.
-HEADLINE_TRAFFIC_BYTES = int((2.0 * 1340.5 + 1.0 * 1024.0) * 1024)
+HEADLINE_TRAFFIC_BYTES = int((2.0 * 1329.5 + 1.0 * 1024.0) * 1024)
 
 
 def algorithmic_bytes(spec, idx, out_dims):
