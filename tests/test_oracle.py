@@ -52,6 +52,41 @@ def test_matmul_is_exact_mod_pq():
     assert np.all(orc.fp_matmul(A, B) == (5000 * (FP_PQ - 1) ** 2) % FP_PQ)
 
 
+def test_signed_byte_residue_planes_reproduce_the_matmul():
+    """The arithmetic the matrix-core fingerprint kernels rely on, restated in numpy: operands
+    split into signed bytes (mod 227 recentred to [-113, 113], mod 113 as it is), exact int32
+    dot products per field, and ONE recombination `(u * 25425 + v * 227) mod 25651` of the
+    unreduced sums u (made non-negative by adding 83715 * 25651) and v equal the oracle's
+    `(r + a*b) % 25651` chain; so does exp taken from the mod-113 sum alone."""
+    rng = np.random.default_rng(7)
+    A = rng.integers(0, FP_PQ, size=(1, 9, 4096)).astype(np.uint16)
+    B = rng.integers(0, FP_PQ, size=(1, 4096, 6)).astype(np.uint16)
+    A[0, 0, :] = (114 * 25425 + 112 * 227) % FP_PQ   # -113 mod 227, 112 mod 113: extreme bytes
+    B[0, :, 0] = (113 * 25425 + 112 * 227) % FP_PQ
+
+    def planes(X):
+        p = X.astype(np.int64) % 227
+        p = np.where(p > 113, p - 227, p)
+        q = X.astype(np.int64) % 113
+        assert p.min() >= -113 and p.max() <= 113 and q.max() <= 112
+        return p, q
+
+    (ap, aq), (bp, bq) = planes(A), planes(B)
+    u, v = ap @ bp, aq @ bq
+    assert np.abs(u).max() < 2 ** 31 - 2 ** 17 and v.min() >= 0 and v.max() < 2 ** 31
+    offset = 83715 * FP_PQ
+    assert offset == 2147373465 and offset < 2 ** 31
+    a = (u + offset) % FP_PQ
+    b = v % FP_PQ
+    assert (a * 25425 + b * 227).max() < 2 ** 32
+    z = (a * 25425 + b * 227) % FP_PQ
+    want = orc.fp_matmul(A, B)
+    assert np.array_equal(z, want)
+    exp_tbl = np.asarray(orc.tables()[0], np.int64)
+    lifted = (exp_tbl[:113] * 25425) % FP_PQ
+    assert np.array_equal(lifted[v % 113], orc.fp_unary("exp", want))
+
+
 def test_add_mul_broadcast_exhaustive_small():
     """every broadcast pattern of <=3 dims of size <=3 against numpy broadcasting"""
     rng = np.random.default_rng(2)
