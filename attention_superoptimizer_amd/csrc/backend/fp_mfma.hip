@@ -1,22 +1,28 @@
 // Fingerprint matmul on the matrix cores (reference src/kernel/cuda/matmul_kernel.cu:145-173
-// computes `r = (r + a*b) % 25651` per multiply-accumulate in one thread per output).
+// computes `r = (r + a*b) % 25651` per multiply-accumulate in one thread per output; the
+// thread-block form is include/mirage/threadblock/cuda/matmul.h:773-804).
 //
 // (sum a*b) mod 25651 is fixed by its residues mod 227 and mod 113.  Every operand is first
 // split, once per matrix, into two planes of signed bytes: the residue mod 227 recentred to
 // [-113, 113] and the residue mod 113; A keeps its orientation [rows][k], B is transposed
 // to [columns][k], k padded with zeros to a multiple of 64.  Both operands of
 // v_mfma_i32_16x16x64_i8 then want the same thing: 16 consecutive k of one row per lane,
-// one 16-byte load.  Planes are stored in blocks of 16 rows x 16 k (plane[row / 16][k / 16]
-// [row % 16][16 bytes]), so the 64 loads of a wavefront's operand fetch are one contiguous
-// kilobyte and a strip of 16 rows is one stream along k.  A 16 x 16 x 64 step per residue is one matrix instruction; the int32
-// sums are exact (|sum| <= 113^2 * k, folded every 131072 k) and are recombined once per
-// output with the reference's CRT multipliers, so results are bit-identical.
+// one 16-byte load.  Planes are stored in blocks of 16 rows x 16 k
+// (plane[row / 16][k / 16][row % 16][16 bytes]), so the 64 loads of a wavefront's operand
+// fetch are one contiguous kilobyte and a strip of 16 rows is one stream along k.  A
+// 16 x 16 x 64 step per residue is one matrix instruction; the int32 sums are exact
+// (|sum| <= 113^2 * k, folded every 131072 k) and are recombined once per output with the
+// reference's CRT multipliers (fp_from_residue_sums), so results are bit-identical.
 //
-// One submission takes many independent matmuls (the kernel-level matmuls of a batch of
-// candidate graphs): one launch splits all operands, one launch multiplies.  A workgroup
-// owns a 64 x 64 output tile (each wavefront a 32 x 32 quadrant over all of k) when its
-// matmul has enough tiles to matter, otherwise a 32 x 32 tile whose k range the four
-// wavefronts share, added up through LDS.
+// Two users.  Kernel-level matmuls: one submission takes many independent ones (those of a
+// batch of candidate graphs): one launch splits all operands, one launch multiplies; a
+// workgroup owns a 64 x 64 output tile (each wavefront a 32 x 32 quadrant over all of k)
+// when its matmul has enough tiles to matter, otherwise a 32 x 32 tile whose k range the
+// four wavefronts share, added up through LDS.  Fused tiled-matmul plans of customized
+// operators (load A tile, load B tile, [exp / silu of a tile], matmul, [exp / silu of the
+// product], accumulate over the for-loop, store): the operand TENSORS are split once per
+// launch and every logical block reads its tiles from the planes through the plan's own
+// strides; see fp_mfma_gemm_block.
 #include "common.h"
 #include "tb_program.h"
 
