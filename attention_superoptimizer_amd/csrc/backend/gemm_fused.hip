@@ -15,10 +15,16 @@
 //    of an iteration before it waits for any, so one compute unit keeps several
 //    whole tiles in flight;
 //  * the reference's generated programs round each iteration's product to fp16 and
-//    add it to an fp16 accumulator in iteration order.  Every workgroup does exactly
-//    that over its own range and writes its fp16 sum to a scratch slab; a second,
-//    tiny launch adds the ranges' sums of each block in range order, again rounding
-//    to fp16 after each add, and stores;
+//    add it to an fp16 accumulator in iteration order (src/kernel/triton_code_gen.cc:
+//    223-232).  A workgroup that owns a whole for-loop does exactly that in registers.
+//    When the for-loop is cut into ranges, summing each range by itself would regroup
+//    the fp16 additions ((t0+t1)+(t2+t3) instead of ((t0+t1)+t2)+t3), which is a
+//    different rounding sequence; so a range's workgroup stores every iteration's fp16
+//    product tile to a scratch slab instead (a few percent of the weight bytes) and a
+//    second, small launch adds the tiles of each block in ITERATION order, rounding to
+//    fp16 after each add: the same sequence of roundings as the unsplit loop;
+//  * products are formed transposed (weights as the first MFMA operand), which leaves a
+//    lane with four consecutive output columns of one row: 8-byte stores;
 //  * weight tiles arrive [k][n] with n contiguous while the MFMA wants k contiguous
 //    per lane, so they are transposed once while being staged into LDS (4 x 16 B
 //    global reads -> 8 x 8 B LDS writes per 4x8 patch), into unpadded rows with a
@@ -55,7 +61,7 @@ struct GemmParams {
   int M, KT;         // rows of the activation tile, k extent of one iteration
   int forloop_range;
   int ksplit;        // workgroups per logical block
-  _Float16 *scratch; // [blocks][ksplit][NB][M][64] fp16 range sums (ksplit > 1)
+  _Float16 *scratch; // [blocks][forloop_range][NB][M][64] fp16 product tiles (ksplit > 1)
 };
 
 __device__ __forceinline__ long long gtile_offset(GTile const &t, int bx, int by, int bz, int it) {
@@ -199,7 +205,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
     stage_weight<1>(src, P.lb.d_cols, 16, 64, lb_lds, tid, NT);
   }
 
-  _Float16 acc16[NB][MT][4];  // O[16mt + 4g + r][16*wave + c], used when ksplit == 1
+  _Float16 acc16[NB][MT][4];  // O[16mt + c][16*wave + 4g + r], used when ksplit == 1
 #pragma unroll
   for (int b = 0; b < NB; b++) {
 #pragma unroll
@@ -285,7 +291,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
       store_weight<LORA ? LPPT : 1>(lreg, KT, 16, la_lds, tid, NT);
     }
   };
-  auto compute = [&]() {
+  bool const split = P.ksplit > 1;
+  auto compute = [&](int it) {
     // ---- lora inner product, transposed: D^T = A^T . X^T (rows past M are zero) -----
     half4 dfrag = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
     if (LORA) {
@@ -317,22 +324,39 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
           half8 a = *reinterpret_cast<half8 const *>(a_lds + sw_chunk(16 * mt + c, ch, KT, kmask));
-          o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, w, o[mt], 0, 0, 0);
+          // weights first: o[mt][r] = O[m = 16mt + c][n = 16 wave + 4g + r]
+          o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, a, o[mt], 0, 0, 0);
         }
       }
       if (LORA) {
         // + [X.A] . B over the 16 concatenated k; B^T rows hold 16 halfs (2 chunks)
         half4 w = *reinterpret_cast<half4 const *>(lb_lds + sw_chunk(16 * wave + c, g >> 1, 16, 1) +
                                                    (g & 1) * 4);
-        o[0] = __builtin_amdgcn_mfma_f32_16x16x16f16(dfrag, w, o[0], 0, 0, 0);
+        o[0] = __builtin_amdgcn_mfma_f32_16x16x16f16(w, dfrag, o[0], 0, 0, 0);
       }
+      if (split) {
+        // this iteration's fp16 product tile goes to its slot of the scratch slab
+        _Float16 *tile = P.scratch + (((long long)block_linear * F + it) * NB + b) * (long long)M * 64;
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) {
+        for (int mt = 0; mt < MT; mt++) {
+          half4 p16;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          _Float16 p16 = static_cast<_Float16>(o[mt][r]);  // this iteration's product tile
-          acc16[b][mt][r] = static_cast<_Float16>(static_cast<float>(acc16[b][mt][r]) +
-                                                  static_cast<float>(p16));
+          for (int r = 0; r < 4; r++) {
+            p16[r] = static_cast<_Float16>(o[mt][r]);
+          }
+          if (16 * mt + c < M) {
+            *reinterpret_cast<half4 *>(tile + (16 * mt + c) * 64 + 16 * wave + 4 * g) = p16;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            _Float16 p16 = static_cast<_Float16>(o[mt][r]);  // this iteration's product tile
+            acc16[b][mt][r] = static_cast<_Float16>(static_cast<float>(acc16[b][mt][r]) +
+                                                    static_cast<float>(p16));
+          }
         }
       }
     }
@@ -348,17 +372,19 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
     __syncthreads();
     fetch(it + 1);
     __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the products
-    compute();
+    compute(it);
   }
   __syncthreads();
   stash();
   __syncthreads();
-  compute();
+  compute(it_end - 1);
 
   // ---- finish ---------------------------------------------------------------------------
-  // The workgroup's fp16 sums go through LDS so that they leave as 16-byte row
-  // segments: straight to the output when the for-loop was not split, else to this
-  // range's slab of the scratch buffer.
+  // A split for-loop has left every iteration's tile in the scratch slab.  Otherwise the
+  // workgroup's fp16 sums go through LDS so that they leave as 16-byte row segments.
+  if (split) {
+    return;
+  }
   constexpr int LDT = 64 + 8;
   _Float16 *t_lds = reinterpret_cast<_Float16 *>(lds);  // the tiles are dead by now
   __syncthreads();
@@ -366,102 +392,75 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
   for (int b = 0; b < NB; b++) {
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
+      half4 v;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        t_lds[(b * 16 * MT + 16 * mt + 4 * g + r) * LDT + 16 * wave + c] = acc16[b][mt][r];
+        v[r] = acc16[b][mt][r];
       }
+      *reinterpret_cast<half4 *>(t_lds + (b * 16 * MT + 16 * mt + c) * LDT + 16 * wave + 4 * g) = v;
     }
   }
   __syncthreads();
   int const chunks = M * 8;  // 16-byte chunks of one [M][64] tile
-  if (P.ksplit == 1) {
-#pragma unroll
-    for (int b = 0; b < NB; b++) {
-      GTile const &ot = b == 0 ? P.o0 : P.o1;
-      _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
-      for (int e = tid; e < chunks; e += NT) {
-        int row = e / 8, col = (e % 8) * 8;
-        *reinterpret_cast<uint4v *>(og + (long long)row * ot.d_cols + col) =
-            *reinterpret_cast<uint4v const *>(t_lds + (b * 16 * MT + row) * LDT + col);
-      }
-    }
-    return;
-  }
-  // scratch layout: [block][range][NB][M][64]
-  long long const slab = (long long)NB * M * 64;
-  _Float16 *mine = P.scratch + ((long long)block_linear * P.ksplit + ks) * slab;
 #pragma unroll
   for (int b = 0; b < NB; b++) {
+    GTile const &ot = b == 0 ? P.o0 : P.o1;
+    _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
     for (int e = tid; e < chunks; e += NT) {
       int row = e / 8, col = (e % 8) * 8;
-      *reinterpret_cast<uint4v *>(mine + (long long)b * M * 64 + row * 64 + col) =
+      *reinterpret_cast<uint4v *>(og + (long long)row * ot.d_cols + col) =
           *reinterpret_cast<uint4v const *>(t_lds + (b * 16 * MT + row) * LDT + col);
     }
   }
 }
 
-// Second pass of a split for-loop: adds the ranges' fp16 sums of every logical block
-// in range order (fp16 rounding after each add, as the sequential loop would) and
-// stores the block's output tile.  A separate launch rather than a last-arriver
+// Second pass of a split for-loop: adds the fp16 product tiles of every logical block in
+// iteration order (fp16 rounding after each add: the rounding sequence of the sequential
+// loop) and stores the block's output tile.  A separate launch rather than a last-arriver
 // fix-up: the kernel boundary makes the slabs visible without device-scope fences,
 // which on this part write back and invalidate a whole L2 each time.
 template <int NB>
 __global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
-  int const tid = threadIdx.x, M = P.M;
+  int const tid = threadIdx.x, M = P.M, F = P.forloop_range;
   int const bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
   int const block_linear = bx + gridDim.x * (by + gridDim.y * bz);
-  long long const slab = (long long)NB * M * 64;
-  _Float16 const *all = P.scratch + (long long)block_linear * P.ksplit * slab;
-  int const chunks = M * 8;
+  long long const slab = (long long)NB * M * 64;  // one iteration's tiles
+  _Float16 const *all = P.scratch + (long long)block_linear * F * slab;
+  // 4-byte pieces (two neighbouring columns), so that even an 8-row tile keeps every thread
+  // busy, and sixteen iterations' loads in flight per piece: the adds are a dependent chain,
+  // the loads are not.
+  typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+  int const pieces = M * 32;
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     GTile const &ot = b == 0 ? P.o0 : P.o1;
     _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
-    for (int e = tid; e < chunks; e += 256) {
-      int row = e / 8, col = (e % 8) * 8;
+    for (int e = tid; e < pieces; e += 256) {
+      int row = e / 32, col = (e % 32) * 2;
       _Float16 const *sp = all + (long long)b * M * 64 + row * 64 + col;
-      half8 acc;
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        acc[j] = (_Float16)0.0f;
-      }
+      float a0 = 0.0f, a1 = 0.0f;  // hold fp16 values between the adds
       int q = 0;
-      for (; q + 8 <= P.ksplit; q += 8) {  // eight loads in flight, adds in order
-        half8 v[8];
+      for (; q + 16 <= F; q += 16) {
+        half2v v[16];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          v[u] = *reinterpret_cast<half8 const *>(sp + (long long)(q + u) * slab);
+        for (int u = 0; u < 16; u++) {
+          v[u] = *reinterpret_cast<half2v const *>(sp + (long long)(q + u) * slab);
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            acc[j] = static_cast<_Float16>(static_cast<float>(acc[j]) + static_cast<float>(v[u][j]));
-          }
+        for (int u = 0; u < 16; u++) {
+          a0 = static_cast<float>(static_cast<_Float16>(a0 + static_cast<float>(v[u][0])));
+          a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[u][1])));
         }
       }
-      for (; q + 4 <= P.ksplit; q += 4) {
-        half8 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-          v[u] = *reinterpret_cast<half8 const *>(sp + (long long)(q + u) * slab);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            acc[j] = static_cast<_Float16>(static_cast<float>(acc[j]) + static_cast<float>(v[u][j]));
-          }
-        }
+      for (; q < F; q++) {
+        half2v v = *reinterpret_cast<half2v const *>(sp + (long long)q * slab);
+        a0 = static_cast<float>(static_cast<_Float16>(a0 + static_cast<float>(v[0])));
+        a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[1])));
       }
-      for (; q < P.ksplit; q++) {
-        half8 v = *reinterpret_cast<half8 const *>(sp + (long long)q * slab);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-          acc[j] = static_cast<_Float16>(static_cast<float>(acc[j]) + static_cast<float>(v[j]));
-        }
-      }
-      *reinterpret_cast<half8 *>(og + (long long)row * ot.d_cols + col) = acc;
+      half2v r;
+      r[0] = static_cast<_Float16>(a0);
+      r[1] = static_cast<_Float16>(a1);
+      *reinterpret_cast<half2v *>(og + (long long)row * ot.d_cols + col) = r;
     }
   }
 }
@@ -672,7 +671,7 @@ int try_launch_gemm(DevProgram const &P) {
       }
     }
   }
-  long long const scratch_elems = blocks * ksplit * G.nb * G.M * 64;
+  long long const scratch_elems = blocks * P.forloop_range * G.nb * G.M * 64;
   if (ksplit > 1 && (scratch_elems * 2 > (long long)s.scratch_bytes)) {
     ksplit = 1;
   }

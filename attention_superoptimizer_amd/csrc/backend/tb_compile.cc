@@ -361,6 +361,24 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
     return MI355_ERR_INVALID;
   }
 
+  // A loader whose tile an operator overwrites in place (exp / silu) runs every iteration even
+  // when its origin does not move with the for-loop: the reference reloads every input tile in
+  // every iteration (customized_kernel.cu:51-56, 323-328), so iteration i must see f(tile), not
+  // f applied i + 1 times to what iteration 0 loaded.
+  if (F > 1) {
+    for (int o = 0; o < prog.num_ops; o++) {
+      DevOp const &u = prog.ops[o];
+      if (u.kind != DOP_UNARY) {
+        continue;
+      }
+      for (int l = 0; l < prog.num_ops; l++) {
+        if (prog.ops[l].kind == DOP_LOAD && prog.ops[l].dst == u.dst) {
+          prog.ops[l].hoist = 0;
+        }
+      }
+    }
+  }
+
   // ---- layouts ---------------------------------------------------------------
   prog.num_tensors = (int)T.size();
   for (int i = 0; i < prog.num_tensors; i++) {

@@ -59,6 +59,8 @@ def lib():
         L.orc_f32_to_f16.argtypes = [vp, vp, sz]
         L.orc_customized.argtypes = [ci, ci, vp, vp, vp, ci, ci, vp, ci, vp, ci, ci, ci]
         L.orc_customized.restype = ci
+        L.orc_customized_blocks.argtypes = [ci, ci, vp, vp, vp, ci, ci, vp, ci, vp, ci, ci, ci, vp, ci]
+        L.orc_customized_blocks.restype = ci
         _lib = L
     return _lib
 
@@ -122,26 +124,43 @@ def fp_reduce(A: np.ndarray, dim: int, size: int = 1) -> np.ndarray:
     return out
 
 
+UNTOUCHED = 0xFFFF  # not a fingerprint (>= 25651); as fp16 bits, a NaN no golden here produces
+
+
 def customized(plan: dict, inputs: List[np.ndarray], f16: bool = False, threads: int = 1,
-               smem_limit: int = 1 << 30, input_layouts=None) -> List[np.ndarray]:
-    """One customized op: build + lower the thread-block graph, run the C interpreter."""
+               smem_limit: int = 1 << 30, input_layouts=None, blocks=None) -> List[np.ndarray]:
+    """One customized op: build + lower the thread-block graph, run the C interpreter.
+
+    `blocks`: linear thread-block indices bx + grid.x * (by + grid.y * bz) to run instead of
+    the whole grid; output elements no listed block writes hold UNTOUCHED (see written())."""
     g = lowering.build_tb_graph(plan, [list(a.shape) for a in inputs], input_layouts, smem_limit)
     types, params = lowering.lower(g)
-    outs = [np.zeros(d, np.uint16) for d in lowering.output_dims(g)]
+    fill = 0 if blocks is None else UNTOUCHED
+    outs = [np.full(d, fill, np.uint16) for d in lowering.output_dims(g)]
     ins = [np.ascontiguousarray(a.view(np.uint16) if a.dtype == np.float16 else a) for a in inputs]
-    run_program(types, params, g.grid_dim, g.forloop_range, g.smem_offset, ins, outs, f16, threads)
+    run_program(types, params, g.grid_dim, g.forloop_range, g.smem_offset, ins, outs, f16, threads,
+                blocks)
     return outs
 
 
-def run_program(types, params, grid, forloop_range, smem_bytes, ins, outs, f16=False, threads=1):
+def written(out: np.ndarray) -> np.ndarray:
+    """Mask of the elements a block-subset run of customized() produced."""
+    return out.view(np.uint16) != UNTOUCHED
+
+
+def run_program(types, params, grid, forloop_range, smem_bytes, ins, outs, f16=False, threads=1,
+                blocks=None):
     t_arr = np.array(types, np.int32)
     p_arr = np.array(params, np.int32)
     g_arr = np.array(grid, np.int32)
     in_ptrs = (ctypes.c_void_p * 4)(*[a.ctypes.data for a in ins])
     out_ptrs = (ctypes.c_void_p * 4)(*[a.ctypes.data for a in outs])
-    rc = lib().orc_customized(len(types), len(params), _p(t_arr), _p(p_arr), _p(g_arr),
-                              int(forloop_range), int(smem_bytes), in_ptrs, len(ins),
-                              out_ptrs, len(outs), 1 if f16 else 0, int(threads))
+    b_arr = None if blocks is None else np.ascontiguousarray(blocks, dtype=np.int32)
+    rc = lib().orc_customized_blocks(len(types), len(params), _p(t_arr), _p(p_arr), _p(g_arr),
+                                     int(forloop_range), int(smem_bytes), in_ptrs, len(ins),
+                                     out_ptrs, len(outs), 1 if f16 else 0, int(threads),
+                                     None if b_arr is None else _p(b_arr),
+                                     0 if b_arr is None else int(b_arr.size))
     assert rc == 0
 
 

@@ -143,6 +143,104 @@ def test_div_inverts_mul_and_zero_convention():
     assert np.array_equal(orc.fp_binary("div", x, np.ones_like(x)), x)
 
 
+# ---- silu (an extension of this backend; the reference has no such operator) -------
+def _silu_closed_form(x: int) -> int:
+    """silu(x) = x / (1 + exp(-x)) residue by residue, in Python integers.  exp lifts to 0
+    mod 113, so the denominator is 1 mod 113 and the mod-113 residue of x passes through;
+    mod 227 the denominator is 1 + 3^((-x) mod 113), never 0 (see the test below)."""
+    neg = (FP_PQ - x) % FP_PQ
+    den = (1 + pow(3, neg % 113, 227)) % 227
+    inv = pow(den, 225, 227)
+    sp, sq = (x % 227) * inv % 227, x % 113
+    return (sp * 25425 + sq * 227) % FP_PQ
+
+
+def test_silu_closed_form_and_invariants():
+    x = np.arange(FP_PQ, dtype=np.uint16)
+    s = orc.fp_unary("silu", x)
+    assert np.array_equal(s, np.array([_silu_closed_form(int(v)) for v in x]))
+    assert s[0] == 0
+    # the same value through the PUBLIC primitives: div(x, add(1, exp(neg x)))
+    neg = ((FP_PQ - x.astype(np.int64)) % FP_PQ).astype(np.uint16)
+    den = orc.fp_binary("add", np.ones_like(x), orc.fp_unary("exp", neg))
+    assert np.array_equal(s, orc.fp_binary("div", x, den))
+    # the denominator is invertible for EVERY x: it is 1 mod 113, and 1 + 3^k = 0 mod 227 would
+    # put -1 into the subgroup generated by 3, whose order 113 is odd.  So silu(x) * (1 +
+    # exp(-x)) == x with no exception, and the zero-divisor convention of div never applies.
+    assert np.all(den % 113 == 1) and np.all(den % 227 != 0)
+    assert np.array_equal(orc.fp_binary("mul", s, den), x)
+    assert np.array_equal(s.astype(np.int64) % 113, x.astype(np.int64) % 113)
+    # mistakes this catches: exp(x) for exp(-x), a dropped "1 +", mul for div
+    wrong_sign = orc.fp_binary("div", x, orc.fp_binary("add", np.ones_like(x), orc.fp_unary("exp", x)))
+    no_one = orc.fp_binary("div", x, orc.fp_unary("exp", neg))
+    assert not np.array_equal(s, wrong_sign) and not np.array_equal(s, no_one)
+
+
+# ---- thread-block add / mul (extensions: the reference's lowering asserts on them) ----
+def tb_add_mul_case():
+    """A customized op built from thread-block add and mul with every broadcast a 3-D tile
+    admits ([1,r,c] with [1,r,1], with [1,1,c], [1,r,1] with [1,1,c], small operand first),
+    over two blocks and a two-iteration for-loop.  119 program ints."""
+    spec = [
+        {"op": "input", "dims": [2, 8, 12]}, {"op": "input", "dims": [2, 8, 12]},
+        {"op": "customized", "in": [[0, 0], [1, 0]], "plan": {
+            "grid_dim": [2, 1, 1], "forloop_range": 2, "reduction_dimx": 4,
+            "input_map": [[0, -1, -1], [0, -1, -1]], "forloop_dim": [2, 2],
+            "output_map": [0, -1, -1],
+            "ops": [["tb_reduction_2_op", [[0, 0]]],            # 2: [1,8,1]
+                    ["tb_reduction_1_op", [[1, 0]]],            # 3: [1,1,6]
+                    ["tb_add_op", [[0, 0], [2, 0]]],            # 4: [1,8,6] + [1,8,1]
+                    ["tb_mul_op", [[4, 0], [3, 0]]],            # 5: [1,8,6] * [1,1,6]
+                    ["tb_add_op", [[2, 0], [3, 0]]],            # 6: [1,8,1] + [1,1,6]
+                    ["tb_mul_op", [[5, 0], [6, 0]]],            # 7
+                    ["tb_mul_op", [[3, 0], [2, 0]]],            # 8: [1,1,6] * [1,8,1]
+                    ["tb_add_op", [[7, 0], [8, 0]]]]}},         # 9
+    ]
+    return spec
+
+
+def tb_add_mul_exact(A, B):
+    """The same computation in Python integers of unbounded size, one modulus at the end."""
+    A, B = A.astype(object), B.astype(object)
+    out = np.zeros((2, 8, 6), object)
+    for b in range(2):
+        for it in range(2):
+            a, bb = A[b][:, it * 6:(it + 1) * 6], B[b][:, it * 6:(it + 1) * 6]
+            r2 = a.sum(axis=1).reshape(8, 1)
+            r1 = bb.sum(axis=0).reshape(1, 6)
+            out[b] = out[b] + ((a + r2) * r1) * (r2 + r1) + r1 * r2
+    return (out % FP_PQ).astype(np.uint16)
+
+
+def test_threadblock_add_mul_exact_integers():
+    spec = tb_add_mul_case()
+    for seed in (1, 2):
+        A, B = uniform_fp([2, 8, 12], seed), uniform_fp([2, 8, 12], seed + 10)
+        got = orc.eval_graph(spec, "fp", {0: A, 1: B})[2]
+        assert len(got) == 1 and got[0].shape == (2, 8, 6)
+        assert np.array_equal(got[0], tb_add_mul_exact(A, B))
+    # worst-case operands: every intermediate product is as large as the ring allows
+    A = np.full((2, 8, 12), FP_PQ - 1, np.uint16)
+    assert np.array_equal(orc.eval_graph(spec, "fp", {0: A, 1: A})[2][0], tb_add_mul_exact(A, A))
+    # an operand swap or add-for-mul changes the answer (the check can fail)
+    bad = tb_add_mul_case()
+    bad[2]["plan"]["ops"][3][0] = "tb_add_op"
+    A, B = uniform_fp([2, 8, 12], 1), uniform_fp([2, 8, 12], 11)
+    assert not np.array_equal(orc.eval_graph(bad, "fp", {0: A, 1: B})[2][0], tb_add_mul_exact(A, B))
+
+
+def test_block_subset_reproduces_those_blocks():
+    """customized(blocks=...) runs the listed thread blocks only: their tiles equal the
+    whole-grid run, everything else is left untouched"""
+    spec, _ = W.config2_gqa_decode()
+    ins = [uniform_fp(spec[i]["dims"], 60 + i) for i in range(3)]
+    full = orc.customized(spec[3]["plan"], ins, threads=8)[0]
+    part = orc.customized(spec[3]["plan"], ins, threads=2, blocks=[1, 6, 31])[0]
+    m = orc.written(part)
+    assert m.sum() == 3 * 256 * 64 and np.array_equal(part[m], full[m])
+    assert m[1, :, 0:64].all() and m[0, :, 3 * 64:4 * 64].all() and m[1, :, 15 * 64:].all()
+
+
 # ---- the interpreter ------------------------------------------------------------
 def test_degenerate_plan_equals_kernel_ops():
     """grid (1,1,1), for-loop 1: a customized op is its kernel-level ops"""
