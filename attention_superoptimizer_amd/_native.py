@@ -107,6 +107,7 @@ ABI = {
     "mi355_mark_wait_queue": (_ci, [_ci, _ci]),
     "mi355_mark_wait_host": (_ci, [_ci]),
     "mi355_customized_fp": (_ci, [_pplan, _pvp, _pvp]),
+    "mi355_customized_fp_static": (_ci, [_pplan, _pvp, _pvp]),
     "mi355_customized_fp_batch": (_ci, [_pplan, _ci, _pvp, _pvp]),
     "mi355_plan_extents": (_ci, [_pplan, _pll, _pll, _pi, _pi]),
     "mi355_customized_run": (_ci, [_pplan, _pvp, _pvp]),

@@ -99,6 +99,9 @@ bool mfma_matmul_pays(int batch, int m, int n, int k);
 int launch_mfma_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m, int n,
                        int k);
 int sync_all_queues();
+// Looks up the device address of the file-scope scratch array behind
+// mi355_customized_fp_static (tb_interp.hip); called by mi355_init with `device` current.
+int static_scratch_setup(int device);
 int fail(int code, char const *fmt, ...);
 
 #define MI355_HIP(expr)                                                             \

@@ -74,6 +74,9 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
       optin > 0) {
     s.max_lds = optin;
   }
+  if (int rc = static_scratch_setup(s.device)) {
+    return rc;
+  }
   for (int i = 0; i < MI355_NUM_QUEUES; i++) {
     MI355_HIP(hipStreamCreate(&s.queues[i]));  // default priority, all of them
   }

@@ -1169,6 +1169,121 @@ extern "C" int mi355_customized_fp(mi355_plan const *plan, void const *const *in
   return launch(prog, false);
 }
 
+// ---- the entry point that allocates nothing ----------------------------------------------
+// The partial sums of a split for-loop normally go to a scratch slab that mi355_init takes
+// from the device allocator.  For callers that cannot have the library allocate or touch
+// allocator-owned memory on their behalf, the same two kernels run with the partial sums in
+// a file-scope device array instead.  `scratch` names the array on the host side only as a
+// symbol: its device address is looked up once per device (static_scratch_setup, from
+// mi355_init, with that device current) and only that address is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[MI355_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 16;
+static void *g_static_scratch[kMaxDevices] = {};
+
+namespace mi355 {
+int static_scratch_setup(int device) {
+  if (device < 0 || device >= kMaxDevices) {
+    return fail(MI355_ERR_INVALID, "device %d out of range", device);
+  }
+  void *ptr = nullptr;
+  MI355_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  if (ptr == nullptr) {
+    return fail(MI355_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch");
+  }
+  g_static_scratch[device] = ptr;
+  // raised here, not lazily at the first large launch: the entry point itself then makes no
+  // call besides its two kernel launches
+  MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_interp_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
+  return MI355_OK;
+}
+}  // namespace mi355
+
+extern "C" int mi355_customized_fp_static(mi355_plan const *plan, void const *const *inputs,
+                                          void *const *outputs) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (plan == nullptr || inputs == nullptr || outputs == nullptr) {
+    return fail(MI355_ERR_INVALID, "null argument");
+  }
+  void *const base = g_static_scratch[s.device];
+  if (base == nullptr) {
+    return fail(MI355_ERR_NOT_INITIALISED, "static scratch of device %d was not set up", s.device);
+  }
+  DevProgram prog;
+  PlanExtents ext;
+  std::string err;
+  int rc = compile_plan(*plan, false, s.max_lds, prog, ext, err);
+  if (rc != MI355_OK) {
+    return fail(rc, "%s", err.c_str());
+  }
+  for (int i = 0; i < plan->num_dmem_inputs; i++) {
+    if (inputs[i] == nullptr) {
+      return fail(MI355_ERR_INVALID, "input %d is null", i);
+    }
+    prog.in[i] = inputs[i];
+  }
+  for (int i = 0; i < plan->num_dmem_outputs; i++) {
+    if (outputs[i] == nullptr) {
+      return fail(MI355_ERR_INVALID, "output %d is null", i);
+    }
+    prog.out[i] = outputs[i];
+  }
+  for (int o = 0; o < prog.num_ops; o++) {
+    DevOp &d = prog.ops[o];
+    if (d.kind == DOP_LOAD && d.vec8 && (reinterpret_cast<uintptr_t>(prog.in[d.io]) & 15) != 0) {
+      d.vec8 = 0;
+    }
+  }
+  // the split rule of mi355_customized_fp; what it needs must fit the array
+  prog.splits = 1;
+  long long const blocks = (long long)prog.grid[0] * prog.grid[1] * prog.grid[2];
+  int const F = prog.forloop_range;
+  if (F >= 2 && blocks < 192) {
+    int const splits = (int)std::min<long long>(std::min(F, 64), (256 + blocks - 1) / blocks);
+    long long elems = 0;
+    for (int i = 0; i < plan->num_dmem_outputs; i++) {
+      elems += (ext.out_elems[i] + 7) / 8 * 8;
+    }
+    long long const need = elems * splits * 2;
+    if (splits >= 2 && need > (long long)MI355_STATIC_SCRATCH_BYTES) {
+      return fail(MI355_ERR_UNSUPPORTED,
+                  "plan needs %lld bytes of partial sums (%d ranges of its for-loop); the static "
+                  "scratch holds %d", need, splits, (int)MI355_STATIC_SCRATCH_BYTES);
+    }
+    if (splits >= 2) {
+      prog.splits = splits;
+      uint16_t *p = static_cast<uint16_t *>(base);
+      for (int i = 0; i < plan->num_dmem_outputs; i++) {
+        prog.part[i] = p;
+        prog.part_elems[i] = ext.out_elems[i];
+        prog.part_stride[i] = (ext.out_elems[i] + 7) / 8 * 8;
+        p += prog.part_stride[i] * splits;
+      }
+    }
+  }
+  if ((long long)prog.grid[0] * prog.splits > 2147483647LL) {
+    return fail(MI355_ERR_UNSUPPORTED, "grid too large");
+  }
+  dim3 grid(prog.grid[0] * prog.splits, prog.grid[1], prog.grid[2]);
+  fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog, s.exp_tbl, s.div_p,
+                                                                        s.div_q);
+  MI355_HIP(hipGetLastError());
+  if (prog.splits > 1) {
+    // every (range, block) workgroup overwrites its whole tile of the slab before this launch
+    // reads it, so nothing needs clearing between calls
+    if (int rc2 = fold_splits(prog)) {
+      return rc2;
+    }
+  }
+  s.last_launch.kernel_id = MI355_KERNEL_FP_INTERP;
+  s.last_launch.workgroups = (int)(grid.x * grid.y * grid.z);
+  s.last_launch.threads = kInterpThreads;
+  s.last_launch.lds_bytes = prog.lds_bytes;
+  s.last_launch.row_split = prog.splits;
+  return MI355_OK;
+}
+
 // One chunk of a batch: every program in one multi-program launch per LDS class, then one
 // launch that folds the partial sums of all split for-loops.  A program whose tiles leave
 // no room in LDS for its own record is launched by itself.

@@ -234,6 +234,21 @@ int mi355_fp_equal_read(int first_slot, int count, uint8_t *equal);
 int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,
                         void *const *outputs);
 
+/* The same fingerprint, for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * It calls no hipMalloc / hipFree and uses none of the memory mi355_init allocated beyond
+ * the lookup tables: the partial sums of a split for-loop go to a file-scope device array
+ * of MI355_STATIC_SCRATCH_BYTES instead of the backend's scratch slab, and the plan always
+ * runs on the generic interpreter (the matrix-core route needs residue planes in allocated
+ * memory).  Bit-identical to mi355_customized_fp.  A plan whose partial sums do not fit
+ * (for-loop ranges x output elements x 2 bytes, ranges chosen as in mi355_customized_fp)
+ * is refused with MI355_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array:
+ * calls that overlap on one GPU (different queues or host threads) race; calls on one
+ * queue are ordered.  Nothing in the array needs clearing between calls. */
+#define MI355_STATIC_SCRATCH_BYTES (8 << 20)
+int mi355_customized_fp_static(mi355_plan const *plan, void const *const *inputs,
+                               void *const *outputs);
+
 /* n independent customized-op fingerprints in one call (the batched form of the entry above
  * for a verification loop that holds many candidates, src/search/search.cc:601-603):
  * operator i reads inputs[4*i .. 4*i+3] and writes outputs[4*i .. 4*i+3].  The operators must
