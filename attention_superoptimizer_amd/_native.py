@@ -163,12 +163,22 @@ FACADE = {
     "mirage_verify_batch": (_ci, [_pvp, _ci, _vp, _u64, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_verify_batch_begin": (_vp, [_pvp, _ci, _vp, _u64, _ci]),
     "mirage_verify_set_queues_per_batch": (None, [_ci]),
+    "mirage_verify_ring_create": (_vp, []),
+    "mirage_verify_ring_destroy": (None, [_vp]),
+    "mirage_verify_ring_acquire": (_ci, [_vp, _ci, _pi, _pi]),
+    "mirage_verify_ring_release": (None, [_vp, _ci]),
     "mirage_verify_batch_end": (_ci, [_vp, _ci, _vp, ctypes.POINTER(MirageVerifyStats)]),
     "mirage_optimize_layout": (_ci, [_vp, ctypes.c_longlong, LAYOUT_COST_FN, _vp,
                                      ctypes.POINTER(MirageLayoutStats)]),
     "mirage_graph_generate_hip_program": (_ci, [_vp, ctypes.c_char_p]),
     "mirage_graph_from_json": (_vp, [ctypes.c_char_p]),
     "mirage_graph_to_json": (ctypes.c_longlong, [_vp, ctypes.c_char_p, ctypes.c_longlong]),
+    "mirage_checkpoint_load": (_vp, [ctypes.c_char_p]),
+    "mirage_checkpoint_destroy": (None, [_vp]),
+    "mirage_checkpoint_num_graphs": (_ci, [_vp]),
+    "mirage_checkpoint_summary": (ctypes.c_float, [_vp, _pll]),
+    "mirage_checkpoint_json": (ctypes.c_longlong, [_vp, _ci, ctypes.c_char_p, ctypes.c_longlong]),
+    "mirage_graph_profile": (ctypes.c_float, [_vp, _pf, _ci]),
     "mirage_set_smem_budget": (None, [_sz]),
     "mirage_get_smem_budget": (_sz, []),
     "mirage_device_ready": (_ci, []),

@@ -2,6 +2,7 @@
 
   libmi355_backend.so   HIP kernels + the C ABI of include/mi355_abi.h
   libmirage_runtime.so  the mirage:: host API (C++) + its C facade for ctypes
+  mirage_profile        the reference's cpp_examples/profile.cc over that API
   generated/            HIP programs written by Graph::generate_hip_program for the example
                         graphs of codegen.py, compiled as libraries and executables
 
@@ -61,6 +62,14 @@ def build_runtime():
          ["-L" + HERE, "-lmi355_backend", "-Wl,-rpath,$ORIGIN", "-pthread"])
 
 
+def build_tools():
+    """mirage_profile: loads a graph / checkpoint JSON, fingerprints and times it (the
+    reference's cpp_examples/profile.cc)."""
+    _run(["g++", "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", INCLUDE, "-I", "/opt/rocm/include",
+          "-o", os.path.join(HERE, "mirage_profile"), os.path.join(CSRC, "examples", "profile.cc"),
+          "-L" + HERE, "-lmirage_runtime", "-lmi355_backend", "-Wl,-rpath,$ORIGIN"])
+
+
 def build_generated():
     """Generated HIP programs of the example graphs (codegen.py), in a process of their own:
     building the graphs loads the runtime just built, in host-only mode."""
@@ -77,6 +86,7 @@ def main():
     build_backend()
     if os.path.isdir(os.path.join(CSRC, "host")):
         build_runtime()
+        build_tools()
         build_generated()
     return 0
 

@@ -33,6 +33,7 @@
 //    16-byte row segments.
 #include "common.h"
 #include "tb_program.h"
+#include <atomic>
 #include <cstdlib>
 
 namespace mi355 {
@@ -1178,7 +1179,7 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_direct_kernel(AttnParams co
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
 int launch_direct_one(AttnParams const &A, dim3 grid, int lds) {
   auto *fn = attn_direct_kernel<D, NK, DV, HAS_DIV, RG, IP>;
-  static int granted = 0;  // per instantiation
+  static std::atomic<int> granted{0};  // per instantiation
   if (lds > 65536 && lds > granted) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
@@ -1203,7 +1204,7 @@ int launch_direct(AttnParams const &A, dim3 grid, int rg, int ip, int lds) {
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
 int launch_one(AttnParams const &A, dim3 grid, int lds) {
   auto *fn = attn_fused_kernel<D, NK, DV, HAS_DIV, RG, IP>;
-  static int granted = 0;  // per instantiation
+  static std::atomic<int> granted{0};  // per instantiation
   if (lds > 65536 && lds > granted) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
@@ -1327,11 +1328,11 @@ int try_launch_attention(DevProgram const &P) {
         int rc = M.D == 64 ? launch_stream<64, 64, 64>(A, M.has_div, grid, rgs, lds)
                            : launch_stream<128, 64, 128>(A, M.has_div, grid, rgs, lds);
         if (rc == 1) {
-          s.last_launch.kernel_id = MI355_KERNEL_F16_ATTENTION;
-          s.last_launch.workgroups = grid.x * grid.y * grid.z;
-          s.last_launch.threads = rgs * 64;
-          s.last_launch.lds_bytes = lds;
-          s.last_launch.row_split = A.split;
+          s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
+          s.last().workgroups = grid.x * grid.y * grid.z;
+          s.last().threads = rgs * 64;
+          s.last().lds_bytes = lds;
+          s.last().row_split = A.split;
         }
         return rc;
       }
@@ -1391,11 +1392,11 @@ int try_launch_attention(DevProgram const &P) {
     rc = M.has_div ? launch_direct<true>(B, direct_grid, 1, ip, direct_lds)
                    : launch_direct<false>(B, direct_grid, 1, ip, direct_lds);
     if (rc == 1) {
-      s.last_launch.kernel_id = MI355_KERNEL_F16_ATTENTION;
-      s.last_launch.workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
-      s.last_launch.threads = ip * 64;
-      s.last_launch.lds_bytes = direct_lds;
-      s.last_launch.row_split = B.split;
+      s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
+      s.last().workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
+      s.last().threads = ip * 64;
+      s.last().lds_bytes = direct_lds;
+      s.last().row_split = B.split;
       return rc;
     }
   }
@@ -1410,11 +1411,11 @@ int try_launch_attention(DevProgram const &P) {
     rc = launch_shape<128, 64, 128>(A, M.has_div, grid, rg, ip, lds);
   }
   if (rc == 1) {
-    s.last_launch.kernel_id = MI355_KERNEL_F16_ATTENTION;
-    s.last_launch.workgroups = grid.x * grid.y * grid.z;
-    s.last_launch.threads = nw * 64;
-    s.last_launch.lds_bytes = lds;
-    s.last_launch.row_split = A.split;
+    s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
+    s.last().workgroups = grid.x * grid.y * grid.z;
+    s.last().threads = nw * 64;
+    s.last().lds_bytes = lds;
+    s.last().row_split = A.split;
   }
   return rc;
 }

@@ -180,11 +180,11 @@ int try_launch_combine(DevProgram const &P) {
   dim3 grid(P.grid[0], P.grid[1], P.grid[2]);
   combine_fused_kernel<<<grid, 256, 0, s.stream()>>>(A);
   MI355_HIP(hipGetLastError());
-  s.last_launch.kernel_id = MI355_KERNEL_F16_COMBINE;
-  s.last_launch.workgroups = (int)(grid.x * grid.y * grid.z);
-  s.last_launch.threads = 256;
-  s.last_launch.lds_bytes = 0;
-  s.last_launch.row_split = 1;
+  s.last().kernel_id = MI355_KERNEL_F16_COMBINE;
+  s.last().workgroups = (int)(grid.x * grid.y * grid.z);
+  s.last().threads = 256;
+  s.last().lds_bytes = 0;
+  s.last().row_split = 1;
   return 1;
 }
 

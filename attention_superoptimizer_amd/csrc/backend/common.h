@@ -52,13 +52,15 @@ struct State {
   size_t arena_bytes = 0;
   // device copies of the lookup tables, reference layout
   uint16_t *exp_tbl = nullptr, *div_p = nullptr, *div_q = nullptr;
-  int *flag = nullptr;        // 4-byte device scratch for mi355_fp_equal
-  int *flag_host = nullptr;   // pinned mirror
+  int *flag = nullptr;        // device scratch of mi355_fp_equal: one int per queue, 64 bytes apart
+  int *flag_host = nullptr;   // pinned mirror, same layout
+  int *queue_flag() const { return flag + 16 * tls_queue; }
+  int *queue_flag_host() const { return flag_host + 16 * tls_queue; }
   int *cmp_host = nullptr;    // MI355_COMPARE_SLOTS mismatch flags of deferred compares, in
                               // pinned host memory
   int *cmp_slots = nullptr;   // the same memory as the device addresses it
   hipEvent_t marks[MI355_NUM_MARKS][MI355_NUM_QUEUES] = {};
-  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  hipEvent_t ev0[MI355_NUM_QUEUES] = {}, ev1[MI355_NUM_QUEUES] = {};  // timer pair per queue
   int max_lds = 65536;
   // staging of batched launches (mi355_customized_fp_batch): per queue a small ring of
   // pinned host / device buffer pairs that carry the program records of one call
@@ -71,7 +73,10 @@ struct State {
   };
   BatchSlot batch[MI355_NUM_QUEUES][kBatchSlots];
   int batch_next[MI355_NUM_QUEUES] = {};
-  mi355_launch_info last_launch{};
+  // what the last customized-op call of each queue launched (a queue is driven by one host
+  // thread at a time, so per-queue records never mix)
+  mi355_launch_info launches[MI355_NUM_QUEUES] = {};
+  mi355_launch_info &last() { return launches[tls_queue]; }
   int force_interpreter = 0;
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
   int fp_vector_dot_only = 0;  // 1: fingerprint matmuls never take the matrix-core kernels
@@ -133,7 +138,7 @@ __device__ __forceinline__ uint32_t mod_q(uint32_t x) { return x % FP_Q; }
 // sum_p may be negative (operands recentred to [-113, 113]), |sum_p| < 2^31 - 2^17; adding
 // 83715 * 25651 makes it non-negative without changing a residue.  sum_q >= 0.
 __device__ __forceinline__ uint32_t fp_from_residue_sums(int sum_p, int sum_q) {
-  uint32_t const a = static_cast<uint32_t>(sum_p + 2147373465) % FP_PQ;
+  uint32_t const a = (static_cast<uint32_t>(sum_p) + 2147373465u) % FP_PQ;  // unsigned: wraps by definition
   uint32_t const b = static_cast<uint32_t>(sum_q) % FP_PQ;
   return (a * FP_Q_MUL_P_MOD_1 + b * FP_P_MUL_Q_MOD_1) % FP_PQ;
 }

@@ -15,6 +15,7 @@
 // Integer only: residues mod 227 / 113 packed four to a dword, v_dot4_u32_u8.
 #include "common.h"
 #include "tb_program.h"
+#include <atomic>
 
 namespace mi355 {
 
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(kThreads) void fp_gemm_multi_kernel(
 
 template <int TPT>
 int raise_lds(int lds_total) {
-  static int granted_single = 0, granted_multi = 0;
+  static std::atomic<int> granted_single{0}, granted_multi{0};
   State &s = state();
   if (lds_total > 65536 && (granted_single < s.max_lds || granted_multi < s.max_lds)) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_gemm_kernel<TPT>),

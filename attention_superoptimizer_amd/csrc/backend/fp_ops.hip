@@ -808,14 +808,14 @@ extern "C" int mi355_fp_equal(uint16_t const *a, uint16_t const *b, size_t n, in
   if (int rc = sync_all_queues()) {  // the operands may come from any queue
     return rc;
   }
-  set_flag_kernel<<<1, 1, 0, s.stream()>>>(s.flag, 1);
+  set_flag_kernel<<<1, 1, 0, s.stream()>>>(s.queue_flag(), 1);
   if (n > 0) {
-    fp_equal_kernel<<<grid_for(n, kThreads, 2048), kThreads, 0, s.stream()>>>(a, b, n, s.flag);
+    fp_equal_kernel<<<grid_for(n, kThreads, 2048), kThreads, 0, s.stream()>>>(a, b, n, s.queue_flag());
   }
   MI355_HIP(hipGetLastError());
-  MI355_HIP(hipMemcpyAsync(s.flag_host, s.flag, sizeof(int), hipMemcpyDeviceToHost, s.stream()));
+  MI355_HIP(hipMemcpyAsync(s.queue_flag_host(), s.queue_flag(), sizeof(int), hipMemcpyDeviceToHost, s.stream()));
   MI355_HIP(hipStreamSynchronize(s.stream()));
-  *equal = *s.flag_host;
+  *equal = *s.queue_flag_host();
   return MI355_OK;
 }
 

@@ -708,11 +708,11 @@ int try_launch_gemm(DevProgram const &P) {
     MI355_HIP(hipGetLastError());
   }
   if (rc == 1) {
-    s.last_launch.kernel_id = MI355_KERNEL_F16_GEMM;
-    s.last_launch.workgroups = grid.x * grid.y * grid.z;
-    s.last_launch.threads = 256;
-    s.last_launch.lds_bytes = lds;
-    s.last_launch.row_split = ksplit;
+    s.last().kernel_id = MI355_KERNEL_F16_GEMM;
+    s.last().workgroups = grid.x * grid.y * grid.z;
+    s.last().threads = 256;
+    s.last().lds_bytes = lds;
+    s.last().row_split = ksplit;
   }
   return rc;
 }

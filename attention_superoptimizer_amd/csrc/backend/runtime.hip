@@ -125,8 +125,10 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
     }
     g_mark_bits[m].store(0);
   }
-  MI355_HIP(hipEventCreate(&s.ev0));
-  MI355_HIP(hipEventCreate(&s.ev1));
+  for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+    MI355_HIP(hipEventCreate(&s.ev0[q]));
+    MI355_HIP(hipEventCreate(&s.ev1[q]));
+  }
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     for (int b = 0; b < State::kBatchSlots; b++) {
       State::BatchSlot &slot = s.batch[q][b];
@@ -158,8 +160,10 @@ extern "C" int mi355_shutdown(void) {
   if (int rc = sync_all_queues()) {
     return rc;
   }
-  MI355_HIP(hipEventDestroy(s.ev0));
-  MI355_HIP(hipEventDestroy(s.ev1));
+  for (int q = 0; q < MI355_NUM_QUEUES; q++) {
+    MI355_HIP(hipEventDestroy(s.ev0[q]));
+    MI355_HIP(hipEventDestroy(s.ev1[q]));
+  }
   MI355_HIP(hipFree(s.arena));
   MI355_HIP(hipFree(s.exp_tbl));
   MI355_HIP(hipFree(s.flag));
@@ -195,7 +199,8 @@ extern "C" int mi355_get_device_info(mi355_device_info *info) {
   hipDeviceProp_t prop;
   MI355_HIP(hipGetDeviceProperties(&prop, state().device));
   memset(info, 0, sizeof(*info));
-  strncpy(info->name, prop.name, sizeof(info->name) - 1);
+  // some driver stacks report an empty marketing name: fall back to the architecture string
+  strncpy(info->name, prop.name[0] != '\0' ? prop.name : prop.gcnArchName, sizeof(info->name) - 1);
   strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
   info->compute_units = prop.multiProcessorCount;
   info->clock_mhz = prop.clockRate / 1000;
@@ -307,14 +312,14 @@ extern "C" int mi355_launch_floor(int iters, float *us) {
   for (int i = 0; i < 64; i++) {
     empty_kernel<<<1, 64, 0, s.stream()>>>();
   }
-  MI355_HIP(hipEventRecord(s.ev0, s.stream()));
+  MI355_HIP(hipEventRecord(s.ev0[tls_queue], s.stream()));
   for (int i = 0; i < iters; i++) {
     empty_kernel<<<1, 64, 0, s.stream()>>>();
   }
-  MI355_HIP(hipEventRecord(s.ev1, s.stream()));
-  MI355_HIP(hipEventSynchronize(s.ev1));
+  MI355_HIP(hipEventRecord(s.ev1[tls_queue], s.stream()));
+  MI355_HIP(hipEventSynchronize(s.ev1[tls_queue]));
   float ms = 0.0f;
-  MI355_HIP(hipEventElapsedTime(&ms, s.ev0, s.ev1));
+  MI355_HIP(hipEventElapsedTime(&ms, s.ev0[tls_queue], s.ev1[tls_queue]));
   *us = ms * 1000.0f / iters;
   return MI355_OK;
 }
@@ -372,15 +377,15 @@ extern "C" int mi355_sync(void) {
 
 extern "C" int mi355_timer_start(void) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipEventRecord(state().ev0, state().stream()));
+  MI355_HIP(hipEventRecord(state().ev0[tls_queue], state().stream()));
   return MI355_OK;
 }
 
 extern "C" int mi355_timer_stop(float *ms) {
   MI355_REQUIRE_INIT();
-  MI355_HIP(hipEventRecord(state().ev1, state().stream()));
-  MI355_HIP(hipEventSynchronize(state().ev1));
-  MI355_HIP(hipEventElapsedTime(ms, state().ev0, state().ev1));
+  MI355_HIP(hipEventRecord(state().ev1[tls_queue], state().stream()));
+  MI355_HIP(hipEventSynchronize(state().ev1[tls_queue]));
+  MI355_HIP(hipEventElapsedTime(ms, state().ev0[tls_queue], state().ev1[tls_queue]));
   return MI355_OK;
 }
 
@@ -388,6 +393,6 @@ extern "C" int mi355_last_launch(mi355_launch_info *info) {
   if (info == nullptr) {
     return fail(MI355_ERR_INVALID, "null info");
   }
-  *info = state().last_launch;
+  *info = state().last();
   return MI355_OK;
 }

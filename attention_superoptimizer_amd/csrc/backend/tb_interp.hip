@@ -10,6 +10,7 @@
 //                       src/kernel/triton_code_gen.cc:223-333)
 #include "common.h"
 #include "tb_program.h"
+#include <atomic>
 
 #include <algorithm>
 #include <string>
@@ -1072,11 +1073,11 @@ static int launch(DevProgram const &prog, bool f16) {
         return rc;
       }
     }
-    s.last_launch.kernel_id = MI355_KERNEL_FP_GEMM;
-    s.last_launch.workgroups = (int)fp_program_blocks(prog);
-    s.last_launch.threads = kInterpThreads;
-    s.last_launch.lds_bytes = prog.lds_bytes;
-    s.last_launch.row_split = prog.splits;
+    s.last().kernel_id = MI355_KERNEL_FP_GEMM;
+    s.last().workgroups = (int)fp_program_blocks(prog);
+    s.last().threads = kInterpThreads;
+    s.last().lds_bytes = prog.lds_bytes;
+    s.last().row_split = prog.splits;
     return MI355_OK;
   }
   if (prog.fused != 0) {
@@ -1089,8 +1090,10 @@ static int launch(DevProgram const &prog, bool f16) {
     return rc < 0 ? rc : fail(MI355_ERR_UNSUPPORTED, "fused kernel declined the launch");
   }
   dim3 grid(prog.grid[0] * (f16 ? 1 : prog.splits), prog.grid[1], prog.grid[2]);
-  static int fp_lds_set = 0, f16_lds_set = 0;
-  int &cur = f16 ? f16_lds_set : fp_lds_set;
+  // atomics: host threads of different queues may get here together (raising the limit twice
+  // is harmless, a torn flag is not)
+  static std::atomic<int> fp_lds_set{0}, f16_lds_set{0};
+  std::atomic<int> &cur = f16 ? f16_lds_set : fp_lds_set;
   if (prog.lds_bytes > 65536 && prog.lds_bytes > cur) {
     if (f16) {
       MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(f16_interp_kernel),
@@ -1113,11 +1116,11 @@ static int launch(DevProgram const &prog, bool f16) {
     }
   }
   MI355_HIP(hipGetLastError());
-  s.last_launch.kernel_id = f16 ? MI355_KERNEL_F16_INTERP : MI355_KERNEL_FP_INTERP;
-  s.last_launch.workgroups = (int)(grid.x * grid.y * grid.z);
-  s.last_launch.threads = kInterpThreads;
-  s.last_launch.lds_bytes = prog.lds_bytes;
-  s.last_launch.row_split = 1;
+  s.last().kernel_id = f16 ? MI355_KERNEL_F16_INTERP : MI355_KERNEL_FP_INTERP;
+  s.last().workgroups = (int)(grid.x * grid.y * grid.z);
+  s.last().threads = kInterpThreads;
+  s.last().lds_bytes = prog.lds_bytes;
+  s.last().row_split = 1;
   return MI355_OK;
 }
 
@@ -1276,11 +1279,11 @@ extern "C" int mi355_customized_fp_static(mi355_plan const *plan, void const *co
       return rc2;
     }
   }
-  s.last_launch.kernel_id = MI355_KERNEL_FP_INTERP;
-  s.last_launch.workgroups = (int)(grid.x * grid.y * grid.z);
-  s.last_launch.threads = kInterpThreads;
-  s.last_launch.lds_bytes = prog.lds_bytes;
-  s.last_launch.row_split = prog.splits;
+  s.last().kernel_id = MI355_KERNEL_FP_INTERP;
+  s.last().workgroups = (int)(grid.x * grid.y * grid.z);
+  s.last().threads = kInterpThreads;
+  s.last().lds_bytes = prog.lds_bytes;
+  s.last().row_split = prog.splits;
   return MI355_OK;
 }
 
@@ -1422,7 +1425,7 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
         return rc;
       }
     }
-    static bool lds_raised = false;
+    static std::atomic<bool> lds_raised{false};
     DevProgram const *dp = reinterpret_cast<DevProgram const *>(slot.dev);
     int const *df = reinterpret_cast<int const *>(slot.dev + off_first);
     for (int c = 0; c < kClasses; c++) {
@@ -1479,14 +1482,14 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
       if (rc != MI355_OK) {
         return rc;
       }
-      launched += s.last_launch.workgroups;
+      launched += s.last().workgroups;
     }
   }
-  s.last_launch.kernel_id = MI355_KERNEL_FP_INTERP;
-  s.last_launch.workgroups = launched;
-  s.last_launch.threads = kInterpThreads;
-  s.last_launch.lds_bytes = 0;
-  s.last_launch.row_split = 1;
+  s.last().kernel_id = MI355_KERNEL_FP_INTERP;
+  s.last().workgroups = launched;
+  s.last().threads = kInterpThreads;
+  s.last().lds_bytes = 0;
+  s.last().row_split = 1;
   return MI355_OK;
 }
 
@@ -1572,17 +1575,17 @@ extern "C" int mi355_customized_profile(mi355_plan const *plan, void const *cons
       return rc;
     }
   }
-  MI355_HIP(hipEventRecord(s.ev0, s.stream()));
+  MI355_HIP(hipEventRecord(s.ev0[tls_queue], s.stream()));
   for (int i = 0; i < iters; i++) {
     rc = launch(prog, fingerprint == 0);
     if (rc != MI355_OK) {
       return rc;
     }
   }
-  MI355_HIP(hipEventRecord(s.ev1, s.stream()));
-  MI355_HIP(hipEventSynchronize(s.ev1));
+  MI355_HIP(hipEventRecord(s.ev1[tls_queue], s.stream()));
+  MI355_HIP(hipEventSynchronize(s.ev1[tls_queue]));
   float total = 0.0f;
-  MI355_HIP(hipEventElapsedTime(&total, s.ev0, s.ev1));
+  MI355_HIP(hipEventElapsedTime(&total, s.ev0[tls_queue], s.ev1[tls_queue]));
   *ms = total / iters;
   return MI355_OK;
 }

@@ -3,6 +3,9 @@
 // operator and the NLOHMANN_DEFINE_TYPE_NON_INTRUSIVE lists of DTensor / STensor /
 // ExecutionPlan).  Host only.
 #include "mirage/utils/json_utils.h"
+#include <istream>
+#include <iterator>
+#include <ostream>
 
 #include "mirage/utils/hip_types.h"
 
@@ -836,6 +839,66 @@ void to_json(json &j, Graph const &g) {
   j["smem_offset"] = g.smem_offset;
 }
 
+}  // namespace threadblock
+}  // namespace mirage
+
+std::istream &operator>>(std::istream &in, mirage::utils::Json &j) {
+  std::string text((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+  j = mirage::utils::Json::parse(text);
+  return in;
+}
+
+std::ostream &operator<<(std::ostream &out, mirage::utils::Json const &j) { return out << j.dump(); }
+
+// ---- operator json() of the operator classes ---------------------------------------------
+// One definition per class, as in the reference (src/kernel/{operator,matmul,element_unary,
+// element_binary,reduction,customized}.cc, src/threadblock/{input_loader,output,matmul,
+// element_unary,element_binary,reduction,concat,graph}.cc): each gives the entry that
+// to_json writes for it, so `json(*op)` and `to_json(j, *op)` agree by construction.
+namespace mirage {
+namespace kernel {
+#define MIRAGE_KN_JSON(CLASS)                          \
+  CLASS::operator json() const {                       \
+    json j;                                            \
+    to_json(j, static_cast<KNOperator const &>(*this)); \
+    return j;                                          \
+  }
+MIRAGE_KN_JSON(KNInputOp)
+MIRAGE_KN_JSON(KNMatmulOp)
+MIRAGE_KN_JSON(KNElementUnaryOp)
+MIRAGE_KN_JSON(KNElementBinaryOp)
+MIRAGE_KN_JSON(KNReductionOp)
+MIRAGE_KN_JSON(KNCustomizedOp)
+#undef MIRAGE_KN_JSON
+
+Graph::operator json() const {
+  json j;
+  to_json(j, *this);
+  return j;
+}
+}  // namespace kernel
+
+namespace threadblock {
+#define MIRAGE_TB_JSON(CLASS)                          \
+  CLASS::operator json() const {                       \
+    json j;                                            \
+    to_json(j, static_cast<TBOperator const &>(*this)); \
+    return j;                                          \
+  }
+MIRAGE_TB_JSON(TBInputOp)
+MIRAGE_TB_JSON(TBOutputOp)
+MIRAGE_TB_JSON(TBMatmulOp)
+MIRAGE_TB_JSON(TBElementUnaryOp)
+MIRAGE_TB_JSON(TBElementBinaryOp)
+MIRAGE_TB_JSON(TBReductionOp)
+MIRAGE_TB_JSON(TBConcatOp)
+#undef MIRAGE_TB_JSON
+
+Graph::operator json() const {
+  json j;
+  to_json(j, *this);
+  return j;
+}
 }  // namespace threadblock
 }  // namespace mirage
 

@@ -343,6 +343,7 @@ struct VerifyTicket {
   std::vector<uint8_t> possible;  // which (reference, candidate) output pairs can be equal at all
   int first_slot = 0, slots = 0;
   int mark_reference = 0, mark_done = 0;
+  int ticket = -1;  // owns mark pair (2 ticket, 2 ticket + 1) and the slot range until the end call
   int reference_queue = 0;
   int workers = 0, first_worker = 0;  // worker w of the batch is pool thread (first_worker + w) % queues
   std::vector<VerifyStats> local;
@@ -353,11 +354,95 @@ struct VerifyTicket {
   std::chrono::steady_clock::time_point t_begin, t_enqueued;
 };
 
-// Slot ranges and marks of the batches in flight come from rings: a range or a mark is reused
-// only MI355_COMPARE_SLOTS compares / 32 batches later.
+// Compare-slot ranges and mark pairs of the batches in flight.  A range or a mark pair is
+// handed out only while no unfinished batch owns it: resetting the slots of a live batch
+// would clear mismatch flags the device has already written (its candidates would then read
+// back as EQUAL), and sharing a mark with a live batch could drop that batch's wait.
+// verify_batch_begin takes both, verify_batch_end gives them back.
+namespace {
+struct InFlight {
+  struct Range {
+    int first, count, ticket;
+  };
+  std::vector<Range> live;
+  int next_slot = 0;
+  int next_ticket = 0;
+  static constexpr int kTickets = MI355_NUM_MARKS / 2;
+
+  bool overlaps(int first, int count, int *end_of_blocker) const {
+    for (Range const &r : live) {
+      if (r.count > 0 && first < r.first + r.count && r.first < first + count) {
+        *end_of_blocker = r.first + r.count;
+        return true;
+      }
+    }
+    return false;
+  }
+
+  // false: every mark pair is owned, or no free stretch of `count` slots exists
+  bool acquire(int count, int *first_slot, int *ticket) {
+    if (count < 0 || count > MI355_COMPARE_SLOTS || (int)live.size() >= kTickets) {
+      return false;
+    }
+    int id = -1;
+    for (int i = 0; i < kTickets && id < 0; i++) {
+      int const cand = (next_ticket + i) % kTickets;
+      bool used = false;
+      for (Range const &r : live) {
+        used = used || r.ticket == cand;
+      }
+      if (!used) {
+        id = cand;
+      }
+    }
+    if (id < 0) {
+      return false;
+    }
+    // first fit from the ring position, wrapping once
+    int pos = next_slot;
+    bool wrapped = false, found = false;
+    for (int guard = 0; guard < 4 * kTickets + 4 && !found; guard++) {
+      if (pos + count > MI355_COMPARE_SLOTS) {
+        if (wrapped) {
+          break;
+        }
+        wrapped = true;
+        pos = 0;
+      }
+      int blocker_end = 0;
+      if (count > 0 && overlaps(pos, count, &blocker_end)) {
+        pos = blocker_end;
+      } else {
+        found = true;
+      }
+      if (wrapped && pos >= next_slot && !found) {
+        break;
+      }
+    }
+    if (!found) {
+      return false;
+    }
+    live.push_back(Range{pos, count, id});
+    next_slot = pos + count;
+    next_ticket = (id + 1) % kTickets;
+    *first_slot = pos;
+    *ticket = id;
+    return true;
+  }
+
+  void release(int ticket) {
+    for (size_t i = 0; i < live.size(); i++) {
+      if (live[i].ticket == ticket) {
+        live.erase(live.begin() + (long)i);
+        return;
+      }
+    }
+  }
+};
+}  // namespace
+
 static std::mutex g_ring_mutex;
-static int g_next_slot = 0;
-static int g_next_ticket = 0;
+static InFlight g_in_flight;
 static int g_queues_per_batch = MI355_NUM_QUEUES;
 static int g_next_queue = 0;
 
@@ -388,13 +473,12 @@ VerifyTicket *verify_batch_begin(std::vector<kernel::Graph *> const &candidates,
   MIRAGE_CHECK(t->slots <= MI355_COMPARE_SLOTS, "too many compares for one verify_batch call");
   {
     std::lock_guard<std::mutex> lock(g_ring_mutex);
-    if (g_next_slot + t->slots > MI355_COMPARE_SLOTS) {
-      g_next_slot = 0;
-    }
-    t->first_slot = g_next_slot;
-    g_next_slot += t->slots;
-    int const ticket = g_next_ticket;
-    g_next_ticket = (g_next_ticket + 1) % (MI355_NUM_MARKS / 2);
+    int ticket = -1;
+    bool const ok = g_in_flight.acquire(t->slots, &t->first_slot, &ticket);
+    MIRAGE_CHECK(ok, "too many verification batches in flight: every verify_batch_begin needs a "
+                     "free mark pair (32 in all) and a free stretch of compare slots; call "
+                     "verify_batch_end on an earlier ticket first");
+    t->ticket = ticket;
     t->mark_reference = 2 * ticket;
     t->mark_done = 2 * ticket + 1;
     t->workers = g_queues_per_batch;
@@ -503,6 +587,10 @@ void verify_batch_end(VerifyTicket *ticket, std::vector<uint8_t> &equal, VerifyS
   MI355_CALL(mi355_mark_wait_host(t->mark_done));
   std::vector<uint8_t> same((size_t)t->slots, 0);
   MI355_CALL(mi355_fp_equal_read(t->first_slot, t->slots, same.data()));
+  {
+    std::lock_guard<std::mutex> lock(g_ring_mutex);
+    g_in_flight.release(t->ticket);  // slots read, marks waited for: both may be handed out again
+  }
   if (stats != nullptr) {
     auto const t_done = std::chrono::steady_clock::now();
     for (VerifyStats const &l : t->local) {
@@ -589,6 +677,16 @@ void *mirage_verify_batch_begin(void *const *candidates, int n, void *reference,
   return mirage::search::verify_batch_begin(c, mirage::search::graph_outputs(*ref), input_seed,
                                             fingerprint_reference ? ref : nullptr);
 }
+
+// The bookkeeping of slot ranges and mark pairs by itself (no device): a scratch instance for
+// host-side tests.  acquire returns 0 and fills first_slot / ticket, or -1 when nothing is free.
+using mirage::search::InFlight;
+void *mirage_verify_ring_create(void) { return new InFlight(); }
+void mirage_verify_ring_destroy(void *ring) { delete static_cast<InFlight *>(ring); }
+int mirage_verify_ring_acquire(void *ring, int slots, int *first_slot, int *ticket) {
+  return static_cast<InFlight *>(ring)->acquire(slots, first_slot, ticket) ? 0 : -1;
+}
+void mirage_verify_ring_release(void *ring, int ticket) { static_cast<InFlight *>(ring)->release(ticket); }
 
 void mirage_verify_set_queues_per_batch(int queues) {
   mirage::search::set_verify_queues_per_batch(queues);

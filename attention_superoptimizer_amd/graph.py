@@ -9,6 +9,7 @@ python/mirage/_cython/core.pyx:180-236), bound over the C facade with ctypes.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -256,11 +257,61 @@ class KNGraph:
         """Mean milliseconds per launch (reference profile() protocol)."""
         return float(self._rt.mirage_op_profile(self._g, idx))
 
+    def profile_all(self):
+        """What the reference's cpp_examples/profile.cc does with a graph (:25-34):
+        fingerprint() of every operator, then profile() of every operator.  Returns
+        (sum of the mean milliseconds per launch, per-operator list)."""
+        n = self.num_operators
+        per_op = (ctypes.c_float * n)()
+        total = float(self._rt.mirage_graph_profile(self._g, per_op, n))
+        return total, [float(per_op[i]) for i in range(n)]
+
     def lowered(self, idx: int, fingerprint: bool = True) -> N.Mi355Plan:
         p = N.Mi355Plan()
         rc = self._rt.mirage_op_lowered(self._g, idx, 1 if fingerprint else 0, ctypes.byref(p), None)
         assert rc == 0
         return p
+
+
+class Checkpoint:
+    """A search checkpoint (reference include/mirage/search/search.h:46-68) or a single graph
+    file, loaded by the host runtime: the computation graph, the generated graphs in wire
+    format, best_profile_result, config / callstack (uninterpreted) and the counters."""
+
+    def __init__(self, handle):
+        self._rt = N.runtime()
+        self._h = ctypes.c_void_p(handle)
+        counters = (ctypes.c_longlong * 3)()
+        self.best_run_time = float(self._rt.mirage_checkpoint_summary(self._h, counters))
+        self.counters = tuple(int(c) for c in counters)
+        self.num_graphs = int(self._rt.mirage_checkpoint_num_graphs(self._h))
+
+    @classmethod
+    def load(cls, path: str) -> "Checkpoint":
+        h = N.runtime().mirage_checkpoint_load(os.fsencode(path))
+        if not h:
+            raise ValueError(f"cannot load a checkpoint or graph from {path}")
+        return cls(h)
+
+    def graph_json(self, index: int) -> str:
+        """-2: the whole checkpoint, -1: the computation graph, i >= 0: generated graph i."""
+        n = self._rt.mirage_checkpoint_json(self._h, index, None, 0)
+        if n < 0:
+            raise IndexError(index)
+        buf = ctypes.create_string_buffer(n + 1)
+        self._rt.mirage_checkpoint_json(self._h, index, buf, n + 1)
+        return buf.value.decode()
+
+    def to_json(self) -> str:
+        return self.graph_json(-2)
+
+    def graph(self, index: int) -> "KNGraph":
+        return KNGraph.from_json(self.graph_json(index))
+
+    def close(self):
+        if self._h is not None:
+            self._rt.mirage_checkpoint_destroy(self._h)
+            self._h = None
 
 
 def _stats(st) -> dict:

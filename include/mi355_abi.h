@@ -9,8 +9,13 @@
  * sizes only; every function returns 0 on success and a negative code on
  * failure, with mi355_last_error() giving the text.  All device pointers must
  * come from the arena returned by mi355_init() (or any hipMalloc'ed memory).
- * Work is enqueued on one backend-owned HIP stream; calls are asynchronous
- * unless stated otherwise.  Single caller thread, like the reference.
+ * Work is enqueued on one of MI355_NUM_QUEUES backend-owned in-order queues (HIP streams):
+ * the queue the calling host thread selected with mi355_queue_select, queue 0 by default.
+ * Calls are asynchronous unless stated otherwise.  Several host threads may call at once
+ * provided each drives a queue of its own (a queue is driven by one thread at a time);
+ * timers, the blocking compare and the launch record are kept per queue.  The reference
+ * itself has one stream and a single caller thread; a caller that never selects a queue
+ * gets exactly that.
  */
 #ifndef MI355_ABI_H
 #define MI355_ABI_H

@@ -21,6 +21,7 @@ public:
   bool profile(ProfileResult &profile) override;
   void run(void);  // one fp16 launch on the backend stream, no synchronisation
   bool fingerprint(void) override;
+  operator json() const override;  // adds bgraph and plan (src/kernel/customized.cc:315-321)
 
   mirage::threadblock::ExecutionPlan plan;
   mirage::threadblock::Graph bgraph;

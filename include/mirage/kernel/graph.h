@@ -66,6 +66,11 @@ public:
   // as there).
   void generate_hip_program(char const *filepath);
 
+  // the graph as the array of its operators' JSON entries (what to_json(json &, Graph
+  // const &) writes, src/kernel/graph.cc:33-37), so that `json(g)` reads as in the
+  // reference's cpp_examples/profile.cc:22
+  operator json() const;
+
   // Operators in creation order.  The graph deletes them newest-first on
   // destruction (the arena is LIFO); callers that pop an operator delete it
   // themselves, as the reference's search does.

@@ -8,6 +8,7 @@
 
 #include "mirage/kernel/device_tensor.h"
 #include "mirage/profile_result.h"
+#include "mirage/utils/json_value.h"
 #include <vector>
 
 namespace mirage {
@@ -24,6 +25,9 @@ public:
   virtual bool profile(ProfileResult &result) = 0;
   // uint16: evaluate the operator over the fingerprint ring into fp_ptr
   virtual bool fingerprint(void) = 0;
+  // the operator's entry in the JSON form of its graph (reference operator.h:41,
+  // src/kernel/graph.cc:35 `json(*op)`)
+  virtual operator json() const = 0;
 
   mirage::type::KNOperatorType op_type;
   std::vector<DTensor> input_tensors;
@@ -40,6 +44,7 @@ public:
   ~KNInputOp();
   bool profile(ProfileResult &profile) override;
   bool fingerprint(void) override;
+  operator json() const override;
 };
 
 class KNMatmulOp : public KNOperator {
@@ -48,6 +53,7 @@ public:
   ~KNMatmulOp();
   bool profile(ProfileResult &profile) override;
   bool fingerprint(void) override;
+  operator json() const override;
 };
 
 class KNElementUnaryOp : public KNOperator {
@@ -56,6 +62,7 @@ public:
   ~KNElementUnaryOp();
   bool profile(ProfileResult &profile) override;
   bool fingerprint(void) override;
+  operator json() const override;
 };
 
 class KNElementBinaryOp : public KNOperator {
@@ -65,6 +72,7 @@ public:
   ~KNElementBinaryOp();
   bool profile(ProfileResult &profile) override;
   bool fingerprint(void) override;
+  operator json() const override;
 };
 
 class KNReductionOp : public KNOperator {
@@ -73,6 +81,7 @@ public:
   ~KNReductionOp();
   bool profile(ProfileResult &profile) override;
   bool fingerprint(void) override;
+  operator json() const override;
 
   int reduction_dim_idx, reduction_dim_size;
 };

@@ -52,7 +52,10 @@ void verify_batch(std::vector<mirage::kernel::Graph *> const &candidates,
 // is fingerprinted as part of the batch; nullptr: the caller has already enqueued its
 // fingerprints on its own queue.  Between the two calls the caller must not enqueue device
 // work on the worker queues itself, and the candidates, the reference and their tensors
-// must stay alive.  At most 32 batches, MI355_COMPARE_SLOTS compares in all, in flight.
+// must stay alive.  At most 32 batches, MI355_COMPARE_SLOTS compares in all, may be in flight
+// (begun and not yet ended): a batch owns its compare slots and its pair of marks until
+// verify_batch_end has read them, and a verify_batch_begin that finds no free pair or no free
+// stretch of slots aborts with a message rather than reuse what a live batch still owns.
 // How many backend queues (and worker threads) a batch is dealt over, MI355_NUM_QUEUES by
 // default.  Successive batches take successive groups of queues, so with two batches in
 // flight and 2 queues per batch each batch has half of the queues to itself: twice as many

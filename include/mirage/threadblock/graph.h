@@ -71,6 +71,10 @@ public:
   static void set_smem_budget(size_t bytes);
   static size_t smem_budget();
 
+  // {graph_level, grid_dim, block_dim, forloop_range, reduction_dimx, operators,
+  // smem_offset} (reference threadblock/graph.h:107, src/threadblock/graph.cc:476-489)
+  operator json() const;
+
   dim3 grid_dim, block_dim;
   int forloop_range;
   int reduction_dimx;

@@ -8,6 +8,7 @@
 #include "mirage/threadblock/smem_tensor.h"
 #include "mirage/type.h"
 #include "mirage/utils/hip_types.h"
+#include "mirage/utils/json_value.h"
 #include <vector>
 
 namespace mirage {
@@ -23,6 +24,9 @@ public:
              STensor const &input2);
   TBOperator(Graph *graph, mirage::type::TBOperatorType, std::vector<STensor> const &inputs);
   virtual ~TBOperator();
+  // the operator's entry in the JSON form of its thread-block graph (reference
+  // threadblock/operator.h:41, src/threadblock/graph.cc:485 `json(*op)`)
+  virtual operator json() const = 0;
 
   Graph *bgraph;
   mirage::type::TBOperatorType op_type;
@@ -36,6 +40,7 @@ public:
   TBInputOp(Graph *_graph, mirage::kernel::DTensor const &dtensor, int3 input_map,
             int forloop_dim, mirage::layout::SmemLayout layout);
   ~TBInputOp();
+  operator json() const override;
 
   mirage::kernel::DTensor dtensor;
   int3 input_map;
@@ -48,6 +53,7 @@ class TBOutputOp : public TBOperator {
 public:
   TBOutputOp(Graph *_graph, STensor const &stensor, int3 output_map);
   ~TBOutputOp();
+  operator json() const override;
 
   mirage::kernel::DTensor dtensor;
   int3 output_map;
@@ -57,12 +63,14 @@ class TBMatmulOp : public TBOperator {
 public:
   TBMatmulOp(Graph *_graph, STensor const &A, STensor const &B);
   ~TBMatmulOp();
+  operator json() const override;
 };
 
 class TBElementUnaryOp : public TBOperator {  // in place
 public:
   TBElementUnaryOp(Graph *_graph, STensor const &A, mirage::type::TBOperatorType _type);
   ~TBElementUnaryOp();
+  operator json() const override;
 };
 
 class TBElementBinaryOp : public TBOperator {
@@ -70,12 +78,14 @@ public:
   TBElementBinaryOp(Graph *_graph, STensor const &A, STensor const &B,
                     mirage::type::TBOperatorType _type);
   ~TBElementBinaryOp();
+  operator json() const override;
 };
 
 class TBReductionOp : public TBOperator {
 public:
   TBReductionOp(Graph *graph, STensor const &input, int dim, int size);
   ~TBReductionOp();
+  operator json() const override;
 
   int reduce_dim, reduce_size;
 };
@@ -84,6 +94,7 @@ class TBConcatOp : public TBOperator {
 public:
   TBConcatOp(Graph *graph, STensor const &A, STensor const &B, int dim);
   ~TBConcatOp();
+  operator json() const override;
 
   int concat_dim;
 };

@@ -10,9 +10,11 @@ tensor guids), dims/layouts of inputs, and each customized op's plan.  The
 older schema has no `reduction_dimx`; the reference default 64 applies
 (include/mirage/threadblock/graph.h:40).
 
-It also keeps an excerpt of the file in its ORIGINAL schema (the computation graph
-and every ninth generated graph, verbatim JSON objects): the data the JSON wire format
-of the host API is tested against.
+It also keeps an excerpt of the file in its ORIGINAL schema: the whole checkpoint object
+(include/mirage/search/search.h:46-68: best_graph, best_profile_result, config, callstack,
+the three counters, the computation graph) with every ninth generated graph, verbatim JSON
+objects: the data the JSON wire format and the checkpoint loader of the host API are
+tested against.
 
 Usage: python tests/golden/extract_gqa_checkpoint.py [reference_root]
 Writes tests/golden/gqa_spec_decode_69.json and
@@ -84,12 +86,12 @@ def main():
     with open(dst, "w") as f:
         json.dump(doc, f, separators=(",", ":"))
     picks = list(range(0, len(j["generated_graphs"]), 9))
-    excerpt = {
+    excerpt = {k: v for k, v in j.items() if k != "generated_graphs"}
+    excerpt.update({
         "source": "demo/checkpoint_group_query_attn_spec_decode.json",
         "indices": picks,
-        "computation_graph": j["computation_graph"],
         "generated_graphs": [j["generated_graphs"][i] for i in picks],
-    }
+    })
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)),
                        "gqa_spec_decode_checkpoint_excerpt.json")
     with open(dst, "w") as f:

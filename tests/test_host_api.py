@@ -195,3 +195,66 @@ def test_plan_extents_and_validation():
     p.operator_types[2] = 2050
     assert ab.mi355_plan_extents(ctypes.byref(p), ie, oe, None, None) == -4
     g.close()
+
+
+def test_verify_ring_never_hands_out_what_a_live_batch_owns():
+    """Compare-slot ranges and mark pairs of verification batches in flight (verify.cc): a new
+    batch never overlaps a live one; ranges and marks come back when a batch ends; the 33rd
+    batch in flight, or a range no free stretch can hold, is refused."""
+    import ctypes
+    from attention_superoptimizer_amd import _native as N
+    rt = N.runtime()
+    ring = ctypes.c_void_p(rt.mirage_verify_ring_create())
+    try:
+        first, ticket = ctypes.c_int(), ctypes.c_int()
+        live = {}
+
+        def acquire(n):
+            rc = rt.mirage_verify_ring_acquire(ring, n, ctypes.byref(first), ctypes.byref(ticket))
+            if rc != 0:
+                return None
+            for f, c in live.values():
+                assert n == 0 or c == 0 or first.value >= f + c or f >= first.value + n, "overlap"
+            assert ticket.value not in live and 0 <= ticket.value < 32
+            assert 0 <= first.value and first.value + n <= 65536
+            live[ticket.value] = (first.value, n)
+            return ticket.value
+
+        def release(t):
+            rt.mirage_verify_ring_release(ring, t)
+            del live[t]
+
+        # three batches of 30,000 slots: the third does not fit until the first has ended
+        a, b = acquire(30000), acquire(30000)
+        assert a is not None and b is not None
+        assert acquire(30000) is None
+        release(a)
+        c = acquire(30000)
+        assert c is not None and live[c][0] == 0          # wrapped into the freed stretch, not onto b
+        assert acquire(10000) is None                     # 5,536 free slots at the end only
+        d = acquire(5000)
+        assert d is not None and live[d][0] == 60000
+        for t in list(live):
+            release(t)
+        # 32 batches in flight use every mark pair; the 33rd is refused until one ends
+        ts = [acquire(16) for _ in range(32)]
+        assert None not in ts and len(set(ts)) == 32
+        assert acquire(16) is None
+        release(ts[7])
+        assert acquire(16) == ts[7]
+        # long run of begin / end with a few in flight: wraps the ring many times
+        for t in list(live):
+            release(t)
+        import random
+        rnd = random.Random(5)
+        order = []
+        for _ in range(2000):
+            if len(order) < 4 or (len(order) < 20 and rnd.random() < 0.5):
+                t = acquire(rnd.choice([0, 1, 64, 4096, 9000]))
+                if t is not None:
+                    order.append(t)
+                    continue
+            release(order.pop(0))
+        assert acquire(65537) is None
+    finally:
+        rt.mirage_verify_ring_destroy(ring)
