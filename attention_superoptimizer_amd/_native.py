@@ -113,6 +113,7 @@ ABI = {
     "mi355_customized_run": (_ci, [_pplan, _pvp, _pvp]),
     "mi355_customized_profile": (_ci, [_pplan, _pvp, _pvp, _ci, _ci, _ci, _pf]),
     "mi355_last_launch": (_ci, [ctypes.POINTER(Mi355LaunchInfo)]),
+    "mi355_phase_trace_read": (_ci, [ctypes.POINTER(ctypes.c_ulonglong), _sz]),
     "mi355_f16_fill_iota": (_ci, [_vp, _sz, _ci]),
     "mi355_f16_fill_normal": (_ci, [_vp, _sz, ctypes.c_float, _u64]),
     "mi355_f16_matmul": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci]),

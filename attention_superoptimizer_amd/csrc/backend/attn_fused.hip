@@ -94,6 +94,12 @@ struct AttnParams {
   int stages;  // for-loop iterations staged per barrier
   int lds_stage_bytes;
   int perm[3];  // grid dims from fastest to slowest varying in the renumbered workgroup id
+  // extents of the launch grid in that order, their multiply-high division magics
+  // (fast_div_magic: q = mulhi(id, magic), 0 stands for extent 1) and the magic of `split`
+  unsigned perm_ext[3], perm_magic[3], split_magic;
+  int rows;     // query rows of the last row group that exist (16, or 8 for an 8-row tile: the
+                // missing rows are zeros in the Q fragment and are never stored)
+  unsigned long long *trace;  // per-wavefront phase timestamps (attn_direct_kernel<.., TRACE>)
 };
 
 __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int by, int bz,
@@ -181,13 +187,16 @@ __device__ __forceinline__ void decode_block(AttnParams const &P, int &bx, int &
   if (total % 8 == 0) {
     id = (id % 8) * (total / 8) + id / 8;
   }
+  // divisions by the extents are multiply-highs with magics the host computed (exact while
+  // id * extent < 2^32, which the host checks): this runs before the first load can go out
   unsigned coord[3] = {0, 0, 0};
 #pragma unroll
   for (int i = 0; i < 3; i++) {
     int const d = P.perm[i];
-    unsigned const e = d == 0 ? ext[0] : (d == 1 ? ext[1] : ext[2]);
-    unsigned const v = id % e;
-    id /= e;
+    unsigned const e = P.perm_ext[i], m = P.perm_magic[i];
+    unsigned const q = m == 0 ? id : __umulhi(id, m);
+    unsigned const v = id - q * e;
+    id = q;
     if (d == 0) {
       coord[0] = v;
     } else if (d == 1) {
@@ -196,8 +205,9 @@ __device__ __forceinline__ void decode_block(AttnParams const &P, int &bx, int &
       coord[2] = v;
     }
   }
-  bx = coord[0] / P.split;
-  slice = coord[0] % P.split;
+  unsigned const b = P.split_magic == 0 ? coord[0] : __umulhi(coord[0], P.split_magic);
+  bx = (int)b;
+  slice = (int)(coord[0] - b * (unsigned)P.split);
   by = coord[1];
   bz = coord[2];
 }
@@ -236,7 +246,12 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
                         (long long)(row_base + c) * P.q.d_cols + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < DK; kk++) {
-      qf[kk] = *reinterpret_cast<half8 const *>(q + 32 * kk);
+      half8 z;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        z[e] = (_Float16)0.0f;
+      }
+      qf[kk] = c < P.rows ? *reinterpret_cast<half8 const *>(q + 32 * kk) : z;
     }
   }
 
@@ -434,12 +449,12 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
     _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
                    tile_offset(P.o, bx, by, bz, 0) + (long long)row_base * P.o.d_cols;
     constexpr int CH = DV / 8;  // 16-byte chunks per row
-    for (int e = lane; e < 16 * CH; e += 64) {
+    for (int e = lane; e < P.rows * CH; e += 64) {
       int rr = e / CH, cc = (e % CH) * 8;
       *reinterpret_cast<uint4v *>(og + (long long)rr * P.o.d_cols + cc) =
           *reinterpret_cast<uint4v const *>(ow + rr * LDO + cc);
     }
-    if (!HAS_DIV && g == 0) {
+    if (!HAS_DIV && g == 0 && c < P.rows) {
       _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
                       tile_offset(P.r, bx, by, bz, 0);
       rgp[(long long)(row_base + c) * P.r.d_cols] = racc;
@@ -937,7 +952,8 @@ bool match(DevProgram const &P, Match &M) {
   M.D = tq.cols;
   M.NK = tk.cols;
   M.DV = tv.cols;
-  if (tk.rows != M.D || tv.rows != M.NK || M.m % 16 != 0) {
+  // query tiles of whole 16-row groups, or a single group of 8 rows (padded with zero rows)
+  if (tk.rows != M.D || tv.rows != M.NK || (M.m % 16 != 0 && M.m != 8)) {
     return false;
   }
   // Q must be loop invariant; all tiles reachable with 16-byte accesses
@@ -957,246 +973,427 @@ bool match(DevProgram const &P, Match &M) {
   return true;
 }
 
-// Latency variant for short for-loops (every iteration has a wavefront of its own: F <= IP)
-// with the staging of the throughput variant: each wavefront streams the K and V tile of ITS
-// iteration from global memory straight into its own 16 KB of LDS, in their row-major layout
-// (sixteen direct loads, no registers, no transposing stores, and no workgroup barrier before
-// the arithmetic: a wavefront only waits for its own loads), and gathers the MFMA operands
-// with transposing LDS reads under the same chunk swizzle.  Arithmetic, rounding points, the
-// ordered hand-over of the iterations' results and the store are those of attn_fused_kernel.
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
-__global__ __launch_bounds__(64 * RG * IP) void attn_direct_kernel(AttnParams const P) {
-  static_assert(NK == 64 && DV == 64, "the chunk swizzles assume rows of 128 bytes");
-  constexpr int LDO = DV + 8;
+// Direct-staging variant: one row group of (up to) 16 query rows per workgroup, IP wavefronts
+// as iteration lanes.  Wavefront ip owns iterations ip, ip + IP, ip + 2 IP, ... and streams the
+// K and V tile of each from global memory straight into ITS OWN LDS buffers, in their row-major
+// layout (sixteen direct loads per tile pair: no registers, no transposing stores), NBUF tile
+// pairs deep: while it multiplies one pair the next is in flight.  No workgroup barrier inside
+// the loop: a wavefront waits for its own loads only (`s_waitcnt vmcnt`), so the workgroup is
+// IP independent streams -- what a bandwidth-bound decode (8 or 16 query rows against a long
+// key range) needs -- and with one iteration per wavefront (F <= IP) the shortest chain from
+// launch to result.  MFMA operands are gathered with transposing LDS reads under the chunk
+// swizzle of the throughput variant.  Arithmetic and rounding points are those of
+// attn_fused_kernel.  Every iteration's fp16 result is kept (packed, in registers) until the
+// wavefront has finished, then written to LDS (into its own, now dead, tile buffers); after
+// ONE barrier all threads add the F results element by element in ITERATION order, rounding
+// to fp16 after each add as the sequential loop does, and store straight from registers.
+//
+// The loads are inline assembly (see lds_dma16), so the compiler's own count of outstanding
+// vector-memory operations knows nothing of them and the waits are written by hand.  Every
+// load of this kernel is a direct-to-LDS load, the Q tile included: a wait for "all but the
+// newest n" relies on loads completing in issue order, which holds among loads of one kind
+// but not between direct-to-LDS loads and loads into registers (a register load issued after
+// a tile's direct loads was seen to complete before them).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+#pragma clang diagnostic pop
+
+template <int D, int NK, int DV, bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, bool TRACE>
+__global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P) {
+  static_assert(D == 64 && NK == 64 && DV == 64, "the chunk swizzles assume rows of 128 bytes");
+  static_assert(NBUF == 1 || NBUF == 2, "one or two tile pairs per wavefront");
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
-  constexpr int NW = RG * IP;
   constexpr int KI = D * NK / 8 / 64, VI = NK * DV / 8 / 64;  // direct loads per tile
-  constexpr int WAVE_HALFS = D * NK + NK * DV;
-  constexpr int SLOT_DW = DB * 2 + 1;
+  constexpr int PAIR_HALFS = D * NK + NK * DV;                // one K tile + one V tile
+  constexpr int ROWS = 16 * RPW;                              // query rows of one wavefront
+  constexpr int Q_HALFS = ROWS * D;                           // this wavefront's copy of the Q tile
+  constexpr int QI = Q_HALFS / 8 / 64;                        // direct loads of the Q tile
+  constexpr int WAVE_HALFS = NBUF * PAIR_HALFS + Q_HALFS;
+  constexpr int LDO = DV + 4;          // row stride of a result slot (halfs): 8-byte aligned rows
+  constexpr int SLOT_HALFS = ROWS * LDO + ROWS;  // one iteration's O tile + its row sums
+  static_assert(NIT * SLOT_HALFS <= NBUF * PAIR_HALFS, "a wavefront's results must fit its own buffers");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
+  unsigned long long t_start = 0, t_issued = 0, t_landed = 0, t_computed = 0, t_joined = 0;
+  if (TRACE) {
+    t_start = __builtin_amdgcn_s_memrealtime();
+  }
   int const tid = threadIdx.x;
-  int const lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
-  int const rg = wave / IP, ip = wave % IP;
+  int const lane = tid % 64, ip = __builtin_amdgcn_readfirstlane(tid / 64);
   int const g = lane / 16, c = lane % 16;
   int bx, by, bz, slice;
   decode_block(P, bx, by, bz, slice);
-  int const row_base = (slice * RG + rg) * 16;
-  bool const active = ip < P.forloop_range;
+  int const row_base = slice * ROWS;
+  int const rows = RPW == 1 ? P.rows : ROWS;  // rows that exist (only a lone row group may be short)
+  int const F = P.forloop_range;
+  int const nit = ip < F ? (F - ip + IP - 1) / IP : 0;  // iterations of this wavefront
 
-  _Float16 *const kt = reinterpret_cast<_Float16 *>(lds) + wave * WAVE_HALFS;
-  _Float16 *const vt = kt + D * NK;
-  if (active) {
-    // this lane's chunk of direct load i is (row r, position pos) of the tile and comes from
-    // global chunk pos ^ 2 * key(r) of row r
-    uint32_t const lds_k = lds_address(kt), lds_v = lds_address(vt);
-    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, ip);
-    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, ip);
+  _Float16 *const wbuf = reinterpret_cast<_Float16 *>(lds) + ip * WAVE_HALFS;
+  uint32_t const lds_w = lds_address(wbuf);
+  // Direct load i of a tile fills LDS chunks 64 i .. 64 i + 63: this lane's chunk is
+  // (row 8 i + lane / 8, position lane % 8) and comes from global chunk pos ^ 2 * key(row) of
+  // that row.  The swizzle keys depend on i only through its parity (K) or not at all (V), so
+  // three lane offsets serve all sixteen loads and the row advance 8 i is added to the
+  // wavefront-uniform base address.
+  int const l3 = lane >> 3, pos = lane & 7;
+  static_assert(stream_swizzle_key<NK, true>(8 + 5) == (stream_swizzle_key<NK, true>(5) | 2) &&
+                    stream_swizzle_key<DV, false>(8 + 5) == stream_swizzle_key<DV, false>(5),
+                "row advance by 8 flips bit 1 of the K key and leaves the V key unchanged");
+  uint32_t const k_off_even = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(l3))));
+  uint32_t const k_off_odd = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(8 + l3))));
+  uint32_t const v_off = 2u * (uint32_t)(l3 * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(l3))));
+  auto fetch = [&](int it, int b) {
+    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
+    uint32_t const base = lds_w + 2u * (uint32_t)(b * PAIR_HALFS);
 #pragma unroll
     for (int i = 0; i < KI; i++) {
-      int const q = i * 64 + lane, r = q / (NK / 8), pos = q % (NK / 8);
-      uint32_t const off = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(r))));
-      lds_dma16(kg, off, lds_k + 1024u * (uint32_t)i);
+      lds_dma16(kg + (long long)(8 * i) * P.k.d_cols, (i & 1) ? k_off_odd : k_off_even,
+                base + 1024u * (uint32_t)i);
     }
 #pragma unroll
     for (int i = 0; i < VI; i++) {
-      int const q = i * 64 + lane, r = q / (DV / 8), pos = q % (DV / 8);
-      uint32_t const off = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(r))));
-      lds_dma16(vg, off, lds_v + 1024u * (uint32_t)i);
+      lds_dma16(vg + (long long)(8 * i) * P.v.d_cols, v_off,
+                base + 2u * (uint32_t)(D * NK) + 1024u * (uint32_t)i);
     }
-  }
-  // Q fragments (B operand of S^T): Q[row c][32kk + 8g .. +7]
-  half8 qf[DK];
-  {
-    _Float16 const *q = static_cast<_Float16 const *>(P.q.ptr) + tile_offset(P.q, bx, by, bz, 0) +
-                        (long long)(row_base + c) * P.q.d_cols + 8 * g;
+  };
+  // The Q tile (rows that do not exist re-read row 0 and are zeroed below), then the first
+  // one or two tile pairs: everything this wavefront needs to start is in flight at once.
+  // (A wavefront without an iteration loads nothing: no transfer may outlive its waits.)
+  half8 qf[RPW][DK];
+  if (nit > 0) {
+    _Float16 const *qg = static_cast<_Float16 const *>(P.q.ptr) + tile_offset(P.q, bx, by, bz, 0) +
+                         (long long)row_base * P.q.d_cols;
 #pragma unroll
-    for (int kk = 0; kk < DK; kk++) {
-      qf[kk] = *reinterpret_cast<half8 const *>(q + 32 * kk);
+    for (int i = 0; i < QI; i++) {
+      int const r = 8 * i + l3;
+      uint32_t const off = 2u * (uint32_t)((r < rows ? r : 0) * P.q.d_cols + 8 * pos);
+      lds_dma16(qg, off, lds_w + 2u * (uint32_t)(NBUF * PAIR_HALFS) + 1024u * (uint32_t)i);
     }
+    fetch(ip, 0);
+  }
+  if (NBUF == 2 && nit > 1) {
+    fetch(ip + IP, 1);
+  }
+  if (TRACE) {
+    t_issued = __builtin_amdgcn_s_memrealtime();
   }
   int const a4 = c >> 2, b4 = c & 3;
   int const k_lane = (8 * g + a4) * NK + ((b4 >> 1) << 3) + (b4 & 1) * 4;
   int const v_lane = (4 * g + a4) * DV + ((b4 >> 1) << 3) + (b4 & 1) * 4;
   int const sw_k = stream_swizzle_key<NK, true>(8 * g + a4) << 4;
   int const sw_v = stream_swizzle_key<DV, false>(4 * g + a4) << 4;
+  // where this thread's share of the result goes (address arithmetic done while loads fly)
+  constexpr int EPT = ROWS * DV / (64 * IP);  // elements per thread (16 rows: 8 / 4 / 2 for IP = 2 / 4 / 8)
+  static_assert(EPT == 2 || EPT == 4 || EPT == 8, "2, 4 or 8 wavefronts");
+  int const out_row = tid / (DV / EPT), out_col = (tid % (DV / EPT)) * EPT;
+  _Float16 *const og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
+                       tile_offset(P.o, bx, by, bz, 0) +
+                       (long long)(row_base + out_row) * P.o.d_cols + out_col;
 
-  unsigned char *const tail = lds + NW * WAVE_HALFS * 2;
-  _Float16 *const o_stage = reinterpret_cast<_Float16 *>(tail);
-  uint32_t *const slots = reinterpret_cast<uint32_t *>(tail + RG * 16 * LDO * 2);
-
-  _Float16 o16[DB][4];
-  _Float16 r16 = (_Float16)0.0f;
+  // results of this wavefront's iterations, packed fp16: keep[j][rp][2t], [2t+1] =
+  // O[row 16rp + c][16t + 4g + r] for r = 0,1 / 2,3; keep[j][rp][2 DB] = the row sum of row c
+  uint32_t keep[NIT][RPW][2 * DB + 1];
 #pragma unroll
-  for (int t = 0; t < DB; t++) {
+  for (int j = 0; j < NIT; j++) {
+    if (j < nit) {
+      int const b = NBUF == 2 ? (j & 1) : 0;
+      // the tile pair of iteration j (and everything older) has landed when at most the next
+      // pair's loads are outstanding
+      if (NBUF == 2 && j + 1 < nit) {
+        wait_vm<KI + VI>();
+      } else {
+        wait_vm<0>();
+      }
+      if (j == 0) {
+        // Q fragments (B operand of S^T): Q[row c][32kk + 8g .. +7]
+        _Float16 const *ql = wbuf + NBUF * PAIR_HALFS + c * D + 8 * g;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      o16[t][r] = (_Float16)0.0f;
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's own tiles have landed
-  if (active) {
-    uint32_t pk[KB / 2][4];
-    float rs = 0.0f;
-    half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
-    constexpr float LOG2E = 1.44269504088896340736f;
+        for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
-    for (int j = 0; j < KB; j++) {
-      float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+          for (int kk = 0; kk < DK; kk++) {
+            qf[rp][kk] = *reinterpret_cast<half8 const *>(ql + 16 * rp * D + 32 * kk);
+            if (RPW == 1 && c >= rows) {
+#pragma unroll
+              for (int e = 0; e < 8; e++) {
+                qf[rp][kk][e] = (_Float16)0.0f;
+              }
+            }
+          }
+        }
+        if (TRACE) {
+          t_landed = __builtin_amdgcn_s_memrealtime();
+        }
+      }
+      _Float16 const *kt = wbuf + b * PAIR_HALFS;
+      _Float16 const *vt = kt + D * NK;
+      // Four phases, each with all of its independent work issued before anything waits:
+      // every K operand read, the KB independent S^T accumulation chains interleaved, every
+      // V operand read (their latency hides under the exp stretch), the DB independent P.V
+      // chains interleaved.
+      half8 ka[KB][DK];
+#pragma unroll
+      for (int jb = 0; jb < KB; jb++) {
+#pragma unroll
+        for (int kk = 0; kk < DK; kk++) {
+          // K[32kk + 8g + 0..7][16jb + c]
+          _Float16 const *kp = kt + k_lane + 32 * kk * NK + (sw_k ^ (jb << 4));
+          half4 const a_lo = lds_read_tr16(kp), a_hi = lds_read_tr16(kp + 4 * NK);
+          ka[jb][kk] = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      }
+      float4v acc[RPW][KB];
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int jb = 0; jb < KB; jb++) {
+          acc[rp][jb] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+      }
 #pragma unroll
       for (int kk = 0; kk < DK; kk++) {
-        // K[32kk + 8g + 0..7][16j + c]
-        _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw_k ^ (j << 4));
-        half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
-        half8 const a = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kk], acc, 0, 0, 0);
-      }
 #pragma unroll
-      for (int h = 0; h < 2; h++) {
-        half2v const s2 = {static_cast<_Float16>(acc[2 * h]), static_cast<_Float16>(acc[2 * h + 1])};
-        float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
-        float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
-        half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
-        rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);
-        pk[j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
-      }
-    }
-    rs += __shfl_xor(rs, 16, 64);
-    rs += __shfl_xor(rs, 32, 64);
-    r16 = static_cast<_Float16>(rs);
-    if (HAS_DIV) {
-      float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
+        for (int jb = 0; jb < KB; jb++) {
 #pragma unroll
-      for (int jj = 0; jj < KB / 2; jj++) {
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-          half2v const e2 = __builtin_bit_cast(half2v, pk[jj][w]);
-          half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
-                             static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
-          pk[jj][w] = __builtin_bit_cast(uint32_t, p2);
+          for (int rp = 0; rp < RPW; rp++) {
+            acc[rp][jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[jb][kk], qf[rp][kk], acc[rp][jb], 0, 0, 0);
+          }
         }
       }
-    }
-#pragma unroll
-    for (int t = 0; t < DB; t++) {
-      float4v o = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int jj = 0; jj < KB / 2; jj++) {
-        // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
-        _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
-        half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
-        half8 const b = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        uint4v const a = {pk[jj][0], pk[jj][1], pk[jj][2], pk[jj][3]};
-        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o, 0, 0, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        o16[t][r] = static_cast<_Float16>(o[r]);
-      }
-    }
-  }
-  // hand the iteration's result to the row group's first wavefront, which adds the
-  // iterations in order, rounding to fp16 after each add as the sequential loop would
-  _Float16 oacc[DB][4];
-  _Float16 racc = (_Float16)0.0f;
-  if (IP > 1) {
-    if (ip > 0 && active) {
-      uint32_t *slot = slots + ((rg * (IP - 1) + (ip - 1)) * SLOT_DW) * 64 + lane;
+      half8 vb[DB][KB / 2];
 #pragma unroll
       for (int t = 0; t < DB; t++) {
-        half2v lo = {o16[t][0], o16[t][1]}, hi = {o16[t][2], o16[t][3]};
-        slot[(2 * t) * 64] = __builtin_bit_cast(uint32_t, lo);
-        slot[(2 * t + 1) * 64] = __builtin_bit_cast(uint32_t, hi);
-      }
-      half2v rr = {r16, (_Float16)0.0f};
-      slot[(2 * DB) * 64] = __builtin_bit_cast(uint32_t, rr);
-    }
-    __syncthreads();
-  }
-  _Float16 *ow = o_stage + rg * 16 * LDO;
-  if (ip == 0) {
 #pragma unroll
-    for (int t = 0; t < DB; t++) {
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        oacc[t][r] = (_Float16)0.0f;
-      }
-    }
-#pragma unroll
-    for (int q = 0; q < IP; q++) {
-      if (q < P.forloop_range) {
-        if (q > 0) {
-          uint32_t const *slot = slots + ((rg * (IP - 1) + (q - 1)) * SLOT_DW) * 64 + lane;
-#pragma unroll
-          for (int t = 0; t < DB; t++) {
-            half2v lo = __builtin_bit_cast(half2v, slot[(2 * t) * 64]);
-            half2v hi = __builtin_bit_cast(half2v, slot[(2 * t + 1) * 64]);
-            o16[t][0] = lo[0];
-            o16[t][1] = lo[1];
-            o16[t][2] = hi[0];
-            o16[t][3] = hi[1];
-          }
-          r16 = __builtin_bit_cast(half2v, slot[(2 * DB) * 64])[0];
+        for (int jj = 0; jj < KB / 2; jj++) {
+          // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
+          _Float16 const *vp = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
+          half4 const b_lo = lds_read_tr16(vp), b_hi = lds_read_tr16(vp + 16 * DV);
+          vb[t][jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      uint32_t pk[RPW][KB / 2][4];
+      _Float16 r16[RPW];
+      half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
+      constexpr float LOG2E = 1.44269504088896340736f;
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        float rs = 0.0f;
+#pragma unroll
+        for (int jb = 0; jb < KB; jb++) {
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            half2v const s2 = {static_cast<_Float16>(acc[rp][jb][2 * h]),
+                               static_cast<_Float16>(acc[rp][jb][2 * h + 1])};
+            float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
+            float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
+            half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
+            rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);
+            pk[rp][jb / 2][2 * (jb & 1) + h] = __builtin_bit_cast(uint32_t, e2);
+          }
+        }
+        rs += __shfl_xor(rs, 16, 64);
+        rs += __shfl_xor(rs, 32, 64);
+        r16[rp] = static_cast<_Float16>(rs);
+        if (HAS_DIV) {
+          float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16[rp]));
+#pragma unroll
+          for (int jj = 0; jj < KB / 2; jj++) {
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              half2v const e2 = __builtin_bit_cast(half2v, pk[rp][jj][w]);
+              half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
+                                 static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+              pk[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
+            }
+          }
+        }
+      }
+      float4v o[RPW][DB];
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int t = 0; t < DB; t++) {
+          o[rp][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < KB / 2; jj++) {
 #pragma unroll
         for (int t = 0; t < DB; t++) {
 #pragma unroll
-          for (int r = 0; r < 4; r++) {
-            oacc[t][r] = static_cast<_Float16>(static_cast<float>(oacc[t][r]) + static_cast<float>(o16[t][r]));
+          for (int rp = 0; rp < RPW; rp++) {
+            // V^T as the first operand: the product comes out transposed, which leaves a lane
+            // with four consecutive columns of one row, o[rp][t][r] = O[row c][16t + 4g + r]
+            uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
+            o[rp][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb[t][jj], __builtin_bit_cast(half8, a),
+                                                              o[rp][t], 0, 0, 0);
           }
         }
-        if (!HAS_DIV) {
-          racc = static_cast<_Float16>(static_cast<float>(racc) + static_cast<float>(r16));
+      }
+      if (NBUF == 2 && j + 2 < nit) {
+        // every operand of this buffer is in registers: the loads of iteration j + 2 go out
+        // behind those of iteration j + 1
+        fetch(ip + (j + 2) * IP, b);
+      }
+      if (NBUF == 1 && j + 1 < nit) {
+        fetch(ip + (j + 1) * IP, 0);
+      }
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int t = 0; t < DB; t++) {
+          half2v const lo = {static_cast<_Float16>(o[rp][t][0]), static_cast<_Float16>(o[rp][t][1])};
+          half2v const hi = {static_cast<_Float16>(o[rp][t][2]), static_cast<_Float16>(o[rp][t][3])};
+          keep[j][rp][2 * t] = __builtin_bit_cast(uint32_t, lo);
+          keep[j][rp][2 * t + 1] = __builtin_bit_cast(uint32_t, hi);
         }
+        half2v const rr = {r16[rp], (_Float16)0.0f};
+        keep[j][rp][2 * DB] = __builtin_bit_cast(uint32_t, rr);
       }
     }
+  }
+  if (TRACE) {
+    t_computed = __builtin_amdgcn_s_memrealtime();
+  }
+  // ---- results to LDS: iteration it = ip + j IP goes to slot j of this wavefront's buffers --
 #pragma unroll
-    for (int t = 0; t < DB; t++) {
+  for (int j = 0; j < NIT; j++) {
+    if (j < nit) {
+      _Float16 *slot = wbuf + j * SLOT_HALFS;
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        ow[(4 * g + r) * LDO + 16 * t + c] = oacc[t][r];
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int t = 0; t < DB; t++) {
+          uint2v const w = {keep[j][rp][2 * t], keep[j][rp][2 * t + 1]};
+          *reinterpret_cast<uint2v *>(slot + (16 * rp + c) * LDO + 16 * t + 4 * g) = w;
+        }
+        if (g == 0) {
+          slot[ROWS * LDO + 16 * rp + c] = __builtin_bit_cast(half2v, keep[j][rp][2 * DB])[0];
+        }
       }
     }
   }
   __syncthreads();
-  if (ip == 0) {
-    _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
-                   tile_offset(P.o, bx, by, bz, 0) + (long long)row_base * P.o.d_cols;
-    constexpr int CH = DV / 8;
-    for (int e = lane; e < 16 * CH; e += 64) {
-      int rr = e / CH, cc = (e % CH) * 8;
-      *reinterpret_cast<uint4v *>(og + (long long)rr * P.o.d_cols + cc) =
-          *reinterpret_cast<uint4v const *>(ow + rr * LDO + cc);
+  if (TRACE) {
+    t_joined = __builtin_amdgcn_s_memrealtime();
+  }
+  // ---- ordered accumulation: every thread owns EPT consecutive columns of one row; the
+  // slots of up to four iterations are read before their (dependent) adds ---------------
+  {
+    float acc[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; e++) {
+      acc[e] = 0.0f;  // holds an fp16 value between the adds
     }
-    if (!HAS_DIV && g == 0) {
+    _Float16 const *all = reinterpret_cast<_Float16 const *>(lds) + out_row * LDO + out_col;
+    auto slot_of = [&](int it) { return all + (it % IP) * WAVE_HALFS + (it / IP) * SLOT_HALFS; };
+    // (a slot no iteration filled holds whatever the tiles left there: it is read, never added)
+    constexpr int BATCH = NIT == 1 ? IP : 4;
+    int const it_end = NIT == 1 ? IP : F;
+#pragma unroll
+    for (int it0 = 0; it0 < it_end; it0 += BATCH) {
+      half2v v[BATCH][EPT / 2];
+#pragma unroll
+      for (int u = 0; u < BATCH; u++) {
+        _Float16 const *src = slot_of(NIT == 1 ? it0 + u : (it0 + u < F ? it0 + u : 0));
+#pragma unroll
+        for (int e = 0; e < EPT / 2; e++) {
+          v[u][e] = *reinterpret_cast<half2v const *>(src + 2 * e);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < BATCH; u++) {
+        if (it0 + u < F) {
+#pragma unroll
+          for (int e = 0; e < EPT / 2; e++) {
+            acc[2 * e] = static_cast<float>(static_cast<_Float16>(acc[2 * e] + static_cast<float>(v[u][e][0])));
+            acc[2 * e + 1] = static_cast<float>(static_cast<_Float16>(acc[2 * e + 1] + static_cast<float>(v[u][e][1])));
+          }
+        }
+      }
+    }
+    if (out_row < rows) {
+      half2v out[EPT / 2];
+#pragma unroll
+      for (int e = 0; e < EPT / 2; e++) {
+        out[e] = half2v{static_cast<_Float16>(acc[2 * e]), static_cast<_Float16>(acc[2 * e + 1])};
+      }
+      if (EPT == 8) {
+        uint4v const w = {__builtin_bit_cast(uint32_t, out[0]), __builtin_bit_cast(uint32_t, out[1]),
+                          __builtin_bit_cast(uint32_t, out[(EPT / 2 > 2) ? 2 : 0]),
+                          __builtin_bit_cast(uint32_t, out[(EPT / 2 > 3) ? 3 : 0])};
+        *reinterpret_cast<uint4v *>(og) = w;
+      } else if (EPT == 4) {
+        uint2v const w = {__builtin_bit_cast(uint32_t, out[0]),
+                          __builtin_bit_cast(uint32_t, out[(EPT / 2 > 1) ? 1 : 0])};
+        *reinterpret_cast<uint2v *>(og) = w;
+      } else {
+        *reinterpret_cast<uint32_t *>(og) = __builtin_bit_cast(uint32_t, out[0]);
+      }
+    }
+    if (!HAS_DIV && tid < rows) {
+      _Float16 const *sums = reinterpret_cast<_Float16 const *>(lds) + ROWS * LDO + tid;
+      float ra = 0.0f;
+      for (int it = 0; it < F; it++) {
+        _Float16 const v = sums[(it % IP) * WAVE_HALFS + (it / IP) * SLOT_HALFS];
+        ra = static_cast<float>(static_cast<_Float16>(ra + static_cast<float>(v)));
+      }
       _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
                       tile_offset(P.r, bx, by, bz, 0);
-      rgp[(long long)(row_base + c) * P.r.d_cols] = racc;
+      rgp[(long long)(row_base + tid) * P.r.d_cols] = static_cast<_Float16>(ra);
     }
   }
-}
-
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
-int launch_direct_one(AttnParams const &A, dim3 grid, int lds) {
-  auto *fn = attn_direct_kernel<D, NK, DV, HAS_DIV, RG, IP>;
-  static std::atomic<int> granted{0};  // per instantiation
-  if (lds > 65536 && lds > granted) {
-    MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
-    granted = state().max_lds;
+  if (TRACE && lane == 0) {
+    // start, loads issued, first tile pair landed, arithmetic done, joined, stores issued
+    unsigned const wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    unsigned long long *t = P.trace + ((size_t)wg * IP + ip) * 6;
+    t[0] = t_start;
+    t[1] = t_issued;
+    t[2] = t_landed;
+    t[3] = t_computed;
+    t[4] = t_joined;
+    t[5] = __builtin_amdgcn_s_memrealtime();
   }
-  fn<<<grid, 64 * RG * IP, lds, state().stream()>>>(A);
-  MI355_HIP(hipGetLastError());
-  return 1;
 }
 
-// 64 / 64 / 64 tiles only; 0: no instantiation for these wavefront counts
+template <bool HAS_DIV, int IP, int RPW, int NBUF, int NIT>
+int launch_direct_one(AttnParams const &A, dim3 grid, int lds) {
+  auto go = [&](auto *fn) -> int {
+    static std::atomic<int> granted{0};  // per instantiation
+    if (lds > 65536 && lds > granted) {
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, state().max_lds));
+      granted = state().max_lds;
+    }
+    fn<<<grid, 64 * IP, lds, state().stream()>>>(A);
+    MI355_HIP(hipGetLastError());
+    return 1;
+  };
+  if (A.trace != nullptr) {
+    return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, true>);
+  }
+  return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, false>);
+}
+
+// 64 / 64 / 64 tiles only.  `ip` wavefronts of `rpw` row groups each, `nbuf` tile pairs per
+// wavefront, up to `nit` iterations per wavefront; 0: no instantiation.
 template <bool HAS_DIV>
-int launch_direct(AttnParams const &A, dim3 grid, int rg, int ip, int lds) {
-  switch (rg * 16 + ip) {
-    case 1 * 16 + 2: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 2>(A, grid, lds);
-    case 1 * 16 + 4: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 4>(A, grid, lds);
-    case 1 * 16 + 8: return launch_direct_one<64, 64, 64, HAS_DIV, 1, 8>(A, grid, lds);
+int launch_direct(AttnParams const &A, dim3 grid, int ip, int rpw, int nbuf, int nit, int lds) {
+  switch (ip * 1000 + rpw * 100 + nbuf * 10 + nit) {
+    case 2111: return launch_direct_one<HAS_DIV, 2, 1, 1, 1>(A, grid, lds);
+    case 4111: return launch_direct_one<HAS_DIV, 4, 1, 1, 1>(A, grid, lds);
+    case 8111: return launch_direct_one<HAS_DIV, 8, 1, 1, 1>(A, grid, lds);
+    case 4211: return launch_direct_one<HAS_DIV, 4, 2, 1, 1>(A, grid, lds);
+    case 4122: return launch_direct_one<HAS_DIV, 4, 1, 2, 2>(A, grid, lds);
+    case 4124: return launch_direct_one<HAS_DIV, 4, 1, 2, 4>(A, grid, lds);
+    case 4128: return launch_direct_one<HAS_DIV, 4, 1, 2, 8>(A, grid, lds);
+    case 8112: return launch_direct_one<HAS_DIV, 8, 1, 1, 2>(A, grid, lds);
+    case 8114: return launch_direct_one<HAS_DIV, 8, 1, 1, 4>(A, grid, lds);
     default: return 0;
   }
 }
@@ -1261,6 +1458,26 @@ int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds)
 
 }  // namespace
 
+// Fills the division magics decode_block uses for this launch grid; false when an id times an
+// extent could leave 32 bits (the magics are exact only below that).
+static bool set_grid_magics(AttnParams &A, dim3 grid) {
+  unsigned const ext[3] = {grid.x, grid.y, grid.z};
+  unsigned long long const total = (unsigned long long)grid.x * grid.y * grid.z;
+  for (int i = 0; i < 3; i++) {
+    unsigned const e = ext[A.perm[i]];
+    if (total * e >= (1ull << 32)) {
+      return false;
+    }
+    A.perm_ext[i] = e;
+    A.perm_magic[i] = fast_div_magic((int)e);
+  }
+  if ((unsigned long long)grid.x * (unsigned)A.split >= (1ull << 32)) {
+    return false;
+  }
+  A.split_magic = fast_div_magic(A.split);
+  return true;
+}
+
 static bool shape_supported(Match const &M) {
   return (M.D == 64 && M.DV == 64 && (M.NK == 64 || M.NK == 128 || M.NK == 256)) ||
          (M.D == 128 && M.DV == 128 && M.NK == 64);
@@ -1284,6 +1501,8 @@ int try_launch_attention(DevProgram const &P) {
   A.o = tile_addr(P.ops[M.out_o], P.out[P.ops[M.out_o].io]);
   A.r = M.out_r >= 0 ? tile_addr(P.ops[M.out_r], P.out[P.ops[M.out_r].io]) : A.o;
   A.forloop_range = P.forloop_range;
+  A.rows = M.m < 16 ? M.m : 16;
+  A.trace = nullptr;
   {
     // grid dims the K / V tiles do not depend on vary fastest in the workgroup id
     int n = 0;
@@ -1325,6 +1544,9 @@ int try_launch_attention(DevProgram const &P) {
       lds = lds > out_bytes ? lds : out_bytes;
       if (lds <= s.max_lds && (long long)P.grid[0] * A.split <= 2147483647LL) {
         dim3 grid(P.grid[0] * A.split, P.grid[1], P.grid[2]);
+        if (!set_grid_magics(A, grid)) {
+          return 0;
+        }
         int rc = M.D == 64 ? launch_stream<64, 64, 64>(A, M.has_div, grid, rgs, lds)
                            : launch_stream<128, 64, 128>(A, M.has_div, grid, rgs, lds);
         if (rc == 1) {
@@ -1342,7 +1564,7 @@ int try_launch_attention(DevProgram const &P) {
   // Row groups per workgroup: up to 4, fewer when that is what it takes to put a
   // workgroup on every compute unit.  Iteration lanes: whatever is left of 8
   // wavefronts, at most the for-loop range.
-  int const groups = M.m / 16;
+  int const groups = (M.m + 15) / 16;
   int rg = groups % 4 == 0 ? 4 : (groups % 2 == 0 ? 2 : 1);
   long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
   while (rg > 1 && blocks * (groups / rg) < 256) {
@@ -1378,27 +1600,63 @@ int try_launch_attention(DevProgram const &P) {
   dim3 grid(P.grid[0] * A.split, P.grid[1], P.grid[2]);
   int const nw = rg * ip;
   int rc = 0;
-  // every iteration on a wavefront of its own and tiles of 64 x 64: the variant that streams
-  // the tiles straight into LDS (attention mode 3 keeps the register-transposed staging)
-  // (one row group per workgroup there: nothing is shared between row groups, and smaller
-  // workgroups start sooner; C2: 5.28 us against 5.38 with two)
-  int const direct_lds = ip * stage_bytes + 16 * (M.DV + 8) * 2 + (ip - 1) * (M.DV / 8 + 1) * 64 * 4;
-  if (M.D == 64 && M.NK == 64 && M.DV == 64 && P.forloop_range <= ip && ip > 1 &&
-      direct_lds <= s.max_lds && s.attention_mode != 3 &&
+  // Tiles of 64 x 64 x 64 take the direct-staging variant (attention mode 3 keeps the
+  // register-transposed staging) in two cases.
+  // (a) Every iteration has a wavefront of its own (F <= 4 or 8 lanes).  A wavefront takes
+  //     two row groups when that still puts a workgroup on every compute unit: each K / V
+  //     operand read from LDS then feeds two MFMAs, and half as many wavefronts stream the
+  //     tiles (C2: 256 workgroups of 4 wavefronts x 32 rows; the L2 -> LDS traffic and the
+  //     LDS reads, both per-CU bandwidth limits at this size, halve).
+  // (b) A single row group (decode: 8 or 16 query rows) with a longer for-loop: eight
+  //     wavefronts that each stream every eighth iteration through a tile pair of their own,
+  //     or (DIRECT_LANES = 4) four wavefronts with two tile pairs each.
+  if (M.D == 64 && M.NK == 64 && M.DV == 64 && s.attention_mode != 3 &&
       (long long)P.grid[0] * groups <= 2147483647LL) {
-    AttnParams B = A;
-    B.split = groups;
-    dim3 const direct_grid(P.grid[0] * B.split, P.grid[1], P.grid[2]);
-    rc = M.has_div ? launch_direct<true>(B, direct_grid, 1, ip, direct_lds)
-                   : launch_direct<false>(B, direct_grid, 1, ip, direct_lds);
-    if (rc == 1) {
-      s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
-      s.last().workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
-      s.last().threads = ip * 64;
-      s.last().lds_bytes = direct_lds;
-      s.last().row_split = B.split;
-      return rc;
+    int const F = P.forloop_range;
+    int dip = 0, rpw = 1, nbuf = 1, nit = 1;
+    if (F <= ip && ip > 1) {
+      dip = ip;
+      if (dip == 4 && groups % 2 == 0 && blocks * (groups / 2) >= 256 && s.direct_lanes != 1) {
+        rpw = 2;
+      }
+    } else if (groups == 1 && F > 1) {
+      int const per8 = (F + 7) / 8, per4 = (F + 3) / 4;
+      if (s.direct_lanes != 4 && per8 <= 4) {
+        dip = 8;
+        nit = per8 <= 1 ? 1 : (per8 <= 2 ? 2 : 4);
+      } else if (per4 <= 8) {
+        dip = 4;
+        nbuf = 2;
+        nit = per4 <= 2 ? 2 : (per4 <= 4 ? 4 : 8);
+      }
     }
+    int const direct_lds = dip * (nbuf * stage_bytes + rpw * 16 * M.D * 2);  // + a Q tile per wavefront
+    if (dip > 0 && direct_lds <= s.max_lds) {
+      AttnParams B = A;
+      B.split = groups / rpw;
+      B.trace = s.phase_trace;
+      dim3 const direct_grid(P.grid[0] * B.split, P.grid[1], P.grid[2]);
+      if (!set_grid_magics(B, direct_grid)) {
+        return 0;
+      }
+      if (B.trace != nullptr &&
+          (size_t)direct_grid.x * direct_grid.y * direct_grid.z * dip * 6 * 8 > s.phase_trace_bytes) {
+        B.trace = nullptr;
+      }
+      rc = M.has_div ? launch_direct<true>(B, direct_grid, dip, rpw, nbuf, nit, direct_lds)
+                     : launch_direct<false>(B, direct_grid, dip, rpw, nbuf, nit, direct_lds);
+      if (rc == 1) {
+        s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
+        s.last().workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
+        s.last().threads = dip * 64;
+        s.last().lds_bytes = direct_lds;
+        s.last().row_split = B.split;
+        return rc;
+      }
+    }
+  }
+  if (!set_grid_magics(A, grid)) {
+    return 0;
   }
   if (rc == 1) {
   } else if (M.D == 64 && M.NK == 64) {

@@ -81,6 +81,12 @@ struct State {
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
   int fp_vector_dot_only = 0;  // 1: fingerprint matmuls never take the matrix-core kernels
   int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
+  int direct_lanes = 0;      // MI355_OPT_DIRECT_LANES
+  // phase timestamps of the direct-staging attention kernel (MI355_OPT_PHASE_TRACE): while
+  // set, launches of that kernel record six wall-clock stamps per wavefront here
+  unsigned long long *phase_trace = nullptr;        // null while tracing is off
+  unsigned long long *phase_trace_store = nullptr;  // the allocation (first use of the option)
+  size_t phase_trace_bytes = 0;
   // fused-kernel workspace: fp16 range sums of split for-loops
   // (each queue has its own slice of scratch_base, so concurrent queues never share)
   size_t scratch_bytes = 0;  // per queue

@@ -177,6 +177,9 @@ extern "C" int mi355_shutdown(void) {
   MI355_HIP(hipFree(s.scratch_base));
   MI355_HIP(hipFree(s.planes_base));
   s.planes_base = nullptr;
+  if (s.phase_trace_store != nullptr) {
+    MI355_HIP(hipFree(s.phase_trace_store));
+  }
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     for (int b = 0; b < State::kBatchSlots; b++) {
       MI355_HIP(hipHostFree(s.batch[q][b].host));
@@ -260,6 +263,20 @@ extern "C" int mi355_set_option(int option, int value) {
   }
   if (option == MI355_OPT_FP_MATMUL_ROUTE && (value == 0 || value == 1)) {
     state().fp_vector_dot_only = value;
+    return MI355_OK;
+  }
+  if (option == MI355_OPT_DIRECT_LANES && (value == 0 || value == 1 || value == 4)) {
+    state().direct_lanes = value;
+    return MI355_OK;
+  }
+  if (option == MI355_OPT_PHASE_TRACE && (value == 0 || value == 1)) {
+    MI355_REQUIRE_INIT();
+    State &s = state();
+    if (value == 1 && s.phase_trace_store == nullptr) {
+      s.phase_trace_bytes = (size_t)8 << 20;
+      MI355_HIP(hipMalloc(reinterpret_cast<void **>(&s.phase_trace_store), s.phase_trace_bytes));
+    }
+    s.phase_trace = value == 1 ? s.phase_trace_store : nullptr;
     return MI355_OK;
   }
   return fail(MI355_ERR_INVALID, "unknown option %d", option);
@@ -386,6 +403,19 @@ extern "C" int mi355_timer_stop(float *ms) {
   MI355_HIP(hipEventRecord(state().ev1[tls_queue], state().stream()));
   MI355_HIP(hipEventSynchronize(state().ev1[tls_queue]));
   MI355_HIP(hipEventElapsedTime(ms, state().ev0[tls_queue], state().ev1[tls_queue]));
+  return MI355_OK;
+}
+
+extern "C" int mi355_phase_trace_read(unsigned long long *stamps, size_t count) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  if (stamps == nullptr || s.phase_trace_store == nullptr || count * 8 > s.phase_trace_bytes) {
+    return fail(MI355_ERR_INVALID, "no trace buffer, or more stamps asked for than it holds");
+  }
+  if (int rc = sync_all_queues()) {
+    return rc;
+  }
+  MI355_HIP(hipMemcpy(stamps, s.phase_trace_store, count * 8, hipMemcpyDeviceToHost));
   return MI355_OK;
 }
 

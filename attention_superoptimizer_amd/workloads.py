@@ -223,6 +223,24 @@ def config2_gqa_decode_long():
     return config2_gqa_decode(groups=32, seq=16384, kv_blocks=16, F=16)
 
 
+def gqa_inc_decode(groups=2, rows=8, seq=4096, kv_blocks=16, F=4):
+    """The reference's GQA incremental-decode plan (cpp_examples/group_query_attn_inc_decode.cc:
+    47-101: Q[2,8,64], grid (2,16,1), for-loop 4; op1 accumulates numerator and denominator per
+    KV block, op2 folds the KV blocks and divides), with its sizes as arguments: 8 query rows
+    against a long key range is the bandwidth-bound decode case (about 8 flop per byte)."""
+    q = [groups, rows, 64]
+    k, v = [groups, 64, seq], [groups, seq, 64]
+    g = attention_two_stage(q, k, v, (0, -1, -1), (0, 2, -1), (groups, kv_blocks, 1), F,
+                            (0, -1, -1), (groups, 1, 1))
+    return g, attention_reference(q, k, v)
+
+
+def gqa_inc_decode_long():
+    """64 kv-head groups x 8 query rows x 16,384 cached keys (K and V 134 MB each): the
+    reference's incremental-decode plan at a size where the launch no longer dominates."""
+    return gqa_inc_decode(groups=64, rows=8, seq=16384, kv_blocks=16, F=16)
+
+
 def config3_mha_prefill(heads=32, seq=2048, hd=128, q_split=16, kv_split=1, F=32, rows2=32):
     """MHA prefill, non-causal: op1 accumulates exp(QK^T)V and rowsum(exp(QK^T))
     over a seq-tiled for-loop per (head, kv block, q block); op2 folds the kv
@@ -315,6 +333,7 @@ BASELINE_CONFIGS = {
 # the same plans at other sizes (reported beside the baseline configurations, not instead)
 SCALED_CONFIGS = {
     "C2_gqa_decode_long": config2_gqa_decode_long,
+    "gqa_inc_decode_long": gqa_inc_decode_long,
 }
 
 # fp16 input distributions per config (std of N(0, std)), keyed by input op index
@@ -322,6 +341,7 @@ INPUT_STD = {
     "C1_fused_matmul": {0: 0.1, 1: 0.1},
     "C2_gqa_decode": {0: 0.125, 1: 0.125, 2: 0.125},
     "C2_gqa_decode_long": {0: 0.125, 1: 0.125, 2: 0.125},
+    "gqa_inc_decode_long": {0: 0.125, 1: 0.125, 2: 0.125},
     "C3_mha_prefill": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
     # the configurations leave X's distribution open; N(0, 0.25) keeps every partial
     # sum below 2, where one fp16 ulp is still under the 1e-3 absolute tolerance

@@ -112,6 +112,18 @@ typedef struct mi355_launch_info {
  * take the int8 matrix-core kernels whenever their shapes allow (default); 1 = always the
  * packed 4 x 8-bit vector-dot kernels.  Results are bit-identical; tests run both. */
 #define MI355_OPT_FP_MATMUL_ROUTE 4
+/* PHASE_TRACE: 1 = launches of the direct-staging attention kernel record six wall-clock
+ * stamps (100 MHz) per wavefront -- start, loads issued, first tiles landed, arithmetic done,
+ * joined, stores issued -- read back with mi355_phase_trace_read; 0 = off (default).  A
+ * measurement aid: the traced kernel is a separate instantiation, the normal one carries no
+ * trace code. */
+#define MI355_OPT_PHASE_TRACE 5
+/* DIRECT_LANES: shape of the direct-staging attention kernel.  0 = chosen by the backend
+ * (default: wavefronts of two row groups where that still fills the chip; eight
+ * single-buffered iteration lanes for a lone row group with a long for-loop); 1 = one row
+ * group per wavefront always; 4 = four double-buffered lanes for a lone row group.  Results
+ * are identical; a measurement knob that the tests use to cover every instantiation. */
+#define MI355_OPT_DIRECT_LANES 6
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor
@@ -284,6 +296,9 @@ int mi355_customized_profile(mi355_plan const *plan, void const *const *inputs,
                              float *ms);
 /* What the last mi355_customized_{fp,run,profile} call launched. */
 int mi355_last_launch(mi355_launch_info *info);
+/* Copies the first `count` 64-bit stamps the last traced launch wrote (blocking):
+ * wavefront w of workgroup g (linear block index) is at [(g * wavefronts + w) * 6 .. + 5]. */
+int mi355_phase_trace_read(unsigned long long *stamps, size_t count);
 
 /* init_input<half>, src/kernel/cuda/input_kernel.cu:29-54: x[i] = (half)(i % last_dim) */
 int mi355_f16_fill_iota(void *x, size_t n, int last_dim);

@@ -196,10 +196,58 @@ def test_reference_examples_f16(rt, path):
         spec, ref = W.REFERENCE_EXAMPLES[name]
         ins = _inputs(spec, 0.05, 60)
         _check(rt, spec, ins, name)
-        # query tiles with a multiple of 16 rows take the fused kernel (8-row tiles do not)
-        if path == "fused" and name in ("group_query_attn_spec_decode", "multi_head_attn_inc_decode",
-                                        "multi_head_attn_prefill", "multi_query_attn_inc_decode", "dnn"):
-            assert _last_kernels[0] == KERNEL_ATTENTION, name
+        # every attention plan takes the fused kernel, the 8-row decode tile included (padded
+        # with zero rows)
+        if path == "fused" and name in ("group_query_attn_inc_decode", "group_query_attn_spec_decode",
+                                        "multi_head_attn_inc_decode", "multi_head_attn_prefill",
+                                        "multi_query_attn_inc_decode", "dnn"):
+            assert _last_kernels[0] == KERNEL_ATTENTION, (name, _last_kernels)
+
+
+@pytest.mark.parametrize("rows,F,kv_blocks,lanes", [
+    (8, 4, 16, 0),     # the reference's plan: one iteration per wavefront
+    (8, 8, 4, 0),      # two iterations per wavefront, two tile pairs in flight
+    (8, 16, 2, 0),     # four
+    (16, 16, 2, 0),    # a full row group
+    (8, 19, 1, 0),     # uneven: wavefronts with five and four iterations
+    (8, 30, 1, 0),     # eight lanes, up to four iterations each
+    (8, 16, 2, 4),     # four lanes with two tile pairs each, by request
+    (8, 30, 1, 4),     # ... eight iterations per lane
+    (8, 40, 1, 0),     # too long for the direct variant: register-transposed staging
+    (16, 3, 2, 0),     # fewer iterations than lanes
+])
+def test_decode_row_groups_on_the_direct_staging_kernel(rt, abi, rows, F, kv_blocks, lanes):
+    """8- and 16-row query tiles (incremental decode) against a for-loop of any length: the
+    looped direct-staging kernel, both forms (two outputs + combine; single op with div),
+    against the golden.  Also on the register-transposed variant (attention mode 3)."""
+    from attention_superoptimizer_amd import workloads as W
+    seq = 64 * F * kv_blocks
+    spec, _ = W.gqa_inc_decode(groups=3, rows=rows, seq=seq, kv_blocks=kv_blocks, F=F)
+    single, _ = W.config2_gqa_decode(groups=3, rows=rows, seq=seq, kv_blocks=kv_blocks, F=F)
+    assert abi.mi355_set_option(6, lanes) == 0
+    try:
+        for what, sp in (("two-stage", spec), ("single op", single)):
+            ins = _inputs(sp, 0.125, 200 + F)
+            _check(rt, sp, ins, f"decode {what} rows {rows} F {F}")
+            assert _last_kernels[0] == KERNEL_ATTENTION, (what, _last_kernels)
+            info = N_launch_info()
+        assert abi.mi355_set_option(2, 3) == 0
+        try:
+            ins = _inputs(spec, 0.125, 300 + F)
+            _check(rt, spec, ins, f"decode rows {rows} F {F}, register-transposed variant")
+            assert _last_kernels[0] == KERNEL_ATTENTION
+        finally:
+            assert abi.mi355_set_option(2, 0) == 0
+    finally:
+        assert abi.mi355_set_option(6, 0) == 0
+
+
+def N_launch_info():
+    import ctypes
+    from attention_superoptimizer_amd import _native as N
+    info = N.Mi355LaunchInfo()
+    N.backend().mi355_last_launch(ctypes.byref(info))
+    return info
 
 
 def test_gqa_fixture_graphs_f16(rt, path):
@@ -244,17 +292,20 @@ def test_attention_latency_variants_agree(rt, abi):
     for spec, stds, what in cases:
         ins = _inputs(spec, stds, 95)
         outs = {}
-        for mode in (0, 3):
-            assert abi.mi355_set_option(2, mode) == 0
+        # (attention mode, direct-lanes knob): streamed with two row groups per wavefront where
+        # the size allows, streamed with one, register-transposed
+        for mode, lanes in ((0, 0), (0, 1), (3, 0)):
+            assert abi.mi355_set_option(2, mode) == 0 and abi.mi355_set_option(6, lanes) == 0
             try:
-                got = _check(rt, spec, ins, f"{what} mode {mode}")
+                got = _check(rt, spec, ins, f"{what} mode {mode} lanes {lanes}")
                 assert _last_kernels[0] == KERNEL_ATTENTION
-                outs[mode] = [got[i] for i in range(len(spec)) if spec[i]["op"] == "customized"]
+                outs[mode, lanes] = [got[i] for i in range(len(spec)) if spec[i]["op"] == "customized"]
             finally:
-                assert abi.mi355_set_option(2, 0) == 0
-        for a, b in zip(outs[0], outs[3]):
-            for x, y in zip(a, b):
-                assert np.array_equal(x, y), what
+                assert abi.mi355_set_option(2, 0) == 0 and abi.mi355_set_option(6, 0) == 0
+        for other in ((0, 1), (3, 0)):
+            for a, b in zip(outs[0, 0], outs[other]):
+                for x, y in zip(a, b):
+                    assert np.array_equal(x, y), (what, other)
 
 
 def test_full_size_configs_routes_agree(rt, abi):
