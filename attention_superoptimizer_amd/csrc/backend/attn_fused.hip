@@ -1002,9 +1002,23 @@ __device__ __forceinline__ void wait_vm() {
 }
 #pragma clang diagnostic pop
 
-template <int D, int NK, int DV, bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, bool TRACE>
+// Key tiles of other widths ride on the same 64-key strips.  A wavefront's unit of work is
+// max(one iteration, one strip of 64 keys):
+//   SPI strips per iteration (key tiles of 128 / 256): the strips of an iteration are streamed
+//     one after the other, the row sum and the fp32 P.V accumulators run across them and the
+//     iteration's result is rounded once at its end (form without the division only: the
+//     division needs the whole row sum before the first P.V);
+//   IPS iterations per strip (key tiles of 32 / 16, whose tiles of consecutive iterations lie
+//     side by side in memory -- the host checks the loader strides): one load of 64 keys, then
+//     every 32- or 16-key slice gets its own exp / row sum / [division] / P.V and its own
+//     rounded result.  Slices of 16 keys take the 16 x 16 x 16 matrix instruction.
+template <int D, int NK, int DV, bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, int SPI, int IPS,
+          bool TRACE>
 __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P) {
   static_assert(D == 64 && NK == 64 && DV == 64, "the chunk swizzles assume rows of 128 bytes");
+  static_assert((SPI == 1 || IPS == 1) && (SPI == 1 || SPI == 2 || SPI == 4) &&
+                    (IPS == 1 || IPS == 2 || IPS == 4) && !(HAS_DIV && SPI > 1),
+                "strips per iteration or iterations per strip, not both");
   static_assert(NBUF == 1 || NBUF == 2, "one or two tile pairs per wavefront");
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
   constexpr int KI = D * NK / 8 / 64, VI = NK * DV / 8 / 64;  // direct loads per tile
@@ -1015,7 +1029,8 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   constexpr int WAVE_HALFS = NBUF * PAIR_HALFS + Q_HALFS;
   constexpr int LDO = DV + 4;          // row stride of a result slot (halfs): 8-byte aligned rows
   constexpr int SLOT_HALFS = ROWS * LDO + ROWS;  // one iteration's O tile + its row sums
-  static_assert(NIT * SLOT_HALFS <= NBUF * PAIR_HALFS, "a wavefront's results must fit its own buffers");
+  // (the Q tile is in registers by then, so its region counts)
+  static_assert(NIT * IPS * SLOT_HALFS <= WAVE_HALFS, "a wavefront's results must fit its own buffers");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
   unsigned long long t_start = 0, t_issued = 0, t_landed = 0, t_computed = 0, t_joined = 0;
@@ -1030,7 +1045,8 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   int const row_base = slice * ROWS;
   int const rows = RPW == 1 ? P.rows : ROWS;  // rows that exist (only a lone row group may be short)
   int const F = P.forloop_range;
-  int const nit = ip < F ? (F - ip + IP - 1) / IP : 0;  // iterations of this wavefront
+  int const units = F / IPS;                                     // units of work of the for-loop
+  int const nit = ip < units ? (units - ip + IP - 1) / IP : 0;  // units of this wavefront
 
   _Float16 *const wbuf = reinterpret_cast<_Float16 *>(lds) + ip * WAVE_HALFS;
   uint32_t const lds_w = lds_address(wbuf);
@@ -1046,9 +1062,12 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   uint32_t const k_off_even = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(l3))));
   uint32_t const k_off_odd = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(8 + l3))));
   uint32_t const v_off = 2u * (uint32_t)(l3 * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(l3))));
-  auto fetch = [&](int it, int b) {
-    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
-    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
+  // strip `strip` (64 keys) of unit `unit`: the unit's first iteration names the tile origin
+  auto fetch = [&](int unit, int strip, int b) {
+    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) +
+                         tile_offset(P.k, bx, by, bz, unit * IPS) + 64 * strip;
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) +
+                         tile_offset(P.v, bx, by, bz, unit * IPS) + (long long)(64 * strip) * P.v.d_cols;
     uint32_t const base = lds_w + 2u * (uint32_t)(b * PAIR_HALFS);
 #pragma unroll
     for (int i = 0; i < KI; i++) {
@@ -1074,10 +1093,12 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       uint32_t const off = 2u * (uint32_t)((r < rows ? r : 0) * P.q.d_cols + 8 * pos);
       lds_dma16(qg, off, lds_w + 2u * (uint32_t)(NBUF * PAIR_HALFS) + 1024u * (uint32_t)i);
     }
-    fetch(ip, 0);
+    fetch(ip, 0, 0);
   }
-  if (NBUF == 2 && nit > 1) {
-    fetch(ip + IP, 1);
+  // strips of this wavefront in the order it walks them: q = j * SPI + s (unit ip + j IP)
+  int const nstrips = nit * SPI;
+  if (NBUF == 2 && nstrips > 1) {
+    fetch(ip + (1 / SPI) * IP, 1 % SPI, 1);
   }
   if (TRACE) {
     t_issued = __builtin_amdgcn_s_memrealtime();
@@ -1097,19 +1118,22 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
 
   // results of this wavefront's iterations, packed fp16: keep[j][rp][2t], [2t+1] =
   // O[row 16rp + c][16t + 4g + r] for r = 0,1 / 2,3; keep[j][rp][2 DB] = the row sum of row c
-  uint32_t keep[NIT][RPW][2 * DB + 1];
+  uint32_t keep[NIT][IPS][RPW][2 * DB + 1];
+  float4v o[RPW][DB];  // P.V accumulators of the iteration in progress (SPI > 1: across strips)
+  float rs_run[RPW];   // its running row sums
 #pragma unroll
-  for (int j = 0; j < NIT; j++) {
-    if (j < nit) {
-      int const b = NBUF == 2 ? (j & 1) : 0;
+  for (int q = 0; q < NIT * SPI; q++) {
+    int const j = q / SPI, sidx = q % SPI;
+    if (q < nstrips) {
+      int const b = NBUF == 2 ? (q & 1) : 0;
       // the tile pair of iteration j (and everything older) has landed when at most the next
       // pair's loads are outstanding
-      if (NBUF == 2 && j + 1 < nit) {
+      if (NBUF == 2 && q + 1 < nstrips) {
         wait_vm<KI + VI>();
       } else {
         wait_vm<0>();
       }
-      if (j == 0) {
+      if (q == 0) {
         // Q fragments (B operand of S^T): Q[row c][32kk + 8g .. +7]
         _Float16 const *ql = wbuf + NBUF * PAIR_HALFS + c * D + 8 * g;
 #pragma unroll
@@ -1176,15 +1200,17 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      // exp of every 16-key block, packed fp16 as the next matrix instruction wants it, and
+      // the blocks' row-sum parts (each lane: its four keys of the block)
       uint32_t pk[RPW][KB / 2][4];
-      _Float16 r16[RPW];
+      float rsb[RPW][KB];
       half2v const ones = {(_Float16)1.0f, (_Float16)1.0f};
       constexpr float LOG2E = 1.44269504088896340736f;
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
-        float rs = 0.0f;
 #pragma unroll
         for (int jb = 0; jb < KB; jb++) {
+          float part = 0.0f;
 #pragma unroll
           for (int h = 0; h < 2; h++) {
             half2v const s2 = {static_cast<_Float16>(acc[rp][jb][2 * h]),
@@ -1192,68 +1218,146 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
             float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
             float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
             half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
-            rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);
+            part = __builtin_amdgcn_fdot2(e2, ones, part, false);
             pk[rp][jb / 2][2 * (jb & 1) + h] = __builtin_bit_cast(uint32_t, e2);
           }
+          rsb[rp][jb] = part;
         }
+      }
+      // row sum of a slice (blocks jb0 .. jb0 + nb - 1 plus `carry`) over the four lane groups
+      auto row_sum = [&](int rp, int jb0, int nb, float carry) {
+        float rs = carry;
+#pragma unroll
+        for (int x = 0; x < KB; x++) {
+          if (x >= jb0 && x < jb0 + nb) {
+            rs += rsb[rp][x];
+          }
+        }
+        return rs;
+      };
+      auto across = [&](float rs) {
         rs += __shfl_xor(rs, 16, 64);
         rs += __shfl_xor(rs, 32, 64);
-        r16[rp] = static_cast<_Float16>(rs);
-        if (HAS_DIV) {
-          float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16[rp]));
+        return rs;
+      };
+      auto normalise = [&](int rp, int w0, int nw, _Float16 r16) {
+        float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
 #pragma unroll
-          for (int jj = 0; jj < KB / 2; jj++) {
+        for (int w = 0; w < 4 * (KB / 2); w++) {
+          if (w >= w0 && w < w0 + nw) {
+            half2v const e2 = __builtin_bit_cast(half2v, pk[rp][w / 4][w % 4]);
+            half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
+                               static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+            pk[rp][w / 4][w % 4] = __builtin_bit_cast(uint32_t, p2);
+          }
+        }
+      };
+      auto store_result = [&](int sub, int rp, float4v const (&res)[DB], _Float16 r16) {
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-              half2v const e2 = __builtin_bit_cast(half2v, pk[rp][jj][w]);
-              half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
-                                 static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
-              pk[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
+        for (int t = 0; t < DB; t++) {
+          half2v const lo = {static_cast<_Float16>(res[t][0]), static_cast<_Float16>(res[t][1])};
+          half2v const hi = {static_cast<_Float16>(res[t][2]), static_cast<_Float16>(res[t][3])};
+          keep[j][sub][rp][2 * t] = __builtin_bit_cast(uint32_t, lo);
+          keep[j][sub][rp][2 * t + 1] = __builtin_bit_cast(uint32_t, hi);
+        }
+        half2v const rr = {r16, (_Float16)0.0f};
+        keep[j][sub][rp][2 * DB] = __builtin_bit_cast(uint32_t, rr);
+      };
+      // V^T is the first operand of every P.V instruction: the product comes out transposed,
+      // which leaves a lane with four consecutive columns of one row,
+      // res[t][r] = O[row c][16t + 4g + r]
+      if (IPS == 1) {
+#pragma unroll
+        for (int rp = 0; rp < RPW; rp++) {
+          rs_run[rp] = row_sum(rp, 0, KB, sidx == 0 ? 0.0f : rs_run[rp]);
+        }
+        _Float16 r16[RPW];
+        if (sidx == SPI - 1) {
+#pragma unroll
+          for (int rp = 0; rp < RPW; rp++) {
+            r16[rp] = static_cast<_Float16>(across(rs_run[rp]));
+            if (HAS_DIV) {
+              normalise(rp, 0, 4 * (KB / 2), r16[rp]);
             }
           }
         }
-      }
-      float4v o[RPW][DB];
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-#pragma unroll
-        for (int t = 0; t < DB; t++) {
-          o[rp][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
-        }
-      }
-#pragma unroll
-      for (int jj = 0; jj < KB / 2; jj++) {
-#pragma unroll
-        for (int t = 0; t < DB; t++) {
+        if (sidx == 0) {
 #pragma unroll
           for (int rp = 0; rp < RPW; rp++) {
-            // V^T as the first operand: the product comes out transposed, which leaves a lane
-            // with four consecutive columns of one row, o[rp][t][r] = O[row c][16t + 4g + r]
-            uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
-            o[rp][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb[t][jj], __builtin_bit_cast(half8, a),
-                                                              o[rp][t], 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < DB; t++) {
+              o[rp][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+          }
+        }
+#pragma unroll
+        for (int jj = 0; jj < KB / 2; jj++) {
+#pragma unroll
+          for (int t = 0; t < DB; t++) {
+#pragma unroll
+            for (int rp = 0; rp < RPW; rp++) {
+              uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
+              o[rp][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb[t][jj], __builtin_bit_cast(half8, a),
+                                                                o[rp][t], 0, 0, 0);
+            }
+          }
+        }
+        if (sidx == SPI - 1) {
+#pragma unroll
+          for (int rp = 0; rp < RPW; rp++) {
+            store_result(0, rp, o[rp], r16[rp]);
+          }
+        }
+      } else if (IPS == 2) {
+        // two iterations of 32 keys: blocks {0, 1} and {2, 3}, one matrix instruction each
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+          for (int rp = 0; rp < RPW; rp++) {
+            _Float16 const r16 = static_cast<_Float16>(across(row_sum(rp, 2 * sub, 2, 0.0f)));
+            if (HAS_DIV) {
+              normalise(rp, 4 * sub, 4, r16);
+            }
+            float4v res[DB];
+            uint4v const a = {pk[rp][sub][0], pk[rp][sub][1], pk[rp][sub][2], pk[rp][sub][3]};
+#pragma unroll
+            for (int t = 0; t < DB; t++) {
+              res[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb[t][sub], __builtin_bit_cast(half8, a),
+                                                              float4v{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            }
+            store_result(sub, rp, res, r16);
+          }
+        }
+      } else {
+        // four iterations of 16 keys: one block each, the 16-deep matrix instruction
+#pragma unroll
+        for (int sub = 0; sub < 4; sub++) {
+#pragma unroll
+          for (int rp = 0; rp < RPW; rp++) {
+            _Float16 const r16 = static_cast<_Float16>(across(row_sum(rp, sub, 1, 0.0f)));
+            if (HAS_DIV) {
+              normalise(rp, 2 * sub, 2, r16);
+            }
+            float4v res[DB];
+            uint2v const a = {pk[rp][sub / 2][2 * (sub & 1)], pk[rp][sub / 2][2 * (sub & 1) + 1]};
+#pragma unroll
+            for (int t = 0; t < DB; t++) {
+              // rows 32 (sub / 2) + 16 (sub & 1) + 4g .. + 3 of V: the low or the high half of
+              // the operand read for the pair of blocks
+              half4 const vh = (sub & 1) ? __builtin_shufflevector(vb[t][sub / 2], vb[t][sub / 2], 4, 5, 6, 7)
+                                         : __builtin_shufflevector(vb[t][sub / 2], vb[t][sub / 2], 0, 1, 2, 3);
+              res[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(vh, __builtin_bit_cast(half4, a),
+                                                             float4v{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            }
+            store_result(sub, rp, res, r16);
           }
         }
       }
-      if (NBUF == 2 && j + 2 < nit) {
-        // every operand of this buffer is in registers: the loads of iteration j + 2 go out
-        // behind those of iteration j + 1
-        fetch(ip + (j + 2) * IP, b);
-      }
-      if (NBUF == 1 && j + 1 < nit) {
-        fetch(ip + (j + 1) * IP, 0);
-      }
-#pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
-#pragma unroll
-        for (int t = 0; t < DB; t++) {
-          half2v const lo = {static_cast<_Float16>(o[rp][t][0]), static_cast<_Float16>(o[rp][t][1])};
-          half2v const hi = {static_cast<_Float16>(o[rp][t][2]), static_cast<_Float16>(o[rp][t][3])};
-          keep[j][rp][2 * t] = __builtin_bit_cast(uint32_t, lo);
-          keep[j][rp][2 * t + 1] = __builtin_bit_cast(uint32_t, hi);
-        }
-        half2v const rr = {r16[rp], (_Float16)0.0f};
-        keep[j][rp][2 * DB] = __builtin_bit_cast(uint32_t, rr);
+      // every operand of this buffer is in registers: the next strip this buffer serves goes
+      // out now (behind the one already in flight when there are two buffers)
+      if (q + NBUF < nstrips) {
+        int const qn = q + NBUF;
+        fetch(ip + (qn / SPI) * IP, qn % SPI, b);
       }
     }
   }
@@ -1264,16 +1368,19 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
 #pragma unroll
   for (int j = 0; j < NIT; j++) {
     if (j < nit) {
-      _Float16 *slot = wbuf + j * SLOT_HALFS;
 #pragma unroll
-      for (int rp = 0; rp < RPW; rp++) {
+      for (int sub = 0; sub < IPS; sub++) {
+        _Float16 *slot = wbuf + (j * IPS + sub) * SLOT_HALFS;
 #pragma unroll
-        for (int t = 0; t < DB; t++) {
-          uint2v const w = {keep[j][rp][2 * t], keep[j][rp][2 * t + 1]};
-          *reinterpret_cast<uint2v *>(slot + (16 * rp + c) * LDO + 16 * t + 4 * g) = w;
-        }
-        if (g == 0) {
-          slot[ROWS * LDO + 16 * rp + c] = __builtin_bit_cast(half2v, keep[j][rp][2 * DB])[0];
+        for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+          for (int t = 0; t < DB; t++) {
+            uint2v const w = {keep[j][sub][rp][2 * t], keep[j][sub][rp][2 * t + 1]};
+            *reinterpret_cast<uint2v *>(slot + (16 * rp + c) * LDO + 16 * t + 4 * g) = w;
+          }
+          if (g == 0) {
+            slot[ROWS * LDO + 16 * rp + c] = __builtin_bit_cast(half2v, keep[j][sub][rp][2 * DB])[0];
+          }
         }
       }
     }
@@ -1291,16 +1398,22 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       acc[e] = 0.0f;  // holds an fp16 value between the adds
     }
     _Float16 const *all = reinterpret_cast<_Float16 const *>(lds) + out_row * LDO + out_col;
-    auto slot_of = [&](int it) { return all + (it % IP) * WAVE_HALFS + (it / IP) * SLOT_HALFS; };
+    // iteration `it` is slice it % IPS of unit it / IPS, which wavefront unit % IP kept as its
+    // result number unit / IP
+    auto slot_of = [&](int it) {
+      int const unit = it / IPS;
+      return all + (unit % IP) * WAVE_HALFS + ((unit / IP) * IPS + it % IPS) * SLOT_HALFS;
+    };
     // (a slot no iteration filled holds whatever the tiles left there: it is read, never added)
-    constexpr int BATCH = NIT == 1 ? IP : 4;
-    int const it_end = NIT == 1 ? IP : F;
+    constexpr bool ALL = NIT == 1 && IPS == 1;  // one slot per wavefront: read them all at once
+    constexpr int BATCH = ALL ? IP : 4;
+    int const it_end = ALL ? IP : F;
 #pragma unroll
     for (int it0 = 0; it0 < it_end; it0 += BATCH) {
       half2v v[BATCH][EPT / 2];
 #pragma unroll
       for (int u = 0; u < BATCH; u++) {
-        _Float16 const *src = slot_of(NIT == 1 ? it0 + u : (it0 + u < F ? it0 + u : 0));
+        _Float16 const *src = slot_of(ALL ? it0 + u : (it0 + u < F ? it0 + u : 0));
 #pragma unroll
         for (int e = 0; e < EPT / 2; e++) {
           v[u][e] = *reinterpret_cast<half2v const *>(src + 2 * e);
@@ -1340,7 +1453,8 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       _Float16 const *sums = reinterpret_cast<_Float16 const *>(lds) + ROWS * LDO + tid;
       float ra = 0.0f;
       for (int it = 0; it < F; it++) {
-        _Float16 const v = sums[(it % IP) * WAVE_HALFS + (it / IP) * SLOT_HALFS];
+        int const unit = it / IPS;
+        _Float16 const v = sums[(unit % IP) * WAVE_HALFS + ((unit / IP) * IPS + it % IPS) * SLOT_HALFS];
         ra = static_cast<float>(static_cast<_Float16>(ra + static_cast<float>(v)));
       }
       _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
@@ -1361,8 +1475,11 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   }
 }
 
-template <bool HAS_DIV, int IP, int RPW, int NBUF, int NIT>
-int launch_direct_one(AttnParams const &A, dim3 grid, int lds) {
+template <bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, int SPI, int IPS>
+int launch_direct_one(AttnParams const &A, dim3 grid, int lds, bool dry) {
+  if (dry) {
+    return 1;  // the question was only whether this shape is built
+  }
   auto go = [&](auto *fn) -> int {
     static std::atomic<int> granted{0};  // per instantiation
     if (lds > 65536 && lds > granted) {
@@ -1374,28 +1491,63 @@ int launch_direct_one(AttnParams const &A, dim3 grid, int lds) {
     MI355_HIP(hipGetLastError());
     return 1;
   };
-  if (A.trace != nullptr) {
-    return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, true>);
+  if (SPI == 1 && IPS == 1 && A.trace != nullptr) {
+    return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, SPI, IPS, SPI == 1 && IPS == 1>);
   }
-  return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, false>);
+  return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, SPI, IPS, false>);
 }
 
-// 64 / 64 / 64 tiles only.  `ip` wavefronts of `rpw` row groups each, `nbuf` tile pairs per
-// wavefront, up to `nit` iterations per wavefront; 0: no instantiation.
+// The shape of a direct-staging launch: `ip` wavefronts of `rpw` row groups each, `nbuf` tile
+// pairs per wavefront, up to `nit` units of work per wavefront, `spi` strips per iteration or
+// `ips` iterations per strip.
+struct DirectShape {
+  int ip = 0, rpw = 1, nbuf = 1, nit = 1, spi = 1, ips = 1;
+  int code() const { return ((((ip * 10 + rpw) * 10 + nbuf) * 10 + nit) * 10 + spi) * 10 + ips; }
+};
+
+// 0: no instantiation for this shape
 template <bool HAS_DIV>
-int launch_direct(AttnParams const &A, dim3 grid, int ip, int rpw, int nbuf, int nit, int lds) {
-  switch (ip * 1000 + rpw * 100 + nbuf * 10 + nit) {
-    case 2111: return launch_direct_one<HAS_DIV, 2, 1, 1, 1>(A, grid, lds);
-    case 4111: return launch_direct_one<HAS_DIV, 4, 1, 1, 1>(A, grid, lds);
-    case 8111: return launch_direct_one<HAS_DIV, 8, 1, 1, 1>(A, grid, lds);
-    case 4211: return launch_direct_one<HAS_DIV, 4, 2, 1, 1>(A, grid, lds);
-    case 4122: return launch_direct_one<HAS_DIV, 4, 1, 2, 2>(A, grid, lds);
-    case 4124: return launch_direct_one<HAS_DIV, 4, 1, 2, 4>(A, grid, lds);
-    case 4128: return launch_direct_one<HAS_DIV, 4, 1, 2, 8>(A, grid, lds);
-    case 8112: return launch_direct_one<HAS_DIV, 8, 1, 1, 2>(A, grid, lds);
-    case 8114: return launch_direct_one<HAS_DIV, 8, 1, 1, 4>(A, grid, lds);
-    default: return 0;
+int launch_direct(AttnParams const &A, dim3 grid, DirectShape const &d, int lds, bool dry = false) {
+#define MI355_DIRECT(IPV, RPWV, NBUFV, NITV, SPIV, IPSV) \
+  case ((((IPV * 10 + RPWV) * 10 + NBUFV) * 10 + NITV) * 10 + SPIV) * 10 + IPSV: \
+    return launch_direct_one<HAS_DIV, IPV, RPWV, NBUFV, NITV, SPIV, IPSV>(A, grid, lds, dry);
+  switch (d.code()) {
+    // one 64-key tile per iteration
+    MI355_DIRECT(2, 1, 1, 1, 1, 1)
+    MI355_DIRECT(4, 1, 1, 1, 1, 1)
+    MI355_DIRECT(8, 1, 1, 1, 1, 1)
+    MI355_DIRECT(4, 2, 1, 1, 1, 1)
+    MI355_DIRECT(4, 1, 2, 2, 1, 1)
+    MI355_DIRECT(4, 1, 2, 4, 1, 1)
+    MI355_DIRECT(4, 1, 2, 8, 1, 1)
+    MI355_DIRECT(8, 1, 1, 2, 1, 1)
+    MI355_DIRECT(8, 1, 1, 4, 1, 1)
+    // key tiles of 32 and 16: two / four iterations per strip
+    MI355_DIRECT(4, 1, 1, 1, 1, 2)
+    MI355_DIRECT(4, 2, 1, 1, 1, 2)
+    MI355_DIRECT(8, 1, 1, 1, 1, 2)
+    MI355_DIRECT(8, 1, 1, 2, 1, 2)
+    MI355_DIRECT(4, 1, 1, 1, 1, 4)
+    MI355_DIRECT(4, 2, 1, 1, 1, 4)
+    MI355_DIRECT(8, 1, 1, 1, 1, 4)
+    default: break;
   }
+  if constexpr (!HAS_DIV) {
+    switch (d.code()) {
+      // key tiles of 128 and 256: two / four strips per iteration (no division inside)
+      MI355_DIRECT(4, 1, 1, 1, 2, 1)
+      MI355_DIRECT(8, 1, 1, 1, 2, 1)
+      MI355_DIRECT(8, 1, 1, 2, 2, 1)
+      MI355_DIRECT(8, 1, 1, 4, 2, 1)
+      MI355_DIRECT(4, 1, 1, 1, 4, 1)
+      MI355_DIRECT(8, 1, 1, 1, 4, 1)
+      MI355_DIRECT(8, 1, 1, 2, 4, 1)
+      MI355_DIRECT(8, 1, 1, 4, 4, 1)
+      default: break;
+    }
+  }
+#undef MI355_DIRECT
+  return 0;
 }
 
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
@@ -1478,19 +1630,97 @@ static bool set_grid_magics(AttnParams &A, dim3 grid) {
   return true;
 }
 
+// Shapes the register-transposed and the throughput variants are built for.
 static bool shape_supported(Match const &M) {
-  return (M.D == 64 && M.DV == 64 && (M.NK == 64 || M.NK == 128 || M.NK == 256)) ||
-         (M.D == 128 && M.DV == 128 && M.NK == 64);
+  return (M.m % 16 == 0 || M.m == 8) &&
+         ((M.D == 64 && M.DV == 64 && (M.NK == 64 || M.NK == 128 || M.NK == 256)) ||
+          (M.D == 128 && M.DV == 128 && M.NK == 64));
+}
+
+// Whether (and in which shape) the direct-staging variant takes the plan: head size 64,
+// key tiles of 16 ... 256 on 64-key strips.
+static bool choose_direct(DevProgram const &P, Match const &M, DirectShape &d, int &lds) {
+  State &s = state();
+  if (M.D != 64 || M.DV != 64 || s.attention_mode == 3 || !(M.m % 16 == 0 || M.m == 8)) {
+    return false;
+  }
+  int const F = P.forloop_range;
+  d = DirectShape{};
+  if (M.NK == 16 || M.NK == 32) {
+    // consecutive iterations' tiles must lie side by side: K advances by NK columns, V by NK rows
+    DevOp const &lk = P.ops[M.k], &lv = P.ops[M.v];
+    d.ips = 64 / M.NK;
+    if (lk.col_fs != M.NK || lk.row_fs != 0 || lk.g_fs != 0 || lv.row_fs != M.NK || lv.col_fs != 0 ||
+        lv.g_fs != 0 || F % d.ips != 0) {
+      return false;
+    }
+  } else if (M.NK == 128 || M.NK == 256) {
+    d.spi = M.NK / 64;
+    if (M.has_div) {
+      return false;
+    }
+  } else if (M.NK != 64) {
+    return false;
+  }
+  int const units = F / d.ips;
+  int const groups = (M.m + 15) / 16;
+  long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
+  auto round_nit = [](int per) { return per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : 8)); };
+  if (groups == 1 && units > 1) {
+    // a lone row group: eight lanes with a tile pair each, or (DIRECT_LANES = 4, whole-tile
+    // iterations only) four lanes with two
+    int const per8 = (units + 7) / 8, per4 = (units + 3) / 4;
+    if (s.direct_lanes == 4 && d.spi == 1 && d.ips == 1 && per4 <= 8 && units > 4) {
+      d.ip = 4;
+      d.nbuf = 2;
+      d.nit = round_nit(per4) < 2 ? 2 : round_nit(per4);
+    } else if (units <= 4 && d.spi == 1) {
+      d.ip = units <= 2 ? 2 : 4;
+      if (d.ips > 1) {
+        d.ip = 4;
+      }
+    } else {
+      d.ip = 8;
+      d.nit = round_nit(per8);
+    }
+  } else if (units >= 1 && units <= 8 && (groups > 1 || units == 1)) {
+    // every unit on a wavefront of its own, one slab of one or two row groups per workgroup
+    d.ip = units <= 2 && d.ips == 1 && d.spi == 1 ? 2 : (units <= 4 ? 4 : 8);
+    if (d.ip == 4 && d.spi == 1 && groups % 2 == 0 && blocks * (groups / 2) >= 256 && s.direct_lanes != 1) {
+      d.rpw = 2;
+    }
+    if (d.ip == 2 && units == 1) {
+      return false;  // a single iteration: nothing to hand over, the other variants serve it
+    }
+  } else {
+    return false;
+  }
+  int const pair_bytes = (64 * 64 + 64 * 64) * 2;
+  lds = d.ip * (d.nbuf * pair_bytes + d.rpw * 16 * M.D * 2);  // + a Q tile per wavefront
+  if (lds > s.max_lds || (long long)P.grid[0] * (groups / d.rpw) > 2147483647LL) {
+    return false;
+  }
+  AttnParams none{};
+  return (M.has_div ? launch_direct<true>(none, dim3(1, 1, 1), d, lds, true)
+                    : launch_direct<false>(none, dim3(1, 1, 1), d, lds, true)) == 1;
 }
 
 bool attention_applicable(DevProgram const &P) {
   Match M;
-  return match(P, M) && shape_supported(M);
+  DirectShape d;
+  int lds = 0;
+  return match(P, M) && (shape_supported(M) || choose_direct(P, M, d, lds));
 }
 
 int try_launch_attention(DevProgram const &P) {
   Match M;
-  if (!match(P, M) || !shape_supported(M)) {
+  if (!match(P, M)) {
+    return 0;
+  }
+  DirectShape dshape;
+  int direct_lds = 0;
+  bool const direct = choose_direct(P, M, dshape, direct_lds);
+  if (!direct && !shape_supported(M)) {
     return 0;
   }
   State &s = state();
@@ -1561,6 +1791,45 @@ int try_launch_attention(DevProgram const &P) {
     }
   }
 
+  // ---- direct-staging variant (attention mode 3 keeps the register-transposed staging):
+  // head size 64, key tiles of 16 ... 256, in two situations.
+  // (a) Every unit of work (an iteration, or a 64-key strip of several) has a wavefront of
+  //     its own.  A wavefront takes two row groups when that still puts a workgroup on every
+  //     compute unit: each K / V operand read from LDS then feeds two MFMAs and half as many
+  //     wavefronts stream the tiles (C2: 256 workgroups of 4 wavefronts x 32 rows; the
+  //     L2 -> LDS traffic and the LDS reads, both per-CU bandwidth limits at this size, halve).
+  // (b) A lone row group (decode: 8 or 16 query rows) with a longer for-loop: eight
+  //     wavefronts that each stream every eighth unit through a tile pair of their own, or
+  //     (DIRECT_LANES = 4) four wavefronts with two tile pairs each.
+  if (direct) {
+    int const groups = (M.m + 15) / 16;
+    AttnParams B = A;
+    B.split = groups / dshape.rpw;
+    B.trace = s.phase_trace;
+    dim3 const direct_grid(P.grid[0] * B.split, P.grid[1], P.grid[2]);
+    if (set_grid_magics(B, direct_grid)) {
+      if (B.trace != nullptr && (size_t)direct_grid.x * direct_grid.y * direct_grid.z * dshape.ip * 6 * 8 >
+                                    s.phase_trace_bytes) {
+        B.trace = nullptr;
+      }
+      int const rc = M.has_div ? launch_direct<true>(B, direct_grid, dshape, direct_lds)
+                               : launch_direct<false>(B, direct_grid, dshape, direct_lds);
+      if (rc != 0) {
+        if (rc == 1) {
+          s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
+          s.last().workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
+          s.last().threads = dshape.ip * 64;
+          s.last().lds_bytes = direct_lds;
+          s.last().row_split = B.split;
+        }
+        return rc;
+      }
+    }
+    if (!shape_supported(M)) {
+      return 0;
+    }
+  }
+
   // Row groups per workgroup: up to 4, fewer when that is what it takes to put a
   // workgroup on every compute unit.  Iteration lanes: whatever is left of 8
   // wavefronts, at most the for-loop range.
@@ -1600,66 +1869,10 @@ int try_launch_attention(DevProgram const &P) {
   dim3 grid(P.grid[0] * A.split, P.grid[1], P.grid[2]);
   int const nw = rg * ip;
   int rc = 0;
-  // Tiles of 64 x 64 x 64 take the direct-staging variant (attention mode 3 keeps the
-  // register-transposed staging) in two cases.
-  // (a) Every iteration has a wavefront of its own (F <= 4 or 8 lanes).  A wavefront takes
-  //     two row groups when that still puts a workgroup on every compute unit: each K / V
-  //     operand read from LDS then feeds two MFMAs, and half as many wavefronts stream the
-  //     tiles (C2: 256 workgroups of 4 wavefronts x 32 rows; the L2 -> LDS traffic and the
-  //     LDS reads, both per-CU bandwidth limits at this size, halve).
-  // (b) A single row group (decode: 8 or 16 query rows) with a longer for-loop: eight
-  //     wavefronts that each stream every eighth iteration through a tile pair of their own,
-  //     or (DIRECT_LANES = 4) four wavefronts with two tile pairs each.
-  if (M.D == 64 && M.NK == 64 && M.DV == 64 && s.attention_mode != 3 &&
-      (long long)P.grid[0] * groups <= 2147483647LL) {
-    int const F = P.forloop_range;
-    int dip = 0, rpw = 1, nbuf = 1, nit = 1;
-    if (F <= ip && ip > 1) {
-      dip = ip;
-      if (dip == 4 && groups % 2 == 0 && blocks * (groups / 2) >= 256 && s.direct_lanes != 1) {
-        rpw = 2;
-      }
-    } else if (groups == 1 && F > 1) {
-      int const per8 = (F + 7) / 8, per4 = (F + 3) / 4;
-      if (s.direct_lanes != 4 && per8 <= 4) {
-        dip = 8;
-        nit = per8 <= 1 ? 1 : (per8 <= 2 ? 2 : 4);
-      } else if (per4 <= 8) {
-        dip = 4;
-        nbuf = 2;
-        nit = per4 <= 2 ? 2 : (per4 <= 4 ? 4 : 8);
-      }
-    }
-    int const direct_lds = dip * (nbuf * stage_bytes + rpw * 16 * M.D * 2);  // + a Q tile per wavefront
-    if (dip > 0 && direct_lds <= s.max_lds) {
-      AttnParams B = A;
-      B.split = groups / rpw;
-      B.trace = s.phase_trace;
-      dim3 const direct_grid(P.grid[0] * B.split, P.grid[1], P.grid[2]);
-      if (!set_grid_magics(B, direct_grid)) {
-        return 0;
-      }
-      if (B.trace != nullptr &&
-          (size_t)direct_grid.x * direct_grid.y * direct_grid.z * dip * 6 * 8 > s.phase_trace_bytes) {
-        B.trace = nullptr;
-      }
-      rc = M.has_div ? launch_direct<true>(B, direct_grid, dip, rpw, nbuf, nit, direct_lds)
-                     : launch_direct<false>(B, direct_grid, dip, rpw, nbuf, nit, direct_lds);
-      if (rc == 1) {
-        s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
-        s.last().workgroups = direct_grid.x * direct_grid.y * direct_grid.z;
-        s.last().threads = dip * 64;
-        s.last().lds_bytes = direct_lds;
-        s.last().row_split = B.split;
-        return rc;
-      }
-    }
-  }
   if (!set_grid_magics(A, grid)) {
     return 0;
   }
-  if (rc == 1) {
-  } else if (M.D == 64 && M.NK == 64) {
+  if (M.D == 64 && M.NK == 64) {
     rc = launch_shape<64, 64, 64>(A, M.has_div, grid, rg, ip, lds);
   } else if (M.D == 64 && M.NK == 128) {
     rc = launch_shape<64, 128, 64>(A, M.has_div, grid, rg, ip, lds);

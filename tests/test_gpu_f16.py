@@ -242,6 +242,38 @@ def test_decode_row_groups_on_the_direct_staging_kernel(rt, abi, rows, F, kv_blo
         assert abi.mi355_set_option(6, 0) == 0
 
 
+@pytest.mark.parametrize("rows,nk,F,kv_blocks,groups", [
+    (64, 32, 8, 2, 3),      # two iterations per 64-key strip, a wavefront per strip
+    (64, 32, 16, 1, 3),     # ... eight strips
+    (16, 32, 32, 1, 3),     # a lone row group: eight lanes, two strips each
+    (64, 16, 16, 2, 3),     # four iterations per strip (16-deep matrix instruction)
+    (16, 16, 32, 1, 3),
+    (8, 16, 8, 2, 3),       # 8-row tile
+    (64, 32, 8, 16, 8),     # two row groups per wavefront (enough blocks to fill the chip)
+    (64, 16, 16, 16, 8),
+    (16, 128, 4, 2, 3),     # two strips per iteration
+    (64, 128, 4, 2, 3),
+    (16, 256, 16, 1, 3),    # four strips per iteration, two iterations per lane
+    (16, 256, 5, 1, 3),
+    (32, 256, 2, 2, 3),
+])
+def test_attention_key_tiles_of_other_widths(rt, abi, rows, nk, F, kv_blocks, groups):
+    """Key tiles of 16 / 32 / 128 / 256 on the direct-staging kernel's 64-key strips, against
+    the golden: the two-output form always, the form with the division inside where the
+    kernel takes it (tiles up to 64 keys)."""
+    from attention_superoptimizer_amd import workloads as W
+    seq = nk * F * kv_blocks
+    two_stage, _ = W.gqa_inc_decode(groups=groups, rows=rows, seq=seq, kv_blocks=kv_blocks, F=F)
+    single, _ = W.config2_gqa_decode(groups=groups, rows=rows, seq=seq, kv_blocks=kv_blocks, F=F)
+    cases = [("two-stage", two_stage)] + ([("single op", single)] if nk <= 64 else [])
+    for what, spec in cases:
+        # (small values: the un-normalised numerators stay below 1, where an fp16 ulp of the
+        # accumulator is inside the absolute tolerance)
+        ins = _inputs(spec, 0.05, 400 + nk + F)
+        _check(rt, spec, ins, f"{what}: rows {rows}, key tile {nk}, for-loop {F}")
+        assert _last_kernels[0] == KERNEL_ATTENTION, (what, _last_kernels)
+
+
 def N_launch_info():
     import ctypes
     from attention_superoptimizer_amd import _native as N
