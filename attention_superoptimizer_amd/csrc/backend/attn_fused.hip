@@ -100,6 +100,10 @@ struct AttnParams {
   int rows;     // query rows of the last row group that exist (16, or 8 for an 8-row tile: the
                 // missing rows are zeros in the Q fragment and are never stored)
   unsigned long long *trace;  // per-wavefront phase timestamps (attn_direct_kernel<.., TRACE>)
+  // attn_direct_kernel: the row sums are stored r_copies times, r_copy_stride elements apart
+  // (a plan whose blocks each take a few value columns and all store the same row sums runs
+  // as one block with the whole value tile)
+  int r_copies, r_copy_stride;
 };
 
 __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int by, int bz,
@@ -880,7 +884,8 @@ struct Match {
   int m, D, NK, DV;
 };
 
-bool match(DevProgram const &P, Match &M) {
+// `pieces`: the value tile may be narrower than 16 bytes (checked by merge_column_pieces)
+bool match(DevProgram const &P, Match &M, bool pieces = false) {
   if (P.num_ops < 9 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
       P.ops[2].kind != DOP_LOAD || P.ops[3].kind != DOP_MATMUL) {
     return false;
@@ -961,7 +966,8 @@ bool match(DevProgram const &P, Match &M) {
   if (lq.row_fs != 0 || lq.col_fs != 0 || lq.g_fs != 0) {
     return false;
   }
-  if (!lq.galign || !P.ops[M.k].galign || !P.ops[M.v].galign || !P.ops[M.out_o].galign) {
+  if (!lq.galign || !P.ops[M.k].galign ||
+      (!pieces && (!P.ops[M.v].galign || !P.ops[M.out_o].galign))) {
     return false;
   }
   for (void const *p : {P.in[lq.io], P.in[P.ops[M.k].io], P.in[P.ops[M.v].io],
@@ -971,6 +977,67 @@ bool match(DevProgram const &P, Match &M) {
     }
   }
   return true;
+}
+
+// A plan that cuts the value columns into pieces along one grid dimension -- every block of
+// that dimension loads the same Q and K tiles, takes DV / G columns of V, stores its columns of
+// the result and, in the row-sum form, its own copy of the same row sums -- computes the scores
+// G times.  Column j of the result depends on column j of V only, so the G blocks are one block
+// with the whole value tile: Q gets that program (grid dimension `g` of extent 1, V and the
+// result 64 columns wide, the row sums stored G times).  False when P is not of this shape.
+bool merge_column_pieces(DevProgram const &P, Match &M, DevProgram &Q, int &copies, int &copy_stride) {
+  if (!match(P, M, true) || M.DV >= 64 || 64 % M.DV != 0) {
+    return false;
+  }
+  int const G = 64 / M.DV;
+  DevOp const &lq = P.ops[M.q], &lk = P.ops[M.k], &lv = P.ops[M.v], &oo = P.ops[M.out_o];
+  for (int g = 0; g < 3; g++) {
+    if (P.grid[g] != G) {
+      continue;
+    }
+    auto free_of = [&](DevOp const &op) { return !op.row_bs[g] && !op.col_bs[g] && !op.g_bs[g]; };
+    auto pieced = [&](DevOp const &op) { return !op.row_bs[g] && !op.g_bs[g] && op.col_bs[g] == M.DV; };
+    if (!free_of(lq) || !free_of(lk) || !pieced(lv) || !pieced(oo)) {
+      continue;
+    }
+    copies = 1;
+    copy_stride = 0;
+    if (M.out_r >= 0) {
+      DevOp const &orr = P.ops[M.out_r];
+      if (orr.row_bs[g] || orr.g_bs[g]) {
+        continue;
+      }
+      copies = G;
+      copy_stride = orr.col_bs[g];
+    }
+    Q = P;
+    Q.grid[g] = 1;
+    Q.ops[M.v].col_bs[g] = 0;
+    Q.ops[M.out_o].col_bs[g] = 0;
+    if (M.out_r >= 0) {
+      Q.ops[M.out_r].col_bs[g] = 0;
+    }
+    // 16-byte reachability of the widened tiles
+    for (int o : {M.v, M.out_o}) {
+      DevOp &d = Q.ops[o];
+      bool al = d.d_cols % 8 == 0 && d.col_fs % 8 == 0 && d.g_fs % 8 == 0;
+      for (int e = 0; e < 3; e++) {
+        al = al && d.col_bs[e] % 8 == 0 && d.g_bs[e] % 8 == 0;
+      }
+      if (!al) {
+        return false;
+      }
+      d.galign = d.vec8 = 1;
+      Q.t[d.dst].cols = 64;
+    }
+    void const *vp = P.in[lv.io], *op = P.out[oo.io];
+    if (((reinterpret_cast<uintptr_t>(vp) | reinterpret_cast<uintptr_t>(op)) & 15) != 0) {
+      return false;
+    }
+    M.DV = 64;
+    return true;
+  }
+  return false;
 }
 
 // Direct-staging variant: one row group of (up to) 16 query rows per workgroup, IP wavefronts
@@ -1459,7 +1526,9 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       }
       _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
                       tile_offset(P.r, bx, by, bz, 0);
-      rgp[(long long)(row_base + tid) * P.r.d_cols] = static_cast<_Float16>(ra);
+      for (int c = 0; c < P.r_copies; c++) {
+        rgp[(long long)(row_base + tid) * P.r.d_cols + c * P.r_copy_stride] = static_cast<_Float16>(ra);
+      }
     }
   }
   if (TRACE && lane == 0) {
@@ -1666,9 +1735,10 @@ static bool choose_direct(DevProgram const &P, Match const &M, DirectShape &d, i
   int const groups = (M.m + 15) / 16;
   long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
   auto round_nit = [](int per) { return per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : 8)); };
-  if (groups == 1 && units > 1) {
-    // a lone row group: eight lanes with a tile pair each, or (DIRECT_LANES = 4, whole-tile
-    // iterations only) four lanes with two
+  if ((groups == 1 && units > 1) || units > 8) {
+    // a lone row group (or a loop too long for a wavefront per unit: then every row group is
+    // a workgroup of its own): eight lanes with a tile pair each, or (DIRECT_LANES = 4,
+    // whole-tile iterations only) four lanes with two
     int const per8 = (units + 7) / 8, per4 = (units + 3) / 4;
     if (s.direct_lanes == 4 && d.spi == 1 && d.ips == 1 && per4 <= 8 && units > 4) {
       d.ip = 4;
@@ -1709,22 +1779,37 @@ bool attention_applicable(DevProgram const &P) {
   Match M;
   DirectShape d;
   int lds = 0;
-  return match(P, M) && (shape_supported(M) || choose_direct(P, M, d, lds));
+  if (match(P, M)) {
+    return shape_supported(M) || choose_direct(P, M, d, lds);
+  }
+  DevProgram merged;
+  int copies = 1, stride = 0;
+  return merge_column_pieces(P, M, merged, copies, stride) && choose_direct(merged, M, d, lds);
 }
 
-int try_launch_attention(DevProgram const &P) {
+int try_launch_attention(DevProgram const &P0) {
   Match M;
-  if (!match(P, M)) {
-    return 0;
+  DevProgram merged;
+  DevProgram const *run = &P0;
+  int r_copies = 1, r_copy_stride = 0;
+  bool const pieces = !match(P0, M);
+  if (pieces) {
+    if (!merge_column_pieces(P0, M, merged, r_copies, r_copy_stride)) {
+      return 0;
+    }
+    run = &merged;
   }
+  DevProgram const &P = *run;
   DirectShape dshape;
   int direct_lds = 0;
   bool const direct = choose_direct(P, M, dshape, direct_lds);
-  if (!direct && !shape_supported(M)) {
-    return 0;
+  if (!direct && (pieces || !shape_supported(M))) {
+    return 0;  // (only the direct-staging variant stores copies of the row sums)
   }
   State &s = state();
   AttnParams A;
+  A.r_copies = r_copies;
+  A.r_copy_stride = r_copy_stride;
   A.q = tile_addr(P.ops[M.q], P.in[P.ops[M.q].io]);
   A.k = tile_addr(P.ops[M.k], P.in[P.ops[M.k].io]);
   A.v = tile_addr(P.ops[M.v], P.in[P.ops[M.v].io]);
@@ -1759,7 +1844,7 @@ int try_launch_attention(DevProgram const &P) {
     int const slabs = M.m / 32;
     int rgs = (M.m % 128 == 0) ? 4 : ((M.m % 64 == 0) ? 2 : 0);
     bool const shape = (M.D == 64 && M.NK == 64 && M.DV == 64) || (M.D == 128 && M.NK == 64 && M.DV == 128);
-    bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512;
+    bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512 && !pieces;
     if (s.attention_mode == 1 || s.attention_mode == 3) {
       want = false;
     } else if (s.attention_mode == 2) {
@@ -1825,7 +1910,7 @@ int try_launch_attention(DevProgram const &P) {
         return rc;
       }
     }
-    if (!shape_supported(M)) {
+    if (pieces || !shape_supported(M)) {
       return 0;
     }
   }

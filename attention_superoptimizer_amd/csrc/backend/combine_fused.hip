@@ -1,14 +1,23 @@
 // Fused kernel for the "fold the partial results and divide" family of thread-block
 // graphs: the second operator of the reference's split-KV attention plans
-// (cpp_examples/multi_head_attn_prefill.cc:75-98 and its siblings),
+// (cpp_examples/multi_head_attn_prefill.cc:75-98 and its siblings) and of the programs its
+// search records for them.  With N the partial numerators (S pieces of X columns per row, side
+// by side or one per for-loop iteration) and D the partial denominators (SD per row, or the
+// finished one), the members differ in where the division sits:
 //
-//   O[r][x] = fp16( fp16(sum_s N[r][s*X + x]) / fp16(sum_s D[r][s]) )
+//   sum, then divide   O[r][x] = fp16( fp16(sum_s N[r][s X + x]) / d[r] )
+//                      (loader, loader, reduction_to_dimx, [reduction], div, saver)
+//   divide, then sum   O[r][x] = fp16( sum_s fp16(N[r][s X + x] / d[r]) )
+//                      (loader, loader, [reduction], div, reduction_to_dimx, saver)
+//   divide, then the saver's for-loop accumulation
+//                      O[r][x] = acc_F,  acc_i = fp16(acc_{i-1} + fp16(N_i[r][x] / d[r]))
+//                      (loader, loader, [reduction], div, saver; any for-loop range)
 //
-// i.e. loader, loader, reduction_to_dimx over the partial numerators, reduction over the
-// partial denominators, div, saver, with a for-loop of one iteration.  Nothing is reused,
-// so nothing goes through LDS: each thread folds eight output columns of one row with
-// 16-byte loads and stores.  Sums run in fp32 over s = 0, 1, ... and are rounded to fp16
-// where the thread-block graph materialises a tile, the division is IEEE fp32.
+// with d[r] = fp16(sum_s D[r][s]) (or D[r] itself when the plan has no reduction over it).
+// Nothing is reused, so nothing goes through LDS: each thread folds eight (or, for tiles of
+// 4 columns, four) output columns of one row with vector loads and stores.  Sums run in
+// fp32 over s = 0, 1, ... and are rounded to fp16 where the thread-block graph materialises a
+// tile, the division is IEEE fp32.
 #include "common.h"
 #include "tb_program.h"
 
@@ -22,11 +31,14 @@ struct CTile {
   int d_cols;
 };
 
+enum { SUM_THEN_DIV = 0, DIV_THEN_SUM = 1, DIV_THEN_SAVE = 2 };
+
 struct CombineParams {
   CTile n, d, o;
-  int rows;  // tile rows
-  int X, S;  // output columns, partial results folded
-  uint32_t mx8;  // division magic of X / 8
+  int rows;        // tile rows
+  int X, S, SD;    // output columns, numerator pieces folded, denominators folded
+  long long step;  // elements from one numerator piece to the next
+  uint32_t mxv;    // division magic of X / VEC
 };
 
 __device__ __forceinline__ long long ctile_origin(CTile const &t) {
@@ -40,34 +52,51 @@ __device__ __forceinline__ long long ctile_origin(CTile const &t) {
   return base + row0 * t.d_cols + col0;
 }
 
+template <int VEC, int MODE>
 __global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const P) {
+  typedef _Float16 halfv __attribute__((ext_vector_type(VEC)));
   _Float16 const *n = static_cast<_Float16 const *>(P.n.ptr) + ctile_origin(P.n);
   _Float16 const *d = static_cast<_Float16 const *>(P.d.ptr) + ctile_origin(P.d);
   _Float16 *o = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) + ctile_origin(P.o);
-  int const x8 = P.X / 8, items = P.rows * x8;
+  int const xv = P.X / VEC, items = P.rows * xv;
   for (int e = threadIdx.x; e < items; e += 256) {
-    int const r = P.mx8 ? (int)__umulhi((uint32_t)e, P.mx8) : e;
-    int const x = (e - r * x8) * 8;
-    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    float den = 0.0f;
+    int const r = P.mxv ? (int)__umulhi((uint32_t)e, P.mxv) : e;
+    int const x = (e - r * xv) * VEC;
     _Float16 const *nr = n + (long long)r * P.n.d_cols + x;
     _Float16 const *dr = d + (long long)r * P.d.d_cols;
-    for (int s = 0; s < P.S; s++) {
-      half8 v = *reinterpret_cast<half8 const *>(nr + (long long)s * P.X);
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        acc[j] += static_cast<float>(v[j]);
-      }
+    float den = 0.0f;
+    for (int s = 0; s < P.SD; s++) {
       den += static_cast<float>(dr[s]);
     }
     float const den16 = static_cast<float>(static_cast<_Float16>(den));
-    half8 out;
+    float acc[VEC];
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      float const num16 = static_cast<float>(static_cast<_Float16>(acc[j]));
-      out[j] = static_cast<_Float16>(num16 / den16);
+    for (int j = 0; j < VEC; j++) {
+      acc[j] = 0.0f;
     }
-    *reinterpret_cast<half8 *>(o + (long long)r * P.o.d_cols + x) = out;
+#pragma unroll 4
+    for (int s = 0; s < P.S; s++) {
+      halfv const v = *reinterpret_cast<halfv const *>(nr + s * P.step);
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        float const t = static_cast<float>(v[j]);
+        if (MODE == SUM_THEN_DIV) {
+          acc[j] += t;
+        } else if (MODE == DIV_THEN_SUM) {
+          acc[j] += static_cast<float>(static_cast<_Float16>(t / den16));
+        } else {
+          acc[j] = static_cast<float>(
+              static_cast<_Float16>(acc[j] + static_cast<float>(static_cast<_Float16>(t / den16))));
+        }
+      }
+    }
+    halfv out;
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+      float const sum16 = static_cast<float>(static_cast<_Float16>(acc[j]));
+      out[j] = static_cast<_Float16>(MODE == SUM_THEN_DIV ? sum16 / den16 : sum16);
+    }
+    *reinterpret_cast<halfv *>(o + (long long)r * P.o.d_cols + x) = out;
   }
 }
 
@@ -87,15 +116,16 @@ CTile ctile(DevOp const &op, void const *ptr) {
 
 struct CMatch {
   int ln, ld, out;  // op indices: numerator loader, denominator loader, saver
-  int rows, X, S;
+  int rows, X, S, SD, mode, vec;
+  long long step;
 };
 
-bool aligned16(CTile const &t) {
-  if ((reinterpret_cast<uintptr_t>(t.ptr) & 15) != 0 || t.d_cols % 8 != 0) {
+bool aligned(CTile const &t, int vec) {
+  if ((reinterpret_cast<uintptr_t>(t.ptr) & (2 * vec - 1)) != 0 || t.d_cols % vec != 0) {
     return false;
   }
   for (int i = 0; i < 3; i++) {
-    if (t.col_bs[i] % 8 != 0 || t.g_bs[i] % 8 != 0) {
+    if (t.col_bs[i] % vec != 0 || t.g_bs[i] % vec != 0) {
       return false;
     }
   }
@@ -103,56 +133,112 @@ bool aligned16(CTile const &t) {
 }
 
 bool cmatch(DevProgram const &P, CMatch &M) {
-  if (P.forloop_range != 1 || P.num_ops != 6) {
+  int const last = P.num_ops - 1, F = P.forloop_range;
+  if (P.num_ops < 4 || P.num_ops > 6 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
+      P.ops[last].kind != DOP_OUTPUT) {
     return false;
   }
-  DevOp const &l0 = P.ops[0], &l1 = P.ops[1], &r0 = P.ops[2], &r1 = P.ops[3], &dv = P.ops[4],
-              &out = P.ops[5];
-  if (l0.kind != DOP_LOAD || l1.kind != DOP_LOAD || r0.kind != DOP_REDUCE ||
-      r1.kind != DOP_REDUCE || dv.kind != DOP_BINARY || dv.sub != TB_DIV_OP ||
-      out.kind != DOP_OUTPUT) {
-    return false;
-  }
-  // either reduction may come first; the numerator is the one the div takes as src0
-  DevOp const *rn = nullptr, *rd = nullptr;
-  for (DevOp const *r : {&r0, &r1}) {
-    if (r->dst == dv.src0) {
-      rn = r;
-    } else if (r->dst == dv.src1) {
-      rd = r;
+  DevOp const &out = P.ops[last];
+  auto loader_of = [&](int tensor) { return P.ops[0].dst == tensor ? 0 : (P.ops[1].dst == tensor ? 1 : -1); };
+  auto producer = [&](int tensor) {  // a middle statement writing `tensor`, or -1
+    for (int o = 2; o < last; o++) {
+      if (P.ops[o].dst == tensor) {
+        return o;
+      }
+    }
+    return -1;
+  };
+  // the one division
+  int dv = -1;
+  for (int o = 2; o < last; o++) {
+    if (P.ops[o].kind == DOP_BINARY && P.ops[o].sub == TB_DIV_OP) {
+      if (dv >= 0) {
+        return false;
+      }
+      dv = o;
     }
   }
-  if (rn == nullptr || rd == nullptr || out.src0 != dv.dst) {
+  if (dv < 0) {
     return false;
   }
-  DevOp const *ln = nullptr, *ld = nullptr;
-  for (DevOp const *l : {&l0, &l1}) {
-    if (l->dst == rn->src0) {
-      ln = l;
-    } else if (l->dst == rd->src0) {
-      ld = l;
+  int used = 1;
+  // its divisor: a one-column tile, loaded as such or folded from the SD columns of a loaded tile
+  int ld = loader_of(P.ops[dv].src1), SD = 1;
+  if (ld < 0) {
+    int const rd = producer(P.ops[dv].src1);
+    if (rd < 0 || P.ops[rd].kind != DOP_REDUCE || P.ops[rd].red_inner != 1) {
+      return false;
     }
+    ld = loader_of(P.ops[rd].src0);
+    if (ld < 0) {
+      return false;
+    }
+    SD = P.ops[rd].red_deg;
+    used++;
   }
-  if (ln == nullptr || ld == nullptr) {
+  DevTensor const &td = P.t[P.ops[ld].dst], &tden = P.t[P.ops[dv].src1];
+  if (td.cols != SD || tden.cols != 1 || tden.rows != td.rows) {
     return false;
   }
-  DevTensor const &tn = P.t[ln->dst], &td = P.t[ld->dst], &to = P.t[dv.dst];
-  int const S = rn->red_deg, X = rn->red_inner;
-  if (tn.cols != S * X || td.rows != tn.rows || td.cols != S || rd->red_deg != S ||
-      rd->red_inner != 1 || P.t[rn->dst].rows != tn.rows || P.t[rn->dst].cols != X ||
-      P.t[rd->dst].rows != tn.rows || P.t[rd->dst].cols != 1 || to.rows != tn.rows ||
-      to.cols != X || X % 8 != 0 || S < 1) {
+  // a fold over S pieces of X columns
+  auto to_dimx = [&](DevOp const &r, int &S, int &X) {
+    DevTensor const &ti = P.t[r.src0], &to = P.t[r.dst];
+    S = r.red_deg;
+    X = r.red_inner;
+    return r.kind == DOP_REDUCE && to.rows == ti.rows && to.cols == X && ti.cols == S * X && S >= 1;
+  };
+  int ln = loader_of(P.ops[dv].src0), S = 1, X = 0, mode;
+  if (ln < 0) {
+    // sum, then divide
+    int const rn = producer(P.ops[dv].src0);
+    if (rn < 0 || !to_dimx(P.ops[rn], S, X) || out.src0 != P.ops[dv].dst || F != 1) {
+      return false;
+    }
+    ln = loader_of(P.ops[rn].src0);
+    mode = SUM_THEN_DIV;
+    used++;
+  } else if (out.src0 == P.ops[dv].dst) {
+    // divide, then the saver accumulates over the for-loop
+    mode = DIV_THEN_SAVE;
+    S = F;
+    X = P.t[P.ops[ln].dst].cols;
+  } else {
+    // divide, then sum
+    int const rn = producer(out.src0);
+    if (rn < 0 || !to_dimx(P.ops[rn], S, X) || P.ops[rn].src0 != P.ops[dv].dst || F != 1) {
+      return false;
+    }
+    mode = DIV_THEN_SUM;
+    used++;
+  }
+  if (ln < 0 || ln == ld || used != P.num_ops - 3) {
     return false;
   }
-  if (!aligned16(ctile(*ln, P.in[ln->io])) || !aligned16(ctile(out, P.out[out.io]))) {
+  DevOp const &opn = P.ops[ln], &opd = P.ops[ld];
+  DevTensor const &tn = P.t[opn.dst], &to = P.t[out.src0];
+  int const pieces = mode == DIV_THEN_SAVE ? 1 : S;
+  if (tn.rows != td.rows || tn.cols != pieces * X || to.rows != tn.rows || to.cols != X ||
+      P.t[P.ops[dv].dst].cols != (mode == SUM_THEN_DIV ? X : tn.cols)) {
     return false;
   }
-  M.ln = (int)(ln - P.ops);
-  M.ld = (int)(ld - P.ops);
-  M.out = 5;
+  // the divisor does not move with the for-loop; the numerator may (one piece an iteration)
+  if (opd.row_fs != 0 || opd.col_fs != 0 || opd.g_fs != 0) {
+    return false;
+  }
+  M.step = mode == DIV_THEN_SAVE ? (long long)opn.g_fs + (long long)opn.row_fs * opn.d_cols + opn.col_fs : X;
+  M.vec = X % 8 == 0 ? 8 : (X % 4 == 0 ? 4 : 0);
+  if (M.vec == 0 || M.step % M.vec != 0 || !aligned(ctile(opn, P.in[opn.io]), M.vec) ||
+      !aligned(ctile(out, P.out[out.io]), M.vec)) {
+    return false;
+  }
+  M.ln = ln;
+  M.ld = ld;
+  M.out = last;
   M.rows = tn.rows;
   M.X = X;
   M.S = S;
+  M.SD = SD;
+  M.mode = mode;
   return true;
 }
 
@@ -176,9 +262,28 @@ int try_launch_combine(DevProgram const &P) {
   A.rows = M.rows;
   A.X = M.X;
   A.S = M.S;
-  A.mx8 = fast_div_magic(M.X / 8);
+  A.SD = M.SD;
+  A.step = M.step;
+  A.mxv = fast_div_magic(M.X / M.vec);
   dim3 grid(P.grid[0], P.grid[1], P.grid[2]);
-  combine_fused_kernel<<<grid, 256, 0, s.stream()>>>(A);
+  hipStream_t const q = s.stream();
+  if (M.vec == 8) {
+    if (M.mode == SUM_THEN_DIV) {
+      combine_fused_kernel<8, SUM_THEN_DIV><<<grid, 256, 0, q>>>(A);
+    } else if (M.mode == DIV_THEN_SUM) {
+      combine_fused_kernel<8, DIV_THEN_SUM><<<grid, 256, 0, q>>>(A);
+    } else {
+      combine_fused_kernel<8, DIV_THEN_SAVE><<<grid, 256, 0, q>>>(A);
+    }
+  } else {
+    if (M.mode == SUM_THEN_DIV) {
+      combine_fused_kernel<4, SUM_THEN_DIV><<<grid, 256, 0, q>>>(A);
+    } else if (M.mode == DIV_THEN_SUM) {
+      combine_fused_kernel<4, DIV_THEN_SUM><<<grid, 256, 0, q>>>(A);
+    } else {
+      combine_fused_kernel<4, DIV_THEN_SAVE><<<grid, 256, 0, q>>>(A);
+    }
+  }
   MI355_HIP(hipGetLastError());
   s.last().kernel_id = MI355_KERNEL_F16_COMBINE;
   s.last().workgroups = (int)(grid.x * grid.y * grid.z);

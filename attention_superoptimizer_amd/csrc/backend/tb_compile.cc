@@ -391,9 +391,9 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       dt.cs = 1;
       ti.bytes = round_up(ti.rows * ti.cols * 2, 16);
     } else {
-      // k-contiguous for the matrix-core B operand: column-major, padded columns;
-      // everything else row-major, padded rows -- unless the plan's declaration rules
-      bool column_major = ti.as_b && !ti.as_a;
+      // every tile row-major with padded rows, as it is loaded (the matrix-core B operand is
+      // gathered with transposing LDS reads) -- unless the plan's declaration rules
+      bool column_major = false;
       int p = pad;
       if (declared_layouts && declared_known(ti.declared)) {
         column_major = declared_column_major(ti.declared);

@@ -598,10 +598,37 @@ __device__ __forceinline__ _Float16 *tile_ptr(unsigned char *lds, DevTensor cons
   return reinterpret_cast<_Float16 *>(lds + t.off);
 }
 
-// C[m][n] = A[m][k] . B[k][n] on the matrix cores.  A is k-contiguous per row
-// (cs == 1), B is k-contiguous per column (rs == 1); both strides are multiples
-// of 8 so every operand fetch is one 16-byte LDS read.  Wavefronts take output
-// tiles round-robin.  Rows past m are clamped on read and masked on write.
+// C[m][n] = A[m][k] . B[k][n] on the matrix cores.  A is k-contiguous per row (cs == 1).
+// B is either k-contiguous per column (rs == 1: one 16-byte LDS read per operand) or, the
+// default, row-major as it was loaded (cs == 1): its operand is then gathered with
+// transposing LDS reads (two 8-byte reads per operand, four k of sixteen columns each), so
+// no tile is ever transposed while it is staged.  Row strides are multiples of 8 halfs.
+// Wavefronts take output tiles round-robin.  Rows and columns past the end are clamped on
+// read and masked on write.
+// Transposing read: within 16 lanes, lane 4a + b names four halfs T[row0 + a][col0 + 4b ..]
+// and lane i receives T[row0 + 0..3][col0 + i].
+__device__ __forceinline__ half4 lds_tr16(_Float16 const *p) {
+  typedef short short4v __attribute__((ext_vector_type(4)));
+  short4v const v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (short4v __attribute__((address_space(3))) *)(__attribute__((address_space(3))) void *)(p));
+  return __builtin_bit_cast(half4, v);
+}
+// B[krow .. krow + 7][col0 + lane % 16] for the 16 lanes of a group: `bp` is this lane's
+// address inside rows krow .. krow + 3 (see b_tr_lane), rows + 4 are `rs` * 4 halfs further
+__device__ __forceinline__ half8 b_frag_tr(_Float16 const *bp, int rs) {
+  half4 const lo = lds_tr16(bp), hi = lds_tr16(bp + 4 * rs);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// this lane's address for the reads above: row (lane % 16) / 4, columns col0 + 4 * (lane % 4),
+// kept inside the row when the tile has fewer than col0 + 16 columns (those output columns
+// are masked)
+__device__ __forceinline__ int b_tr_lane(int lane, int col0, int n, int rs) {
+  int const a = (lane % 16) / 4;
+  int col = col0 + 4 * (lane % 4);
+  int const last = ((n + 3) / 4) * 4 - 4;
+  col = col < last ? col : last;
+  return a * rs + col;
+}
 template <int TILE>
 __device__ __forceinline__ void mfma_matmul(unsigned char *lds, DevTensor const &ta,
                                             DevTensor const &tb, DevTensor const &tc, int wave,
@@ -610,14 +637,17 @@ __device__ __forceinline__ void mfma_matmul(unsigned char *lds, DevTensor const 
   _Float16 const *B = tile_ptr(lds, tb);
   _Float16 *C = tile_ptr(lds, tc);
   int const m = ta.rows, k = ta.cols, n = tb.cols;
-  int const tiles_m = (m + TILE - 1) / TILE, tiles_n = n / TILE;
+  int const tiles_m = (m + TILE - 1) / TILE, tiles_n = (n + TILE - 1) / TILE;
   for (int tile = wave; tile < tiles_m * tiles_n; tile += num_waves) {
     int const tm = tile / tiles_n, tn = tile % tiles_n;
     if constexpr (TILE == 32) {
       int arow = tm * 32 + lane % 32;
       arow = arow < m ? arow : m - 1;
       _Float16 const *ap = A + arow * ta.rs + 8 * (lane / 32);
-      _Float16 const *bp = B + (tn * 32 + lane % 32) * tb.cs + 8 * (lane / 32);
+      bool const b_rows = tb.cs == 1;  // row-major B: transposing reads
+      _Float16 const *bp = b_rows ? B + (8 * (lane / 32)) * tb.rs +
+                                        b_tr_lane(lane, tn * 32 + 16 * ((lane / 16) % 2), n, tb.rs)
+                                  : B + (tn * 32 + lane % 32) * tb.cs + 8 * (lane / 32);
       float16v acc;
 #pragma unroll
       for (int i = 0; i < 16; i++) {
@@ -625,7 +655,7 @@ __device__ __forceinline__ void mfma_matmul(unsigned char *lds, DevTensor const 
       }
       for (int k0 = 0; k0 < k; k0 += 16) {
         half8 a = *reinterpret_cast<half8 const *>(ap + k0);
-        half8 b = *reinterpret_cast<half8 const *>(bp + k0);
+        half8 b = b_rows ? b_frag_tr(bp + k0 * tb.rs, tb.rs) : *reinterpret_cast<half8 const *>(bp + k0);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
       }
 #pragma unroll
@@ -640,24 +670,29 @@ __device__ __forceinline__ void mfma_matmul(unsigned char *lds, DevTensor const 
       int arow = tm * 16 + lane % 16;
       arow = arow < m ? arow : m - 1;
       _Float16 const *ap = A + arow * ta.rs;
-      _Float16 const *bp = B + (tn * 16 + lane % 16) * tb.cs;
+      bool const b_rows = tb.cs == 1;  // row-major B: transposing reads
+      int bcol = tn * 16 + lane % 16;
+      bcol = bcol < n ? bcol : n - 1;
+      _Float16 const *bp = b_rows ? B + b_tr_lane(lane, tn * 16, n, tb.rs) : B + bcol * tb.cs;
       float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
       int k0 = 0;
       for (; k0 + 32 <= k; k0 += 32) {
         half8 a = *reinterpret_cast<half8 const *>(ap + k0 + 8 * (lane / 16));
-        half8 b = *reinterpret_cast<half8 const *>(bp + k0 + 8 * (lane / 16));
+        half8 b = b_rows ? b_frag_tr(bp + (k0 + 8 * (lane / 16)) * tb.rs, tb.rs)
+                         : *reinterpret_cast<half8 const *>(bp + k0 + 8 * (lane / 16));
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
       }
       for (; k0 + 16 <= k; k0 += 16) {
         half4 a = *reinterpret_cast<half4 const *>(ap + k0 + 4 * (lane / 16));
-        half4 b = *reinterpret_cast<half4 const *>(bp + k0 + 4 * (lane / 16));
+        half4 b = b_rows ? lds_tr16(bp + (k0 + 4 * (lane / 16)) * tb.rs)
+                         : *reinterpret_cast<half4 const *>(bp + k0 + 4 * (lane / 16));
         acc = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, acc, 0, 0, 0);
       }
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         int row = tm * 16 + (lane / 16) * 4 + r;
         int col = tn * 16 + lane % 16;
-        if (row < m) {
+        if (row < m && col < n) {
           C[row * tc.rs + col * tc.cs] = static_cast<_Float16>(acc[r]);
         }
       }
@@ -665,10 +700,28 @@ __device__ __forceinline__ void mfma_matmul(unsigned char *lds, DevTensor const 
   }
 }
 
-__global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram const P) {
+// rows of 16-byte pieces: element-wise statements then move eight halfs per LDS access
+__device__ __forceinline__ bool vec_tile(DevTensor const &t) {
+  return t.cs == 1 && t.rs % 8 == 0 && t.cols % 8 == 0;
+}
+__device__ __forceinline__ half8 splat8(_Float16 x) {
+  half8 v = {x, x, x, x, x, x, x, x};
+  return v;
+}
+
+// `trace` (null unless the phase trace option is on): the first workgroup's first thread
+// stamps the 100 MHz clock at its start and after every statement's barrier; trace[0] counts
+// the stamps that follow it.
+__global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram const P,
+                                                                    unsigned long long *trace) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   int const tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   int const F = P.forloop_range;
+  bool const tracing = trace != nullptr && tid == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;
+  unsigned long long stamps = 0;
+  if (tracing) {
+    trace[++stamps] = __builtin_amdgcn_s_memrealtime();
+  }
   for (int it = 0; it < F; it++) {
     for (int o = 0; o < P.num_ops; o++) {
       DevOp const &op = P.ops[o];
@@ -684,7 +737,7 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           if (op.vec8) {
             int const cpr = t.cols / 8, n = t.rows * cpr;
             for (int e = tid; e < n; e += kInterpThreads) {
-              int r = e / cpr, c = (e % cpr) * 8;
+              int const r = fdiv(e, t.mcpr), c = (e - r * cpr) * 8;
               half8 v = *reinterpret_cast<half8 const *>(
                   g + (long long)(org.row0 + r) * op.d_cols + org.col0 + c);
               if (op.vec8 == 1) {
@@ -699,7 +752,7 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           } else {
             int const n = t.rows * t.cols;
             for (int e = tid; e < n; e += kInterpThreads) {
-              int r = e / t.cols, c = e % t.cols;
+              int const r = fdiv(e, t.mcols), c = e - r * t.cols;
               s[r * t.rs + c * t.cs] = g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c];
             }
           }
@@ -708,8 +761,9 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
         case DOP_MATMUL: {
           DevTensor const &ta = P.t[op.src0], &tb = P.t[op.src1], &tc = P.t[op.dst];
           int const m = ta.rows, k = ta.cols, n = tb.cols;
-          bool const fast = ta.cs == 1 && tb.rs == 1 && ta.rs % 8 == 0 && tb.cs % 8 == 0 &&
-                            k % 16 == 0 && n % 16 == 0;
+          // (any m and n: rows and columns past the end are clamped on read, masked on write)
+          bool const fast = ta.cs == 1 && ta.rs % 8 == 0 && k % 16 == 0 &&
+                            ((tb.rs == 1 && tb.cs % 8 == 0) || (tb.cs == 1 && tb.rs % 4 == 0 && n >= 4));
           if (fast && m % 32 == 0 && n % 32 == 0) {
             mfma_matmul<32>(lds, ta, tb, tc, wave, lane, kInterpThreads / 64);
           } else if (fast) {
@@ -719,7 +773,7 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
             _Float16 const *B = tile_ptr(lds, tb);
             _Float16 *C = tile_ptr(lds, tc);
             for (int e = tid; e < m * n; e += kInterpThreads) {
-              int row = e / n, col = e % n;
+              int const row = fdiv(e, tb.mcols), col = e - row * n;
               float acc = 0.0f;
               for (int kk = 0; kk < k; kk++) {
                 acc = __builtin_fmaf(static_cast<float>(A[row * ta.rs + kk * ta.cs]),
@@ -737,11 +791,27 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           DevTensor const &t = P.t[op.dst];
           _Float16 *p = tile_ptr(lds, t);
           int const n = t.rows * t.cols;
+          bool const is_exp = op.sub == TB_EXP_OP;
+          if (vec_tile(t)) {
+            int const cpr = t.cols / 8;
+            for (int e = tid; e < n / 8; e += kInterpThreads) {
+              int const r = fdiv(e, t.mcpr), c = (e - r * cpr) * 8;
+              half8 *q = reinterpret_cast<half8 *>(p + r * t.rs + c);
+              half8 v = *q;
+#pragma unroll
+              for (int j = 0; j < 8; j++) {
+                float const x = static_cast<float>(v[j]);
+                v[j] = static_cast<_Float16>(is_exp ? __expf(x) : x / (1.0f + __expf(-x)));
+              }
+              *q = v;
+            }
+            break;
+          }
           for (int e = tid; e < n; e += kInterpThreads) {
-            int r = e / t.cols, c = e % t.cols;
+            int const r = fdiv(e, t.mcols), c = e - r * t.cols;
             _Float16 *q = p + r * t.rs + c * t.cs;
             float x = static_cast<float>(*q);
-            float y = (op.sub == TB_EXP_OP) ? __expf(x) : x / (1.0f + __expf(-x));
+            float y = is_exp ? __expf(x) : x / (1.0f + __expf(-x));
             *q = static_cast<_Float16>(y);
           }
           break;
@@ -752,10 +822,33 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           _Float16 const *x2 = tile_ptr(lds, t2);
           _Float16 *y = tile_ptr(lds, to);
           int const n = to.rows * to.cols;
+          // an operand dim is either the output's or 1 (checked by the lowering): broadcast = index 0
+          bool const r1 = t1.rows > 1, c1 = t1.cols > 1, r2 = t2.rows > 1, c2 = t2.cols > 1;
+          // an operand with columns is read eight at a time, one without is one value per row
+          bool const v1 = !c1 || (t1.cs == 1 && (t1.rs % 8 == 0 || !r1));
+          bool const v2 = !c2 || (t2.cs == 1 && (t2.rs % 8 == 0 || !r2));
+          if (vec_tile(to) && v1 && v2) {
+            int const cpr = to.cols / 8;
+            for (int e = tid; e < n / 8; e += kInterpThreads) {
+              int const r = fdiv(e, to.mcpr), c = (e - r * cpr) * 8;
+              _Float16 const *p1 = x1 + (r1 ? r : 0) * t1.rs, *p2 = x2 + (r2 ? r : 0) * t2.rs;
+              half8 const a8 = c1 ? *reinterpret_cast<half8 const *>(p1 + c) : splat8(*p1);
+              half8 const b8 = c2 ? *reinterpret_cast<half8 const *>(p2 + c) : splat8(*p2);
+              half8 z8;
+#pragma unroll
+              for (int j = 0; j < 8; j++) {
+                float const a = static_cast<float>(a8[j]), b = static_cast<float>(b8[j]);
+                float const z = (op.sub == TB_DIV_OP) ? a / b : (op.sub == TB_ADD_OP) ? a + b : a * b;
+                z8[j] = static_cast<_Float16>(z);
+              }
+              *reinterpret_cast<half8 *>(y + r * to.rs + c) = z8;
+            }
+            break;
+          }
           for (int e = tid; e < n; e += kInterpThreads) {
-            int r = e / to.cols, c = e % to.cols;
-            float a = static_cast<float>(x1[(r % t1.rows) * t1.rs + (c % t1.cols) * t1.cs]);
-            float b = static_cast<float>(x2[(r % t2.rows) * t2.rs + (c % t2.cols) * t2.cs]);
+            int const r = fdiv(e, to.mcols), c = e - r * to.cols;
+            float a = static_cast<float>(x1[(r1 ? r : 0) * t1.rs + (c1 ? c : 0) * t1.cs]);
+            float b = static_cast<float>(x2[(r2 ? r : 0) * t2.rs + (c2 ? c : 0) * t2.cs]);
             float z = (op.sub == TB_DIV_OP) ? a / b : (op.sub == TB_ADD_OP) ? a + b : a * b;
             y[r * to.rs + c * to.cs] = static_cast<_Float16>(z);
           }
@@ -766,13 +859,99 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           _Float16 const *x = tile_ptr(lds, ti);
           _Float16 *y = tile_ptr(lds, to);
           int const n = to.rows * to.cols, deg = op.red_deg, inner = op.red_inner;
-          for (int e = tid; e < n; e += kInterpThreads) {
-            int pos = (e / inner) * (inner * deg) + e % inner;
-            float r = 0.0f;
-            for (int kk = 0; kk < deg; kk++, pos += inner) {
-              r += static_cast<float>(x[(pos / ti.cols) * ti.rs + (pos % ti.cols) * ti.cs]);
+          // Along the columns of a row (output (r, c) = sum over j of x[r][c + j inner]) or along
+          // the rows (output (r, c) = sum over j of x[r + j to.rows][c]): no division in the sum.
+          // Long sums are shared by 16 lanes (fp32 parts, added across the lanes at the end).
+          bool const along_cols = to.rows == ti.rows;
+          int const lanes = (deg >= 64 && n * 16 <= 4 * kInterpThreads) ? 16 : 1;
+          int const step = along_cols ? inner * ti.cs : to.rows * ti.rs;
+          if (along_cols && inner == 1 && ti.cs == 1 && ti.rs % 8 == 0 && deg % 8 == 0) {
+            // a run of consecutive elements: each lane adds pieces of eight, one after the
+            // other in element order (with one lane this is the plain order)
+            for (int e0 = 0; e0 < n; e0 += kInterpThreads / lanes) {
+              int const e = e0 + tid / lanes, part = tid % lanes;
+              float r = 0.0f;
+              if (e < n) {
+                int const orow = fdiv(e, to.mcols), ocol = e - orow * to.cols;
+                _Float16 const *src = x + orow * ti.rs + ocol;
+                for (int kk = 8 * part; kk < deg; kk += 8 * lanes) {
+                  half8 const v = *reinterpret_cast<half8 const *>(src + kk);
+#pragma unroll
+                  for (int j = 0; j < 8; j++) {
+                    r += static_cast<float>(v[j]);
+                  }
+                }
+              }
+              if (lanes == 16) {
+                r += __shfl_xor(r, 1, 64);
+                r += __shfl_xor(r, 2, 64);
+                r += __shfl_xor(r, 4, 64);
+                r += __shfl_xor(r, 8, 64);
+              }
+              if (e < n && part == 0) {
+                int const orow = fdiv(e, to.mcols), ocol = e - orow * to.cols;
+                y[orow * to.rs + ocol * to.cs] = static_cast<_Float16>(r);
+              }
             }
-            y[(e / to.cols) * to.rs + (e % to.cols) * to.cs] = static_cast<_Float16>(r);
+            break;
+          }
+          if (vec_tile(to) && ti.cs == 1 && ti.rs % 8 == 0 && (!along_cols || inner % 8 == 0)) {
+            // eight neighbouring outputs per lane, each with the element order of the plain loop
+            int const cpr = to.cols / 8;
+            for (int e0 = 0; e0 < n / 8; e0 += kInterpThreads / lanes) {
+              int const e = e0 + tid / lanes, part = tid % lanes;
+              float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+              int const orow = fdiv(e, to.mcpr), ocol = (e - orow * cpr) * 8;
+              if (e < n / 8) {
+                _Float16 const *src = x + orow * ti.rs + ocol + part * step;
+                for (int kk = part; kk < deg; kk += lanes, src += lanes * step) {
+                  half8 const v = *reinterpret_cast<half8 const *>(src);
+#pragma unroll
+                  for (int j = 0; j < 8; j++) {
+                    r[j] += static_cast<float>(v[j]);
+                  }
+                }
+              }
+              if (lanes == 16) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                  r[j] += __shfl_xor(r[j], 1, 64);
+                  r[j] += __shfl_xor(r[j], 2, 64);
+                  r[j] += __shfl_xor(r[j], 4, 64);
+                  r[j] += __shfl_xor(r[j], 8, 64);
+                }
+              }
+              if (e < n / 8 && part == 0) {
+                half8 h;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                  h[j] = static_cast<_Float16>(r[j]);
+                }
+                *reinterpret_cast<half8 *>(y + orow * to.rs + ocol) = h;
+              }
+            }
+            break;
+          }
+          for (int e0 = 0; e0 < n; e0 += kInterpThreads / lanes) {
+            int const e = e0 + tid / lanes, part = tid % lanes;
+            float r = 0.0f;
+            if (e < n) {
+              int const orow = fdiv(e, to.mcols), ocol = e - orow * to.cols;
+              _Float16 const *src = x + orow * ti.rs + ocol * ti.cs + part * step;
+              for (int kk = part; kk < deg; kk += lanes, src += lanes * step) {
+                r += static_cast<float>(*src);
+              }
+            }
+            if (lanes == 16) {
+              r += __shfl_xor(r, 1, 64);
+              r += __shfl_xor(r, 2, 64);
+              r += __shfl_xor(r, 4, 64);
+              r += __shfl_xor(r, 8, 64);
+            }
+            if (e < n && part == 0) {
+              int const orow = fdiv(e, to.mcols), ocol = e - orow * to.cols;
+              y[orow * to.rs + ocol * to.cs] = static_cast<_Float16>(r);
+            }
           }
           break;
         }
@@ -784,7 +963,7 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           int const n = to.rows * to.cols;
           bool const along_cols = (op.cat_inner == 1 && t1.rows == to.rows);
           for (int e = tid; e < n; e += kInterpThreads) {
-            int r = e / to.cols, c = e % to.cols;
+            int const r = fdiv(e, to.mcols), c = e - r * to.cols;
             _Float16 v;
             if (along_cols) {
               v = c < t1.cols ? A[r * t1.rs + c * t1.cs] : B[r * t2.rs + (c - t1.cols) * t2.cs];
@@ -805,8 +984,28 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           bool const last = (it == F - 1);
           TileOrigin org = tile_origin(op, 0, blockIdx.x);
           _Float16 *g = static_cast<_Float16 *>(P.out[op.io]) + org.base;
+          if (op.vec8 && vec_tile(ti)) {
+            int const cpr = ta.cols / 8;
+            for (int e = tid; e < n / 8; e += kInterpThreads) {
+              int const r = fdiv(e, ta.mcpr), c = (e - r * cpr) * 8;
+              half8 v = *reinterpret_cast<half8 const *>(x + r * ti.rs + c);
+              if (it > 0) {
+                half8 const a = *reinterpret_cast<half8 const *>(acc + r * ta.rs + c);
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                  v[j] = static_cast<_Float16>(static_cast<float>(v[j]) + static_cast<float>(a[j]));
+                }
+              }
+              if (last) {
+                *reinterpret_cast<half8 *>(g + (long long)(org.row0 + r) * op.d_cols + org.col0 + c) = v;
+              } else {
+                *reinterpret_cast<half8 *>(acc + r * ta.rs + c) = v;
+              }
+            }
+            break;
+          }
           for (int e = tid; e < n; e += kInterpThreads) {
-            int r = e / ta.cols, c = e % ta.cols;
+            int const r = fdiv(e, ta.mcols), c = e - r * ta.cols;
             float v = static_cast<float>(x[r * ti.rs + c * ti.cs]);
             if (it > 0) {
               v += static_cast<float>(acc[r * ta.rs + c * ta.cs]);
@@ -824,7 +1023,13 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           break;
       }
       __syncthreads();
+      if (tracing && stamps < 4000) {
+        trace[++stamps] = __builtin_amdgcn_s_memrealtime();
+      }
     }
+  }
+  if (tracing) {
+    trace[0] = stamps;
   }
 }
 
@@ -1105,7 +1310,7 @@ static int launch(DevProgram const &prog, bool f16) {
     cur = s.max_lds;
   }
   if (f16) {
-    f16_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog);
+    f16_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog, s.phase_trace);
   } else {
     fp_interp_kernel<<<grid, kInterpThreads, prog.lds_bytes, s.stream()>>>(prog, s.exp_tbl,
                                                                           s.div_p, s.div_q);

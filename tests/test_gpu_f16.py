@@ -292,6 +292,47 @@ def test_gqa_fixture_graphs_f16(rt, path):
         _check(rt, spec, ins, f"fixture graph {gi}")
 
 
+def test_value_columns_cut_into_pieces_run_as_one_block(rt, abi):
+    """The recorded programs whose grid cuts the 64 value columns into 16 pieces of 4 (every
+    piece's block repeats the same scores and stores its own copy of the row sums): the fused
+    route runs each (batch, query tile) as one block with the whole value tile -- 32
+    workgroups (2 x 4 query tiles x 4 row groups) instead of 128 blocks -- and matches the golden
+    on both outputs, every copy of the row sums included."""
+    from helpers import load_gqa_fixture
+    fx = load_gqa_fixture()
+    for gi in (60, 65):
+        spec = fx["generated_graphs"][gi]
+        plan = spec[3]["plan"]
+        assert plan["grid_dim"] == [2, 16, 4] and spec[3]["out_dims"] == [[2, 256, 16], [2, 256, 64]]
+        ins = _inputs(spec, 0.05, 170 + gi)
+        # (values of one sign: the 4096-key sums then grow steadily, and an fp16 ulp of the
+        # accumulator stays inside the relative tolerance of the final value)
+        ins[2] = np.abs(ins[2])
+        _check(rt, spec, ins, f"fixture graph {gi}", threads=16)
+        assert _last_kernels[0] == KERNEL_ATTENTION, _last_kernels
+
+
+@pytest.mark.parametrize("gi, what", [
+    (1, "div of a [16,64] tile by its [16,1] row sums"),
+    (7, "div of [256,4] column pieces by whole-tile row sums"),
+    (13, "div, tiles cut along the last dim of both inputs, stored along rows"),
+    (22, "partial denominators folded, div, then the partial numerators folded"),
+    (23, "both folds first, then div"),
+    (28, "div inside a for-loop of 16, the saver accumulates"),
+    (60, "div of [256,4] column pieces by their own copy of the row sums"),
+])
+def test_recorded_second_operators_take_the_fused_fold(rt, abi, gi, what):
+    """Every shape of second operator in the recorded programs -- the division before, after or
+    without the folds, inside a for-loop, on 4-column pieces -- runs on the fused fold kernel
+    and matches the golden."""
+    from helpers import load_gqa_fixture
+    spec = load_gqa_fixture()["generated_graphs"][gi]
+    ins = _inputs(spec, 0.05, 270 + gi)
+    ins[2] = np.abs(ins[2])  # (steadily growing sums in the first operator, see above)
+    _check(rt, spec, ins, f"fixture graph {gi}: {what}", threads=16)
+    assert _last_kernels == [KERNEL_ATTENTION, KERNEL_COMBINE], _last_kernels
+
+
 def test_attention_throughput_variant(rt, abi):
     """the pipelined 32-rows-per-wavefront variant, forced on small problems: both forms,
     both head sizes"""

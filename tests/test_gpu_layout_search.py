@@ -98,17 +98,18 @@ def test_optimize_layout_measured(rt, abi):
 
 
 def test_a_pruned_layout_is_slower(rt, abi, declared_layouts):
-    """What the validity rules are for: B declared row-major is not k-contiguous, the tile
-    matmul leaves the matrix cores, and the op takes several times longer."""
+    """What the validity rules are for: A declared column-major is not k-contiguous, the tile
+    matmul leaves the matrix cores, and the op takes several times longer.  (B may be staged
+    either way: a row-major B tile is gathered with transposing LDS reads.)"""
     times = {}
-    for lb in ("SmemColumnMajorTensorOpMultiplicand_Crosswise32", "SmemRowMajor"):
+    for la in ("SmemRowMajorTensorOpMultiplicand_Crosswise32", "SmemColumnMajor"):
         g, vals = rt.build_from_spec(
-            _matmul_spec(["SmemRowMajorTensorOpMultiplicand_Crosswise32", lb]))
+            _matmul_spec([la, "SmemColumnMajorTensorOpMultiplicand_Crosswise32"]))
         try:
             vals[0][0].write_data(normal_f16([64, 1024], 0.1, 10))
             vals[1][0].write_data(normal_f16([1024, 1024], 0.1, 11))
-            times[lb] = g.profile(2)
+            times[la] = g.profile(2)
         finally:
             g.close()
     print("ms per launch:", times, flush=True)
-    assert times["SmemRowMajor"] > 2.0 * times["SmemColumnMajorTensorOpMultiplicand_Crosswise32"]
+    assert times["SmemColumnMajor"] > 2.0 * times["SmemRowMajorTensorOpMultiplicand_Crosswise32"]
