@@ -222,10 +222,13 @@ bool cmatch(DevProgram const &P, CMatch &M) {
     return false;
   }
   // the divisor does not move with the for-loop; the numerator may (one piece an iteration)
-  if (opd.row_fs != 0 || opd.col_fs != 0 || opd.g_fs != 0) {
+  // (the strides of a single iteration mean nothing)
+  if (F > 1 && (opd.row_fs != 0 || opd.col_fs != 0 || opd.g_fs != 0)) {
     return false;
   }
-  M.step = mode == DIV_THEN_SAVE ? (long long)opn.g_fs + (long long)opn.row_fs * opn.d_cols + opn.col_fs : X;
+  M.step = mode != DIV_THEN_SAVE ? X
+           : F > 1 ? (long long)opn.g_fs + (long long)opn.row_fs * opn.d_cols + opn.col_fs
+                   : 0;
   M.vec = X % 8 == 0 ? 8 : (X % 4 == 0 ? 4 : 0);
   if (M.vec == 0 || M.step % M.vec != 0 || !aligned(ctile(opn, P.in[opn.io]), M.vec) ||
       !aligned(ctile(out, P.out[out.io]), M.vec)) {

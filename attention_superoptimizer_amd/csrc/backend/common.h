@@ -82,6 +82,7 @@ struct State {
   int fp_vector_dot_only = 0;  // 1: fingerprint matmuls never take the matrix-core kernels
   int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
   int direct_lanes = 0;      // MI355_OPT_DIRECT_LANES
+  int gemm_mode = 0;         // MI355_OPT_GEMM_MODE
   // phase timestamps of the direct-staging attention kernel (MI355_OPT_PHASE_TRACE): while
   // set, launches of that kernel record six wall-clock stamps per wavefront here
   unsigned long long *phase_trace = nullptr;        // null while tracing is off

@@ -8,7 +8,10 @@
 //                                                                 cpp_examples/lora.cc:45-67)
 //
 // These are HBM-bound: what matters is how many bytes of weights are in flight, not
-// the MFMAs.  Design:
+// the MFMAs.  Two kernels.  gemm_lanes_kernel (further down) runs a plan in ONE launch with
+// the output tile cut into 16 x 16 pieces, one workgroup each, whose wavefronts take the
+// for-loop's iterations side by side; it serves the launch-bound members.  gemm_fused_kernel
+// cuts the for-loop instead and needs a second launch to add the ranges.  Its design:
 //  * the plan's grid is a lower bound on parallelism.  Each logical block's for-loop
 //    is cut into `ksplit` contiguous ranges handled by different workgroups, sized so
 //    that a few workgroups sit on every compute unit; a workgroup issues every load
@@ -465,6 +468,249 @@ __global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
   }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// One launch, no scratch: the output tile of a logical block is cut into 16-row x 16-column
+// pieces and every piece is a workgroup of its own (four pieces across the 64 columns, one
+// row of pieces per 16 activation rows), so a plan with a handful of blocks still covers the
+// chip.  Inside a workgroup the wavefronts are ITERATION LANES: lane ip takes iterations ip,
+// ip + IP, ... of the for-loop and needs nobody else for them --
+//   * its activation rows arrive as MFMA operands straight from global memory (a lane's eight
+//     consecutive k of one row are 16 contiguous bytes), the element-wise prologue is applied
+//     in registers;
+//   * its 16-column strip of each weight tile ([KT][16], 32 contiguous bytes per k) is copied
+//     by direct-to-LDS loads into a buffer of its own and read back with transposing LDS
+//     reads, which hand a lane the eight consecutive k of one column;
+//   * one wait for all of its loads, then KT / 32 MFMAs per weight matrix (weights as the
+//     first operand: a lane ends up with four consecutive columns of one row);
+// so the workgroup is IP independent streams with no barrier in the loop.  Every iteration's
+// product piece is rounded to fp16 into an LDS slot of its own; after ONE barrier the
+// pieces are added in ITERATION order, rounding to fp16 after each add -- the arithmetic of
+// the sequential loop (src/kernel/triton_code_gen.cc:223-232) -- and stored.
+// Workgroup ids put the four column pieces of a block on ids that are equal modulo 8, i.e. on
+// one XCD: the 128-byte lines of a weight row that the pieces share are fetched into one L2.
+struct LaneParams {
+  GemmParams g;
+  int gx, gy;        // the plan's grid (x, y): the logical block index is decoded from a flat id
+  int blocks;        // logical blocks
+  int mtiles;        // 16-row pieces per block
+  int slot_base;     // byte offset of the product slots in LDS (after the lanes' buffers)
+};
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void lane_dma16(_Float16 const *gbase, uint32_t lane_byte_offset,
+                                           uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(lane_byte_offset),
+                 "s"(gbase)
+               : "m0", "memory");
+}
+#pragma clang diagnostic pop
+__device__ __forceinline__ uint32_t lane_lds_address(void const *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void const *)p;
+}
+// within 16 lanes, lane 4a + b names four halfs T[row0 + a][col0 + 4b ..]; lane i receives
+// T[row0 + 0..3][col0 + i]
+__device__ __forceinline__ half4 lane_tr16(_Float16 const *p) {
+  typedef short short4v __attribute__((ext_vector_type(4)));
+  short4v const v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (short4v __attribute__((address_space(3))) *)(__attribute__((address_space(3))) void *)(p));
+  return __builtin_bit_cast(half4, v);
+}
+
+template <int KT, int NB, int PRO, bool LORA>
+__global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
+  GemmParams const &P = L.g;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  constexpr int KS = KT / 32;                                // MFMA steps (and 1 KB loads) per strip
+  constexpr int STRIPS = NB + (LORA ? 1 : 0);
+  constexpr int WAVE_BYTES = STRIPS * KT * 32 + (LORA ? 512 : 0);  // + the [16][16] piece of lora B
+  int const tid = threadIdx.x, lane = tid % 64, IP = blockDim.x / 64;
+  int const ip = __builtin_amdgcn_readfirstlane(tid / 64);  // (wave-uniform: addresses stay scalar)
+  int const g = lane / 16, c = lane % 16;
+  int const F = P.forloop_range, M = P.M;
+
+  // flat id -> (logical block, row piece, column piece): ids that differ by 8 x piece index
+  // share a block
+  int const S = 4 * L.mtiles;
+  int const id = blockIdx.x;
+  int const blk = (id / (8 * S)) * 8 + id % 8, sub = (id / 8) % S;
+  if (blk >= L.blocks) {
+    return;
+  }
+  int const piece = sub % 4, mt = sub / 4;
+  int const bx = blk % L.gx, by = (blk / L.gx) % L.gy, bz = blk / (L.gx * L.gy);
+  int const n0 = 16 * piece;
+
+  unsigned char *mine = lds + ip * WAVE_BYTES;
+  _Float16 const *strip[STRIPS];
+#pragma unroll
+  for (int b = 0; b < STRIPS; b++) {
+    strip[b] = reinterpret_cast<_Float16 const *>(mine + b * KT * 32);
+  }
+  _Float16 const *lb_piece = reinterpret_cast<_Float16 const *>(mine + STRIPS * KT * 32);
+  _Float16 *slots = reinterpret_cast<_Float16 *>(lds + L.slot_base);  // [F][NB][16][16]
+
+  // this lane's place in a strip load (64 lanes x 16 bytes = 32 rows of 32 bytes) and in the
+  // transposing reads
+  int const ld_row = lane / 2, ld_half = lane % 2;
+  int const tr_off = (c / 4) * 16 + 4 * (c % 4);
+  int const row = 16 * mt + c;                 // activation row of this lane's fragments
+  bool const row_ok = row < M;
+  int const row_ld = row_ok ? row : M - 1;
+
+  if (LORA) {
+    // lora B [16][64], loop invariant: this piece's 16 columns, rows of 32 bytes
+    _Float16 const *src = static_cast<_Float16 const *>(P.lb.ptr) + gtile_offset(P.lb, bx, by, bz, 0) + n0;
+    if (lane < 32) {
+      lane_dma16(src, (uint32_t)((ld_row * P.lb.d_cols + 8 * ld_half) * 2), lane_lds_address(lb_piece));
+    }
+  }
+
+  for (int it = ip; it < F; it += IP) {
+    // ---- issue everything this iteration needs -------------------------------------------
+#pragma unroll
+    for (int b = 0; b < STRIPS; b++) {
+      GTile const &bt = b == NB ? P.la : (b == 0 ? P.b0 : P.b1);
+      int const col0 = b == NB ? 0 : n0;  // the lora A tile is [KT][16]: whole
+      _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it) + col0;
+      uint32_t const off = (uint32_t)((ld_row * bt.d_cols + 8 * ld_half) * 2);
+#pragma unroll
+      for (int j = 0; j < KS; j++) {
+        lane_dma16(src + (long long)(32 * j) * bt.d_cols, off, lane_lds_address(strip[b]) + j * 1024);
+      }
+    }
+    _Float16 const *a0 = static_cast<_Float16 const *>(P.a0.ptr) + gtile_offset(P.a0, bx, by, bz, it) +
+                         (long long)row_ld * P.a0.d_cols + 8 * g;
+    uint4v xr[KS], ur[PRO == PRO_SILU_MUL ? KS : 1];
+#pragma unroll
+    for (int j = 0; j < KS; j++) {
+      xr[j] = *reinterpret_cast<uint4v const *>(a0 + 32 * j);
+    }
+    if (PRO == PRO_SILU_MUL) {
+      _Float16 const *a1 = static_cast<_Float16 const *>(P.a1.ptr) + gtile_offset(P.a1, bx, by, bz, it) +
+                           (long long)row_ld * P.a1.d_cols + 8 * g;
+#pragma unroll
+      for (int j = 0; j < KS; j++) {
+        ur[j] = *reinterpret_cast<uint4v const *>(a1 + 32 * j);
+      }
+    }
+    // ---- one wait for all of it (direct-to-LDS loads and register loads do not complete in
+    // one order, so nothing short of "all" says that a particular one has landed) ------------
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+    for (int j = 0; j < KS; j++) {
+      asm volatile("" : "+v"(xr[j]));  // (no use of a fragment moves above the wait)
+      if (PRO == PRO_SILU_MUL) {
+        asm volatile("" : "+v"(ur[j]));
+      }
+    }
+#pragma clang diagnostic pop
+    // ---- activation fragments: rows past M are zero, prologue in registers -----------------
+    half8 x[KS];
+#pragma unroll
+    for (int j = 0; j < KS; j++) {
+      half8 v = __builtin_bit_cast(half8, xr[j]);
+      if (PRO == PRO_EXP || PRO == PRO_SILU) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          v[e] = static_cast<_Float16>(prologue(PRO, static_cast<float>(v[e])));
+        }
+      } else if (PRO == PRO_SILU_MUL) {
+        half8 const u = __builtin_bit_cast(half8, ur[j]);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          _Float16 const sg = static_cast<_Float16>(prologue(PRO_SILU, static_cast<float>(v[e])));
+          v[e] = static_cast<_Float16>(static_cast<float>(sg) * static_cast<float>(u[e]));
+        }
+      }
+      if (!row_ok) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          v[e] = (_Float16)0.0f;
+        }
+      }
+      x[j] = v;
+    }
+    // ---- lora inner product, transposed: d[r] = (X.A)[m = c][n = 4g + r] -------------------
+    half4 dfrag = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
+    if (LORA) {
+      float4v d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < KS; j++) {
+        _Float16 const *ap = strip[NB] + (32 * j + 8 * g) * 16 + tr_off;
+        half4 const lo = lane_tr16(ap), hi = lane_tr16(ap + 64);
+        half8 const a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, x[j], d, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        dfrag[r] = static_cast<_Float16>(d[r]);
+      }
+    }
+    // ---- products: o[r] = O[m = c][n = n0 + 4g + r] ----------------------------------------
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      float4v o = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < KS; j++) {
+        _Float16 const *wp = strip[b] + (32 * j + 8 * g) * 16 + tr_off;
+        half4 const lo = lane_tr16(wp), hi = lane_tr16(wp + 64);
+        half8 const w = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, x[j], o, 0, 0, 0);
+      }
+      if (LORA) {
+        half4 const w = lane_tr16(lb_piece + (4 * g) * 16 + tr_off);  // B[k = 4g ..][n = c]
+        o = __builtin_amdgcn_mfma_f32_16x16x16f16(w, dfrag, o, 0, 0, 0);
+      }
+      half4 p16;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        p16[r] = static_cast<_Float16>(o[r]);
+      }
+      *reinterpret_cast<half4 *>(slots + ((it * NB + b) * 16 + c) * 16 + 4 * g) = p16;
+    }
+  }
+  __syncthreads();
+  // ---- the saver: pieces added in iteration order, two neighbouring columns per thread ----
+  typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+  for (int e = tid; e < NB * 128; e += blockDim.x) {
+    int const b = e / 128, r = (e % 128) / 8, col = (e % 8) * 2;
+    _Float16 const *sp = slots + (b * 16 + r) * 16 + col;
+    float a0 = 0.0f, a1 = 0.0f;  // hold fp16 values between the adds
+    int q = 0;
+    for (; q + 8 <= F; q += 8) {
+      half2v v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        v[u] = *reinterpret_cast<half2v const *>(sp + (q + u) * NB * 256);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        a0 = static_cast<float>(static_cast<_Float16>(a0 + static_cast<float>(v[u][0])));
+        a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[u][1])));
+      }
+    }
+    for (; q < F; q++) {
+      half2v const v = *reinterpret_cast<half2v const *>(sp + q * NB * 256);
+      a0 = static_cast<float>(static_cast<_Float16>(a0 + static_cast<float>(v[0])));
+      a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[1])));
+    }
+    if (16 * mt + r < M) {
+      GTile const &ot = b == 0 ? P.o0 : P.o1;
+      _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(ot.ptr)) + gtile_offset(ot, bx, by, bz, 0);
+      half2v out;
+      out[0] = static_cast<_Float16>(a0);
+      out[1] = static_cast<_Float16>(a1);
+      *reinterpret_cast<half2v *>(og + (long long)(16 * mt + r) * ot.d_cols + n0 + col) = out;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // host: recognise the family and launch
 // ---------------------------------------------------------------------------------------
@@ -624,6 +870,92 @@ int launch_kt(GemmParams const &A, dim3 grid, int lds) {
   return go(gemm_fused_kernel<MT, NB, PRO, LORA, 512>);
 }
 
+// gemm_lanes_kernel for this plan, or 0 when it is not the better choice (see the rule in
+// try_launch_lanes); k extents 64 / 128 / 256.
+template <int NB, int PRO, bool LORA>
+int launch_lanes_kt(LaneParams const &L, int grid, int threads, int lds) {
+  State &s = state();
+  auto go = [&](auto *fn) -> int {
+    if (lds > 65536) {
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    }
+    fn<<<grid, threads, lds, s.stream()>>>(L);
+    MI355_HIP(hipGetLastError());
+    return 1;
+  };
+  switch (L.g.KT) {
+    case 64:
+      return go(gemm_lanes_kernel<64, NB, PRO, LORA>);
+    case 128:
+      return go(gemm_lanes_kernel<128, NB, PRO, LORA>);
+    case 256:
+      return go(gemm_lanes_kernel<256, NB, PRO, LORA>);
+    default:
+      return 0;
+  }
+}
+
+int try_launch_lanes(DevProgram const &P, GMatch const &G, GemmParams const &A) {
+  State &s = state();
+  if (s.gemm_mode == 1 || !(G.KT == 64 || G.KT == 128 || G.KT == 256)) {
+    return 0;
+  }
+  long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
+  int const mtiles = (G.M + 15) / 16, S = 4 * mtiles, F = P.forloop_range;
+  long long const groups = (blocks + 7) / 8;
+  if (groups * 8 * S > 2147483647LL) {
+    return 0;
+  }
+  // By itself only where the launch, not the traffic, sets the time (weights of a few MB): a
+  // 16-column strip uses 32 bytes of every 128-byte line it pulls into a compute unit's L1, and
+  // every piece re-reads the activation rows, so the L2 -> L1 traffic is 4-5 x the bytes of the
+  // plan (measured on the LoRA plan: 202 MB of requests for 34 MB), which is what bounds a plan
+  // of tens of MB; the range-splitting kernel moves whole lines once.
+  long long const weight_bytes = blocks * F * (long long)(G.nb * G.KT * 64 + (G.lora ? G.KT * 16 : 0)) * 2;
+  if (s.gemm_mode == 0 && (blocks * S > 1024 || weight_bytes > (8LL << 20))) {
+    return 0;
+  }
+  int const strips = G.nb + (G.lora ? 1 : 0);
+  int const wave_bytes = strips * G.KT * 32 + (G.lora ? 512 : 0);
+  int const slot_bytes = F * G.nb * 512;
+  int ip = F < 16 ? F : 16;
+  while (ip > 1 && ip * wave_bytes + slot_bytes > s.max_lds) {
+    ip = (ip + 1) / 2;
+  }
+  if (ip * wave_bytes + slot_bytes > s.max_lds) {
+    return 0;
+  }
+  LaneParams L{};
+  L.g = A;
+  L.gx = P.grid[0];
+  L.gy = P.grid[1];
+  L.blocks = (int)blocks;
+  L.mtiles = mtiles;
+  L.slot_base = ip * wave_bytes;
+  int const lds = ip * wave_bytes + slot_bytes, grid = (int)(groups * 8 * S);
+  int rc = 0;
+#define MI355_LANES_CASE(NBV, PROV, LORAV)                                  \
+  if (G.nb == NBV && G.pro == PROV && G.lora == LORAV) {                    \
+    rc = launch_lanes_kt<NBV, PROV, LORAV>(L, grid, ip * 64, lds);          \
+  }
+  MI355_LANES_CASE(1, PRO_NONE, false)
+  MI355_LANES_CASE(1, PRO_EXP, false)
+  MI355_LANES_CASE(1, PRO_SILU, false)
+  MI355_LANES_CASE(2, PRO_NONE, false)
+  MI355_LANES_CASE(1, PRO_SILU_MUL, false)
+  MI355_LANES_CASE(1, PRO_NONE, true)
+#undef MI355_LANES_CASE
+  if (rc == 1) {
+    s.last().kernel_id = MI355_KERNEL_F16_GEMM;
+    s.last().workgroups = grid;
+    s.last().threads = ip * 64;
+    s.last().lds_bytes = lds;
+    s.last().row_split = S;
+  }
+  return rc;
+}
+
 }  // namespace
 
 bool gemm_applicable(DevProgram const &P) {
@@ -650,6 +982,9 @@ int try_launch_gemm(DevProgram const &P) {
   A.M = G.M;
   A.KT = G.KT;
   A.forloop_range = P.forloop_range;
+  if (int const rc = try_launch_lanes(P, G, A)) {
+    return rc;
+  }
   int const mt = (G.M + 15) / 16;
   long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
   // Ranges per block: the split that minimises (rounds of resident workgroups) x

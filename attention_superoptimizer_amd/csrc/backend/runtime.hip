@@ -269,6 +269,10 @@ extern "C" int mi355_set_option(int option, int value) {
     state().direct_lanes = value;
     return MI355_OK;
   }
+  if (option == MI355_OPT_GEMM_MODE && value >= 0 && value <= 2) {
+    state().gemm_mode = value;
+    return MI355_OK;
+  }
   if (option == MI355_OPT_PHASE_TRACE && (value == 0 || value == 1)) {
     MI355_REQUIRE_INIT();
     State &s = state();

@@ -124,6 +124,13 @@ typedef struct mi355_launch_info {
  * group per wavefront always; 4 = four double-buffered lanes for a lone row group.  Results
  * are identical; a measurement knob that the tests use to cover every instantiation. */
 #define MI355_OPT_DIRECT_LANES 6
+/* GEMM_MODE: which fused kernel runs a skinny-GEMM plan.  0 = chosen by the backend (one
+ * launch with the output tile cut into 16 x 16 pieces for plans that would otherwise leave
+ * most of the chip idle; the for-loop cut into ranges, plus a launch that adds them, for
+ * plans whose traffic, not the launch, sets the time); 1 = always the range-splitting kernel; 2 = the one-launch
+ * kernel wherever it applies.  Both keep the accumulation order of the sequential loop;
+ * results agree to the last bit.  A measurement knob that the tests use to cover both. */
+#define MI355_OPT_GEMM_MODE 7
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor

@@ -26,6 +26,18 @@ def path(request, abi):
     assert abi.mi355_set_option(1, 0) == 0
 
 
+@pytest.fixture(params=["ranges", "pieces", "interpreter"])
+def gemm_path(request, abi):
+    """The skinny-GEMM plans on each route: the fused kernel that cuts the for-loop into ranges
+    (plus the launch that adds them), the one-launch kernel that cuts the output tile into
+    pieces, and the generic LDS interpreter."""
+    assert abi.mi355_set_option(1, 1 if request.param == "interpreter" else 0) == 0
+    assert abi.mi355_set_option(7, {"ranges": 1, "pieces": 2, "interpreter": 0}[request.param]) == 0
+    yield "fused" if request.param != "interpreter" else "interpreter"
+    assert abi.mi355_set_option(7, 0) == 0
+    assert abi.mi355_set_option(1, 0) == 0
+
+
 def _graph_f16(rt, spec, inputs):
     import ctypes
     from attention_superoptimizer_amd import _native as N
@@ -83,7 +95,8 @@ def _expect(path, fused_kernel):
     return fused_kernel if path == "fused" else KERNEL_INTERP
 
 
-def test_config1_fused_matmul(rt, path):
+def test_config1_fused_matmul(rt, gemm_path):
+    path = gemm_path
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config1_fused_matmul()
     ins = _inputs(spec, W.INPUT_STD["C1_fused_matmul"], 10)
@@ -139,7 +152,8 @@ def test_config3_single_kv_block(rt, path):
                              else [KERNEL_INTERP, KERNEL_INTERP])
 
 
-def test_config4_lora(rt, path):
+def test_config4_lora(rt, gemm_path):
+    path = gemm_path
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config4_lora()
     ins = _inputs(spec, W.INPUT_STD["C4_lora"], 40)
@@ -150,7 +164,8 @@ def test_config4_lora(rt, path):
     assert_f16_close(got, X @ Wm + (X @ A) @ B, rtol=1e-2, atol=4e-3, what="C4 vs float64")
 
 
-def test_config5_gated_mlp_small(rt, path):
+def test_config5_gated_mlp_small(rt, gemm_path):
+    path = gemm_path
     from attention_superoptimizer_amd import workloads as W
     spec, ref = W.config5_gated_mlp(m=8, d=1024, h=3584, grid1=56, F1=4, grid2=16, F2=14)
     ins = _inputs(spec, W.INPUT_STD["C5a_gated_mlp"], 50)
@@ -162,9 +177,10 @@ def test_config5_gated_mlp_small(rt, path):
     assert_f16_close(got, exact, rtol=2e-2, atol=4e-3, what="C5a vs float64")
 
 
-def test_gemm_family_shapes(rt, path):
+def test_gemm_family_shapes(rt, gemm_path):
     """for-loop split over workgroups (few blocks) and unsplit (many blocks), 16/32/64-row
     tiles, exp prologue"""
+    path = gemm_path
     from attention_superoptimizer_amd import workloads as W
     cases = {
         "unsplit": W.tiled_matmul(1024, 4096, 128, (16, 64, 1), 2, (0, -1, -1), (-1, 1, -1), (0, 1, -1)),
@@ -379,6 +395,30 @@ def test_attention_latency_variants_agree(rt, abi):
             for a, b in zip(outs[0, 0], outs[other]):
                 for x, y in zip(a, b):
                     assert np.array_equal(x, y), (what, other)
+
+
+def test_gemm_kernels_agree_to_the_last_bit(rt, abi):
+    """Full-size C1, C4 and C5a on the two fused GEMM kernels: both round every iteration's
+    product tile to fp16 and add the tiles in iteration order, so they agree bit for bit."""
+    from attention_superoptimizer_amd import workloads as W
+    for name in ("C1_fused_matmul", "C4_lora", "C5a_gated_mlp"):
+        spec, _ = W.BASELINE_CONFIGS[name]()
+        ins = _inputs(spec, W.INPUT_STD[name], 0xBEEF00)
+        outs = {}
+        for mode in (1, 2):
+            assert abi.mi355_set_option(7, mode) == 0
+            try:
+                outs[mode] = _graph_f16(rt, spec, ins)
+                assert all(k == KERNEL_GEMM for k in _last_kernels), (name, mode, _last_kernels)
+                info = N_launch_info()
+                print(name, "mode", mode, "workgroups", info.workgroups, "threads", info.threads,
+                      "lds", info.lds_bytes, "split", info.row_split, flush=True)
+            finally:
+                assert abi.mi355_set_option(7, 0) == 0
+        for i, op in enumerate(spec):
+            if op["op"] == "customized":
+                for a, b in zip(outs[1][i], outs[2][i]):
+                    assert np.array_equal(a, b), (name, i)
 
 
 def test_full_size_configs_routes_agree(rt, abi):
