@@ -86,6 +86,7 @@ struct Searcher {
   LayoutSearchConfig const &cfg;
   LayoutSearchResult res;
   std::map<std::pair<int, std::vector<int>>, float> known;  // (operator, loader layouts) -> ms
+  std::map<int, float> fused_cost;  // operators that took a fused kernel: their (only) time
   std::vector<int> best;                                    // snapshot of every layout
   bool have_best = false;
 
@@ -148,6 +149,12 @@ struct Searcher {
     if (it != known.end()) {
       return it->second;
     }
+    // an operator that ran on a fused kernel keeps its tiles in registers / its own LDS
+    // layout: no declared layout can change its time, one measurement stands for all
+    auto fl = fused_cost.find(op_idx);
+    if (fl != fused_cost.end()) {
+      return fl->second;
+    }
     float ms;
     if (cfg.cost) {
       ms = cfg.cost(op);
@@ -155,6 +162,11 @@ struct Searcher {
       ProfileResult r;
       op->profile(r);
       ms = r.run_time;
+      mi355_launch_info li{};
+      if (op->op_type == KN_CUSTOMIZED_OP && mi355_last_launch(&li) == MI355_OK &&
+          li.kernel_id != MI355_KERNEL_F16_INTERP) {
+        fused_cost[op_idx] = ms;
+      }
     }
     res.measurements++;
     known[{op_idx, key}] = ms;

@@ -41,7 +41,9 @@ struct LayoutSearchConfig {
 
 struct LayoutSearchResult {
   long long assignments = 0;   // complete layout assignments evaluated
-  long long measurements = 0;  // operator costs actually measured (the rest were known)
+  long long measurements = 0;  // operator costs actually measured (the rest were known: same
+                               // loader layouts seen before, or an operator that ran on a fused
+                               // kernel, whose time no declared layout can change)
   bool truncated = false;
   float first_run_time = 0.0f;  // total of the first assignment evaluated
   float best_run_time = 0.0f;

@@ -113,3 +113,22 @@ def test_a_pruned_layout_is_slower(rt, abi, declared_layouts):
             g.close()
     print("ms per launch:", times, flush=True)
     assert times["SmemColumnMajor"] > 2.0 * times["SmemRowMajorTensorOpMultiplicand_Crosswise32"]
+
+
+def test_a_fused_operator_is_measured_once(rt, abi):
+    """With the fused routes on (the default), C1's customized op runs on a fused GEMM kernel
+    that keeps its tiles in its own layout: the search measures the kernel that actually runs,
+    once, and every one of the 72 assignments gets that time."""
+    from attention_superoptimizer_amd import graph as G
+    g, vals = rt.build_from_spec(_matmul_spec(["SmemUnknownLayout"] * 2))
+    try:
+        vals[0][0].write_data(normal_f16([64, 1024], 0.1, 10))
+        vals[1][0].write_data(normal_f16([1024, 1024], 0.1, 11))
+        fused_ms = g.profile(2)
+        st = G.optimize_layout(g)
+        print("layout search on the fused route:", st, "fused", fused_ms, flush=True)
+        assert st["assignments"] == 72 and st["measurements"] == 3 and not st["truncated"]
+        assert st["best_ms"] == st["worst_ms"]
+        assert st["best_ms"] < 3.0 * fused_ms
+    finally:
+        g.close()
