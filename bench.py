@@ -216,12 +216,19 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
         "candidates_per_s_by_family": {k: round(v[0] / v[1], 1) for k, v in sorted(fam.items())},
         "inputs": "uniform [0, 25651) from (seed, input index)",
     }
-    if in_flight > 1:
+    if in_flight > 1 and per_problem == 64:
         one = fingerprint_throughput(G, False, num_problems, per_problem, 1, 4)
         G.set_verify_queues_per_batch(4)
         rec["one_submission_in_flight"] = {k: one[k] for k in (
             "candidates_per_s", "verify_s", "host_enqueue_s", "final_wait_s",
             "candidates_per_s_by_family")}
+        # the same number of candidates against a quarter of the problems: what a submission
+        # costs is mostly its chain of launches, which 256 candidates share instead of 64
+        big = fingerprint_throughput(G, False, num_problems // 4, per_problem * 4, 2, 4)
+        G.set_verify_queues_per_batch(4)
+        rec["submissions_of_256_candidates"] = {k: big[k] for k in (
+            "candidates", "problems", "candidates_per_s", "verify_s", "verdicts_as_constructed",
+            "submissions_in_flight", "queues_per_submission", "candidates_per_s_by_family")}
     if cpu_baseline:
         # the scalar C restatement over a bounded sample: every candidate of every 4th
         # problem, once on one core and once with one candidate per host thread
