@@ -1779,8 +1779,8 @@ bool attention_applicable(DevProgram const &P) {
   Match M;
   DirectShape d;
   int lds = 0;
-  if (match(P, M)) {
-    return shape_supported(M) || choose_direct(P, M, d, lds);
+  if (match(P, M) && (shape_supported(M) || choose_direct(P, M, d, lds))) {
+    return true;
   }
   DevProgram merged;
   int copies = 1, stride = 0;
@@ -1792,7 +1792,13 @@ int try_launch_attention(DevProgram const &P0) {
   DevProgram merged;
   DevProgram const *run = &P0;
   int r_copies = 1, r_copy_stride = 0;
-  bool const pieces = !match(P0, M);
+  // as the plan states it, or (value tiles narrower than 64 columns) with its column pieces merged
+  bool pieces = !match(P0, M);
+  if (!pieces) {
+    DirectShape probe;
+    int probe_lds = 0;
+    pieces = !shape_supported(M) && !choose_direct(P0, M, probe, probe_lds);
+  }
   if (pieces) {
     if (!merge_column_pieces(P0, M, merged, r_copies, r_copy_stride)) {
       return 0;

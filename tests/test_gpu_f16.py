@@ -349,6 +349,30 @@ def test_recorded_second_operators_take_the_fused_fold(rt, abi, gi, what):
     assert _last_kernels == [KERNEL_ATTENTION, KERNEL_COMBINE], _last_kernels
 
 
+def test_column_pieces_with_the_division_inside(rt, abi):
+    """A single-op attention plan (division inside the block) whose grid cuts the value columns
+    into 4 pieces of 16: merged into one block per query tile on the fused route, same result as
+    the interpreter's block-by-block evaluation and the golden."""
+    spec = [
+        {"op": "input", "dims": [2, 64, 64]}, {"op": "input", "dims": [2, 64, 256]},
+        {"op": "input", "dims": [2, 256, 64]},
+        {"op": "customized", "in": [[0, 0], [1, 0], [2, 0]], "plan": {
+            "grid_dim": [2, 4, 2], "forloop_range": 4,
+            "input_map": [[0, -1, 1], [0, -1, -1], [0, 2, -1]], "forloop_dim": [-1, 2, 1],
+            "output_map": [0, 2, 1],
+            "ops": [["tb_matmul_op", [[0, 0], [1, 0]]], ["tb_exp_op", [[3, 0]]],
+                    ["tb_reduction_2_op", [[4, 0]]], ["tb_div_op", [[4, 0], [5, 0]]],
+                    ["tb_matmul_op", [[6, 0], [2, 0]]]]}},
+    ]
+    for force in (0, 1):
+        assert abi.mi355_set_option(1, force) == 0
+        try:
+            _check(rt, spec, _inputs(spec, 0.1, 610), f"column pieces, division inside, forced={force}")
+            assert _last_kernels == [KERNEL_INTERP if force else KERNEL_ATTENTION], _last_kernels
+        finally:
+            assert abi.mi355_set_option(1, 0) == 0
+
+
 def test_attention_throughput_variant(rt, abi):
     """the pipelined 32-rows-per-wavefront variant, forced on small problems: both forms,
     both head sizes"""
@@ -395,6 +419,30 @@ def test_attention_latency_variants_agree(rt, abi):
             for a, b in zip(outs[0, 0], outs[other]):
                 for x, y in zip(a, b):
                     assert np.array_equal(x, y), (what, other)
+
+
+def test_one_launch_gemm_shapes(rt, abi):
+    """The one-launch kernel on the shapes its lanes and pieces must cover: 8 / 16 / 48 / 64
+    activation rows, k tiles of 64 / 128 / 256, for-loops of 1, 3 (fewer iterations than lanes),
+    16 and 40 (several per lane), a block count that is no multiple of 8, a 3-D grid, LoRA with
+    a small k tile, two weights, silu * mul."""
+    from attention_superoptimizer_amd import workloads as W
+    assert abi.mi355_set_option(7, 2) == 0
+    try:
+        cases = {
+            "rows8 k64 F3": W.tiled_matmul(8, 192, 192, (3, 1, 1), 3, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),
+            "rows48 k128 F1": W.tiled_matmul(48, 320, 128, (5, 1, 1), 1, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),
+            "rows64 k256 F40": W.tiled_matmul(64, 128, 10240, (2, 1, 1), 40, (-1, -1, -1), (1, -1, -1), (1, -1, -1)),
+            "grid 2x3": W.tiled_matmul(32, 192, 256, (2, 3, 1), 4, (0, -1, -1), (-1, 1, -1), (0, 1, -1)),
+            "lora k64": W.config4_lora(m=16, d=256, r=16, grid=4, F=4),
+            "gated mlp": W.config5_gated_mlp(m=8, d=512, h=640, grid1=10, F1=4, grid2=8, F2=5),
+        }
+        for name, (spec, _) in cases.items():
+            ins = _inputs(spec, 0.1, 90)
+            _check(rt, spec, ins, name)
+            assert all(k == KERNEL_GEMM for k in _last_kernels), (name, _last_kernels)
+    finally:
+        assert abi.mi355_set_option(7, 0) == 0
 
 
 def test_gemm_kernels_agree_to_the_last_bit(rt, abi):
