@@ -455,10 +455,22 @@ __global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
           a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[u][1])));
         }
       }
-      for (; q < F; q++) {
-        half2v v = *reinterpret_cast<half2v const *>(sp + (long long)q * slab);
-        a0 = static_cast<float>(static_cast<_Float16>(a0 + static_cast<float>(v[0])));
-        a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[1])));
+      if (q < F) {
+        // the tail's loads go out together as well (past the end: the last tile again, left out
+        // of the sums), not one latency after the other
+        half2v v[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+          int const it = q + u < F ? q + u : F - 1;
+          v[u] = *reinterpret_cast<half2v const *>(sp + (long long)it * slab);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+          if (q + u < F) {
+            a0 = static_cast<float>(static_cast<_Float16>(a0 + static_cast<float>(v[u][0])));
+            a1 = static_cast<float>(static_cast<_Float16>(a1 + static_cast<float>(v[u][1])));
+          }
+        }
       }
       half2v r;
       r[0] = static_cast<_Float16>(a0);
