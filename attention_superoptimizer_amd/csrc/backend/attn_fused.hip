@@ -1589,6 +1589,9 @@ int launch_direct(AttnParams const &A, dim3 grid, DirectShape const &d, int lds,
     MI355_DIRECT(4, 1, 2, 2, 1, 1)
     MI355_DIRECT(4, 1, 2, 4, 1, 1)
     MI355_DIRECT(4, 1, 2, 8, 1, 1)
+    MI355_DIRECT(4, 1, 1, 2, 1, 1)
+    MI355_DIRECT(4, 1, 1, 4, 1, 1)
+    MI355_DIRECT(4, 1, 1, 8, 1, 1)
     MI355_DIRECT(8, 1, 1, 2, 1, 1)
     MI355_DIRECT(8, 1, 1, 4, 1, 1)
     // key tiles of 32 and 16: two / four iterations per strip
@@ -1737,8 +1740,9 @@ static bool choose_direct(DevProgram const &P, Match const &M, DirectShape &d, i
   auto round_nit = [](int per) { return per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : 8)); };
   if ((groups == 1 && units > 1) || units > 8) {
     // a lone row group (or a loop too long for a wavefront per unit: then every row group is
-    // a workgroup of its own): eight lanes with a tile pair each, or (DIRECT_LANES = 4,
-    // whole-tile iterations only) four lanes with two
+    // a workgroup of its own): eight lanes with a tile pair each; four when the grid is large
+    // enough to put two workgroups on every compute unit; or (DIRECT_LANES = 4, whole-tile
+    // iterations only) four lanes with two tile pairs each
     int const per8 = (units + 7) / 8, per4 = (units + 3) / 4;
     if (s.direct_lanes == 4 && d.spi == 1 && d.ips == 1 && per4 <= 8 && units > 4) {
       d.ip = 4;
@@ -1749,6 +1753,12 @@ static bool choose_direct(DevProgram const &P, Match const &M, DirectShape &d, i
       if (d.ips > 1) {
         d.ip = 4;
       }
+    } else if (s.direct_lanes == 0 && blocks >= 512 && units > 4 && per4 <= 8 && d.spi == 1 && d.ips == 1) {
+      // enough blocks for two workgroups on every compute unit: four single-buffered lanes (half
+      // the LDS), so that one workgroup streams while its neighbour starts up or adds up its
+      // results (the HBM-bound decode: 5.75 -> 6.3 TB/s)
+      d.ip = 4;
+      d.nit = round_nit(per4);
     } else {
       d.ip = 8;
       d.nit = round_nit(per8);

@@ -258,6 +258,19 @@ def test_decode_row_groups_on_the_direct_staging_kernel(rt, abi, rows, F, kv_blo
         assert abi.mi355_set_option(6, 0) == 0
 
 
+@pytest.mark.parametrize("F, units_per_lane", [(8, 2), (16, 4), (32, 8)])
+def test_decode_grid_large_enough_for_two_workgroups_per_cu(rt, abi, F, units_per_lane):
+    """512 blocks (64 groups x 8 key blocks) of 8 query rows: the direct-staging kernel runs them
+    as workgroups of four single-buffered lanes (73,728 B of LDS: two per compute unit), each
+    lane streaming F / 4 tile pairs, against the golden."""
+    from attention_superoptimizer_amd import workloads as W
+    spec, _ = W.gqa_inc_decode(groups=64, rows=8, seq=64 * F * 8, kv_blocks=8, F=F)
+    ins = _inputs(spec, 0.125, 700 + F)
+    ins[2] = np.abs(ins[2])  # (sums that grow steadily: an accumulator ulp stays inside the tolerance)
+    _check(rt, spec, ins, f"decode 512 blocks, F {F}", threads=16)
+    assert _last_kernels[0] == KERNEL_ATTENTION, _last_kernels
+
+
 @pytest.mark.parametrize("rows,nk,F,kv_blocks,groups", [
     (64, 32, 8, 2, 3),      # two iterations per 64-key strip, a wavefront per strip
     (64, 32, 16, 1, 3),     # ... eight strips
