@@ -1424,6 +1424,11 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       // out now (behind the one already in flight when there are two buffers)
       if (q + NBUF < nstrips) {
         int const qn = q + NBUF;
+        // (nothing of this strip may still be on its way out of LDS when the transfers that
+        // overwrite the buffer are issued, and the compiler may not move them up among the
+        // matrix instructions: the operand reads' completion is what it would move them past)
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         fetch(ip + (qn / SPI) * IP, qn % SPI, b);
       }
     }
@@ -1658,9 +1663,9 @@ int launch_shape(AttnParams const &A, bool has_div, dim3 grid, int rg, int ip, i
                  : launch_waves<D, NK, DV, false>(A, grid, rg, ip, lds);
 }
 
-template <int D, int NK, int DV, bool HAS_DIV, int RG>
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW = 2>
 int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
-  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, 2>;
+  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, RPW>;
   if (lds > 65536) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -1671,7 +1676,13 @@ int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
 }
 
 template <int D, int NK, int DV>
-int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds) {
+int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds, bool wide = false) {
+  if constexpr (D == 64) {
+    if (wide) {  // four wavefronts of 64 rows
+      return has_div ? launch_stream_one<D, NK, DV, true, 4, 4>(A, grid, lds)
+                     : launch_stream_one<D, NK, DV, false, 4, 4>(A, grid, lds);
+    }
+  }
   if (has_div) {
     return rg == 4 ? launch_stream_one<D, NK, DV, true, 4>(A, grid, lds)
                    : launch_stream_one<D, NK, DV, true, 2>(A, grid, lds);
@@ -1861,10 +1872,22 @@ int try_launch_attention(DevProgram const &P0) {
     int rgs = (M.m % 128 == 0) ? 4 : ((M.m % 64 == 0) ? 2 : 0);
     bool const shape = (M.D == 64 && M.NK == 64 && M.DV == 64) || (M.D == 128 && M.NK == 64 && M.DV == 128);
     bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512 && !pieces;
+    // Head size 64 with 256-row query tiles and enough of them for two wavefronts per SIMD:
+    // wavefronts of 64 rows.  The kernel is bound by its transposing LDS operand reads (every
+    // wavefront reads the whole K and V tile of a pass), and a 64-row wavefront reads half as
+    // much per MFMA; at head size 64 its registers still fit two wavefronts per SIMD.
+    bool wide = false;
     if (s.attention_mode == 1 || s.attention_mode == 3) {
       want = false;
     } else if (s.attention_mode == 2) {
       want = rgs != 0 && shape;
+    }
+    // (measured on the 32-group x 16,384-key decode plan: 68.8 -> 67.0 us; at head size 64 the
+    // exp / rounding work, not the LDS, is the larger share)
+    wide = want && M.D == 64 && M.m % 256 == 0 &&
+           (s.attention_mode == 2 || blocks_all * (M.m / 64) >= 2048);
+    if (wide) {
+      rgs = 8;
     }
     if (want) {
       A.split = slabs / rgs;
@@ -1878,12 +1901,12 @@ int try_launch_attention(DevProgram const &P0) {
         if (!set_grid_magics(A, grid)) {
           return 0;
         }
-        int rc = M.D == 64 ? launch_stream<64, 64, 64>(A, M.has_div, grid, rgs, lds)
+        int rc = M.D == 64 ? launch_stream<64, 64, 64>(A, M.has_div, grid, rgs, lds, wide)
                            : launch_stream<128, 64, 128>(A, M.has_div, grid, rgs, lds);
         if (rc == 1) {
           s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
           s.last().workgroups = grid.x * grid.y * grid.z;
-          s.last().threads = rgs * 64;
+          s.last().threads = wide ? 256 : rgs * 64;
           s.last().lds_bytes = lds;
           s.last().row_split = A.split;
         }

@@ -582,6 +582,11 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
   }
 
   for (int it = ip; it < F; it += IP) {
+    // (the previous iteration's operand reads must be out of LDS before the transfers that
+    // overwrite the strips are issued; the compiler would otherwise move them up among that
+    // iteration's last matrix instructions, past the waits for those reads)
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     // ---- issue everything this iteration needs -------------------------------------------
 #pragma unroll
     for (int b = 0; b < STRIPS; b++) {

@@ -386,6 +386,40 @@ def test_column_pieces_with_the_division_inside(rt, abi):
             assert abi.mi355_set_option(1, 0) == 0
 
 
+def test_streaming_kernels_are_deterministic(rt, abi):
+    """The kernels whose wavefronts stream several tiles through ONE LDS buffer each (a strip is
+    overwritten by direct-to-LDS transfers as soon as its operands have been read): 60 launches
+    of the same operator give the same bits.  (A transfer issued while operand reads of the
+    buffer were still outstanding once made whole 16-column blocks differ from run to run.)"""
+    from helpers import load_gqa_fixture
+    from attention_superoptimizer_amd import workloads as W
+    cases = [("recorded program 0, 256-key tiles as four strips, two iterations per lane",
+              load_gqa_fixture()["generated_graphs"][0], 3, 0),
+             ("direct-staging decode, four tile pairs per lane",
+              W.gqa_inc_decode(groups=64, rows=8, seq=64 * 16 * 8, kv_blocks=8, F=16)[0], 3, 0),
+             ("one-launch GEMM, five iterations per lane",
+              W.tiled_matmul(64, 128, 10240, (2, 1, 1), 40, (-1, -1, -1), (1, -1, -1), (1, -1, -1))[0], 2, 2)]
+    for what, spec, op, gemm_mode in cases:
+        assert abi.mi355_set_option(7, gemm_mode) == 0
+        g, vals = rt.build_from_spec(spec)
+        try:
+            for i, o in enumerate(spec):
+                if o["op"] == "input":
+                    vals[i][0].write_data(normal_f16(o["dims"], 0.05, 800 + i))
+            first = None
+            for run in range(60):
+                g.execute(op)
+                outs = [t.read_data().view(np.uint16).copy() for t in vals[op]]
+                if first is None:
+                    first = outs
+                else:
+                    for a, b in zip(first, outs):
+                        assert np.array_equal(a, b), f"{what}: launch {run} differs in {int((a != b).sum())} elements"
+        finally:
+            g.close()
+            assert abi.mi355_set_option(7, 0) == 0
+
+
 def test_attention_throughput_variant(rt, abi):
     """the pipelined 32-rows-per-wavefront variant, forced on small problems: both forms,
     both head sizes"""
@@ -401,6 +435,11 @@ def test_attention_throughput_variant(rt, abi):
         spec, _ = W.REFERENCE_EXAMPLES["multi_head_attn_prefill"]   # Q tile [64, 64], form B
         _check(rt, spec, _inputs(spec, 0.05, 92), "mha prefill throughput variant")
         assert _last_kernels[0] == KERNEL_ATTENTION
+        # 256-row query tiles at head size 64 run as wavefronts of 64 rows (C2 above: the form
+        # with the division inside; here the two-output form)
+        spec, _ = W.gqa_inc_decode(groups=2, rows=256, seq=1024, kv_blocks=2, F=8)
+        _check(rt, spec, _inputs(spec, 0.05, 93), "256-row tiles, two outputs, throughput variant")
+        assert _last_kernels[0] == KERNEL_ATTENTION and N_launch_info is not None
     finally:
         assert abi.mi355_set_option(2, 0) == 0
 
