@@ -388,7 +388,8 @@ def test_column_pieces_with_the_division_inside(rt, abi):
 
 def test_streaming_kernels_are_deterministic(rt, abi):
     """The kernels whose wavefronts stream several tiles through ONE LDS buffer each (a strip is
-    overwritten by direct-to-LDS transfers as soon as its operands have been read): 60 launches
+    overwritten by direct-to-LDS transfers as soon as its operands have been read), and the other
+    fused kernels: 40 launches
     of the same operator give the same bits.  (A transfer issued while operand reads of the
     buffer were still outstanding once made whole 16-column blocks differ from run to run.)"""
     from helpers import load_gqa_fixture
@@ -399,6 +400,16 @@ def test_streaming_kernels_are_deterministic(rt, abi):
               W.gqa_inc_decode(groups=64, rows=8, seq=64 * 16 * 8, kv_blocks=8, F=16)[0], 3, 0),
              ("one-launch GEMM, five iterations per lane",
               W.tiled_matmul(64, 128, 10240, (2, 1, 1), 40, (-1, -1, -1), (1, -1, -1), (1, -1, -1))[0], 2, 2)]
+    fx = load_gqa_fixture()["generated_graphs"]
+    cases += [("recorded program 22 (32-key tiles, two iterations per strip)", fx[22], 3, 0),
+              ("recorded program 41 (16-key tiles, four iterations per strip)", fx[41], 3, 0),
+              ("recorded program 60 (value columns in pieces)", fx[60], 3, 0),
+              ("C2, the headline plan", W.config2_gqa_decode()[0], 3, 0),
+              ("the reference's dnn example (8-row tiles, 8 iterations)", W.REFERENCE_EXAMPLES["dnn"][0], 3, 0),
+              ("C3 at reduced size, throughput kernel",
+               W.config3_mha_prefill(heads=4, seq=1024, hd=128, q_split=8, kv_split=1, F=16)[0], 3, 0),
+              ("LoRA, range-splitting kernel", W.config4_lora(m=16, d=1024, r=16, grid=16, F=4)[0], 4, 1),
+              ("LoRA, one-launch kernel", W.config4_lora(m=16, d=1024, r=16, grid=16, F=4)[0], 4, 2)]
     for what, spec, op, gemm_mode in cases:
         assert abi.mi355_set_option(7, gemm_mode) == 0
         g, vals = rt.build_from_spec(spec)
@@ -407,7 +418,7 @@ def test_streaming_kernels_are_deterministic(rt, abi):
                 if o["op"] == "input":
                     vals[i][0].write_data(normal_f16(o["dims"], 0.05, 800 + i))
             first = None
-            for run in range(60):
+            for run in range(40):
                 g.execute(op)
                 outs = [t.read_data().view(np.uint16).copy() for t in vals[op]]
                 if first is None:
