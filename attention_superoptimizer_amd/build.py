@@ -68,6 +68,10 @@ def build_tools():
     _run(["g++", "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", INCLUDE, "-I", "/opt/rocm/include",
           "-o", os.path.join(HERE, "mirage_profile"), os.path.join(CSRC, "examples", "profile.cc"),
           "-L" + HERE, "-lmirage_runtime", "-lmi355_backend", "-Wl,-rpath,$ORIGIN"])
+    # mirage_gfx950_rates: the MFMA / vector co-issue and LDS read-rate measurements the design
+    # notes of the fused attention kernels cite (stand-alone, links nothing of this package)
+    _run([HIPCC, "--offload-arch=gfx950", "-O3", "-w", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-o", os.path.join(HERE, "mirage_gfx950_rates"), os.path.join(CSRC, "examples", "gfx950_rates.hip")])
 
 
 def build_generated():
