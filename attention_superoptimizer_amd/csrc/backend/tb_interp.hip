@@ -1501,55 +1501,16 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
   int const n = (int)progs.size();
   // fused matmul plans take the matrix cores while the residue planes of their operand
   // tensors fit what is left of this queue's plane memory
-  // Members that multiply the same operand tensor (candidates of one problem share their
-  // inputs) share its planes: the first one splits it, the others point at the result.
-  struct SplitOperand {
-    void const *src;
-    int which, unary, slabs, rows, cols;
-    char *planes;
-  };
-  std::vector<SplitOperand> split;
   std::vector<DevProgram const *> on_matrix_cores;
   size_t planes_used = 0;
   for (int i = 0; i < n; i++) {
     size_t need = 0;
-    if (progs[i].fused == 4 && fp_mfma_gemm_fits(progs[i], exts[i], &need)) {
-      DevProgram &P = progs[i];
-      size_t bytes[2];
-      fp_mfma_plane_bytes(P, &bytes[0], &bytes[1]);
-      char *place[2] = {nullptr, nullptr};
-      int shared = 0;
-      size_t fresh = 0;
-      for (int which = 0; which < 2; which++) {
-        DevOp const &op = P.ops[P.fg[which]];
-        for (SplitOperand const &o : split) {
-          if (o.src == P.in[op.io] && o.which == which && o.unary == P.fp_unary[which] &&
-              o.slabs == P.pl_geo[3 * which] && o.rows == op.d_rows && o.cols == op.d_cols) {
-            place[which] = o.planes;
-            shared |= 1 << which;
-            break;
-          }
-        }
-        if (place[which] == nullptr) {
-          fresh += (bytes[which] + 255) / 256 * 256;
-        }
-      }
-      if (planes_used + fresh <= s.planes_bytes) {
-        for (int which = 0; which < 2; which++) {
-          if (place[which] == nullptr) {
-            DevOp const &op = P.ops[P.fg[which]];
-            place[which] = s.planes() + planes_used;
-            planes_used += (bytes[which] + 255) / 256 * 256;
-            split.push_back(SplitOperand{P.in[op.io], which, P.fp_unary[which], P.pl_geo[3 * which],
-                                         op.d_rows, op.d_cols, place[which]});
-          }
-        }
-        fp_mfma_gemm_bind(P, place[0], place[1], shared);
-        on_matrix_cores.push_back(&progs[i]);
-        continue;
-      }
-    }
-    if (progs[i].fused == 4 && fp_needs_matrix_cores(progs[i])) {
+    if (progs[i].fused == 4 && fp_mfma_gemm_fits(progs[i], exts[i], &need) &&
+        planes_used + need <= s.planes_bytes) {
+      fp_mfma_gemm_bind(progs[i], s.planes() + planes_used);
+      planes_used += (need + 255) / 256 * 256;
+      on_matrix_cores.push_back(&progs[i]);
+    } else if (progs[i].fused == 4 && fp_needs_matrix_cores(progs[i])) {
       // (the caller cuts chunks so that the planes of their members fit together)
       return fail(MI355_ERR_UNSUPPORTED, "operand prologue without the matrix-core route");
     }
