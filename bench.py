@@ -280,6 +280,9 @@ def main() -> int:
     ap.add_argument("--gemm-mode", type=int, default=0, choices=(0, 1, 2),
                     help="with --only: which fused skinny-GEMM kernel runs (0 the backend's choice, 1 the "
                          "range-splitting kernel, 2 the one-launch kernel)")
+    ap.add_argument("--attention-mode", type=int, default=0, choices=(0, 1, 2, 3),
+                    help="with --only: which fused attention kernel runs (0 the backend's choice; see "
+                         "MI355_OPT_ATTENTION_MODE)")
     ap.add_argument("--fp-matmul", default="", metavar="B,M,N,K",
                     help="time the kernel-level fingerprint matmul of that shape on the matrix-core "
                          "route and on the vector-dot route and print both (used under the profiler)")
@@ -395,6 +398,7 @@ def main() -> int:
     if args.only:
         spec, g, vals = setup(args.only)
         assert abi.mi355_set_option(7, args.gemm_mode) == 0
+        assert abi.mi355_set_option(2, args.attention_mode) == 0
         out = {}
         for i, op in enumerate(spec):
             if op["op"] != "customized":
