@@ -1873,8 +1873,8 @@ int try_launch_attention(DevProgram const &P0) {
     bool const shape = (M.D == 64 && M.NK == 64 && M.DV == 64) || (M.D == 128 && M.NK == 64 && M.DV == 128);
     bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512 && !pieces;
     // Head size 64 with 256-row query tiles and enough of them for two wavefronts per SIMD:
-    // wavefronts of 64 rows.  The kernel is bound by its transposing LDS operand reads (every
-    // wavefront reads the whole K and V tile of a pass), and a 64-row wavefront reads half as
+    // wavefronts of 64 rows.  The transposing LDS operand reads are the largest share of a pass
+    // (every wavefront reads the whole K and V tile), and a 64-row wavefront reads half as
     // much per MFMA; at head size 64 its registers still fit two wavefronts per SIMD.
     bool wide = false;
     if (s.attention_mode == 1 || s.attention_mode == 3) {
