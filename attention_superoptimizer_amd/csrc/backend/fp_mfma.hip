@@ -388,16 +388,19 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
   int const F = P.forloop_range;
   int const it_begin = (int)((long long)F * split / P.splits);
   int const it_end = (int)((long long)F * (split + 1) / P.splits);
-  int const Q = (it_end - it_begin) * cpi, steps = (Q + 3) / 4;
-  // An operator applied to every iteration's product (k tiles are multiples of 64 then, so an
-  // iteration is a whole number of steps): after its last step the two sums become a
-  // fingerprint value, the operator is applied and the result added to a running sum.
-  int const epi = P.fp_unary[2], spi = cpi / 4;
+  // An operator applied to every iteration's product: an iteration is a whole number of steps
+  // (k tiles of 16, 32 or 48 take one step in which only the first one, two or three lane
+  // groups hold a chunk; longer k tiles are multiples of 64); after its last step the two sums
+  // become a fingerprint value, the operator is applied and the result added to a running sum.
+  int const epi = P.fp_unary[2];
+  int const cps = epi != 0 && cpi < 4 ? cpi : 4;  // chunks per step
+  int const spi = cpi / cps;                        // steps per iteration (with an operator)
+  int const Q = (it_end - it_begin) * cpi, steps = (Q + cps - 1) / cps;
   int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
   int const a0 = bx * P.pl_a[0] + by * P.pl_a[1] + bz * P.pl_a[2] + it_begin * P.pl_a[3];
   int const b0 = bx * P.pl_b[0] + by * P.pl_b[1] + bz * P.pl_b[2] + it_begin * P.pl_b[3];
   int const a_it = P.pl_a[3], b_it = P.pl_b[3];
-  int const dq_it = 4 / cpi, dq_c = 4 % cpi;
+  int const dq_it = cps / cpi, dq_c = cps % cpi;
   int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
   int const ways = mt >= 3 ? 1 : (mt == 2 ? 2 : 4);  // wavefronts sharing one piece's chunks
   uint16_t *const gout = (P.splits > 1 ? P.part[so.io] + (long long)split * P.part_stride[so.io]
@@ -428,15 +431,15 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
       a_base[i] = a0 + (sa / spb_m) * P.pl_a[1] + (sa % spb_m) * P.pl_a[4] + r * 16;
       b_base[i] = b0 + (sb / spb_n) * P.pl_b[0] + (sb % spb_n) * P.pl_b[4] + r * 16;
     }
-    // this lane's chunk of step s: number 4 s + g of the sequence
-    int q = 4 * s_begin + g;
+    // this lane's chunk of step s: number cps s + g of the sequence (none if g >= cps)
+    int q = cps * s_begin + g;
     int itr = q / cpi, c = q - itr * cpi;
     // operands of two steps are in flight while a third is multiplied
     struct Operands {
       v4i ap[2], aq[2], bp[2], bq[2];
     } o0, o1;
     auto fetch = [&](Operands &o) {
-      bool const valid = q < Q;
+      bool const valid = g < cps && q < Q;
       int const oa = itr * a_it + c * 256, ob = itr * b_it + c * 256;
       v4i const zero = {0, 0, 0, 0};
 #pragma unroll
@@ -446,7 +449,7 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
         o.bp[i] = valid ? *reinterpret_cast<v4i const *>(pb + b_base[i] + ob) : zero;
         o.bq[i] = valid ? *reinterpret_cast<v4i const *>(qb + b_base[i] + ob) : zero;
       }
-      q += 4;
+      q += cps;
       itr += dq_it;
       c += dq_c;
       if (c >= cpi) {
@@ -887,7 +890,7 @@ bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_byte
   }
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]];
   int const m = P.t[la.dst].rows, kt = P.t[la.dst].cols, n = P.t[lb.dst].cols;
-  if (m % 16 != 0 || n % 16 != 0 || kt % 16 != 0 || (P.fp_unary[2] != 0 && kt % 64 != 0)) {
+  if (m % 16 != 0 || n % 16 != 0 || kt % 16 != 0 || (P.fp_unary[2] != 0 && kt > 48 && kt % 64 != 0)) {
     return false;
   }
   size_t total = 0;
@@ -917,7 +920,7 @@ bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_byte
   return true;
 }
 
-void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
+void fp_mfma_gemm_bind(DevProgram &P, char *planes, int min_blocks) {
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]];
   size_t const a_plane = (size_t)P.pl_geo[0] * P.pl_geo[1] * P.pl_geo[2];
   size_t const b_plane = (size_t)P.pl_geo[3] * P.pl_geo[4] * P.pl_geo[5];
@@ -954,7 +957,8 @@ void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
   P.fg[5] = 1;
   P.lds_bytes = kFpMfmaLdsBytes;
   // group neighbouring blocks of small tiles up to 64 x 64 outputs per workgroup, as long as
-  // the program keeps a few hundred workgroups
+  // the program keeps `min_blocks` workgroups (a few hundred when it is launched by itself, a
+  // few when many programs share the launch)
   P.pl_group[0] = P.pl_group[1] = 1;
   int const m = P.t[la.dst].rows, n = P.t[lb.dst].cols;
   P.pl_magic[0] = fast_div_magic(m / 16);
@@ -963,7 +967,7 @@ void fp_mfma_gemm_bind(DevProgram &P, char *planes) {
     long long blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
     auto grow = [&](int which, int tile) {
       int &g = P.pl_group[which];
-      while (tile * g * 2 <= 64 && P.grid[which] % (g * 2) == 0 && blocks / 2 >= 256) {
+      while (tile * g * 2 <= 64 && P.grid[which] % (g * 2) == 0 && blocks / 2 >= min_blocks) {
         g *= 2;
         blocks /= 2;
       }

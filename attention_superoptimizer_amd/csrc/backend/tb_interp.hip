@@ -1230,7 +1230,7 @@ static int prepare(mi355_plan const *plan, void const *const *inputs, void *cons
   if (!f16 && prog.fused == 4 && ext_out == nullptr) {
     size_t need = 0;
     if (fp_mfma_gemm_fits(prog, ext, &need) && need <= state().planes_bytes) {
-      fp_mfma_gemm_bind(prog, state().planes());
+      fp_mfma_gemm_bind(prog, state().planes(), 256);
     }
   }
   if (ext_out != nullptr) {
@@ -1507,7 +1507,7 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
     size_t need = 0;
     if (progs[i].fused == 4 && fp_mfma_gemm_fits(progs[i], exts[i], &need) &&
         planes_used + need <= s.planes_bytes) {
-      fp_mfma_gemm_bind(progs[i], s.planes() + planes_used);
+      fp_mfma_gemm_bind(progs[i], s.planes() + planes_used, n >= 8 ? 16 : 256);
       planes_used += (need + 255) / 256 * 256;
       on_matrix_cores.push_back(&progs[i]);
     } else if (progs[i].fused == 4 && fp_needs_matrix_cores(progs[i])) {

@@ -134,7 +134,7 @@ int launch_fp_gemm_multi(DevProgram const *progs, int const *first_block, int n,
 // fp_mfma_gemm_bind: places the planes at `planes` and marks the program; the launches split
 // the operand tensors of the bound programs into their planes first (fp_mfma_split_programs).
 bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_bytes);
-void fp_mfma_gemm_bind(DevProgram &P, char *planes);
+void fp_mfma_gemm_bind(DevProgram &P, char *planes, int min_blocks);
 int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream);
 int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream);
 int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,

@@ -142,7 +142,8 @@ def _spec_inputs(spec, seed):
 
 
 def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_problem: int = 64,
-                           in_flight: int = 4, queues_per_submission: int = 2):
+                           in_flight: int = 16, queues_per_submission: int = 1,
+                           other_shapes: bool = True):
     """Batched verification of 4096 generated candidate mugraphs (8-12 operators, dims in
     [64, 1024]).  Per problem ONE verify_batch submission fingerprints the reference graph and
     its 64 candidates and compares their outputs; `in_flight` submissions overlap, each dealt
@@ -216,15 +217,19 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
         "candidates_per_s_by_family": {k: round(v[0] / v[1], 1) for k, v in sorted(fam.items())},
         "inputs": "uniform [0, 25651) from (seed, input index)",
     }
-    if in_flight > 1 and per_problem == 64:
-        one = fingerprint_throughput(G, False, num_problems, per_problem, 1, 4)
+    if other_shapes:
+        one = fingerprint_throughput(G, False, num_problems, per_problem, 1, 4, False)
         G.set_verify_queues_per_batch(4)
         rec["one_submission_in_flight"] = {k: one[k] for k in (
             "candidates_per_s", "verify_s", "host_enqueue_s", "final_wait_s",
             "candidates_per_s_by_family")}
+        four = fingerprint_throughput(G, False, num_problems, per_problem, 4, 2, False)
+        G.set_verify_queues_per_batch(4)
+        rec["four_submissions_in_flight"] = {k: four[k] for k in (
+            "candidates_per_s", "verify_s", "queues_per_submission", "candidates_per_s_by_family")}
         # the same number of candidates against a quarter of the problems: what a submission
         # costs is mostly its chain of launches, which 256 candidates share instead of 64
-        big = fingerprint_throughput(G, False, num_problems // 4, per_problem * 4, 2, 4)
+        big = fingerprint_throughput(G, False, num_problems // 4, per_problem * 4, 4, 4, False)
         G.set_verify_queues_per_batch(4)
         rec["submissions_of_256_candidates"] = {k: big[k] for k in (
             "candidates", "problems", "candidates_per_s", "verify_s", "verdicts_as_constructed",

@@ -261,7 +261,11 @@ def test_fused_matmul_fingerprint_with_operand_prologues(rt, abi, pro):
     (64, 256, 512, (4, 1, 1), 4, "silu", "exp", True),    # k tile 128, exp(A) before, silu after
     (32, 32, 1024, (1, 1, 1), 16, "exp", None, True),     # one 32 x 32 piece: wavefronts share iterations
     (64, 32, 64 * 37, (1, 1, 1), 37, "exp", None, True),  # two pieces, 37 iterations: uneven shares, split for-loop
-    (64, 256, 512, (4, 1, 1), 16, "exp", None, False),    # k tile 32: not whole steps, interpreter
+    (64, 256, 512, (4, 1, 1), 16, "exp", None, True),     # k tile 32: a step of two chunks per iteration
+    (64, 256, 256, (4, 1, 1), 16, "exp", None, True),     # k tile 16: a step of one chunk
+    (32, 32, 1024, (1, 1, 1), 32, "exp", None, True),     # k tile 32, one piece shared by four wavefronts
+    (64, 32, 48 * 21, (1, 1, 1), 21, "silu", None, True), # k tile 48, two pieces, uneven shares
+    (64, 256, 80 * 4, (4, 1, 1), 4, "exp", None, False),  # k tile 80: not whole steps, interpreter
 ])
 def test_fused_matmul_fingerprint_with_operator_on_the_products(rt, abi, m, n, k, grid, F, epi, pro, fused):
     """exp / silu of every iteration's product before the saver adds it up (sum over
