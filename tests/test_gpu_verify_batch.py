@@ -120,6 +120,40 @@ def test_verify_batches_in_flight_match_one_at_a_time(rt):
     rt.set_verify_queues_per_batch(4)
 
 
+def test_sixteen_batches_in_flight_on_one_queue_each(rt):
+    """The benchmark's shape: sixteen submissions begun before the first is ended, each on one
+    queue, ended newest first and then oldest first: verdicts as constructed and the same
+    candidate outputs as a blocking verify_batch of the same problem."""
+    probs = C.generate(num_problems=16, per_problem=8, seed=0x16F1, max_dim=256)
+    want = [_verify_problem(rt, prob) for prob in probs]
+    rt.set_verify_queues_per_batch(1)
+    try:
+        for order in (list(reversed(range(16))), list(range(16))):
+            built = []
+            try:
+                for prob in probs:
+                    ref_g, ref_vals = rt.build_from_spec(prob["reference"])
+                    cands = [rt.build_from_spec(c["spec"]) for c in prob["candidates"]]
+                    built.append((prob, ref_g, ref_vals, cands))
+                tickets = [rt.verify_batch_begin([g for g, _ in cands], ref_g, prob["input_seed"])
+                           for prob, ref_g, _, cands in built]
+                for k in order:
+                    prob, ref_g, ref_vals, cands = built[k]
+                    verdicts, stats = rt.verify_batch_end(tickets[k])
+                    assert verdicts == [c["expect_equal"] for c in prob["candidates"]], (k, prob["family"])
+                    assert verdicts == want[k][0] and stats["compares"] == len(cands)
+                    for c, (_, vals), w in zip(prob["candidates"], cands, want[k][1]):
+                        got = [t.read_fingerprint() for t in _outputs(c["spec"], vals)]
+                        assert all(np.array_equal(a, b) for a, b in zip(got, w)), (k, prob["family"])
+            finally:
+                for prob, ref_g, _, cands in reversed(built):
+                    for g, _ in reversed(cands):
+                        g.close()
+                    ref_g.close()
+    finally:
+        rt.set_verify_queues_per_batch(4)
+
+
 def test_marks_order_queues_and_report_only_their_work(rt, abi):
     """A compare enqueued on queue 1 behind a mark that queue 0 recorded after filling its
     operand sees the filled values; waiting for the mark queue 1 recorded is enough to read
