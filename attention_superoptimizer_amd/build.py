@@ -26,7 +26,11 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: packed FP32 forms have produced silent wrong results on these boxes
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
+                "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+                # MFMA results stay in VGPRs: with accumulators in AGPRs every use of a product by
+                # vector code costs a v_accvgpr_read (the fingerprint matmul kernels' step: 144 ->
+                # 96 vector instructions, their verification family 271 K -> 340 K candidates/s)
+                "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
 def _sources(sub, exts):
