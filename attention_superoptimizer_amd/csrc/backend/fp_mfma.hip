@@ -377,6 +377,7 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
 // its chunk sequence between wavefronts and adds their sums through `part`.  (bx, by) is the
 // first of pl_group[0] x pl_group[1] logical blocks whose tiles the workgroup treats as one
 // tile of gy * m rows and gx * n columns: strip s of its rows belongs to block by + s / (m / 16).
+template <bool EPI>  // an operator is applied to every iteration's product
 __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables const &tbl, int *part,
                                                    uint16_t const *exp_lds, int bx, int by, int bz,
                                                    int split) {
@@ -392,8 +393,8 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
   // (k tiles of 16, 32 or 48 take one step in which only the first one, two or three lane
   // groups hold a chunk; longer k tiles are multiples of 64); after its last step the two sums
   // become a fingerprint value, the operator is applied and the result added to a running sum.
-  int const epi = P.fp_unary[2];
-  int const cps = epi != 0 && cpi < 4 ? cpi : 4;  // chunks per step
+  int const epi = EPI ? P.fp_unary[2] : 0;
+  int const cps = EPI && cpi < 4 ? cpi : 4;  // chunks per step
   int const spi = cpi / cps;                        // steps per iteration (with an operator)
   int const Q = (it_end - it_begin) * cpi, steps = (Q + cps - 1) / cps;
   int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
@@ -419,7 +420,7 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
     int const ks = ways == 1 ? 0 : wave % ways;
     // wavefronts that share a piece split its steps, by whole iterations if there is an
     // operator on the products
-    int const units = epi ? it_end - it_begin : steps, per_unit = epi ? spi : 1;
+    int const units = EPI ? it_end - it_begin : steps, per_unit = EPI ? spi : 1;
     int const s_begin = (int)((long long)units * ks / ways) * per_unit;
     int const s_end = (int)((long long)units * (ks + 1) / ways) * per_unit;
     int const row_m = (t / mt_n) * 32, col_n = (t % mt_n) * 32;
@@ -477,7 +478,7 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
           acc[1][i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.bq[jn], o.aq[i], acc[1][i][jn], 0, 0, 0);
         }
       }
-      if (epi != 0) {
+      if constexpr (EPI) {
         if (--until == 0) {  // the iteration's product is complete
           until = spi;
           bool const fold = (++folds & 32767) == 0;  // 32768 values below 25651 fit 32 bits
@@ -501,9 +502,7 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
             }
           }
         }
-        return;
-      }
-      if (((s - s_begin) & 2047) == 2047) {
+      } else if (((s - s_begin) & 2047) == 2047) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
 #pragma unroll
@@ -557,7 +556,7 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
       }
       store_values(i, jn, z);
     };
-    if (epi != 0) {
+    if constexpr (EPI) {
       // the running sums are fingerprint values already
       if (ways > 1 && ks != 0) {
 #pragma unroll
@@ -659,8 +658,13 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_gemm_kernel(DevProgram const
     load_exp_table(tbl, exp_lds);
   }
   int const gx = P.grid[0] / P.pl_group[0];
-  fp_mfma_gemm_block(P, tbl, part, exp_lds, (blockIdx.x % gx) * P.pl_group[0], blockIdx.y * P.pl_group[1], blockIdx.z,
-                     blockIdx.x / gx);
+  if (P.fp_unary[2] != 0) {
+    fp_mfma_gemm_block<true>(P, tbl, part, exp_lds, (blockIdx.x % gx) * P.pl_group[0], blockIdx.y * P.pl_group[1],
+                             blockIdx.z, blockIdx.x / gx);
+  } else {
+    fp_mfma_gemm_block<false>(P, tbl, part, exp_lds, (blockIdx.x % gx) * P.pl_group[0], blockIdx.y * P.pl_group[1],
+                              blockIdx.z, blockIdx.x / gx);
+  }
 }
 
 // Many programs in one launch: workgroup -> program by a prefix table, the program record
@@ -694,8 +698,13 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_gemm_multi_kernel(
   int const gx = P.grid[0] / P.pl_group[0], gy = P.grid[1] / P.pl_group[1];
   int const x = v % (gx * P.splits);
   v /= gx * P.splits;
-  fp_mfma_gemm_block(P, tbl, reinterpret_cast<int *>(lds), exp_lds, (x % gx) * P.pl_group[0], (v % gy) * P.pl_group[1],
-                     v / gy, x / gx);
+  if (P.fp_unary[2] != 0) {
+    fp_mfma_gemm_block<true>(P, tbl, reinterpret_cast<int *>(lds), exp_lds, (x % gx) * P.pl_group[0],
+                             (v % gy) * P.pl_group[1], v / gy, x / gx);
+  } else {
+    fp_mfma_gemm_block<false>(P, tbl, reinterpret_cast<int *>(lds), exp_lds, (x % gx) * P.pl_group[0],
+                              (v % gy) * P.pl_group[1], v / gy, x / gx);
+  }
 }
 
 inline size_t round_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
