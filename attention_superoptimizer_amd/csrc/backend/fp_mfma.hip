@@ -929,14 +929,26 @@ bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_byte
   return true;
 }
 
+void fp_mfma_plane_bytes(DevProgram const &P, size_t *a_bytes, size_t *b_bytes) {
+  *a_bytes = 2 * (size_t)P.pl_geo[0] * P.pl_geo[1] * P.pl_geo[2];
+  *b_bytes = 2 * (size_t)P.pl_geo[3] * P.pl_geo[4] * P.pl_geo[5];
+}
+
 void fp_mfma_gemm_bind(DevProgram &P, char *planes, int min_blocks) {
+  size_t a_bytes, b_bytes;
+  fp_mfma_plane_bytes(P, &a_bytes, &b_bytes);
+  fp_mfma_gemm_bind(P, planes, planes + a_bytes, 0, min_blocks);
+}
+
+void fp_mfma_gemm_bind(DevProgram &P, char *a_planes, char *b_planes, int shared, int min_blocks) {
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]];
   size_t const a_plane = (size_t)P.pl_geo[0] * P.pl_geo[1] * P.pl_geo[2];
   size_t const b_plane = (size_t)P.pl_geo[3] * P.pl_geo[4] * P.pl_geo[5];
-  P.pl[0] = reinterpret_cast<int8_t *>(planes);
+  P.pl[0] = reinterpret_cast<int8_t *>(a_planes);
   P.pl[1] = P.pl[0] + a_plane;
-  P.pl[2] = P.pl[1] + a_plane;
+  P.pl[2] = reinterpret_cast<int8_t *>(b_planes);
   P.pl[3] = P.pl[2] + b_plane;
+  P.pl_shared = shared;
   // A: strips follow rows, chunks follow columns
   {
     long long const matrix = (long long)la.d_rows * la.d_cols;
@@ -987,13 +999,18 @@ void fp_mfma_gemm_bind(DevProgram &P, char *planes, int min_blocks) {
 }
 
 int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream) {
-  std::vector<SplitJob> jobs((size_t)(2 * n));
+  std::vector<SplitJob> jobs;
+  jobs.reserve((size_t)(2 * n));
   for (int e = 0; e < n; e++) {
     DevProgram const &P = *progs[e];
     DevOp const *ops[2] = {&P.ops[P.fg[0]], &P.ops[P.fg[1]]};
     for (int which = 0; which < 2; which++) {
+      if (P.pl_shared & (1 << which)) {
+        continue;  // an earlier program of this launch splits the same tensor into these planes
+      }
       DevOp const &op = *ops[which];
-      SplitJob &j = jobs[(size_t)(2 * e + which)];
+      jobs.emplace_back();
+      SplitJob &j = jobs.back();
       j = SplitJob{};
       j.src = static_cast<uint16_t const *>(P.in[op.io]);
       j.plane_p = P.pl[2 * which];
@@ -1016,7 +1033,7 @@ int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t st
       j.blocks = (unsigned)std::min<size_t>(work, 1024);
     }
   }
-  return launch_split_jobs(jobs.data(), 2 * n, stream);
+  return launch_split_jobs(jobs.data(), (int)jobs.size(), stream);
 }
 
 int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream) {

@@ -1492,6 +1492,26 @@ extern "C" int mi355_customized_fp_static(mi355_plan const *plan, void const *co
   return MI355_OK;
 }
 
+// The residue planes of one operand of a fused matmul plan: what identifies them (operand
+// tensor, side, prologue, geometry) and where they are.
+struct SplitOperand {
+  void const *src;
+  int which, unary, slabs, rows, cols;
+  char *planes;
+};
+
+static SplitOperand const *find_split_operand(std::vector<SplitOperand> const &split, DevProgram const &P,
+                                              int which) {
+  DevOp const &op = P.ops[P.fg[which]];
+  for (SplitOperand const &o : split) {
+    if (o.src == P.in[op.io] && o.which == which && o.unary == P.fp_unary[which] &&
+        o.slabs == P.pl_geo[3 * which] && o.rows == op.d_rows && o.cols == op.d_cols) {
+      return &o;
+    }
+  }
+  return nullptr;
+}
+
 // One chunk of a batch: every program in one multi-program launch per LDS class, then one
 // launch that folds the partial sums of all split for-loops.  A program whose tiles leave
 // no room in LDS for its own record is launched by itself.
@@ -1501,16 +1521,46 @@ static int launch_fp_chunk(std::vector<DevProgram> &progs, std::vector<PlanExten
   int const n = (int)progs.size();
   // fused matmul plans take the matrix cores while the residue planes of their operand
   // tensors fit what is left of this queue's plane memory
+  // Members that multiply the same operand tensor (the candidates of one problem read one copy
+  // of their common inputs) share its planes: the first one splits it, the others point at
+  // the result.
+  std::vector<SplitOperand> split;
   std::vector<DevProgram const *> on_matrix_cores;
   size_t planes_used = 0;
   for (int i = 0; i < n; i++) {
     size_t need = 0;
-    if (progs[i].fused == 4 && fp_mfma_gemm_fits(progs[i], exts[i], &need) &&
-        planes_used + need <= s.planes_bytes) {
-      fp_mfma_gemm_bind(progs[i], s.planes() + planes_used, n >= 8 ? 16 : 256);
-      planes_used += (need + 255) / 256 * 256;
-      on_matrix_cores.push_back(&progs[i]);
-    } else if (progs[i].fused == 4 && fp_needs_matrix_cores(progs[i])) {
+    if (progs[i].fused == 4 && fp_mfma_gemm_fits(progs[i], exts[i], &need)) {
+      DevProgram &P = progs[i];
+      size_t bytes[2];
+      fp_mfma_plane_bytes(P, &bytes[0], &bytes[1]);
+      char *place[2] = {nullptr, nullptr};
+      int shared = 0;
+      size_t fresh = 0;
+      for (int which = 0; which < 2; which++) {
+        if (SplitOperand const *o = find_split_operand(split, P, which)) {
+          place[which] = o->planes;
+          shared |= 1 << which;
+        }
+        if (place[which] == nullptr) {
+          fresh += (bytes[which] + 255) / 256 * 256;
+        }
+      }
+      if (planes_used + fresh <= s.planes_bytes) {
+        for (int which = 0; which < 2; which++) {
+          if (place[which] == nullptr) {
+            DevOp const &op = P.ops[P.fg[which]];
+            place[which] = s.planes() + planes_used;
+            planes_used += (bytes[which] + 255) / 256 * 256;
+            split.push_back(SplitOperand{P.in[op.io], which, P.fp_unary[which], P.pl_geo[3 * which],
+                                         op.d_rows, op.d_cols, place[which]});
+          }
+        }
+        fp_mfma_gemm_bind(P, place[0], place[1], shared, n >= 8 ? 16 : 256);
+        on_matrix_cores.push_back(&progs[i]);
+        continue;
+      }
+    }
+    if (progs[i].fused == 4 && fp_needs_matrix_cores(progs[i])) {
       // (the caller cuts chunks so that the planes of their members fit together)
       return fail(MI355_ERR_UNSUPPORTED, "operand prologue without the matrix-core route");
     }
@@ -1712,12 +1762,14 @@ extern "C" int mi355_customized_fp_batch(mi355_plan const *plans, int n,
   std::vector<PlanExtents> exts;
   std::vector<int> nout;
   size_t planes_wanted = 0;
+  std::vector<SplitOperand> wanted;  // operands whose planes the chunk already counts
   auto flush = [&]() {
     int rc = progs.empty() ? MI355_OK : launch_fp_chunk(progs, exts, nout);
     progs.clear();
     exts.clear();
     nout.clear();
     planes_wanted = 0;
+    wanted.clear();
     return rc;
   };
   for (int i = 0; i < n; i++) {
@@ -1730,13 +1782,30 @@ extern "C" int mi355_customized_fp_batch(mi355_plan const *plans, int n,
     }
     size_t need = 0;
     if (prog.fused == 4 && fp_mfma_gemm_fits(prog, ext, &need)) {
-      need = (need + 255) / 256 * 256;
-      if (planes_wanted + need > state().planes_bytes) {
+      size_t bytes[2];
+      fp_mfma_plane_bytes(prog, &bytes[0], &bytes[1]);
+      auto fresh = [&]() {
+        size_t f = 0;
+        for (int which = 0; which < 2; which++) {
+          if (find_split_operand(wanted, prog, which) == nullptr) {
+            f += (bytes[which] + 255) / 256 * 256;
+          }
+        }
+        return f;
+      };
+      if (planes_wanted + fresh() > state().planes_bytes) {
         if (int rc2 = flush()) {
           return rc2;
         }
       }
-      planes_wanted += need;
+      planes_wanted += fresh();
+      for (int which = 0; which < 2; which++) {
+        if (find_split_operand(wanted, prog, which) == nullptr) {
+          DevOp const &op = prog.ops[prog.fg[which]];
+          wanted.push_back(SplitOperand{prog.in[op.io], which, prog.fp_unary[which], prog.pl_geo[3 * which],
+                                        op.d_rows, op.d_cols, nullptr});
+        }
+      }
     }
     progs.push_back(prog);
     exts.push_back(ext);

@@ -87,7 +87,8 @@ struct alignas(16) DevProgram {
   // adds it up.  Only the matrix-core route runs a program that has any of them.
   int fp_unary[3];
   uint32_t pl_magic[2];  // division magics of m / 16 and n / 16 (strips per logical block)
-  int pl_pad2[1];
+  int pl_shared;  // bit 0 / 1: the A / B^T planes belong to an earlier program of the launch
+                  // (same operand tensor, same prologue): this program does not split them
   int grid[3];
   int mm_off;  // uint16 interpreter: LDS offset of the matmul residue scratch
   // uint16 interpreter, split for-loop: workgroup (split, block) runs iterations
@@ -135,6 +136,11 @@ int launch_fp_gemm_multi(DevProgram const *progs, int const *first_block, int n,
 // the operand tensors of the bound programs into their planes first (fp_mfma_split_programs).
 bool fp_mfma_gemm_fits(DevProgram &P, PlanExtents const &ext, size_t *plane_bytes);
 void fp_mfma_gemm_bind(DevProgram &P, char *planes, int min_blocks);
+// The same with the two operands' planes at places of their own (`a_planes`: both planes of A,
+// `b_planes`: both of B^T) and `shared` as in DevProgram::pl_shared; fp_mfma_plane_bytes gives
+// the bytes each side needs once fp_mfma_gemm_fits has filled in the geometry.
+void fp_mfma_gemm_bind(DevProgram &P, char *a_planes, char *b_planes, int shared, int min_blocks);
+void fp_mfma_plane_bytes(DevProgram const &P, size_t *a_bytes, size_t *b_bytes);
 int fp_mfma_split_programs(DevProgram const *const *progs, int n, hipStream_t stream);
 int launch_fp_mfma_gemm(DevProgram const &P, hipStream_t stream);
 int launch_fp_mfma_gemm_multi(DevProgram const *progs, int const *first_block, int n, int blocks,
