@@ -37,7 +37,9 @@ struct VerifyStats {
 // fingerprinted first.  input_seed == 0 fills inputs as the reference does
 // (`idx % 25651`, src/kernel/cuda/input_kernel.cu:56-61); otherwise input number j of
 // each graph holds uniform values generated from (input_seed, j), so graphs built
-// over the same inputs see the same data.  The reference outputs must already hold
+// over the same inputs see the same data (the batched operators read inputs number j of
+// equal element count through the first such graph's tensor, so every candidate's tensors
+// must stay allocated until the verdicts are in).  The reference outputs must already hold
 // their fingerprints.  At most MI355_COMPARE_SLOTS compares per call.
 void verify_batch(std::vector<mirage::kernel::Graph *> const &candidates,
                   std::vector<mirage::kernel::DTensor> const &reference_outputs,
