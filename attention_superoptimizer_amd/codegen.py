@@ -21,6 +21,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # from the fp16 interpreter's chain; "on" keeps every fused multiply-add as written
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-mllvm", "-amdgpu-mfma-vgpr-form",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
 # graphs whose programs the build generates and the GPU tests run
