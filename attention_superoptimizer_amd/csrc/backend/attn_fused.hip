@@ -80,11 +80,14 @@ __device__ __forceinline__ half4 lds_read_tr16(_Float16 const *p) {
   return __builtin_bit_cast(half4, v);
 }
 
+// Where a tile of a device tensor starts: the element offset is linear in the block
+// coordinates and the for-loop iteration, so the host folds the plan's row / column / batch
+// strides into one stride per coordinate (a handful of scalar multiplies per tile address
+// instead of three sums of products; they sit on the path to the first load).
 struct TileAddr {
   void const *ptr;
-  int row_bs[3], col_bs[3], row_fs, col_fs;
-  int g_bs[3], g_fs;
-  int d_cols;
+  long long lin[4];  // elements per step of bx, by, bz and of the iteration
+  int d_cols;        // row stride of the tensor
 };
 
 struct AttnParams {
@@ -108,11 +111,7 @@ struct AttnParams {
 
 __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int by, int bz,
                                                  int it) {
-  int row0 = bx * t.row_bs[0] + by * t.row_bs[1] + bz * t.row_bs[2] + it * t.row_fs;
-  int col0 = bx * t.col_bs[0] + by * t.col_bs[1] + bz * t.col_bs[2] + it * t.col_fs;
-  long long base = (long long)bx * t.g_bs[0] + (long long)by * t.g_bs[1] +
-                   (long long)bz * t.g_bs[2] + (long long)it * t.g_fs;
-  return base + (long long)row0 * t.d_cols + col0;
+  return bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3];
 }
 
 // Element offset of 16-byte chunk `chunk` of row `row` in a swizzled LDS tile whose
@@ -193,21 +192,18 @@ __device__ __forceinline__ void decode_block(AttnParams const &P, int &bx, int &
   }
   // divisions by the extents are multiply-highs with magics the host computed (exact while
   // id * extent < 2^32, which the host checks): this runs before the first load can go out
-  unsigned coord[3] = {0, 0, 0};
+  unsigned digit[3];  // digit i of the id belongs to grid dim perm[i]
 #pragma unroll
   for (int i = 0; i < 3; i++) {
-    int const d = P.perm[i];
     unsigned const e = P.perm_ext[i], m = P.perm_magic[i];
     unsigned const q = m == 0 ? id : __umulhi(id, m);
-    unsigned const v = id - q * e;
+    digit[i] = id - q * e;
     id = q;
-    if (d == 0) {
-      coord[0] = v;
-    } else if (d == 1) {
-      coord[1] = v;
-    } else {
-      coord[2] = v;
-    }
+  }
+  unsigned coord[3];  // (selects, no branches: this is on the path to the first load)
+#pragma unroll
+  for (int k = 0; k < 3; k++) {
+    coord[k] = P.perm[0] == k ? digit[0] : (P.perm[1] == k ? digit[1] : digit[2]);
   }
   unsigned const b = P.split_magic == 0 ? coord[0] : __umulhi(coord[0], P.split_magic);
   bx = (int)b;
@@ -359,8 +355,8 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
 #pragma unroll
             for (int w = 0; w < 4; w++) {
               half2v const e2 = __builtin_bit_cast(half2v, pk[jj][w]);
-              half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
-                                 static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+              half2v const p2 = {static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[0]), inv, 0.0f)),
+                                 static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[1]), inv, 0.0f))};
               pk[jj][w] = __builtin_bit_cast(uint32_t, p2);
             }
           }
@@ -654,8 +650,10 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
 #pragma unroll
           for (int w = 0; w < 4; w++) {
             half2v const e2 = __builtin_bit_cast(half2v, pk[rp][jj][w]);
-            half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
-                               static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+            // (a fused multiply-add with +0: maps to the mixed-precision FMA that reads and
+            // writes fp16; exp values are positive, so the +0 changes nothing)
+            half2v const p2 = {static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[0]), inv, 0.0f)),
+                               static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[1]), inv, 0.0f))};
             pk[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
           }
         }
@@ -866,13 +864,9 @@ TileAddr tile_addr(DevOp const &op, void const *ptr) {
   TileAddr t;
   t.ptr = ptr;
   for (int i = 0; i < 3; i++) {
-    t.row_bs[i] = op.row_bs[i];
-    t.col_bs[i] = op.col_bs[i];
-    t.g_bs[i] = op.g_bs[i];
+    t.lin[i] = op.g_bs[i] + (long long)op.row_bs[i] * op.d_cols + op.col_bs[i];
   }
-  t.row_fs = op.row_fs;
-  t.col_fs = op.col_fs;
-  t.g_fs = op.g_fs;
+  t.lin[3] = op.g_fs + (long long)op.row_fs * op.d_cols + op.col_fs;
   t.d_cols = op.d_cols;
   return t;
 }
@@ -1280,11 +1274,12 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
           float part = 0.0f;
 #pragma unroll
           for (int h = 0; h < 2; h++) {
-            half2v const s2 = {static_cast<_Float16>(acc[rp][jb][2 * h]),
-                               static_cast<_Float16>(acc[rp][jb][2 * h + 1])};
-            float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
-            float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
-            half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
+            // (pairs are rounded to fp16 by one packed conversion each)
+            float2v const f2 = {acc[rp][jb][2 * h], acc[rp][jb][2 * h + 1]};
+            half2v const s2 = __builtin_convertvector(f2, half2v);
+            float2v const x2 = {__builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f)),
+                                __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f))};
+            half2v const e2 = __builtin_convertvector(x2, half2v);
             part = __builtin_amdgcn_fdot2(e2, ones, part, false);
             pk[rp][jb / 2][2 * (jb & 1) + h] = __builtin_bit_cast(uint32_t, e2);
           }
@@ -1313,8 +1308,11 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
         for (int w = 0; w < 4 * (KB / 2); w++) {
           if (w >= w0 && w < w0 + nw) {
             half2v const e2 = __builtin_bit_cast(half2v, pk[rp][w / 4][w % 4]);
-            half2v const p2 = {static_cast<_Float16>(static_cast<float>(e2[0]) * inv),
-                               static_cast<_Float16>(static_cast<float>(e2[1]) * inv)};
+            // (written as a fused multiply-add with +0 so that it maps to the mixed-precision
+            // FMA that reads fp16 and writes fp16: exp values are positive, so adding +0 changes
+            // nothing)
+            half2v const p2 = {static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[0]), inv, 0.0f)),
+                               static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[1]), inv, 0.0f))};
             pk[rp][w / 4][w % 4] = __builtin_bit_cast(uint32_t, p2);
           }
         }
@@ -1322,8 +1320,8 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       auto store_result = [&](int sub, int rp, float4v const (&res)[DB], _Float16 r16) {
 #pragma unroll
         for (int t = 0; t < DB; t++) {
-          half2v const lo = {static_cast<_Float16>(res[t][0]), static_cast<_Float16>(res[t][1])};
-          half2v const hi = {static_cast<_Float16>(res[t][2]), static_cast<_Float16>(res[t][3])};
+          half2v const lo = __builtin_convertvector(float2v{res[t][0], res[t][1]}, half2v);
+          half2v const hi = __builtin_convertvector(float2v{res[t][2], res[t][3]}, half2v);
           keep[j][sub][rp][2 * t] = __builtin_bit_cast(uint32_t, lo);
           keep[j][sub][rp][2 * t + 1] = __builtin_bit_cast(uint32_t, hi);
         }
@@ -1464,10 +1462,12 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   // ---- ordered accumulation: every thread owns EPT consecutive columns of one row; the
   // slots of up to four iterations are read before their (dependent) adds ---------------
   {
-    float acc[EPT];
+    // fp16 sums, two per register: adding two fp16 numbers with one packed fp16 add gives their
+    // exact sum rounded once, which is what adding in fp32 and rounding to fp16 gives
+    half2v acc[EPT / 2];
 #pragma unroll
-    for (int e = 0; e < EPT; e++) {
-      acc[e] = 0.0f;  // holds an fp16 value between the adds
+    for (int e = 0; e < EPT / 2; e++) {
+      acc[e] = half2v{(_Float16)0.0f, (_Float16)0.0f};
     }
     _Float16 const *all = reinterpret_cast<_Float16 const *>(lds) + out_row * LDO + out_col;
     // iteration `it` is slice it % IPS of unit it / IPS, which wavefront unit % IP kept as its
@@ -1496,8 +1496,7 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
         if (it0 + u < F) {
 #pragma unroll
           for (int e = 0; e < EPT / 2; e++) {
-            acc[2 * e] = static_cast<float>(static_cast<_Float16>(acc[2 * e] + static_cast<float>(v[u][e][0])));
-            acc[2 * e + 1] = static_cast<float>(static_cast<_Float16>(acc[2 * e + 1] + static_cast<float>(v[u][e][1])));
+            acc[e] = acc[e] + v[u][e];
           }
         }
       }
@@ -1506,7 +1505,7 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       half2v out[EPT / 2];
 #pragma unroll
       for (int e = 0; e < EPT / 2; e++) {
-        out[e] = half2v{static_cast<_Float16>(acc[2 * e]), static_cast<_Float16>(acc[2 * e + 1])};
+        out[e] = acc[e];
       }
       if (EPT == 8) {
         uint4v const w = {__builtin_bit_cast(uint32_t, out[0]), __builtin_bit_cast(uint32_t, out[1]),
