@@ -38,6 +38,7 @@
 //    never leaves registers and the two concats cost nothing.
 #include "common.h"
 #include "tb_program.h"
+#include <algorithm>
 
 namespace mi355 {
 
@@ -49,11 +50,13 @@ typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 enum { PRO_NONE = 0, PRO_EXP = 1, PRO_SILU = 2, PRO_SILU_MUL = 3 };
 
+// Where a tile of a device tensor starts: the element offset is linear in the block
+// coordinates and the for-loop iteration, so the host folds the plan's row / column / batch
+// strides into one stride per coordinate (a few scalar multiplies per tile address).
 struct GTile {
   void const *ptr;
-  int row_bs[3], col_bs[3], row_fs, col_fs;
-  int g_bs[3], g_fs;
-  int d_cols;
+  long long lin[4];  // elements per step of bx, by, bz and of the iteration
+  int d_cols;        // row stride of the tensor
 };
 
 struct GemmParams {
@@ -68,11 +71,7 @@ struct GemmParams {
 };
 
 __device__ __forceinline__ long long gtile_offset(GTile const &t, int bx, int by, int bz, int it) {
-  int row0 = bx * t.row_bs[0] + by * t.row_bs[1] + bz * t.row_bs[2] + it * t.row_fs;
-  int col0 = bx * t.col_bs[0] + by * t.col_bs[1] + bz * t.col_bs[2] + it * t.col_fs;
-  long long base = (long long)bx * t.g_bs[0] + (long long)by * t.g_bs[1] +
-                   (long long)bz * t.g_bs[2] + (long long)it * t.g_fs;
-  return base + (long long)row0 * t.d_cols + col0;
+  return bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3];
 }
 
 // 16-byte chunk `chunk` of row `row` in a swizzled LDS tile with LD halfs per row.
@@ -507,6 +506,9 @@ struct LaneParams {
   int blocks;        // logical blocks
   int mtiles;        // 16-row pieces per block
   int slot_base;     // byte offset of the product slots in LDS (after the lanes' buffers)
+  // multiply-high division magics (fast_div_magic) of 8 * 4 * mtiles, 4 * mtiles, gx and gy:
+  // the decode of the flat id is on the path to the first load
+  uint32_t m_group, m_pieces, m_gx, m_gy;
 };
 
 #pragma clang diagnostic push
@@ -546,14 +548,19 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
 
   // flat id -> (logical block, row piece, column piece): ids that differ by 8 x piece index
   // share a block
-  int const S = 4 * L.mtiles;
-  int const id = blockIdx.x;
-  int const blk = (id / (8 * S)) * 8 + id % 8, sub = (id / 8) % S;
+  auto div = [](unsigned v, uint32_t magic) { return magic == 0 ? v : __umulhi(v, magic); };
+  unsigned const S = 4 * L.mtiles;
+  unsigned const id = blockIdx.x;
+  unsigned const eighth = id >> 3;
+  int const blk = (int)(div(id, L.m_group) * 8 + (id & 7));
+  int const sub = (int)(eighth - div(eighth, L.m_pieces) * S);
   if (blk >= L.blocks) {
     return;
   }
   int const piece = sub % 4, mt = sub / 4;
-  int const bx = blk % L.gx, by = (blk / L.gx) % L.gy, bz = blk / (L.gx * L.gy);
+  unsigned const q1 = div((unsigned)blk, L.m_gx);  // blk / gx
+  unsigned const q2 = div(q1, L.m_gy);             // blk / (gx * gy)
+  int const bx = (int)((unsigned)blk - q1 * (unsigned)L.gx), by = (int)(q1 - q2 * (unsigned)L.gy), bz = (int)q2;
   int const n0 = 16 * piece;
 
   unsigned char *mine = lds + ip * WAVE_BYTES;
@@ -737,13 +744,9 @@ GTile gtile(DevOp const &op, void const *ptr) {
   GTile t;
   t.ptr = ptr;
   for (int i = 0; i < 3; i++) {
-    t.row_bs[i] = op.row_bs[i];
-    t.col_bs[i] = op.col_bs[i];
-    t.g_bs[i] = op.g_bs[i];
+    t.lin[i] = op.g_bs[i] + (long long)op.row_bs[i] * op.d_cols + op.col_bs[i];
   }
-  t.row_fs = op.row_fs;
-  t.col_fs = op.col_fs;
-  t.g_fs = op.g_fs;
+  t.lin[3] = op.g_fs + (long long)op.row_fs * op.d_cols + op.col_fs;
   t.d_cols = op.d_cols;
   return t;
 }
@@ -921,7 +924,9 @@ int try_launch_lanes(DevProgram const &P, GMatch const &G, GemmParams const &A) 
   long long const blocks = (long long)P.grid[0] * P.grid[1] * P.grid[2];
   int const mtiles = (G.M + 15) / 16, S = 4 * mtiles, F = P.forloop_range;
   long long const groups = (blocks + 7) / 8;
-  if (groups * 8 * S > 2147483647LL) {
+  // (the kernel decodes the flat id with multiply-high magics: exact while id x divisor < 2^32)
+  long long const widest = std::max<long long>(8 * S, std::max(P.grid[0], P.grid[1]));
+  if (groups * 8 * S * widest >= (1LL << 32)) {
     return 0;
   }
   // By itself only where the launch, not the traffic, sets the time (weights of a few MB): a
@@ -950,6 +955,10 @@ int try_launch_lanes(DevProgram const &P, GMatch const &G, GemmParams const &A) 
   L.blocks = (int)blocks;
   L.mtiles = mtiles;
   L.slot_base = ip * wave_bytes;
+  L.m_group = fast_div_magic(8 * 4 * mtiles);
+  L.m_pieces = fast_div_magic(4 * mtiles);
+  L.m_gx = fast_div_magic(P.grid[0]);
+  L.m_gy = fast_div_magic(P.grid[1]);
   int const lds = ip * wave_bytes + slot_bytes, grid = (int)(groups * 8 * S);
   int rc = 0;
 #define MI355_LANES_CASE(NBV, PROV, LORAV)                                  \
