@@ -25,9 +25,11 @@ namespace mi355 {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
+// Where a block's tile starts: linear in the block coordinates, so the host folds the plan's
+// row / column / batch strides into one element stride per coordinate.
 struct CTile {
   void const *ptr;
-  int row_bs[3], col_bs[3], g_bs[3];
+  long long lin[3];
   int d_cols;
 };
 
@@ -42,14 +44,7 @@ struct CombineParams {
 };
 
 __device__ __forceinline__ long long ctile_origin(CTile const &t) {
-  int const bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
-  long long const row0 = (long long)bx * t.row_bs[0] + (long long)by * t.row_bs[1] +
-                         (long long)bz * t.row_bs[2];
-  long long const col0 = (long long)bx * t.col_bs[0] + (long long)by * t.col_bs[1] +
-                         (long long)bz * t.col_bs[2];
-  long long const base = (long long)bx * t.g_bs[0] + (long long)by * t.g_bs[1] +
-                         (long long)bz * t.g_bs[2];
-  return base + row0 * t.d_cols + col0;
+  return (long long)blockIdx.x * t.lin[0] + (long long)blockIdx.y * t.lin[1] + (long long)blockIdx.z * t.lin[2];
 }
 
 template <int VEC, int MODE>
@@ -106,9 +101,7 @@ CTile ctile(DevOp const &op, void const *ptr) {
   CTile t;
   t.ptr = ptr;
   for (int i = 0; i < 3; i++) {
-    t.row_bs[i] = op.row_bs[i];
-    t.col_bs[i] = op.col_bs[i];
-    t.g_bs[i] = op.g_bs[i];
+    t.lin[i] = op.g_bs[i] + (long long)op.row_bs[i] * op.d_cols + op.col_bs[i];
   }
   t.d_cols = op.d_cols;
   return t;
@@ -125,7 +118,7 @@ bool aligned(CTile const &t, int vec) {
     return false;
   }
   for (int i = 0; i < 3; i++) {
-    if (t.col_bs[i] % vec != 0 || t.g_bs[i] % vec != 0) {
+    if (t.lin[i] % vec != 0) {
       return false;
     }
   }
