@@ -381,60 +381,93 @@ template <bool EPI>  // an operator is applied to every iteration's product
 __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables const &tbl, int *part,
                                                    uint16_t const *exp_lds, int bx, int by, int bz,
                                                    int split) {
+  // Everything read from the program record is the same for all lanes; in a multi-program launch
+  // the record sits in LDS, where the compiler cannot know that, so the values are made scalar
+  // here (`uni`) and the address arithmetic below runs on the scalar unit.  Divisions are 32-bit
+  // (products of loop counts and split numbers are small) or multiply-highs with host magics.
+  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  auto uni_ptr = [](auto *ptr) {
+    unsigned long long const v = reinterpret_cast<unsigned long long>(ptr);
+    unsigned const lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    unsigned const hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return reinterpret_cast<decltype(ptr)>(((unsigned long long)hi << 32) | lo);
+  };
+  auto udiv = [](unsigned v, uint32_t magic) { return magic == 0 ? v : __umulhi(v, magic); };
   DevOp const &la = P.ops[P.fg[0]], &lb = P.ops[P.fg[1]], &so = P.ops[P.num_ops - 1];
-  int const bm = P.t[la.dst].rows, kt = P.t[la.dst].cols, bn = P.t[lb.dst].cols;
-  int const m = bm * P.pl_group[1], n = bn * P.pl_group[0];  // the grouped tile
-  int const spb_m = bm / 16, spb_n = bn / 16;                // strips per block
+  int const bm = uni(P.t[la.dst].rows), kt = uni(P.t[la.dst].cols), bn = uni(P.t[lb.dst].cols);
+  int const group_x = uni(P.pl_group[0]), group_y = uni(P.pl_group[1]);
+  int const m = bm * group_y, n = bn * group_x;    // the grouped tile
+  int const spb_m = bm / 16, spb_n = bn / 16;      // strips per block
+  uint32_t const magic_m = (uint32_t)uni((int)P.pl_magic[0]), magic_n = (uint32_t)uni((int)P.pl_magic[1]);
   int const cpi = kt / 16;  // chunks per iteration
-  int const F = P.forloop_range;
-  int const it_begin = (int)((long long)F * split / P.splits);
-  int const it_end = (int)((long long)F * (split + 1) / P.splits);
+  int const F = uni(P.forloop_range), splits = uni(P.splits);
+  bx = uni(bx);
+  by = uni(by);
+  bz = uni(bz);
+  split = uni(split);
+  int const it_begin = (int)((unsigned)(F * split) / (unsigned)splits);
+  int const it_end = (int)((unsigned)(F * (split + 1)) / (unsigned)splits);
   // An operator applied to every iteration's product: an iteration is a whole number of steps
   // (k tiles of 16, 32 or 48 take one step in which only the first one, two or three lane
   // groups hold a chunk; longer k tiles are multiples of 64); after its last step the two sums
   // become a fingerprint value, the operator is applied and the result added to a running sum.
-  int const epi = EPI ? P.fp_unary[2] : 0;
+  int const epi = EPI ? uni(P.fp_unary[2]) : 0;
   int const cps = EPI && cpi < 4 ? cpi : 4;  // chunks per step
-  int const spi = cpi / cps;                        // steps per iteration (with an operator)
+  int const spi = EPI && cpi >= 4 ? cpi / 4 : 1;    // steps per iteration (with an operator)
   int const Q = (it_end - it_begin) * cpi, steps = (Q + cps - 1) / cps;
-  int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
-  int const a0 = bx * P.pl_a[0] + by * P.pl_a[1] + bz * P.pl_a[2] + it_begin * P.pl_a[3];
-  int const b0 = bx * P.pl_b[0] + by * P.pl_b[1] + bz * P.pl_b[2] + it_begin * P.pl_b[3];
-  int const a_it = P.pl_a[3], b_it = P.pl_b[3];
+  int const tid = threadIdx.x, wave = uni(tid / 64), lane = tid % 64, r = lane % 16, g = lane / 16;
+  int const pl_a0 = uni(P.pl_a[0]), pl_a1 = uni(P.pl_a[1]), pl_a2 = uni(P.pl_a[2]), pl_a3 = uni(P.pl_a[3]),
+            pl_a4 = uni(P.pl_a[4]);
+  int const pl_b0 = uni(P.pl_b[0]), pl_b1 = uni(P.pl_b[1]), pl_b2 = uni(P.pl_b[2]), pl_b3 = uni(P.pl_b[3]),
+            pl_b4 = uni(P.pl_b[4]);
+  int const a0 = bx * pl_a0 + by * pl_a1 + bz * pl_a2 + it_begin * pl_a3;
+  int const b0 = bx * pl_b0 + by * pl_b1 + bz * pl_b2 + it_begin * pl_b3;
+  int const a_it = pl_a3, b_it = pl_b3;
   int const dq_it = cps / cpi, dq_c = cps % cpi;
   int const mt_n = (n + 31) / 32, mt = ((m + 31) / 32) * mt_n;
-  int const ways = mt >= 3 ? 1 : (mt == 2 ? 2 : 4);  // wavefronts sharing one piece's chunks
-  uint16_t *const gout = (P.splits > 1 ? P.part[so.io] + (long long)split * P.part_stride[so.io]
-                                       : static_cast<uint16_t *>(P.out[so.io]));
-  // element offset of the output tile of logical block (bx + dx, by + dy, bz)
-  auto out_origin = [&](int dx, int dy) {
-    int const x = bx + dx, y = by + dy;
-    int const row0 = x * so.row_bs[0] + y * so.row_bs[1] + bz * so.row_bs[2];
-    int const col0 = x * so.col_bs[0] + y * so.col_bs[1] + bz * so.col_bs[2];
-    long long const base = (long long)x * so.g_bs[0] + (long long)y * so.g_bs[1] +
-                           (long long)bz * so.g_bs[2];
-    return base + (long long)row0 * so.d_cols + col0;
-  };
-  int8_t const *const pa = P.pl[0], *const qa = P.pl[1], *const pb = P.pl[2], *const qb = P.pl[3];
-  for (int t = ways == 1 ? wave : wave / ways; t < mt; t += 4) {
-    int const ks = ways == 1 ? 0 : wave % ways;
+  int const ways_log2 = mt >= 3 ? 0 : (mt == 2 ? 1 : 2);  // wavefronts sharing one piece's chunks
+  int const ways = 1 << ways_log2;
+  int const so_io = uni(so.io);
+  uint16_t *const gout = uni_ptr(splits > 1 ? P.part[so_io] + (long long)split * P.part_stride[so_io]
+                                            : static_cast<uint16_t *>(P.out[so_io]));
+  // element offset of the output tile of logical block (bx + dx, by + dy, bz): linear in the
+  // block coordinates
+  int const so_cols = uni(so.d_cols);
+  long long const o_x = uni(so.g_bs[0]) + (long long)uni(so.row_bs[0]) * so_cols + uni(so.col_bs[0]);
+  long long const o_y = uni(so.g_bs[1]) + (long long)uni(so.row_bs[1]) * so_cols + uni(so.col_bs[1]);
+  long long const o_z = uni(so.g_bs[2]) + (long long)uni(so.row_bs[2]) * so_cols + uni(so.col_bs[2]);
+  long long const o_base = bx * o_x + by * o_y + bz * o_z;
+  auto out_origin = [&](int dx, int dy) { return o_base + dx * o_x + dy * o_y; };
+  int8_t const *const pa = uni_ptr(P.pl[0]), *const qa = uni_ptr(P.pl[1]), *const pb = uni_ptr(P.pl[2]),
+                      *const qb = uni_ptr(P.pl[3]);
+  for (int t = wave >> ways_log2; t < mt; t += 4) {
+    int const ks = wave & (ways - 1);
     // wavefronts that share a piece split its steps, by whole iterations if there is an
     // operator on the products
     int const units = EPI ? it_end - it_begin : steps, per_unit = EPI ? spi : 1;
-    int const s_begin = (int)((long long)units * ks / ways) * per_unit;
-    int const s_end = (int)((long long)units * (ks + 1) / ways) * per_unit;
-    int const row_m = (t / mt_n) * 32, col_n = (t % mt_n) * 32;
+    int const s_begin = ((units * ks) >> ways_log2) * per_unit;
+    int const s_end = ((units * (ks + 1)) >> ways_log2) * per_unit;
+    int const t_row = (int)((unsigned)t / (unsigned)mt_n);
+    int const row_m = t_row * 32, col_n = (t - t_row * mt_n) * 32;
     int const i1 = row_m + 16 < m ? 1 : 0, j1 = col_n + 16 < n ? 1 : 0;
     int a_base[2], b_base[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       int const sa = row_m / 16 + (i ? i1 : 0), sb = col_n / 16 + (i ? j1 : 0);
-      a_base[i] = a0 + (sa / spb_m) * P.pl_a[1] + (sa % spb_m) * P.pl_a[4] + r * 16;
-      b_base[i] = b0 + (sb / spb_n) * P.pl_b[0] + (sb % spb_n) * P.pl_b[4] + r * 16;
+      int const sa_blk = (int)udiv((unsigned)sa, magic_m), sb_blk = (int)udiv((unsigned)sb, magic_n);
+      a_base[i] = a0 + sa_blk * pl_a1 + (sa - sa_blk * spb_m) * pl_a4 + r * 16;
+      b_base[i] = b0 + sb_blk * pl_b0 + (sb - sb_blk * spb_n) * pl_b4 + r * 16;
     }
     // this lane's chunk of step s: number cps s + g of the sequence (none if g >= cps)
     int q = cps * s_begin + g;
-    int itr = q / cpi, c = q - itr * cpi;
+    int itr = (int)((unsigned)(cps * s_begin) / (unsigned)cpi), c = cps * s_begin - itr * cpi + g;
+#pragma unroll
+    for (int wrap = 0; wrap < 4; wrap++) {  // g <= 3 chunks further on
+      if (c >= cpi) {
+        c -= cpi;
+        itr++;
+      }
+    }
     // operands of two steps are in flight while a third is multiplied
     struct Operands {
       v4i ap[2], aq[2], bp[2], bq[2];
@@ -543,10 +576,9 @@ __device__ __forceinline__ void fp_mfma_gemm_block(DevProgram const &P, FpTables
       w.y = z[2] | (z[3] << 16);
       // strip -> logical block of the grouped tile by multiply-high (magics from the host)
       int const srow = row_m / 16 + i, scol = col_n / 16 + jn;
-      int const dy = P.pl_magic[0] ? (int)__umulhi((uint32_t)srow, P.pl_magic[0]) : srow;
-      int const dx = P.pl_magic[1] ? (int)__umulhi((uint32_t)scol, P.pl_magic[1]) : scol;
+      int const dy = (int)udiv((unsigned)srow, magic_m), dx = (int)udiv((unsigned)scol, magic_n);
       int const row = (srow - dy * spb_m) * 16 + r, col = (scol - dx * spb_n) * 16 + 4 * g;
-      *reinterpret_cast<uint2 *>(gout + out_origin(dx, dy) + (long long)row * so.d_cols + col) = w;
+      *reinterpret_cast<uint2 *>(gout + out_origin(dx, dy) + (long long)row * so_cols + col) = w;
     };
     auto store = [&](int i, int jn, v4i const &sp, v4i const &sq) {
       uint32_t z[4];
