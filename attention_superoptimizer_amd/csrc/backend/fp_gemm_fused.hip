@@ -51,8 +51,10 @@ __device__ __forceinline__ void fp_gemm_block(DevProgram const &P, uint32_t *lds
   int const buf_dwords = 2 * kq * (lda + n);
   int const tid = threadIdx.x;
   int const F = P.forloop_range;
-  int const it_begin = (int)((long long)F * split / P.splits);
-  int const it_end = (int)((long long)F * (split + 1) / P.splits);
+  // (32-bit: a for-loop is cut into at most 64 parts, and 64 F is far below 2^32)
+  unsigned const parts = (unsigned)P.splits;
+  int const it_begin = parts == 1 ? 0 : (int)((unsigned)F * (unsigned)split / parts);
+  int const it_end = parts == 1 ? F : (int)((unsigned)F * (unsigned)(split + 1) / parts);
   int const chunks = kt / kc, steps = (it_end - it_begin) * chunks;
   uint16_t const *inA = static_cast<uint16_t const *>(P.in[la.io]);
   uint16_t const *inB = static_cast<uint16_t const *>(P.in[lb.io]);

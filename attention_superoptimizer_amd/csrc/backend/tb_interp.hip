@@ -315,8 +315,10 @@ __device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned ch
   int const tid = threadIdx.x;
   int const F = P.forloop_range;
   // a split for-loop: this workgroup covers iterations [it_begin, it_end) of block bx
-  int const it_begin = (int)((long long)F * split / P.splits);
-  int const it_end = (int)((long long)F * (split + 1) / P.splits);
+  // (32-bit: a for-loop is cut into at most 64 parts, and 64 F is far below 2^32)
+  unsigned const parts = (unsigned)P.splits;
+  int const it_begin = parts == 1 ? 0 : (int)((unsigned)F * (unsigned)split / parts);
+  int const it_end = parts == 1 ? F : (int)((unsigned)F * (unsigned)(split + 1) / parts);
   for (int it = it_begin; it < it_end; it++) {
     for (int o = 0; o < P.num_ops; o++) {
       DevOp const &op = P.ops[o];
