@@ -32,12 +32,23 @@ struct TileOrigin {
   int row0, col0;
 };
 
+// (Every operand is the same in all lanes.  When the program record sits in LDS the compiler
+// cannot know that, so they are made scalar here: the sums of products then run on the scalar
+// unit instead of as quarter-rate vector integer multiplies.)
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
 __device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it, int bx, int by, int bz) {
   TileOrigin o;
-  o.row0 = bx * op.row_bs[0] + by * op.row_bs[1] + bz * op.row_bs[2] + it * op.row_fs;
-  o.col0 = bx * op.col_bs[0] + by * op.col_bs[1] + bz * op.col_bs[2] + it * op.col_fs;
-  o.base = (long long)bx * op.g_bs[0] + (long long)by * op.g_bs[1] + (long long)bz * op.g_bs[2] +
-           (long long)it * op.g_fs;
+  bx = uniform(bx);
+  by = uniform(by);
+  bz = uniform(bz);
+  it = uniform(it);
+  o.row0 = bx * uniform(op.row_bs[0]) + by * uniform(op.row_bs[1]) + bz * uniform(op.row_bs[2]) +
+           it * uniform(op.row_fs);
+  o.col0 = bx * uniform(op.col_bs[0]) + by * uniform(op.col_bs[1]) + bz * uniform(op.col_bs[2]) +
+           it * uniform(op.col_fs);
+  o.base = (long long)bx * uniform(op.g_bs[0]) + (long long)by * uniform(op.g_bs[1]) +
+           (long long)bz * uniform(op.g_bs[2]) + (long long)it * uniform(op.g_fs);
   return o;
 }
 __device__ __forceinline__ TileOrigin tile_origin(DevOp const &op, int it, int bx) {
@@ -319,31 +330,36 @@ __device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned ch
   unsigned const parts = (unsigned)P.splits;
   int const it_begin = parts == 1 ? 0 : (int)((unsigned)F * (unsigned)split / parts);
   int const it_end = parts == 1 ? F : (int)((unsigned)F * (unsigned)(split + 1) / parts);
+  int const num_ops = uniform(P.num_ops);
   for (int it = it_begin; it < it_end; it++) {
-    for (int o = 0; o < P.num_ops; o++) {
+    for (int o = 0; o < num_ops; o++) {
       DevOp const &op = P.ops[o];
-      switch (op.kind) {
+      switch (uniform(op.kind)) {
         case DOP_LOAD: {
-          if (op.hoist && it > it_begin) {
+          if (uniform(op.hoist) && it > it_begin) {
             break;
           }
-          DevTensor const &t = P.t[op.dst];
-          uint16_t *s = reinterpret_cast<uint16_t *>(lds + t.off);
+          DevTensor const &t = P.t[uniform(op.dst)];
+          uint16_t *s = reinterpret_cast<uint16_t *>(lds + uniform(t.off));
           TileOrigin org = tile_origin(op, it, bx, by, bz);
-          uint16_t const *g = static_cast<uint16_t const *>(P.in[op.io]) + org.base +
-                              (long long)org.row0 * op.d_cols + org.col0;
-          if (op.vec8) {
-            int const cpr = t.cols / 8, n = t.rows * cpr;
+          int const d_cols = uniform(op.d_cols);
+          uint16_t const *g = static_cast<uint16_t const *>(P.in[uniform(op.io)]) + org.base +
+                              (long long)org.row0 * d_cols + org.col0;
+          if (uniform(op.vec8)) {
+            int const cpr = uniform(t.cols) / 8, n = uniform(t.rows) * cpr;
+            int const cols = uniform(t.cols);
+            uint32_t const mcpr = (uint32_t)uniform((int)t.mcpr);
             for (int e = tid; e < n; e += kInterpThreads) {
-              int const r = fdiv(e, t.mcpr), c = (e - r * cpr) * 8;
-              uint4v v = *reinterpret_cast<uint4v const *>(g + (long long)r * op.d_cols + c);
-              *reinterpret_cast<uint4v *>(s + r * t.cols + c) = v;
+              int const r = fdiv(e, mcpr), c = (e - r * cpr) * 8;
+              uint4v v = *reinterpret_cast<uint4v const *>(g + (long long)r * d_cols + c);
+              *reinterpret_cast<uint4v *>(s + r * cols + c) = v;
             }
           } else {
-            int const n = t.rows * t.cols;
+            int const cols = uniform(t.cols), n = uniform(t.rows) * cols;
+            uint32_t const mcols = (uint32_t)uniform((int)t.mcols);
             for (int e = tid; e < n; e += kInterpThreads) {
-              int const r = fdiv(e, t.mcols), c = e - r * t.cols;
-              s[e] = g[(long long)r * op.d_cols + c];
+              int const r = fdiv(e, mcols), c = e - r * cols;
+              s[e] = g[(long long)r * d_cols + c];
             }
           }
           break;
@@ -482,17 +498,19 @@ __device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned ch
         }
         case DOP_OUTPUT: {
           // reference output_saver.h:373-401 (accumulate) and :418-447 (store)
-          DevTensor const &ti = P.t[op.src0], &ta = P.t[op.dst];
-          uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + ti.off);
-          uint16_t *acc = reinterpret_cast<uint16_t *>(lds + ta.off);
-          int const n = ta.rows * ta.cols;
+          DevTensor const &ti = P.t[uniform(op.src0)], &ta = P.t[uniform(op.dst)];
+          uint16_t const *x = reinterpret_cast<uint16_t const *>(lds + uniform(ti.off));
+          uint16_t *acc = reinterpret_cast<uint16_t *>(lds + uniform(ta.off));
+          int const ta_rows = uniform(ta.rows), ta_cols = uniform(ta.cols), n = ta_rows * ta_cols;
           bool const last = (it == it_end - 1), first = (it == it_begin);
           TileOrigin org = tile_origin(op, 0, bx, by, bz);
-          uint16_t *g = (P.splits > 1 ? P.part[op.io] + (long long)split * P.part_stride[op.io]
-                                      : static_cast<uint16_t *>(P.out[op.io])) +
-                        org.base + (long long)org.row0 * op.d_cols + org.col0;
-          if (op.vec8) {
-            int const cpr = ta.cols / 8, n8 = ta.rows * cpr;
+          int const d_cols = uniform(op.d_cols), io = uniform(op.io);
+          uint16_t *g = (P.splits > 1 ? P.part[io] + (long long)split * P.part_stride[io]
+                                      : static_cast<uint16_t *>(P.out[io])) +
+                        org.base + (long long)org.row0 * d_cols + org.col0;
+          if (uniform(op.vec8)) {
+            int const cpr = ta_cols / 8, n8 = ta_rows * cpr;
+            uint32_t const mcpr = (uint32_t)uniform((int)ta.mcpr);
             for (int e = tid; e < n8; e += kInterpThreads) {
               uint4v v = *reinterpret_cast<uint4v const *>(x + e * 8);
               if (!first) {
@@ -503,8 +521,8 @@ __device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned ch
                 }
               }
               if (last) {
-                int const r = fdiv(e, ta.mcpr), c = (e - r * cpr) * 8;
-                *reinterpret_cast<uint4v *>(g + (long long)r * op.d_cols + c) = v;
+                int const r = fdiv(e, mcpr), c = (e - r * cpr) * 8;
+                *reinterpret_cast<uint4v *>(g + (long long)r * d_cols + c) = v;
               } else {
                 *reinterpret_cast<uint4v *>(acc + e * 8) = v;
               }
@@ -516,8 +534,8 @@ __device__ __forceinline__ void fp_interp_block(DevProgram const &P, unsigned ch
                 v = (v + acc[e]) % FP_PQ;
               }
               if (last) {
-                int const r = fdiv(e, ta.mcols), c = e - r * ta.cols;
-                g[(long long)r * op.d_cols + c] = static_cast<uint16_t>(v);
+                int const r = fdiv(e, ta.mcols), c = e - r * ta_cols;
+                g[(long long)r * d_cols + c] = static_cast<uint16_t>(v);
               } else {
                 acc[e] = static_cast<uint16_t>(v);
               }
