@@ -72,6 +72,59 @@ def test_verify_batch_matches_oracle(rt):
             assert verdict == oracle_verdict == c["expect_equal"]
 
 
+def test_inputs_read_through_one_tensor_keep_every_graph_right(rt):
+    """A batch reads inputs number j of equal element count through the first graph's tensor,
+    and a launch splits an operand that several fused matmul plans share into residue planes
+    once.  Graphs of one batch whose inputs have the same counts but other shapes, other
+    operand roles and other prologues (so: the same bytes seen as [64,128] and as [128,64],
+    with and without exp in front) must still each give the oracle's outputs."""
+    from attention_superoptimizer_amd import workloads as W
+
+    def matmul_graph(m, k, n, tiles, exp_on_a):
+        mt, nt, kt = tiles
+        ops = []
+        a_ref = (0, 0)
+        if exp_on_a:
+            ops.append(("tb_exp_op", [(0, 0)]))
+            a_ref = (2, 0)
+        ops.append(("tb_matmul_op", [a_ref, (1, 0)]))
+        gx, gy = n // nt, m // mt
+        return [W._inp([m, k]), W._inp([k, n]),
+                {"op": "customized", "in": [[0, 0], [1, 0]],
+                 "plan": W._plan((gx, gy, 1), k // kt,
+                                 [(-1, 0, -1) if gy > 1 else (-1, -1, -1), (1, -1, -1) if gx > 1 else (-1, -1, -1)],
+                                 (1, 0), (1 if gx > 1 else -1, 0 if gy > 1 else -1, -1), ops)}]
+
+    # inputs 0 and 1 hold 8192 elements in every graph: [64,128].[128,64] and [128,64].[64,128]
+    specs = [matmul_graph(64, 128, 64, (32, 32, 64), False),
+             matmul_graph(128, 64, 128, (32, 64, 32), False),
+             matmul_graph(64, 128, 64, (16, 32, 32), True),
+             matmul_graph(64, 128, 64, (64, 64, 128), False),
+             matmul_graph(128, 64, 128, (64, 32, 64), True),
+             matmul_graph(64, 128, 64, (32, 32, 64), True),
+             matmul_graph(128, 64, 128, (128, 128, 64), False),
+             matmul_graph(64, 128, 64, (16, 64, 16), False)]
+    seed = 0x5A5A0001
+    ref_g, _ = rt.build_from_spec(specs[0])
+    built = [rt.build_from_spec(sp) for sp in specs]
+    try:
+        ref_g.fingerprint_seeded(seed)
+        verdicts, _ = rt.verify_batch([g for g, _ in built], ref_g, seed)
+        want_ref = _outputs(specs[0], orc.eval_graph(specs[0], "fp", _inputs(specs[0], seed), threads=8))[0]
+        for k, (sp, (_, vals)) in enumerate(zip(specs, built)):
+            want = _outputs(sp, orc.eval_graph(sp, "fp", _inputs(sp, seed), threads=8))
+            got = [t.read_fingerprint() for t in _outputs(sp, vals)]
+            assert len(got) == len(want) == 1
+            assert np.array_equal(got[0], want[0]), k
+            assert verdicts[k] == (want[0].shape == want_ref.shape and np.array_equal(want[0], want_ref)), k
+        # the same product under other tiles is equal; other shapes and exp in front are not
+        assert verdicts == [True, False, False, True, False, False, False, True]
+    finally:
+        for g, _ in reversed(built):
+            g.close()
+        ref_g.close()
+
+
 def test_verify_batch_full_size_verdicts(rt):
     """Full dims ([64, 1024]): rewrites verify equal, mutants unequal."""
     probs = C.generate(num_problems=8, per_problem=16, seed=0xBEEF)
