@@ -80,6 +80,7 @@ struct State {
   int force_interpreter = 0;
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
   int fp_vector_dot_only = 0;  // 1: fingerprint matmuls never take the matrix-core kernels
+  int fp_big_tiles = 1;        // 0: large kernel-level matmuls keep 64 x 64 tiles
   int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
   int direct_lanes = 0;      // MI355_OPT_DIRECT_LANES
   int gemm_mode = 0;         // MI355_OPT_GEMM_MODE

@@ -27,6 +27,7 @@
 #include "tb_program.h"
 
 #include <algorithm>
+#include <atomic>
 #include <vector>
 
 namespace mi355 {
@@ -200,7 +201,9 @@ struct GemmJob {
   int batch, m, n, kp;
   int mp, np;                 // m, n rounded up to 16
   int shared_k;               // 1: 32 x 32 tile per workgroup, wavefronts share k
-  int tiles_m, tiles_n;
+  int tiles_m, tiles_n;       // tiles of 32 (shared k), 64, or 128 (fp_mfma_matmul_big_kernel) rows / columns
+  int xcd_order;              // see tile_of_workgroup
+  uint32_t magic_per_batch, magic_width;  // division magics of tiles_m * tiles_n and 8 * tiles_n
   unsigned first_block;
 };
 struct GemmMany {
@@ -209,6 +212,67 @@ struct GemmMany {
 };
 
 __device__ __forceinline__ int fold_signed(int v, int mod) { return v % mod; }
+
+// Four consecutive outputs of row `row` from column `col` on, from their residue sums.
+__device__ __forceinline__ void store_outputs(uint16_t *out, int m, int n, bool whole4, int row, int col,
+                                              v4i const &sp, v4i const &sq) {
+  if (row >= m || col >= n) {
+    return;
+  }
+  uint32_t z[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    z[e] = fp_from_residue_sums(sp[e], sq[e]);
+  }
+  uint16_t *dst = out + (size_t)row * n + col;
+  if (whole4 && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+    uint2 w;
+    w.x = z[0] | (z[1] << 16);
+    w.y = z[2] | (z[3] << 16);
+    *reinterpret_cast<uint2 *>(dst) = w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      if (col + e < n) {
+        dst[e] = (uint16_t)z[e];
+      }
+    }
+  }
+}
+
+// Workgroup t of a job -> (batch, tile row, tile column).  Workgroups go to the 8 XCDs round
+// robin, so XCD x gets the contiguous range of positions [x * total / 8, ...) of the tile order:
+// the tiles that run together on one XCD are neighbours and share operand strips in that XCD's
+// L2.  The order walks eight tile rows at a time, column after column within them.  Divisions
+// by the job's tile counts are multiply-highs with magics from the host (a workgroup's first
+// loads wait for this arithmetic).  The host decides per job whether this order or the plain
+// one (row after row) is used.
+__device__ __forceinline__ void tile_of_workgroup(GemmJob const &J, unsigned t, int *b, int *tm, int *tn) {
+  unsigned const per_batch = (unsigned)(J.tiles_m * J.tiles_n);
+  if (!J.xcd_order) {
+    *b = (int)(t / per_batch);
+    t %= per_batch;
+    *tm = (int)(t / (unsigned)J.tiles_n);
+    *tn = (int)(t % (unsigned)J.tiles_n);
+    return;
+  }
+  unsigned const total = per_batch * (unsigned)J.batch;
+  unsigned const x = t % 8, slot = t / 8, base = total / 8, rem = total % 8;
+  unsigned const pos = x * base + min(x, rem) + slot;
+  unsigned const bb = J.magic_per_batch ? __umulhi(pos, J.magic_per_batch) : pos;
+  unsigned const l = pos - bb * per_batch;
+  unsigned const width = 8u * (unsigned)J.tiles_n;
+  unsigned const group = __umulhi(l, J.magic_width), within = l - group * width;
+  int const first = (int)group * 8, rows = min(J.tiles_m - first, 8);
+  *b = (int)bb;
+  if (rows == 8) {
+    *tm = first + (int)(within & 7u);
+    *tn = (int)(within >> 3);
+  } else {  // the last rows of a tile count that is no multiple of eight
+    *tm = first + (int)(within % (unsigned)rows);
+    *tn = (int)(within / (unsigned)rows);
+  }
+}
 
 __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const G) {
   __shared__ int part[4][32][64];  // shared-k reduction: [wavefront][register][lane]
@@ -220,18 +284,20 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
   int const tid = threadIdx.x, wave = tid / 64, lane = tid % 64, r = lane % 16, g = lane / 16;
   unsigned t = blockIdx.x - J.first_block;
   int const per_batch = J.tiles_m * J.tiles_n;
-  int const b = (int)(t / per_batch);
-  t %= per_batch;
   int const steps = J.kp / 64;
-  int row0, col0, s_begin, s_end;
+  int b, row0, col0, s_begin, s_end;
   if (J.shared_k) {
+    b = (int)(t / per_batch);
+    t %= per_batch;
     row0 = (int)(t / J.tiles_n) * 32;
     col0 = (int)(t % J.tiles_n) * 32;
     s_begin = (int)((long long)steps * wave / 4);
     s_end = (int)((long long)steps * (wave + 1) / 4);
   } else {
-    row0 = (int)(t / J.tiles_n) * 64 + (wave / 2) * 32;
-    col0 = (int)(t % J.tiles_n) * 64 + (wave % 2) * 32;
+    int tm, tn;
+    tile_of_workgroup(J, t, &b, &tm, &tn);
+    row0 = tm * 64 + (wave / 2) * 32;
+    col0 = tn * 64 + (wave % 2) * 32;
     s_begin = 0;
     s_end = steps;
   }
@@ -309,29 +375,7 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
   uint16_t *out = J.out + (size_t)b * J.m * J.n;
   bool const whole4 = J.n % 4 == 0;
   auto store = [&](int i, int jn, v4i const &sp, v4i const &sq) {
-    int const row = row0 + 16 * i + r, col = col0 + 16 * jn + 4 * g;
-    if (row >= J.m || col >= J.n) {
-      return;
-    }
-    uint32_t z[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      z[e] = fp_from_residue_sums(sp[e], sq[e]);
-    }
-    uint16_t *dst = out + (size_t)row * J.n + col;
-    if (whole4 && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
-      uint2 w;
-      w.x = z[0] | (z[1] << 16);
-      w.y = z[2] | (z[3] << 16);
-      *reinterpret_cast<uint2 *>(dst) = w;
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        if (col + e < J.n) {
-          dst[e] = (uint16_t)z[e];
-        }
-      }
-    }
+    store_outputs(out, J.m, J.n, whole4, row0 + 16 * i + r, col0 + 16 * jn + 4 * g, sp, sq);
   };
   if (!J.shared_k) {
 #pragma unroll
@@ -366,6 +410,187 @@ __global__ __launch_bounds__(kThreads) void fp_mfma_matmul_kernel(GemmMany const
     }
   }
   store(wave / 2, wave % 2, sp, sq);
+}
+
+// ---- large kernel-level matmuls: 128 x 128 tiles, operand strips shared through LDS ------
+// Every lane fetches 16 bytes from `gbase` (wave-uniform) + its own byte offset; the wavefront's
+// 64 chunks land in LDS at `lds_wave_base` + 16 * lane without passing through registers
+// (completion is counted by vmcnt).  Inline assembly so that the compiler does not make the
+// next LDS read wait for the transfer; the caller waits before the barrier that publishes it.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void plane_dma16(int8_t const *gbase, uint32_t lane_byte_offset,
+                                            uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(lane_byte_offset), "s"(gbase)
+               : "m0", "memory");
+}
+#pragma clang diagnostic pop
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+// A 16-byte load whose latency the compiler knows nothing of: `dst` holds the data only after
+// landed<N>() on it (N = transfers issued after this one that may still be in flight).  Both
+// stand in the same straight-line piece of code, so the compiler has no reason to move or
+// copy `dst` in between, and only landed values are carried round a loop.
+__device__ __forceinline__ void plane_load16(v4i &dst, int8_t const *gbase, uint32_t lane_byte_offset) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(lane_byte_offset), "s"(gbase) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void landed(v4i (&b)[4]) {
+  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) : "n"(N) : "memory");
+}
+#pragma clang diagnostic pop
+
+constexpr int kBigStage = 16384;  // A of one 64-k step: (mod 227, mod 113) x 8 strips x 1 KB
+constexpr int kBigStages = 4;
+constexpr int kBigLdsBytes = kBigStages * kBigStage;
+constexpr long long kBigMinTiles = 192;  // 128 x 128 tiles from here on (256 compute units)
+constexpr int kBigMaxK = 2048 * 64;
+
+// A workgroup owns a 128 x 128 output tile; wavefront w works in one residue field (w & 1) on
+// one half of the tile's columns (w >> 1): 128 x 64 sums, 32 matrix instructions per step of
+// 64 k.  Operand blocks are 1 KB (16 plane rows x 64 k, contiguous in the blocked planes, lane
+// l's operand of v_mfma_i32_16x16x64_i8 is bytes [16 l, 16 l + 16) of it).  The 16 A blocks of
+// a step (8 row strips x 2 residues) are needed by two wavefronts each: they are copied to LDS
+// three steps ahead (four stages of 16 KB), 4 transfers per wavefront, and read from there one
+// step ahead.  The 4 B^T blocks a wavefront needs are needed by nobody else: it loads them
+// straight into registers, one step ahead.  Against one 64 x 64 tile per workgroup with
+// operands read straight from L2 by every wavefront, a tile's operands cross L2 -> compute
+// unit once per 128 x 128 instead of once per 32 x 32 quadrant.  Two workgroups per compute
+// unit.  The host sends matmuls of at most kBigMaxK k here: 2048 steps x 64 k x 113^2 < 2^31,
+// so the int32 sums need no fold on the way.
+__global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMany const G) {
+  extern __shared__ __attribute__((aligned(16))) int8_t big_lds[];
+  int j = 0;
+  while (j + 1 < G.count && blockIdx.x >= G.job[j + 1].first_block) {
+    j++;
+  }
+  GemmJob const &J = G.job[j];
+  int const tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  int const r = lane % 16, g = lane / 16;
+  int const res = wave & 1, half = wave >> 1;
+  int b, tm, tn;
+  tile_of_workgroup(J, blockIdx.x - J.first_block, &b, &tm, &tn);
+  int const row0 = tm * 128, col0 = tn * 128 + half * 64;
+  int const steps = J.kp / 64;
+  uint32_t const strip_bytes = (uint32_t)J.kp * 16u;
+  // this wavefront copies 4 of the 16 A blocks of a step: residue wave / 2, strips 4 (wave % 2) ..
+  int8_t const *a_plane = (wave / 2 == 0 ? J.a_p : J.a_q) + (size_t)b * (size_t)J.mp * (size_t)J.kp;
+  int8_t const *b_plane = (res == 0 ? J.bt_p : J.bt_q) + (size_t)b * (size_t)J.np * (size_t)J.kp;
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    a_off[i] = (uint32_t)(min(row0 + 16 * ((wave % 2) * 4 + i), J.mp - 16) / 16) * strip_bytes + (uint32_t)lane * 16u;
+    b_off[i] = (uint32_t)(min(col0 + 16 * i, J.np - 16) / 16) * strip_bytes + (uint32_t)lane * 16u;
+  }
+  uint32_t const lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void const *)big_lds;
+  // Transfers are issued for every step up to three past the last one (the last step's data
+  // again, into a stage / registers nobody reads any more): the queue of outstanding transfers
+  // then looks the same at every wait and the waits need no conditions.
+  auto issue_a = [&](int s) {
+    int8_t const *src = a_plane + (size_t)min(s, steps - 1) * 1024;
+    uint32_t const dst = lds0 + (uint32_t)((s % kBigStages) * kBigStage + wave * 4096);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      plane_dma16(src, a_off[i], dst + (uint32_t)i * 1024u);
+    }
+  };
+  auto issue_b = [&](int s, v4i (&buf)[4]) {
+    int8_t const *src = b_plane + (size_t)min(s, steps - 1) * 1024;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      plane_load16(buf[i], src, b_off[i]);
+    }
+  };
+  v4i acc[8][4];
+#pragma unroll
+  for (int e = 0; e < 32; e++) {
+    acc[e / 4][e % 4] = v4i{0, 0, 0, 0};
+  }
+  // A: three steps ahead through the four LDS stages.  B^T: one step ahead in registers; a
+  // load and the wait for it stand in the same iteration, and only values that have landed
+  // are carried round the loop (the compiler knows nothing of the loads' latency).
+  v4i cur[4], next[4], a[8], a_next[8];
+  issue_a(0);
+  issue_a(1);
+  issue_b(0, cur);
+  issue_a(2);
+  landed<4>(cur);  // A(0), A(1) and B(0) are there; A(2) may still be on its way
+  __syncthreads();
+  {
+    int8_t const *stage = big_lds + res * 8192 + lane * 16;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      a[i] = *reinterpret_cast<v4i const *>(stage + i * 1024);
+    }
+  }
+  // one step: multiplies (a_now, b_now) while the next step's operands arrive in (a_new, b_new);
+  // the loop runs it twice with the register sets swapped, so nothing is copied
+  auto step = [&](int s, v4i (&a_now)[8], v4i (&b_now)[4], v4i (&a_new)[8], v4i (&b_new)[4]) {
+    if (s > 0) {
+      __syncthreads();  // A(s + 1) is in LDS; everyone has the stage of step s - 1 in registers
+    }
+    issue_b(s + 1, b_new);
+    issue_a(s + 3);
+    int8_t const *stage = big_lds + ((s + 1) % kBigStages) * kBigStage + res * 8192 + lane * 16;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      a_new[i] = *reinterpret_cast<v4i const *>(stage + i * 1024);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // the next step's operands are on their way before ...
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+      for (int jn = 0; jn < 4; jn++) {
+        acc[i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b_now[jn], a_now[i], acc[i][jn], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // ... this step's products, and awaited after them
+    landed<4>(b_new);  // B(s + 1) and, issued before it, A(s + 2)
+  };
+  for (int s = 0; s < steps; s += 2) {
+    step(s, a, cur, a_next, next);
+    if (s + 1 < steps) {
+      step(s + 1, a_next, next, a, cur);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the transfers past the last step
+  // The two wavefronts of a column half hold the sums mod 227 and mod 113 of the same outputs:
+  // each hands the other one half of its rows (through LDS, lane for lane) and finishes the half
+  // it keeps.
+  __syncthreads();
+  v4i *mine = reinterpret_cast<v4i *>(big_lds) + wave * 1024, *theirs = reinterpret_cast<v4i *>(big_lds) + (wave ^ 1) * 1024;
+  // (row strips 4 - 7 given away by the mod 227 wavefront, 0 - 3 by the mod 113 one; written
+  // with constant register indices under a wave-uniform branch)
+  if (res == 0) {
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      mine[e * 64 + lane] = acc[4 + e / 4][e % 4];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      mine[e * 64 + lane] = acc[e / 4][e % 4];
+    }
+  }
+  __syncthreads();
+  uint16_t *out = J.out + (size_t)b * J.m * J.n;
+  bool const whole4 = J.n % 4 == 0;
+  if (res == 0) {
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      store_outputs(out, J.m, J.n, whole4, row0 + (e / 4) * 16 + r, col0 + (e % 4) * 16 + 4 * g,
+                    acc[e / 4][e % 4], theirs[e * 64 + lane]);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      store_outputs(out, J.m, J.n, whole4, row0 + (4 + e / 4) * 16 + r, col0 + (e % 4) * 16 + 4 * g,
+                    theirs[e * 64 + lane], acc[4 + e / 4][e % 4]);
+    }
+  }
 }
 
 // ---- fused tiled-matmul plans (load A tile, load B tile, matmul, accumulate, store) -------
@@ -780,10 +1005,10 @@ static bool mfma_matmul_fits(int batch, int m, int n, int k, size_t *plane_bytes
 static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B, uint16_t *const *C,
                              int const *batch, int const *m, int const *n, int const *k, int count) {
   std::vector<SplitJob> jobs((size_t)(2 * count));
-  GemmMany G{};
+  GemmMany G{}, Big{};  // jobs of the 64 x 64 / 32 x 32 kernel, jobs of the 128 x 128 kernel
   char *planes = state().planes();
   size_t used = 0;
-  unsigned gemm_blocks = 0;
+  unsigned gemm_blocks = 0, big_blocks = 0;
   for (int e = 0; e < count; e++) {
     int const kp = (int)round_up((size_t)k[e], 64);
     int const mp = (int)round_up((size_t)m[e], 16), np = (int)round_up((size_t)n[e], 16);
@@ -820,7 +1045,7 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     sb.vec = n[e] % 4 == 0 && (reinterpret_cast<uintptr_t>(B[e]) & 7) == 0;
     size_t const b_tiles = (size_t)batch[e] * (kp / 64) * ((n[e] + 63) / 64);
     sb.blocks = (unsigned)std::min<size_t>(b_tiles, 1024);
-    GemmJob &g = G.job[e];
+    GemmJob g{};
     g.a_p = a_p;
     g.a_q = a_q;
     g.bt_p = bt_p;
@@ -832,21 +1057,51 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     g.kp = kp;
     g.mp = mp;
     g.np = np;
-    long long const big_tiles = (long long)((m[e] + 63) / 64) * ((n[e] + 63) / 64) * batch[e];
-    g.shared_k = big_tiles < 64;
-    int const edge = g.shared_k ? 32 : 64;
+    long long const tiles64 = (long long)((m[e] + 63) / 64) * ((n[e] + 63) / 64) * batch[e];
+    long long const tiles128 = (long long)((m[e] + 127) / 128) * ((n[e] + 127) / 128) * batch[e];
+    // 128 x 128 tiles once they fill the device (a tile's plane offsets are 32-bit there)
+    bool const large = tiles128 >= kBigMinTiles && state().fp_big_tiles && kp <= kBigMaxK &&
+                       (size_t)std::max(mp, np) * (size_t)kp < ((size_t)1 << 31);
+    g.shared_k = !large && tiles64 < 64;
+    int const edge = large ? 128 : (g.shared_k ? 32 : 64);
     g.tiles_m = (m[e] + edge - 1) / edge;
     g.tiles_n = (n[e] + edge - 1) / edge;
-    g.first_block = gemm_blocks;
-    gemm_blocks += (unsigned)((long long)g.tiles_m * g.tiles_n * batch[e]);
+    unsigned const blocks = (unsigned)((long long)g.tiles_m * g.tiles_n * batch[e]);
+    // Measured with the split launch in front, as it runs: the XCD-aware order pays once the
+    // tiles no longer all run at once (8 x 1024^3: 40 against 49 us); for fewer it costs a
+    // microsecond although it halves the bytes fetched (1024^3 on 64 x 64 tiles: 16.6 against
+    // 15.1 us).  The magics are exact while dividend * divisor < 2^32 (dividends: below `blocks`).
+    g.xcd_order = large && blocks >= 512u && blocks < 65536u;
+    g.magic_per_batch = fast_div_magic(g.tiles_m * g.tiles_n);
+    g.magic_width = fast_div_magic(8 * g.tiles_n);
+    if (large) {
+      g.first_block = big_blocks;
+      big_blocks += blocks;
+      Big.job[Big.count++] = g;
+    } else {
+      g.first_block = gemm_blocks;
+      gemm_blocks += blocks;
+      G.job[G.count++] = g;
+    }
   }
-  G.count = count;
   hipStream_t st = state().stream();
   if (int rc = launch_split_jobs(jobs.data(), 2 * count, st)) {
     return rc;
   }
-  fp_mfma_matmul_kernel<<<gemm_blocks, kThreads, 0, st>>>(G);
-  MI355_HIP(hipGetLastError());
+  if (G.count > 0) {
+    fp_mfma_matmul_kernel<<<gemm_blocks, kThreads, 0, st>>>(G);
+    MI355_HIP(hipGetLastError());
+  }
+  if (Big.count > 0) {
+    static std::atomic<int> granted{0};
+    if (granted.load(std::memory_order_acquire) < kBigLdsBytes) {
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_mfma_matmul_big_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
+      granted.store(kBigLdsBytes, std::memory_order_release);
+    }
+    fp_mfma_matmul_big_kernel<<<big_blocks, kThreads, kBigLdsBytes, st>>>(Big);
+    MI355_HIP(hipGetLastError());
+  }
   return MI355_OK;
 }
 

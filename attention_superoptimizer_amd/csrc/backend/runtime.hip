@@ -261,8 +261,9 @@ extern "C" int mi355_set_option(int option, int value) {
     state().plan_smem_layout = value;
     return MI355_OK;
   }
-  if (option == MI355_OPT_FP_MATMUL_ROUTE && (value == 0 || value == 1)) {
-    state().fp_vector_dot_only = value;
+  if (option == MI355_OPT_FP_MATMUL_ROUTE && value >= 0 && value <= 2) {
+    state().fp_vector_dot_only = value == 1;
+    state().fp_big_tiles = value != 2;
     return MI355_OK;
   }
   if (option == MI355_OPT_DIRECT_LANES && (value == 0 || value == 1 || value == 4)) {

@@ -110,7 +110,9 @@ typedef struct mi355_launch_info {
 #define MI355_OPT_PLAN_SMEM_LAYOUT 3
 /* FP_MATMUL_ROUTE: 0 = fingerprint matmuls (kernel-level and the fused tiled-matmul plans)
  * take the int8 matrix-core kernels whenever their shapes allow (default); 1 = always the
- * packed 4 x 8-bit vector-dot kernels.  Results are bit-identical; tests run both. */
+ * packed 4 x 8-bit vector-dot kernels; 2 = as 0, but large kernel-level matmuls keep the
+ * 64 x 64 tiles of the smaller ones instead of 128 x 128 tiles staged through LDS.  Results
+ * are bit-identical; tests run all three. */
 #define MI355_OPT_FP_MATMUL_ROUTE 4
 /* PHASE_TRACE: 1 = launches of the direct-staging attention kernel record six wall-clock
  * stamps (100 MHz) per wavefront -- start, loads issued, first tiles landed, arithmetic done,

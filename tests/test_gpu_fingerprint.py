@@ -382,6 +382,29 @@ def test_many_matmuls_on_the_matrix_cores_match_oracle(rt, abi):
         assert np.array_equal(C, orc.fp_matmul(A, B)), s
 
 
+def test_large_matmuls_on_128_tiles_match_oracle(rt, abi):
+    """Matmuls with 192 or more 128 x 128 output tiles take the kernel that stages operand strips
+    through LDS: ragged edges in rows, columns and k, a batch, one k step and an odd number of
+    them, together with small matmuls in the same call; with the option that keeps 64 x 64
+    tiles the same calls give the same bits."""
+    shapes = [(1, 2008, 1544, 200), (3, 1024, 1024, 72), (1, 48, 80, 64), (1, 2048, 2048, 64),
+              (2, 1100, 1500, 330), (1, 16, 16, 16)]
+    fill = lambda i, d: uniform_fp(d, 900 + i)
+    ins, got = _matmul_many(abi, rt, shapes, fill)
+    for (A, B), C, s in zip(ins, got, shapes):
+        assert np.array_equal(C, orc.fp_matmul(A, B)), s
+    assert abi.mi355_set_option(4, 2) == 0
+    try:
+        _, again = _matmul_many(abi, rt, shapes, fill)
+    finally:
+        assert abi.mi355_set_option(4, 0) == 0
+    for C, D, s in zip(got, again, shapes):
+        assert np.array_equal(C, D), s
+    x = (114 * 25425 + 112 * 227) % FP_PQ       # = -113 (mod 227), 112 (mod 113)
+    _, ext = _matmul_many(abi, rt, [(1, 1536, 2048, 8192)], lambda i, d: np.full(d, x, np.uint16))
+    assert np.all(ext[0] == (8192 * x * x) % FP_PQ)
+
+
 def test_matrix_core_matmul_extreme_values_and_long_k(rt, abi):
     """Operands whose residues are the largest in magnitude the planes hold (-113 mod 227,
     112 mod 113), k long enough that a wavefront's int32 sums must be folded on the way."""
