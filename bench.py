@@ -141,6 +141,35 @@ def _spec_inputs(spec, seed):
     return ins
 
 
+def fp_matmul_rate(G, abi, shape, steps: int, warmup: int, both_routes: bool):
+    """Kernel-level fingerprint matmul [b, m, k] x [b, k, n] (reference compute_matmul_fingerprint,
+    src/kernel/cuda/matmul_kernel.cu:145-203): microseconds per matmul, operand splitting included,
+    timed with stream events over back-to-back calls; one multiply-accumulate of the ring counted
+    once.  `both_routes` adds the packed 8-bit dot-product route."""
+    b, m, n, k = shape
+    g = G.KNGraph()
+    A, B = g.new_input((b, m, k)), g.new_input((b, k, n))
+    g.matmul(A, B)
+    g.fingerprint(0)
+    g.fingerprint(1)
+    rec = {"shape": [b, m, n, k], "macs": b * m * n * k}
+    for route, name in ((0, "matrix_cores"), (1, "vector_dot")) if both_routes else ((0, "matrix_cores"),):
+        assert abi.mi355_set_option(4, route) == 0
+        for _ in range(max(1, warmup // 64)):
+            g.fingerprint(2)
+        assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
+        iters = max(1, steps // 16)
+        for _ in range(iters):
+            g.fingerprint(2)
+        ms = ctypes.c_float()
+        assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
+        us = ms.value * 1e3 / iters
+        rec[name] = {"us": round(us, 2), "T_MACps": round(b * m * n * k / us / 1e6, 2)}
+    assert abi.mi355_set_option(4, 0) == 0
+    g.close()
+    return rec
+
+
 def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_problem: int = 64,
                            in_flight: int = 16, queues_per_submission: int = 1,
                            other_shapes: bool = True):
@@ -320,28 +349,8 @@ def main() -> int:
         return 0
 
     if args.fp_matmul:
-        b, m, n, k = (int(x) for x in args.fp_matmul.split(","))
-        g = G.KNGraph()
-        A, B = g.new_input((b, m, k)), g.new_input((b, k, n))
-        g.matmul(A, B)
-        g.fingerprint(0)
-        g.fingerprint(1)
-        rec = {"shape": [b, m, n, k], "macs": b * m * n * k}
-        for route, name in ((0, "matrix_cores"), (1, "vector_dot")):
-            assert abi.mi355_set_option(4, route) == 0
-            for _ in range(max(1, args.warmup // 64)):
-                g.fingerprint(2)
-            assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
-            iters = max(1, args.steps // 16)
-            for _ in range(iters):
-                g.fingerprint(2)
-            ms = ctypes.c_float()
-            assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
-            us = ms.value * 1e3 / iters
-            rec[name] = {"us": round(us, 2), "T_MACps": round(b * m * n * k / us / 1e6, 2)}
-        assert abi.mi355_set_option(4, 0) == 0
-        print(json.dumps(rec), flush=True)
-        g.close()
+        shape = tuple(int(x) for x in args.fp_matmul.split(","))
+        print(json.dumps(fp_matmul_rate(G, abi, shape, args.steps, args.warmup, True)), flush=True)
         return 0
 
     if args.calibrate_copy:
@@ -547,6 +556,9 @@ def main() -> int:
     if not args.headline_only and not args.no_fingerprints:
         g.close()
         result["fingerprint_throughput"] = fingerprint_throughput(G, not args.no_cpu_baseline)
+        result["fingerprint_matmul"] = [fp_matmul_rate(G, abi, sh, steps, 1024, False)
+                                        for sh, steps in (((1, 1024, 1024, 1024), 2048),
+                                                          ((1, 4096, 4096, 4096), 256))]
         spec, g, vals = setup("C2_gqa_decode")
     floor = ctypes.c_float()
     if abi.mi355_launch_floor(2048, ctypes.byref(floor)) == 0:
