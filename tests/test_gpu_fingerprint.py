@@ -385,10 +385,13 @@ def test_many_matmuls_on_the_matrix_cores_match_oracle(rt, abi):
 def test_large_matmuls_on_128_tiles_match_oracle(rt, abi):
     """Matmuls with 192 or more 128 x 128 output tiles take the kernel that stages operand strips
     through LDS: ragged edges in rows, columns and k, a batch, one k step and an odd number of
-    them, together with small matmuls in the same call; with the option that keeps 64 x 64
-    tiles the same calls give the same bits."""
+    them, both tile orders, together with small matmuls in the same call; with the option that
+    keeps 64 x 64 tiles the same calls give the same bits."""
     shapes = [(1, 2008, 1544, 200), (3, 1024, 1024, 72), (1, 48, 80, 64), (1, 2048, 2048, 64),
-              (2, 1100, 1500, 330), (1, 16, 16, 16)]
+              (2, 1100, 1500, 330), (1, 16, 16, 16),
+              # 512 tiles or more: the order in which workgroups take tiles follows the XCDs; tile
+              # rows that are no multiple of 8, tile counts that are no multiple of 8, a batch
+              (1, 2700, 3200, 64), (3, 1700, 1800, 100)]
     fill = lambda i, d: uniform_fp(d, 900 + i)
     ins, got = _matmul_many(abi, rt, shapes, fill)
     for (A, B), C, s in zip(ins, got, shapes):
