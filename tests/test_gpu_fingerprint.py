@@ -408,6 +408,23 @@ def test_large_matmuls_on_128_tiles_match_oracle(rt, abi):
     assert np.all(ext[0] == (8192 * x * x) % FP_PQ)
 
 
+def test_full_size_matmul_checksum_of_checksums(rt, abi):
+    """4096 x 4096 x 4096, uniform inputs: too large for the oracle as a whole, so the check is
+    linear algebra in the ring: (1^T A) B = 1^T (A B) and A (B 1) = (A B) 1.  The two vector
+    products are the oracle's; the sums are exact integer arithmetic."""
+    n = 4096
+    ins, got = _matmul_many(abi, rt, [(1, n, n, n)], lambda i, d: uniform_fp(d, 4000 + i))
+    (A, B), C = ins[0], got[0]
+    A2, B2, C2 = (x.reshape(n, n).astype(np.int64) for x in (A, B, C))
+    assert C2.max() < FP_PQ
+    col_of_a = (A2.sum(axis=0) % FP_PQ).astype(np.uint16).reshape(1, 1, n)
+    row_of_b = (B2.sum(axis=1) % FP_PQ).astype(np.uint16).reshape(1, n, 1)
+    want_cols = orc.fp_matmul(col_of_a, B.reshape(1, n, n)).reshape(n).astype(np.int64)
+    want_rows = orc.fp_matmul(A.reshape(1, n, n), row_of_b).reshape(n).astype(np.int64)
+    assert np.array_equal(C2.sum(axis=0) % FP_PQ, want_cols)
+    assert np.array_equal(C2.sum(axis=1) % FP_PQ, want_rows)
+
+
 def test_matrix_core_matmul_extreme_values_and_long_k(rt, abi):
     """Operands whose residues are the largest in magnitude the planes hold (-113 mod 227,
     112 mod 113), k long enough that a wavefront's int32 sums must be folded on the way."""
