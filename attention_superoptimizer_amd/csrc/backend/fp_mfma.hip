@@ -210,6 +210,7 @@ struct GemmMany {
   GemmJob job[kMaxJobs];
   int count;
 };
+static_assert(sizeof(GemmMany) <= 4096, "kernel arguments are limited to 4 KB");
 
 __device__ __forceinline__ int fold_signed(int v, int mod) { return v % mod; }
 
