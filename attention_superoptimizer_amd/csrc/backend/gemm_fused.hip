@@ -420,7 +420,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
 // iteration order (fp16 rounding after each add: the rounding sequence of the sequential
 // loop) and stores the block's output tile.  A separate launch rather than a last-arriver
 // fix-up: the kernel boundary makes the slabs visible without device-scope fences,
-// which on this part write back and invalidate a whole L2 each time.
+// which on this part write back and invalidate a whole L2 each time (with a fence per
+// workgroup the LoRA plan took 77 us instead of 13).
 template <int NB>
 __global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
   int const tid = threadIdx.x, M = P.M, F = P.forloop_range;
