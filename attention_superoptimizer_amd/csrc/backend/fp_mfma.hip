@@ -434,7 +434,9 @@ __device__ __forceinline__ void plane_dma16(int8_t const *gbase, uint32_t lane_b
 // A 16-byte load whose latency the compiler knows nothing of: `dst` holds the data only after
 // landed<N>() on it (N = transfers issued after this one that may still be in flight).  Both
 // stand in the same straight-line piece of code, so the compiler has no reason to move or
-// copy `dst` in between, and only landed values are carried round a loop.
+// copy `dst` in between, and only landed values are carried round a loop.  A kernel that uses
+// this must not spill registers (a spill of `dst` before its wait would save stale data): the
+// one below builds with 235 vector registers and no scratch memory.
 __device__ __forceinline__ void plane_load16(v4i &dst, int8_t const *gbase, uint32_t lane_byte_offset) {
   asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(lane_byte_offset), "s"(gbase) : "memory");
 }
