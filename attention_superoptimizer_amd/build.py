@@ -33,6 +33,31 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
                 "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
+# source file -> kernels that must build without register spills (see build_backend)
+NO_SPILL_KERNELS = {"fp_mfma.hip": ["fp_mfma_matmul_big_kernel"]}
+
+
+def resource_usage(remarks):
+    """Per kernel (mangled name) the figures of hipcc's -Rpass-analysis=kernel-resource-usage."""
+    usage, name = {}, None
+    for line in remarks.splitlines():
+        if "remark: Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+        elif name and "remark:" in line and ":" in line.split("remark:")[1]:
+            key, _, value = line.split("remark:")[1].partition(":")
+            usage.setdefault(name, {})[key.strip()] = value.split("[")[0].strip()
+    return usage
+
+
+def spilling(usage, kernel):
+    """Resource figures of the kernels named `kernel` that use scratch memory or spill vector
+    registers; raises if the compiler reported nothing for that name."""
+    hits = [u for n, u in usage.items() if kernel in n]
+    if not hits:
+        raise RuntimeError(f"no resource usage reported for {kernel}")
+    return [u for u in hits if u.get("ScratchSize [bytes/lane]") != "0" or u.get("VGPRs Spill") != "0"]
+
+
 def _sources(sub, exts):
     d = os.path.join(CSRC, sub)
     return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(exts))
@@ -50,7 +75,24 @@ def build_backend():
     def compile_one(pair):
         s, o = pair
         lang = ["-x", "hip"] if s.endswith(".hip") else []
-        _run([HIPCC] + DEVICE_FLAGS + ["-I", INCLUDE, "-I", os.path.join(CSRC, "backend"), "-c"] + lang + [s, "-o", o])
+        cmd = [HIPCC] + DEVICE_FLAGS + ["-I", INCLUDE, "-I", os.path.join(CSRC, "backend"), "-c"] + lang + [s, "-o", o]
+        must_not_spill = NO_SPILL_KERNELS.get(os.path.basename(s))
+        if not must_not_spill:
+            _run(cmd)
+            return
+        # kernels whose inline-assembly loads land in registers behind the compiler's back: a
+        # spill between such a load and its wait would save stale data, so the build fails on one
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
+        print(" ".join(cmd), flush=True)
+        done = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+        if done.returncode != 0:
+            sys.stderr.write(done.stderr)
+            raise subprocess.CalledProcessError(done.returncode, cmd)
+        usage = resource_usage(done.stderr)
+        for kernel in must_not_spill:
+            bad = spilling(usage, kernel)
+            if bad:
+                raise RuntimeError(f"{s}: {kernel} spills registers: {bad}")
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         list(pool.map(compile_one, zip(srcs, objs)))

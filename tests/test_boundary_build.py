@@ -110,3 +110,31 @@ def test_checkpoint_object_loads_and_passes_through():
     # a single-graph file (what cpp_examples/profile.cc takes) loads as a one-graph checkpoint
     with pytest.raises(ValueError):
         G.Checkpoint.load(os.path.join(GOLDEN, "no_such_file.json"))
+
+
+def test_build_refuses_register_spills_in_kernels_with_asynchronous_register_loads():
+    """build.py reads the compiler's resource report for the kernels whose inline-assembly
+    loads write registers behind the compiler's back and fails the build when one of them
+    spills (a spill between such a load and its wait would save stale data)."""
+    from attention_superoptimizer_amd import build as B
+
+    def report(name, scratch, spilled):
+        head = "csrc/backend/x.hip:1:1: remark: "
+        tail = " [-Rpass-analysis=kernel-resource-usage]\n"
+        return (head + f"Function Name: _ZN5mi355{len(name)}{name}E" + tail +
+                head + "    VGPRs: 235" + tail +
+                head + f"    ScratchSize [bytes/lane]: {scratch}" + tail +
+                head + "    Occupancy [waves/SIMD]: 2" + tail +
+                head + f"    VGPRs Spill: {spilled}" + tail)
+
+    text = report("fp_mfma_matmul_kernel", 64, 3) + report("fp_mfma_matmul_big_kernel", 0, 0)
+    usage = B.resource_usage(text)
+    assert len(usage) == 2
+    assert B.spilling(usage, "fp_mfma_matmul_big_kernel") == []
+    assert B.spilling(usage, "fp_mfma_matmul_kernel")[0]["VGPRs Spill"] == "3"
+    assert B.spilling(B.resource_usage(report("fp_mfma_matmul_big_kernel", 528, 0)),
+                      "fp_mfma_matmul_big_kernel")[0]["ScratchSize [bytes/lane]"] == "528"
+    with pytest.raises(RuntimeError):
+        B.spilling(usage, "no_such_kernel")
+    for names in B.NO_SPILL_KERNELS.values():
+        assert names
