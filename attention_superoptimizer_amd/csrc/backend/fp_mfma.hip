@@ -444,17 +444,21 @@ template <int N>
 __device__ __forceinline__ void landed(v4i (&b)[4]) {
   asm volatile("s_waitcnt vmcnt(%4)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) : "n"(N) : "memory");
 }
+template <int N>
+__device__ __forceinline__ void landed(v4i (&b)[2]) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(b[0]), "+v"(b[1]) : "n"(N) : "memory");
+}
 #pragma clang diagnostic pop
 
 constexpr int kBigStage = 16384;  // A of one 64-k step: (mod 227, mod 113) x 8 strips x 1 KB
 constexpr int kBigStages = 4;
 constexpr int kBigLdsBytes = kBigStages * kBigStage;
-constexpr long long kBigMinTiles = 192;  // 128 x 128 tiles from here on (256 compute units)
+constexpr long long kBigMinTiles = 256;  // tiles of fp_mfma_matmul_big_kernel from here on (256 compute units)
 constexpr int kBigMaxK = 2048 * 64;
 
-// A workgroup owns a 128 x 128 output tile; wavefront w works in one residue field (w & 1) on
-// one half of the tile's columns (w >> 1): 128 x 64 sums, 32 matrix instructions per step of
-// 64 k.  Operand blocks are 1 KB (16 plane rows x 64 k, contiguous in the blocked planes, lane
+// A workgroup owns a 128 x TN output tile, TN = 128 or (for matmuls with too few of those) 64;
+// wavefront w works in one residue field (w & 1) on one half of the tile's columns (w >> 1):
+// with TN = 128, 128 x 64 sums and 32 matrix instructions per step of 64 k.  Operand blocks are 1 KB (16 plane rows x 64 k, contiguous in the blocked planes, lane
 // l's operand of v_mfma_i32_16x16x64_i8 is bytes [16 l, 16 l + 16) of it).  The 16 A blocks of
 // a step (8 row strips x 2 residues) are needed by two wavefronts each: they are copied to LDS
 // three steps ahead (four stages of 16 KB), 4 transfers per wavefront, and read from there one
@@ -464,7 +468,9 @@ constexpr int kBigMaxK = 2048 * 64;
 // unit once per 128 x 128 instead of once per 32 x 32 quadrant.  Two workgroups per compute
 // unit.  The host sends matmuls of at most kBigMaxK k here: 2048 steps x 64 k x 113^2 < 2^31,
 // so the int32 sums need no fold on the way.
+template <int TN>  // columns of the tile: 128 or 64
 __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMany const G) {
+  constexpr int NB = TN / 32;  // B^T blocks (16 columns each) per wavefront
   extern __shared__ __attribute__((aligned(16))) int8_t big_lds[];
   int j = 0;
   while (j + 1 < G.count && blockIdx.x >= G.job[j + 1].first_block) {
@@ -476,16 +482,19 @@ __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMan
   int const res = wave & 1, half = wave >> 1;
   int b, tm, tn;
   tile_of_workgroup(J, blockIdx.x - J.first_block, &b, &tm, &tn);
-  int const row0 = tm * 128, col0 = tn * 128 + half * 64;
+  int const row0 = tm * 128, col0 = tn * TN + half * (TN / 2);
   int const steps = J.kp / 64;
   uint32_t const strip_bytes = (uint32_t)J.kp * 16u;
   // this wavefront copies 4 of the 16 A blocks of a step: residue wave / 2, strips 4 (wave % 2) ..
   int8_t const *a_plane = (wave / 2 == 0 ? J.a_p : J.a_q) + (size_t)b * (size_t)J.mp * (size_t)J.kp;
   int8_t const *b_plane = (res == 0 ? J.bt_p : J.bt_q) + (size_t)b * (size_t)J.np * (size_t)J.kp;
-  uint32_t a_off[4], b_off[4];
+  uint32_t a_off[4], b_off[NB];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     a_off[i] = (uint32_t)(min(row0 + 16 * ((wave % 2) * 4 + i), J.mp - 16) / 16) * strip_bytes + (uint32_t)lane * 16u;
+  }
+#pragma unroll
+  for (int i = 0; i < NB; i++) {
     b_off[i] = (uint32_t)(min(col0 + 16 * i, J.np - 16) / 16) * strip_bytes + (uint32_t)lane * 16u;
   }
   uint32_t const lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void const *)big_lds;
@@ -500,22 +509,22 @@ __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMan
       plane_dma16(src, a_off[i], dst + (uint32_t)i * 1024u);
     }
   };
-  auto issue_b = [&](int s, v4i (&buf)[4]) {
+  auto issue_b = [&](int s, v4i (&buf)[NB]) {
     int8_t const *src = b_plane + (size_t)min(s, steps - 1) * 1024;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NB; i++) {
       plane_load16(buf[i], src, b_off[i]);
     }
   };
-  v4i acc[8][4];
+  v4i acc[8][NB];
 #pragma unroll
-  for (int e = 0; e < 32; e++) {
-    acc[e / 4][e % 4] = v4i{0, 0, 0, 0};
+  for (int e = 0; e < 8 * NB; e++) {
+    acc[e / NB][e % NB] = v4i{0, 0, 0, 0};
   }
   // A: three steps ahead through the four LDS stages.  B^T: one step ahead in registers; a
   // load and the wait for it stand in the same iteration, and only values that have landed
   // are carried round the loop (the compiler knows nothing of the loads' latency).
-  v4i cur[4], next[4], a[8], a_next[8];
+  v4i cur[NB], next[NB], a[8], a_next[8];
   issue_a(0);
   issue_a(1);
   issue_b(0, cur);
@@ -531,7 +540,7 @@ __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMan
   }
   // one step: multiplies (a_now, b_now) while the next step's operands arrive in (a_new, b_new);
   // the loop runs it twice with the register sets swapped, so nothing is copied
-  auto step = [&](int s, v4i (&a_now)[8], v4i (&b_now)[4], v4i (&a_new)[8], v4i (&b_new)[4]) {
+  auto step = [&](int s, v4i (&a_now)[8], v4i (&b_now)[NB], v4i (&a_new)[8], v4i (&b_new)[NB]) {
     if (s > 0) {
       __syncthreads();  // A(s + 1) is in LDS; everyone has the stage of step s - 1 in registers
     }
@@ -546,7 +555,7 @@ __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMan
 #pragma unroll
     for (int i = 0; i < 8; i++) {
 #pragma unroll
-      for (int jn = 0; jn < 4; jn++) {
+      for (int jn = 0; jn < NB; jn++) {
         acc[i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b_now[jn], a_now[i], acc[i][jn], 0, 0, 0);
       }
     }
@@ -569,13 +578,13 @@ __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMan
   // with constant register indices under a wave-uniform branch)
   if (res == 0) {
 #pragma unroll
-    for (int e = 0; e < 16; e++) {
-      mine[e * 64 + lane] = acc[4 + e / 4][e % 4];
+    for (int e = 0; e < 4 * NB; e++) {
+      mine[e * 64 + lane] = acc[4 + e / NB][e % NB];
     }
   } else {
 #pragma unroll
-    for (int e = 0; e < 16; e++) {
-      mine[e * 64 + lane] = acc[e / 4][e % 4];
+    for (int e = 0; e < 4 * NB; e++) {
+      mine[e * 64 + lane] = acc[e / NB][e % NB];
     }
   }
   __syncthreads();
@@ -583,15 +592,15 @@ __global__ __launch_bounds__(kThreads, 2) void fp_mfma_matmul_big_kernel(GemmMan
   bool const whole4 = J.n % 4 == 0;
   if (res == 0) {
 #pragma unroll
-    for (int e = 0; e < 16; e++) {
-      store_outputs(out, J.m, J.n, whole4, row0 + (e / 4) * 16 + r, col0 + (e % 4) * 16 + 4 * g,
-                    acc[e / 4][e % 4], theirs[e * 64 + lane]);
+    for (int e = 0; e < 4 * NB; e++) {
+      store_outputs(out, J.m, J.n, whole4, row0 + (e / NB) * 16 + r, col0 + (e % NB) * 16 + 4 * g,
+                    acc[e / NB][e % NB], theirs[e * 64 + lane]);
     }
   } else {
 #pragma unroll
-    for (int e = 0; e < 16; e++) {
-      store_outputs(out, J.m, J.n, whole4, row0 + (4 + e / 4) * 16 + r, col0 + (e % 4) * 16 + 4 * g,
-                    theirs[e * 64 + lane], acc[4 + e / 4][e % 4]);
+    for (int e = 0; e < 4 * NB; e++) {
+      store_outputs(out, J.m, J.n, whole4, row0 + (4 + e / NB) * 16 + r, col0 + (e % NB) * 16 + 4 * g,
+                    theirs[e * 64 + lane], acc[4 + e / NB][e % NB]);
     }
   }
 }
@@ -1008,10 +1017,10 @@ static bool mfma_matmul_fits(int batch, int m, int n, int k, size_t *plane_bytes
 static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B, uint16_t *const *C,
                              int const *batch, int const *m, int const *n, int const *k, int count) {
   std::vector<SplitJob> jobs((size_t)(2 * count));
-  GemmMany G{}, Big{};  // jobs of the 64 x 64 / 32 x 32 kernel, jobs of the 128 x 128 kernel
+  GemmMany G{}, Big{}, Narrow{};  // jobs of the 64 x 64 / 32 x 32 kernel, of the 128 x 128 and 128 x 64 kernels
   char *planes = state().planes();
   size_t used = 0;
-  unsigned gemm_blocks = 0, big_blocks = 0;
+  unsigned gemm_blocks = 0, big_blocks = 0, narrow_blocks = 0;
   for (int e = 0; e < count; e++) {
     int const kp = (int)round_up((size_t)k[e], 64);
     int const mp = (int)round_up((size_t)m[e], 16), np = (int)round_up((size_t)n[e], 16);
@@ -1062,22 +1071,33 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     g.np = np;
     long long const tiles64 = (long long)((m[e] + 63) / 64) * ((n[e] + 63) / 64) * batch[e];
     long long const tiles128 = (long long)((m[e] + 127) / 128) * ((n[e] + 127) / 128) * batch[e];
-    // 128 x 128 tiles once they fill the device (a tile's plane offsets are 32-bit there)
-    bool const large = tiles128 >= kBigMinTiles && state().fp_big_tiles && kp <= kBigMaxK &&
-                       (size_t)std::max(mp, np) * (size_t)kp < ((size_t)1 << 31);
+    long long const tiles128x64 = (long long)((m[e] + 127) / 128) * ((n[e] + 63) / 64) * batch[e];
+    // 128 x 128 tiles once there is one for every compute unit (a tile's plane offsets are
+    // 32-bit there); below that 128 x 64 tiles if there is one of those for every compute unit
+    // (1536^3: 26.7 us against 33.2 on 64 x 64 tiles; 1536 x 2048 x 1024: 23.2 against 25.7 on
+    // 128 x 128; from 256 wide tiles on the narrow ones are no faster or slower)
+    bool const fits_big = state().fp_big_tiles && kp <= kBigMaxK &&
+                          (size_t)std::max(mp, np) * (size_t)kp < ((size_t)1 << 31);
+    bool const narrow = fits_big && tiles128 < kBigMinTiles && tiles128x64 >= kBigMinTiles;
+    bool const large = fits_big && (tiles128 >= kBigMinTiles || narrow);
     g.shared_k = !large && tiles64 < 64;
     int const edge = large ? 128 : (g.shared_k ? 32 : 64);
+    int const edge_n = narrow ? 64 : edge;
     g.tiles_m = (m[e] + edge - 1) / edge;
-    g.tiles_n = (n[e] + edge - 1) / edge;
+    g.tiles_n = (n[e] + edge_n - 1) / edge_n;
     unsigned const blocks = (unsigned)((long long)g.tiles_m * g.tiles_n * batch[e]);
     // Measured with the split launch in front, as it runs: the XCD-aware order pays once the
     // tiles no longer all run at once (8 x 1024^3: 40 against 49 us); for fewer it costs a
     // microsecond although it halves the bytes fetched (1024^3 on 64 x 64 tiles: 16.6 against
     // 15.1 us).  The magics are exact while dividend * divisor < 2^32 (dividends: below `blocks`).
-    g.xcd_order = large && blocks >= 512u && blocks < 65536u;
+    g.xcd_order = large && !narrow && blocks >= 512u && blocks < 65536u;
     g.magic_per_batch = fast_div_magic(g.tiles_m * g.tiles_n);
     g.magic_width = fast_div_magic(8 * g.tiles_n);
-    if (large) {
+    if (narrow) {
+      g.first_block = narrow_blocks;
+      narrow_blocks += blocks;
+      Narrow.job[Narrow.count++] = g;
+    } else if (large) {
       g.first_block = big_blocks;
       big_blocks += blocks;
       Big.job[Big.count++] = g;
@@ -1095,15 +1115,23 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     fp_mfma_matmul_kernel<<<gemm_blocks, kThreads, 0, st>>>(G);
     MI355_HIP(hipGetLastError());
   }
-  if (Big.count > 0) {
+  if (Big.count > 0 || Narrow.count > 0) {
     static std::atomic<int> granted{0};
     if (granted.load(std::memory_order_acquire) < kBigLdsBytes) {
-      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_mfma_matmul_big_kernel),
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_mfma_matmul_big_kernel<128>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
+      MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fp_mfma_matmul_big_kernel<64>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
       granted.store(kBigLdsBytes, std::memory_order_release);
     }
-    fp_mfma_matmul_big_kernel<<<big_blocks, kThreads, kBigLdsBytes, st>>>(Big);
-    MI355_HIP(hipGetLastError());
+    if (Big.count > 0) {
+      fp_mfma_matmul_big_kernel<128><<<big_blocks, kThreads, kBigLdsBytes, st>>>(Big);
+      MI355_HIP(hipGetLastError());
+    }
+    if (Narrow.count > 0) {
+      fp_mfma_matmul_big_kernel<64><<<narrow_blocks, kThreads, kBigLdsBytes, st>>>(Narrow);
+      MI355_HIP(hipGetLastError());
+    }
   }
   return MI355_OK;
 }

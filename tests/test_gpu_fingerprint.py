@@ -383,8 +383,9 @@ def test_many_matmuls_on_the_matrix_cores_match_oracle(rt, abi):
 
 
 def test_large_matmuls_on_128_tiles_match_oracle(rt, abi):
-    """Matmuls with 192 or more 128 x 128 output tiles take the kernel that stages operand strips
-    through LDS: ragged edges in rows, columns and k, a batch, one k step and an odd number of
+    """Matmuls with 256 or more output tiles of 128 x 128, or of 128 x 64 when there are fewer
+    of the wide ones, take the kernel that stages operand strips through LDS (shapes of both
+    kinds below): ragged edges in rows, columns and k, a batch, one k step and an odd number of
     them, both tile orders, together with small matmuls in the same call; with the option that
     keeps 64 x 64 tiles the same calls give the same bits."""
     shapes = [(1, 2008, 1544, 200), (3, 1024, 1024, 72), (1, 48, 80, 64), (1, 2048, 2048, 64),
