@@ -208,8 +208,10 @@ int mi355_fp_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch
  * operator in the reference, matmul_kernel.cu:175-203): C[i] = A[i] . B[i] with extents
  * batch[i], m[i], n[i], k[i], bit-identical to mi355_fp_matmul of each.  Operands are split
  * once into signed-byte residue planes (mod 227 recentred, mod 113) in backend memory and
- * multiplied with int8 matrix instructions; up to MI355_MAX_MATMULS go out as two launches,
- * longer lists in groups.  Outputs must not alias inputs of the same call. */
+ * multiplied with int8 matrix instructions; up to MI355_MAX_MATMULS go out as two launches
+ * (one more per tile shape when the list holds matmuls large enough for the kernels that
+ * stage operands through LDS), longer lists in groups.  Outputs must not alias inputs of the
+ * same call. */
 #define MI355_MAX_MATMULS 32
 int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *const *B, uint16_t *const *C,
                          int const *batch, int const *m, int const *n, int const *k, int count);
