@@ -80,15 +80,16 @@ __global__ __launch_bounds__(kThreads) void fp_split_planes_kernel(SplitMany con
   if (!J.transpose) {
     // unit = 16 consecutive k of one plane row; the 16 rows of a block go to 16 neighbouring
     // threads, which write one contiguous 256-byte block
-    int const chunks = J.kp / 16;
-    size_t const units = (size_t)J.slabs * J.rp * chunks;
-    for (size_t u = (size_t)block * kThreads + tid; u < units; u += (size_t)J.blocks * kThreads) {
-      int const r = (int)(u % 16);
-      size_t const blk = u / 16;                 // (slab, strip, chunk)
-      int const c = (int)(blk % chunks);
-      size_t const strip = blk / chunks;         // over slabs * rp / 16
-      int const slab = (int)(strip / (J.rp / 16));
-      int const row = (int)(strip % (J.rp / 16)) * 16 + r;
+    // (32-bit index arithmetic: a plane has fewer than 2^31 bytes, so fewer than 2^27 units)
+    unsigned const chunks = (unsigned)J.kp / 16u, strips = (unsigned)J.rp / 16u;
+    unsigned const units = (unsigned)J.slabs * (unsigned)J.rp * chunks;
+    for (unsigned u = block * kThreads + tid; u < units; u += J.blocks * kThreads) {
+      int const r = (int)(u % 16u);
+      unsigned const blk = u / 16u;              // (slab, strip, chunk)
+      unsigned const strip = blk / chunks;       // over slabs * rp / 16
+      int const c = (int)(blk - strip * chunks);
+      int const slab = (int)(strip / strips);
+      int const row = (int)(strip - (unsigned)slab * strips) * 16 + r;
       int const k0 = c * 16;
       uint32_t v[16];
       if (row < J.rows) {
@@ -129,8 +130,8 @@ __global__ __launch_bounds__(kThreads) void fp_split_planes_kernel(SplitMany con
         q[w] = byte_q(v[4 * w]) | (byte_q(v[4 * w + 1]) << 8) | (byte_q(v[4 * w + 2]) << 16) |
                (byte_q(v[4 * w + 3]) << 24);
       }
-      *reinterpret_cast<uint4v *>(J.plane_p + u * 16) = p;  // u = ((strip * chunks + c) * 16 + r)
-      *reinterpret_cast<uint4v *>(J.plane_q + u * 16) = q;
+      *reinterpret_cast<uint4v *>(J.plane_p + (size_t)u * 16) = p;  // u = ((strip * chunks + c) * 16 + r)
+      *reinterpret_cast<uint4v *>(J.plane_q + (size_t)u * 16) = q;
     }
     return;
   }
