@@ -35,6 +35,10 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
 
 # source file -> kernels that must build without register spills (see build_backend)
 NO_SPILL_KERNELS = {"fp_mfma.hip": ["fp_mfma_matmul_big_kernel"]}
+# fewest wavefronts per SIMD those kernels are written for (two workgroups per compute unit):
+# fewer means the register allocation is no longer the one the hand-placed loads and waits
+# were checked against
+MIN_OCCUPANCY = {"fp_mfma_matmul_big_kernel": 2}
 
 
 def resource_usage(remarks):
@@ -55,7 +59,9 @@ def spilling(usage, kernel):
     hits = [u for n, u in usage.items() if kernel in n]
     if not hits:
         raise RuntimeError(f"no resource usage reported for {kernel}")
-    return [u for u in hits if u.get("ScratchSize [bytes/lane]") != "0" or u.get("VGPRs Spill") != "0"]
+    least = MIN_OCCUPANCY.get(kernel, 0)
+    return [u for u in hits if u.get("ScratchSize [bytes/lane]") != "0" or u.get("VGPRs Spill") != "0" or
+            int(u.get("Occupancy [waves/SIMD]", least)) < least]
 
 
 def _sources(sub, exts):
@@ -92,7 +98,7 @@ def build_backend():
         for kernel in must_not_spill:
             bad = spilling(usage, kernel)
             if bad:
-                raise RuntimeError(f"{s}: {kernel} spills registers: {bad}")
+                raise RuntimeError(f"{s}: {kernel} spills registers or lost occupancy: {bad}")
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         list(pool.map(compile_one, zip(srcs, objs)))
@@ -114,10 +120,6 @@ def build_tools():
     _run(["g++", "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", INCLUDE, "-I", "/opt/rocm/include",
           "-o", os.path.join(HERE, "mirage_profile"), os.path.join(CSRC, "examples", "profile.cc"),
           "-L" + HERE, "-lmirage_runtime", "-lmi355_backend", "-Wl,-rpath,$ORIGIN"])
-    # mirage_gfx950_rates: the MFMA / vector co-issue and LDS read-rate measurements the design
-    # notes of the fused attention kernels cite (stand-alone, links nothing of this package)
-    _run([HIPCC, "--offload-arch=gfx950", "-O3", "-w", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-          "-o", os.path.join(HERE, "mirage_gfx950_rates"), os.path.join(CSRC, "examples", "gfx950_rates.hip")])
 
 
 def build_generated():

@@ -26,6 +26,13 @@
 #include "common.h"
 #include "tb_program.h"
 
+// fp_mfma_matmul_big_kernel loads registers by inline assembly and waits for them later: code
+// compiled without optimisation stores every such register to scratch memory right after the
+// load is issued, before its data is there.  Refuse to build that.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__OPTIMIZE__)
+#error "fp_mfma.hip must be compiled with optimisation (-O1 or higher): its asynchronous register loads do not survive -O0"
+#endif
+
 #include <algorithm>
 #include <atomic>
 #include <vector>

@@ -37,11 +37,17 @@ int main(int argc, char **argv) {
   std::vector<float> times;
   for (size_t i = first; i < cp.generated_graphs.size() && i < first + count; i++) {
     kernel::Graph g;
-    from_json(cp.generated_graphs[i], g);
-    if (single) {
-      std::cout << json(g) << std::endl;
+    GraphProfile p;
+    try {
+      from_json(cp.generated_graphs[i], g);
+      if (single) {
+        std::cout << json(g) << std::endl;
+      }
+      p = profile_graph(g);
+    } catch (std::exception const &e) {
+      std::cerr << "graph " << i << ": " << e.what() << std::endl;
+      return 1;
     }
-    GraphProfile const p = profile_graph(g);
     times.push_back(p.run_time);
     if (single) {
       std::cout << "Profiled running time: " << p.run_time << std::endl;

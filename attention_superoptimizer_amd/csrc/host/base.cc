@@ -11,9 +11,11 @@
 
 namespace mirage {
 
+// reference src/profile_result.cc:7-9: "infinity" is a finite sentinel (1000 ms), so a
+// checkpoint whose best profile was never set still serialises as a number
 ProfileResult ProfileResult::infinity() {
   ProfileResult r;
-  r.run_time = std::numeric_limits<float>::infinity();
+  r.run_time = 1000.0f;
   return r;
 }
 

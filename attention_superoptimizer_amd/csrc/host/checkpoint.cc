@@ -20,7 +20,10 @@ void from_json(json const &j, Checkpoint &c) {
   c.computation_graph = j.at("computation_graph");
   c.best_graph = j.contains("best_graph") ? j.at("best_graph") : json();
   c.best_profile_result = ProfileResult::infinity();
-  if (j.contains("best_profile_result") && j.at("best_profile_result").contains("run_time")) {
+  // (a null run_time is how a writer spells a non-finite float: it stays "infinity")
+  if (j.contains("best_profile_result") && j.at("best_profile_result").is_object() &&
+      j.at("best_profile_result").contains("run_time") &&
+      !j.at("best_profile_result").at("run_time").is_null()) {
     c.best_profile_result.run_time = (float)j.at("best_profile_result").at("run_time").as_double();
   }
   c.config = j.contains("config") ? j.at("config") : json::object();
@@ -110,13 +113,20 @@ void *mirage_checkpoint_load(char const *path) {
 
 void mirage_checkpoint_destroy(void *c) { delete static_cast<mirage::search::Checkpoint *>(c); }
 
+// (every accessor below returns an error value for a null handle)
 int mirage_checkpoint_num_graphs(void *c) {
+  if (c == nullptr) {
+    return -1;
+  }
   return (int)static_cast<mirage::search::Checkpoint *>(c)->generated_graphs.size();
 }
 
 // counters[0..2] = num_total_kernel_graphs, num_total_random_tests, num_valid_kernel_graphs;
 // returns best_profile_result.run_time
 float mirage_checkpoint_summary(void *c, long long *counters) {
+  if (c == nullptr) {
+    return -1.0f;
+  }
   auto *cp = static_cast<mirage::search::Checkpoint *>(c);
   if (counters != nullptr) {
     counters[0] = cp->num_total_kernel_graphs;
@@ -129,6 +139,9 @@ float mirage_checkpoint_summary(void *c, long long *counters) {
 // The whole checkpoint (index -2), its computation graph (index -1) or generated graph
 // `index` as JSON text; returns the length, copies at most capacity - 1 bytes.
 long long mirage_checkpoint_json(void *c, int index, char *buf, long long capacity) {
+  if (c == nullptr) {
+    return -1;
+  }
   auto *cp = static_cast<mirage::search::Checkpoint *>(c);
   std::string text;
   if (index == -2) {
@@ -153,6 +166,9 @@ long long mirage_checkpoint_json(void *c, int index, char *buf, long long capaci
 // profile.cc's measurement on an open graph: per-operator mean milliseconds into op_ms (up to
 // capacity entries); returns the sum.
 float mirage_graph_profile(void *graph, float *op_ms, int capacity) {
+  if (graph == nullptr) {
+    return -1.0f;
+  }
   mirage::search::GraphProfile p =
       mirage::search::profile_graph(*static_cast<mirage::kernel::Graph *>(graph));
   for (int i = 0; op_ms != nullptr && i < capacity && i < (int)p.op_ms.size(); i++) {

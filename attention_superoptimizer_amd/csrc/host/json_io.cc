@@ -139,6 +139,11 @@ static void dump_value(Json const &j, int indent, int level, std::string &out) {
     case Json::Bool: out += j.as_bool() ? "true" : "false"; break;
     case Json::Int: out += std::to_string(j.as_int()); break;
     case Json::Float: {
+      // JSON has no spelling for infinities and NaNs: null, as nlohmann-json writes them
+      if (!std::isfinite(j.as_double())) {
+        out += "null";
+        break;
+      }
       char buf[40];
       std::snprintf(buf, sizeof(buf), "%.17g", j.as_double());
       out += buf;

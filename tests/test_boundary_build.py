@@ -107,9 +107,45 @@ def test_checkpoint_object_loads_and_passes_through():
                 g.close()
     finally:
         cp.close()
-    # a single-graph file (what cpp_examples/profile.cc takes) loads as a one-graph checkpoint
     with pytest.raises(ValueError):
         G.Checkpoint.load(os.path.join(GOLDEN, "no_such_file.json"))
+
+
+def test_single_graph_file_round_trips_as_a_checkpoint(tmp_path):
+    """A single-graph file (what cpp_examples/profile.cc takes) loads as a one-graph checkpoint
+    whose best profile was never set; what it writes is valid JSON with a finite run time (the
+    reference's "infinity" is 1000 ms, src/profile_result.cc:7-9) and loads again.  A run time
+    spelled null (how a writer spells a non-finite float) reads back as that same sentinel."""
+    from attention_superoptimizer_amd import graph as G
+    want = json.load(open(os.path.join(GOLDEN, "gqa_spec_decode_checkpoint_excerpt.json")))
+    G.set_smem_budget(1 << 20)
+    single = tmp_path / "single.json"
+    single.write_text(json.dumps(want["generated_graphs"][0]))
+    cp = G.Checkpoint.load(str(single))
+    try:
+        assert cp.num_graphs == 1 and cp.best_run_time == 1000.0
+        text = cp.to_json()
+        back = json.loads(text)  # Python's parser rejects inf / nan spelled any way but null
+        assert back["best_profile_result"]["run_time"] == 1000.0
+        assert back["generated_graphs"] == [want["generated_graphs"][0]]
+    finally:
+        cp.close()
+    again = tmp_path / "again.json"
+    again.write_text(text)
+    cp2 = G.Checkpoint.load(str(again))
+    try:
+        assert cp2.num_graphs == 1 and cp2.best_run_time == 1000.0
+    finally:
+        cp2.close()
+    back["best_profile_result"]["run_time"] = None
+    nulled = tmp_path / "nulled.json"
+    nulled.write_text(json.dumps(back))
+    cp3 = G.Checkpoint.load(str(nulled))
+    try:
+        assert cp3.best_run_time == 1000.0
+        assert json.loads(cp3.to_json())["best_profile_result"]["run_time"] == 1000.0
+    finally:
+        cp3.close()
 
 
 def test_build_refuses_register_spills_in_kernels_with_asynchronous_register_loads():
