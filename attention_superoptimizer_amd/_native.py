@@ -117,6 +117,8 @@ ABI = {
     "mi355_f16_fill_iota": (_ci, [_vp, _sz, _ci]),
     "mi355_f16_fill_normal": (_ci, [_vp, _sz, ctypes.c_float, _u64]),
     "mi355_f16_matmul": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci]),
+    "mi355_f16_matmul_layout": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci]),
+    "mi355_f16_transpose": (_ci, [_vp, _vp, _ci, _ci, _ci]),
     "mi355_f16_unary": (_ci, [_ci, _vp, _vp, _sz]),
     "mi355_f16_binary": (_ci, [_ci, _vp, _pi, _vp, _pi, _vp, _pi, _ci]),
     "mi355_f16_reduce": (_ci, [_vp, _vp, _sz, _ci, _ci, _ci]),

@@ -212,9 +212,29 @@ __device__ __forceinline__ void decode_block(AttnParams const &P, int &bx, int &
   bz = coord[2];
 }
 
+// Column-major K and V (template parameter CM of the kernels below): the K tile lies in memory and in LDS as K^T [NK keys][D], the V
+// tile as V^T [DV][NK keys]: the reduction index of both matrix products is contiguous, and every
+// operand is ONE plain 16-byte LDS read.  Key block j of S^T takes the keys
+// 32 (j / 2) + 8 (c / 4) + 4 (j % 2) + c % 4 for c = 0 .. 15 (any 16 keys may form a block), so
+// that the eight values of P a lane holds after blocks 2jj and 2jj + 1 are the eight CONSECUTIVE
+// keys 32jj + 8g .. + 7: the keys its V^T operand read delivers.  16-byte chunks are swizzled so
+// that the sixteen rows one read phase touches fall on sixteen different bank groups: chunk q of
+// row r sits at position q ^ cm_key<row bytes>(r).
+//   rows of 256 bytes (one row = all 64 banks): K^T rows with D = 128 read at the sixteen keys
+//     above, key(r) = (r & 3) | ((r >> 3) & 3) << 2 (= c); V^T rows with NK = 128 read at sixteen
+//     consecutive rows, key(r) = r & 15 (also for longer rows);
+//   rows of 128 bytes (two rows per bank line, the row's parity picks the half): the key
+//     permutes the eight chunks of the half: K^T with D = 64, key(r) = ((r >> 1) & 1) |
+//     ((r >> 3) & 3) << 1 (= c >> 1); V^T with NK = 64, key(r) = (r >> 1) & 7.
+template <int RowHalfs, bool IsK>
+__device__ __forceinline__ constexpr int cm_swizzle_key(int r) {
+  return IsK ? (RowHalfs == 128 ? ((r & 3) | (((r >> 3) & 3) << 2)) : (((r >> 1) & 1) | (((r >> 3) & 3) << 1)))
+             : (RowHalfs >= 128 ? (r & 15) : ((r >> 1) & 7));
+}
+
 // RG row groups of 16 query rows, IP wavefronts per row group working on IP
 // consecutive for-loop iterations.
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP, bool CM = false>
 __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
@@ -288,7 +308,18 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
           TileAddr const &ta = is_k ? P.k : P.v;
           _Float16 const *src =
               static_cast<_Float16 const *>(ta.ptr) + tile_offset(ta, bx, by, bz, it0 + s0 + u);
-          pt[i] = load_patch(src, ta.d_cols, is_k ? NK / 8 : DV / 8, is_k ? r : r - KP);
+          if (CM) {
+            // column-major tiles need no transpose: item r is four consecutive 16-byte chunks
+            // of K^T [NK][D] or V^T [DV][NK] (chunks per row are multiples of 4)
+            int const cpr = is_k ? D / 8 : NK / 8, q = 4 * (is_k ? r : r - KP);
+            _Float16 const *p4 = src + (long long)(q / cpr) * ta.d_cols + 8 * (q % cpr);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              pt[i].x[e] = *reinterpret_cast<uint4v const *>(p4 + 8 * e);
+            }
+          } else {
+            pt[i] = load_patch(src, ta.d_cols, is_k ? NK / 8 : DV / 8, is_k ? r : r - KP);
+          }
         }
       }
       // phase 2: transpose in registers, write K^T [NK][D] and V^T [DV][NK]
@@ -299,7 +330,16 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
         if (u < SG && s0 + u < n_st) {
           bool const is_k = r < KP;
           _Float16 *kt = reinterpret_cast<_Float16 *>(lds + (s0 + u) * P.lds_stage_bytes);
-          if (is_k) {
+          if (CM) {
+            int const cpr = is_k ? D / 8 : NK / 8, q = 4 * (is_k ? r : r - KP);
+            int const row = q / cpr, pos = q % cpr;
+            int const key = is_k ? cm_swizzle_key<D, true>(row) : cm_swizzle_key<NK, false>(row);
+            _Float16 *dst = (is_k ? kt : kt + NK * D) + row * (is_k ? D : NK);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              *reinterpret_cast<uint4v *>(dst + (((pos + e) ^ key) << 3)) = pt[i].x[e];
+            }
+          } else if (is_k) {
             store_patch_transposed(pt[i], kt, D, NK / 8, r);
           } else {
             store_patch_transposed<true>(pt[i], kt + NK * D, NK, DV / 8, r - KP);
@@ -331,7 +371,15 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
           float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
           for (int kk = 0; kk < DK; kk++) {
-            half8 a = *reinterpret_cast<half8 const *>(kt + swz_chunk(16 * j + c, 4 * kk + g, D));
+            half8 a;
+            if (CM) {
+              // permuted key order inside a pair of blocks, see cm_swizzle_key
+              int const row = 32 * (j >> 1) + 4 * (j & 1) + 8 * (c >> 2) + (c & 3);
+              a = *reinterpret_cast<half8 const *>(
+                  kt + row * D + (((4 * kk + g) ^ cm_swizzle_key<D, true>(8 * (c >> 2) + (c & 3))) << 3));
+            } else {
+              a = *reinterpret_cast<half8 const *>(kt + swz_chunk(16 * j + c, 4 * kk + g, D));
+            }
             acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kk], acc, 0, 0, 0);
           }
 #pragma unroll
@@ -369,7 +417,13 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
 #pragma unroll
           for (int jj = 0; jj < KB / 2; jj++) {
             // paired key groups (see store_patch_transposed): one 16-byte read per operand
-            half8 b = *reinterpret_cast<half8 const *>(vt + swz_chunk(vrow, 4 * jj + g, NK));
+            half8 b;
+            if (CM) {
+              // V^T[16t + c][keys 32jj + 8g + 0..7]
+              b = *reinterpret_cast<half8 const *>(vt + vrow * NK + (((4 * jj + g) ^ cm_swizzle_key<NK, false>(c)) << 3));
+            } else {
+              b = *reinterpret_cast<half8 const *>(vt + swz_chunk(vrow, 4 * jj + g, NK));
+            }
             uint4v const a = {pk[jj][0], pk[jj][1], pk[jj][2], pk[jj][3]};
             o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, o, 0, 0, 0);
           }
@@ -485,7 +539,7 @@ __device__ __forceinline__ constexpr int stream_swizzle_key(int r) {
   return RowHalfs == 128 ? (r & 7) : (IsK ? (((r >> 1) & 1) | (((r >> 3) & 1) << 1)) : ((r >> 1) & 3));
 }
 
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW>
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW, bool CM = false>
 __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams const P) {
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
@@ -513,6 +567,10 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   int const v_lane = (4 * g + a4) * DV + ((b4 >> 1) << 3) + (b4 & 1) * 4;
   int const sw_k = stream_swizzle_key<NK, true>(8 * g + a4) << 4;
   int const sw_v = stream_swizzle_key<DV, false>(4 * g + a4) << 4;
+  // column-major tiles: this lane's K^T row inside a pair of key blocks (block parity adds 4)
+  // and its V^T row inside a block of 16 value columns, with the rows' swizzle keys
+  int const kc_row = 8 * a4 + b4, kc_key = cm_swizzle_key<D, true>(8 * a4 + b4);
+  int const vc_key = cm_swizzle_key<NK, false>(c);
   int const row_base = (slice * RG + wave) * RPW * 16;
   int const F = P.forloop_range;
 
@@ -553,14 +611,24 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
 #pragma unroll
   for (int i = 0; i < KI; i++) {
     int const q = (wave * KI + i) * 64 + lane;
-    int const r = q / (NK / 8), pos = q % (NK / 8);
-    k_goff[i] = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(r))));
+    if (CM) {  // K^T: NK rows of D halfs
+      int const r = q / (D / 8), pos = q % (D / 8);
+      k_goff[i] = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ cm_swizzle_key<D, true>(r)));
+    } else {
+      int const r = q / (NK / 8), pos = q % (NK / 8);
+      k_goff[i] = 2u * (uint32_t)(r * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(r))));
+    }
   }
 #pragma unroll
   for (int i = 0; i < VI; i++) {
     int const q = (wave * VI + i) * 64 + lane;
-    int const r = q / (DV / 8), pos = q % (DV / 8);
-    v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(r))));
+    if (CM) {  // V^T: DV rows of NK halfs
+      int const r = q / (NK / 8), pos = q % (NK / 8);
+      v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ cm_swizzle_key<NK, false>(r)));
+    } else {
+      int const r = q / (DV / 8), pos = q % (DV / 8);
+      v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(r))));
+    }
   }
   auto fetch_k = [&](int it, int b) {
     _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
@@ -590,10 +658,16 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   auto s_fetch = [&](_Float16 const *kt, int j, half8 (&a)[DK]) {
 #pragma unroll
     for (int kk = 0; kk < DK; kk++) {
-      // K[32kk + 8g + 0..7][16j + c]
-      _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw_k ^ (j << 4));
-      half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
-      a[kk] = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      if (CM) {
+        // K^T[key 32 (j / 2) + 8 (c / 4) + 4 (j % 2) + c % 4][32kk + 8g + 0..7]
+        a[kk] = *reinterpret_cast<half8 const *>(kt + (32 * (j >> 1) + 4 * (j & 1) + kc_row) * D +
+                                                 (((4 * kk + g) ^ kc_key) << 3));
+      } else {
+        // K[32kk + 8g + 0..7][16j + c]
+        _Float16 const *ka = kt + k_lane + 32 * kk * NK + (sw_k ^ (j << 4));
+        half4 const a_lo = lds_read_tr16(ka), a_hi = lds_read_tr16(ka + 4 * NK);
+        a[kk] = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
     }
   };
   auto s_mfma = [&](half8 const (&a)[DK], float4v (&acc)[RPW]) {
@@ -667,10 +741,15 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   auto pv_fetch = [&](_Float16 const *vt, int t, half8 (&b)[KB / 2]) {
 #pragma unroll
     for (int jj = 0; jj < KB / 2; jj++) {
-      // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
-      _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
-      half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
-      b[jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      if (CM) {
+        // V^T[16t + c][keys 32jj + 8g + 0..7]: the keys P holds (see the key order of S^T)
+        b[jj] = *reinterpret_cast<half8 const *>(vt + (16 * t + c) * NK + (((4 * jj + g) ^ vc_key) << 3));
+      } else {
+        // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
+        _Float16 const *vb = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
+        half4 const b_lo = lds_read_tr16(vb), b_hi = lds_read_tr16(vb + 16 * DV);
+        b[jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
     }
   };
   auto pv_mfma = [&](half8 const (&b)[KB / 2], uint32_t const (&pk)[RPW][KB / 2][4], float4v (&o)[RPW]) {
@@ -860,14 +939,19 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
 // ---------------------------------------------------------------------------------------
 namespace {
 
+// (a column-major tensor -- DevOp::sub == 1 on its loader -- holds element (r, c) at
+// c * d_rows + r: a step along the rows is one element, a step along the columns d_rows, and
+// `d_cols` of the result is that leading dimension)
 TileAddr tile_addr(DevOp const &op, void const *ptr) {
   TileAddr t;
   t.ptr = ptr;
+  bool const cm = op.kind == DOP_LOAD && op.sub == 1;
+  long long const rstep = cm ? 1 : op.d_cols, cstep = cm ? op.d_rows : 1;
   for (int i = 0; i < 3; i++) {
-    t.lin[i] = op.g_bs[i] + (long long)op.row_bs[i] * op.d_cols + op.col_bs[i];
+    t.lin[i] = op.g_bs[i] + op.row_bs[i] * rstep + op.col_bs[i] * cstep;
   }
-  t.lin[3] = op.g_fs + (long long)op.row_fs * op.d_cols + op.col_fs;
-  t.d_cols = op.d_cols;
+  t.lin[3] = op.g_fs + op.row_fs * rstep + op.col_fs * cstep;
+  t.d_cols = cm ? op.d_rows : op.d_cols;
   return t;
 }
 
@@ -876,6 +960,11 @@ struct Match {
   int out_o, out_r;   // output op indices (out_r < 0 in form A)
   bool has_div;
   int m, D, NK, DV;
+  // K and V are both DmemColumnMajor (the layout every attention plan of the reference declares,
+  // e.g. cpp_examples/group_query_attn_inc_decode.cc:41-44): K [D][keys] is then stored key by key
+  // with the head dim contiguous, V [keys][DV] column by column with the keys contiguous, so both
+  // tiles arrive with the MFMA's reduction index contiguous and no read transposes anything
+  bool kv_colmajor;
 };
 
 // `pieces`: the value tile may be narrower than 16 bytes (checked by merge_column_pieces)
@@ -960,6 +1049,11 @@ bool match(DevProgram const &P, Match &M, bool pieces = false) {
   if (lq.row_fs != 0 || lq.col_fs != 0 || lq.g_fs != 0) {
     return false;
   }
+  // Q row-major; K and V in one storage order (a mixed pair takes the interpreter)
+  if (lq.sub == 1 || P.ops[M.k].sub != P.ops[M.v].sub) {
+    return false;
+  }
+  M.kv_colmajor = P.ops[M.k].sub == 1;
   if (!lq.galign || !P.ops[M.k].galign ||
       (!pieces && (!P.ops[M.v].galign || !P.ops[M.out_o].galign))) {
     return false;
@@ -1014,6 +1108,15 @@ bool merge_column_pieces(DevProgram const &P, Match &M, DevProgram &Q, int &copi
     // 16-byte reachability of the widened tiles
     for (int o : {M.v, M.out_o}) {
       DevOp &d = Q.ops[o];
+      if (d.kind == DOP_LOAD && d.sub == 1) {
+        // column-major V: a wider tile is more columns, i.e. more rows of V^T, each as
+        // reachable with 16-byte accesses as before
+        if (!d.galign) {
+          return false;
+        }
+        Q.t[d.dst].cols = 64;
+        continue;
+      }
       bool al = d.d_cols % 8 == 0 && d.col_fs % 8 == 0 && d.g_fs % 8 == 0;
       for (int e = 0; e < 3; e++) {
         al = al && d.col_bs[e] % 8 == 0 && d.g_bs[e] % 8 == 0;
@@ -1073,9 +1176,15 @@ __device__ __forceinline__ void wait_vm() {
 //     side by side in memory -- the host checks the loader strides): one load of 64 keys, then
 //     every 32- or 16-key slice gets its own exp / row sum / [division] / P.V and its own
 //     rounded result.  Slices of 16 keys take the 16 x 16 x 16 matrix instruction.
+// Column-major K and V (CM): the tiles are K^T [64 keys][64] and V^T [64][64 keys], swizzled and
+// read as in attn_stream_kernel (one plain 16-byte LDS read per operand, keys of a pair of S^T
+// blocks permuted so that P's eight values per lane are consecutive keys).  Slices of 16 keys
+// (IPS == 4) need every block to be 16 consecutive keys: they keep the plain key order and fetch
+// their V^T operand as two 8-byte reads.
 template <int D, int NK, int DV, bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, int SPI, int IPS,
-          bool TRACE>
+          bool TRACE, bool CM>
 __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P) {
+  constexpr bool PERM = CM && IPS != 4;  // permuted key order inside pairs of S^T blocks
   static_assert(D == 64 && NK == 64 && DV == 64, "the chunk swizzles assume rows of 128 bytes");
   static_assert((SPI == 1 || IPS == 1) && (SPI == 1 || SPI == 2 || SPI == 4) &&
                     (IPS == 1 || IPS == 2 || IPS == 4) && !(HAS_DIV && SPI > 1),
@@ -1120,24 +1229,35 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   static_assert(stream_swizzle_key<NK, true>(8 + 5) == (stream_swizzle_key<NK, true>(5) | 2) &&
                     stream_swizzle_key<DV, false>(8 + 5) == stream_swizzle_key<DV, false>(5),
                 "row advance by 8 flips bit 1 of the K key and leaves the V key unchanged");
-  uint32_t const k_off_even = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(l3))));
-  uint32_t const k_off_odd = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<NK, true>(8 + l3))));
-  uint32_t const v_off = 2u * (uint32_t)(l3 * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(l3))));
-  // strip `strip` (64 keys) of unit `unit`: the unit's first iteration names the tile origin
+  // (column-major tiles: the K^T key of row 8 i + l3 depends on i % 4, the V^T key on i % 2)
+  uint32_t k_off[CM ? 4 : 2], v_offs[CM ? 2 : 1];
+#pragma unroll
+  for (int i = 0; i < (CM ? 4 : 2); i++) {
+    int const key = CM ? cm_swizzle_key<D, true>(8 * i + l3) : 2 * stream_swizzle_key<NK, true>(8 * i + l3);
+    k_off[i] = 2u * (uint32_t)(l3 * P.k.d_cols + 8 * (pos ^ key));
+  }
+#pragma unroll
+  for (int i = 0; i < (CM ? 2 : 1); i++) {
+    int const key = CM ? cm_swizzle_key<NK, false>(8 * i + l3) : 2 * stream_swizzle_key<DV, false>(l3);
+    v_offs[i] = 2u * (uint32_t)(l3 * P.v.d_cols + 8 * (pos ^ key));
+  }
+  // strip `strip` (64 keys) of unit `unit`: the unit's first iteration names the tile origin;
+  // 64 keys further is 64 columns of K and 64 rows of V (column-major: 64 rows of K^T, 64
+  // columns of V^T)
   auto fetch = [&](int unit, int strip, int b) {
-    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) +
-                         tile_offset(P.k, bx, by, bz, unit * IPS) + 64 * strip;
-    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) +
-                         tile_offset(P.v, bx, by, bz, unit * IPS) + (long long)(64 * strip) * P.v.d_cols;
+    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, unit * IPS) +
+                         (CM ? (long long)(64 * strip) * P.k.d_cols : (long long)(64 * strip));
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, unit * IPS) +
+                         (CM ? (long long)(64 * strip) : (long long)(64 * strip) * P.v.d_cols);
     uint32_t const base = lds_w + 2u * (uint32_t)(b * PAIR_HALFS);
 #pragma unroll
     for (int i = 0; i < KI; i++) {
-      lds_dma16(kg + (long long)(8 * i) * P.k.d_cols, (i & 1) ? k_off_odd : k_off_even,
+      lds_dma16(kg + (long long)(8 * i) * P.k.d_cols, k_off[CM ? (i & 3) : (i & 1)],
                 base + 1024u * (uint32_t)i);
     }
 #pragma unroll
     for (int i = 0; i < VI; i++) {
-      lds_dma16(vg + (long long)(8 * i) * P.v.d_cols, v_off,
+      lds_dma16(vg + (long long)(8 * i) * P.v.d_cols, v_offs[CM ? (i & 1) : 0],
                 base + 2u * (uint32_t)(D * NK) + 1024u * (uint32_t)i);
     }
   };
@@ -1169,6 +1289,8 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   int const v_lane = (4 * g + a4) * DV + ((b4 >> 1) << 3) + (b4 & 1) * 4;
   int const sw_k = stream_swizzle_key<NK, true>(8 * g + a4) << 4;
   int const sw_v = stream_swizzle_key<DV, false>(4 * g + a4) << 4;
+  int const kc_row = 8 * a4 + b4, kc_key = cm_swizzle_key<D, true>(8 * a4 + b4);
+  int const vc_key = cm_swizzle_key<NK, false>(c);
   // where this thread's share of the result goes (address arithmetic done while loads fly)
   constexpr int EPT = ROWS * DV / (64 * IP);  // elements per thread (16 rows: 8 / 4 / 2 for IP = 2 / 4 / 8)
   static_assert(EPT == 2 || EPT == 4 || EPT == 8, "2, 4 or 8 wavefronts");
@@ -1225,10 +1347,20 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       for (int jb = 0; jb < KB; jb++) {
 #pragma unroll
         for (int kk = 0; kk < DK; kk++) {
-          // K[32kk + 8g + 0..7][16jb + c]
-          _Float16 const *kp = kt + k_lane + 32 * kk * NK + (sw_k ^ (jb << 4));
-          half4 const a_lo = lds_read_tr16(kp), a_hi = lds_read_tr16(kp + 4 * NK);
-          ka[jb][kk] = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          if (PERM) {
+            // K^T[key 32 (jb / 2) + 8 (c / 4) + 4 (jb % 2) + c % 4][32kk + 8g + 0..7]
+            ka[jb][kk] = *reinterpret_cast<half8 const *>(kt + (32 * (jb >> 1) + 4 * (jb & 1) + kc_row) * D +
+                                                          (((4 * kk + g) ^ kc_key) << 3));
+          } else if (CM) {
+            // K^T[key 16jb + c][32kk + 8g + 0..7]
+            ka[jb][kk] = *reinterpret_cast<half8 const *>(
+                kt + (16 * jb + c) * D + (((4 * kk + g) ^ cm_swizzle_key<D, true>(16 * jb + c)) << 3));
+          } else {
+            // K[32kk + 8g + 0..7][16jb + c]
+            _Float16 const *kp = kt + k_lane + 32 * kk * NK + (sw_k ^ (jb << 4));
+            half4 const a_lo = lds_read_tr16(kp), a_hi = lds_read_tr16(kp + 4 * NK);
+            ka[jb][kk] = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          }
         }
       }
       float4v acc[RPW][KB];
@@ -1254,10 +1386,21 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
       for (int t = 0; t < DB; t++) {
 #pragma unroll
         for (int jj = 0; jj < KB / 2; jj++) {
-          // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
-          _Float16 const *vp = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
-          half4 const b_lo = lds_read_tr16(vp), b_hi = lds_read_tr16(vp + 16 * DV);
-          vb[t][jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          if (PERM) {
+            // V^T[16t + c][keys 32jj + 8g + 0..7]: the keys P holds under the permuted order
+            vb[t][jj] = *reinterpret_cast<half8 const *>(vt + (16 * t + c) * NK + (((4 * jj + g) ^ vc_key) << 3));
+          } else if (CM) {
+            // V^T[16t + c][keys 32jj + 4g + 0..3] and [32jj + 16 + 4g + 0..3]: 8 bytes each
+            _Float16 const *vrow = vt + (16 * t + c) * NK + 4 * (g & 1);
+            half4 const b_lo = *reinterpret_cast<half4 const *>(vrow + (((4 * jj + (g >> 1)) ^ vc_key) << 3));
+            half4 const b_hi = *reinterpret_cast<half4 const *>(vrow + (((4 * jj + 2 + (g >> 1)) ^ vc_key) << 3));
+            vb[t][jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          } else {
+            // V[32jj + 4g + 0..3][16t + c] and V[32jj + 16 + 4g + 0..3][16t + c]: the keys P holds
+            _Float16 const *vp = vt + v_lane + 32 * jj * DV + (sw_v ^ (t << 4));
+            half4 const b_lo = lds_read_tr16(vp), b_hi = lds_read_tr16(vp + 16 * DV);
+            vb[t][jj] = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -1548,7 +1691,7 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P
   }
 }
 
-template <bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, int SPI, int IPS>
+template <bool HAS_DIV, bool CM, int IP, int RPW, int NBUF, int NIT, int SPI, int IPS>
 int launch_direct_one(AttnParams const &A, dim3 grid, int lds, bool dry) {
   if (dry) {
     return 1;  // the question was only whether this shape is built
@@ -1565,9 +1708,9 @@ int launch_direct_one(AttnParams const &A, dim3 grid, int lds, bool dry) {
     return 1;
   };
   if (SPI == 1 && IPS == 1 && A.trace != nullptr) {
-    return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, SPI, IPS, SPI == 1 && IPS == 1>);
+    return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, SPI, IPS, SPI == 1 && IPS == 1, CM>);
   }
-  return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, SPI, IPS, false>);
+  return go(attn_direct_kernel<64, 64, 64, HAS_DIV, IP, RPW, NBUF, NIT, SPI, IPS, false, CM>);
 }
 
 // The shape of a direct-staging launch: `ip` wavefronts of `rpw` row groups each, `nbuf` tile
@@ -1579,11 +1722,11 @@ struct DirectShape {
 };
 
 // 0: no instantiation for this shape
-template <bool HAS_DIV>
+template <bool HAS_DIV, bool CM>
 int launch_direct(AttnParams const &A, dim3 grid, DirectShape const &d, int lds, bool dry = false) {
 #define MI355_DIRECT(IPV, RPWV, NBUFV, NITV, SPIV, IPSV) \
   case ((((IPV * 10 + RPWV) * 10 + NBUFV) * 10 + NITV) * 10 + SPIV) * 10 + IPSV: \
-    return launch_direct_one<HAS_DIV, IPV, RPWV, NBUFV, NITV, SPIV, IPSV>(A, grid, lds, dry);
+    return launch_direct_one<HAS_DIV, CM, IPV, RPWV, NBUFV, NITV, SPIV, IPSV>(A, grid, lds, dry);
   switch (d.code()) {
     // one 64-key tile per iteration
     MI355_DIRECT(2, 1, 1, 1, 1, 1)
@@ -1626,9 +1769,9 @@ int launch_direct(AttnParams const &A, dim3 grid, DirectShape const &d, int lds,
   return 0;
 }
 
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP>
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP, bool CM>
 int launch_one(AttnParams const &A, dim3 grid, int lds) {
-  auto *fn = attn_fused_kernel<D, NK, DV, HAS_DIV, RG, IP>;
+  auto *fn = attn_fused_kernel<D, NK, DV, HAS_DIV, RG, IP, CM>;
   static std::atomic<int> granted{0};  // per instantiation
   if (lds > 65536 && lds > granted) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
@@ -1640,31 +1783,35 @@ int launch_one(AttnParams const &A, dim3 grid, int lds) {
   return 1;
 }
 
-template <int D, int NK, int DV, bool HAS_DIV>
+template <int D, int NK, int DV, bool HAS_DIV, bool CM>
 int launch_waves(AttnParams const &A, dim3 grid, int rg, int ip, int lds) {
   switch (rg * 16 + ip) {
-    case 1 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 1, 1>(A, grid, lds);
-    case 1 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 1, 2>(A, grid, lds);
-    case 1 * 16 + 4: return launch_one<D, NK, DV, HAS_DIV, 1, 4>(A, grid, lds);
-    case 1 * 16 + 8: return launch_one<D, NK, DV, HAS_DIV, 1, 8>(A, grid, lds);
-    case 2 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 2, 1>(A, grid, lds);
-    case 2 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 2, 2>(A, grid, lds);
-    case 2 * 16 + 4: return launch_one<D, NK, DV, HAS_DIV, 2, 4>(A, grid, lds);
-    case 4 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 4, 1>(A, grid, lds);
-    case 4 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 4, 2>(A, grid, lds);
+    case 1 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 1, 1, CM>(A, grid, lds);
+    case 1 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 1, 2, CM>(A, grid, lds);
+    case 1 * 16 + 4: return launch_one<D, NK, DV, HAS_DIV, 1, 4, CM>(A, grid, lds);
+    case 1 * 16 + 8: return launch_one<D, NK, DV, HAS_DIV, 1, 8, CM>(A, grid, lds);
+    case 2 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 2, 1, CM>(A, grid, lds);
+    case 2 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 2, 2, CM>(A, grid, lds);
+    case 2 * 16 + 4: return launch_one<D, NK, DV, HAS_DIV, 2, 4, CM>(A, grid, lds);
+    case 4 * 16 + 1: return launch_one<D, NK, DV, HAS_DIV, 4, 1, CM>(A, grid, lds);
+    case 4 * 16 + 2: return launch_one<D, NK, DV, HAS_DIV, 4, 2, CM>(A, grid, lds);
     default: return 0;
   }
 }
 
 template <int D, int NK, int DV>
-int launch_shape(AttnParams const &A, bool has_div, dim3 grid, int rg, int ip, int lds) {
-  return has_div ? launch_waves<D, NK, DV, true>(A, grid, rg, ip, lds)
-                 : launch_waves<D, NK, DV, false>(A, grid, rg, ip, lds);
+int launch_shape(AttnParams const &A, bool has_div, bool cm, dim3 grid, int rg, int ip, int lds) {
+  if (cm) {
+    return has_div ? launch_waves<D, NK, DV, true, true>(A, grid, rg, ip, lds)
+                   : launch_waves<D, NK, DV, false, true>(A, grid, rg, ip, lds);
+  }
+  return has_div ? launch_waves<D, NK, DV, true, false>(A, grid, rg, ip, lds)
+                 : launch_waves<D, NK, DV, false, false>(A, grid, rg, ip, lds);
 }
 
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW = 2>
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW, bool CM>
 int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
-  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, RPW>;
+  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, RPW, CM>;
   if (lds > 65536) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -1674,20 +1821,20 @@ int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
   return 1;
 }
 
-template <int D, int NK, int DV>
+template <int D, int NK, int DV, bool CM>
 int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds, bool wide = false) {
   if constexpr (D == 64) {
     if (wide) {  // four wavefronts of 64 rows
-      return has_div ? launch_stream_one<D, NK, DV, true, 4, 4>(A, grid, lds)
-                     : launch_stream_one<D, NK, DV, false, 4, 4>(A, grid, lds);
+      return has_div ? launch_stream_one<D, NK, DV, true, 4, 4, CM>(A, grid, lds)
+                     : launch_stream_one<D, NK, DV, false, 4, 4, CM>(A, grid, lds);
     }
   }
   if (has_div) {
-    return rg == 4 ? launch_stream_one<D, NK, DV, true, 4>(A, grid, lds)
-                   : launch_stream_one<D, NK, DV, true, 2>(A, grid, lds);
+    return rg == 4 ? launch_stream_one<D, NK, DV, true, 4, 2, CM>(A, grid, lds)
+                   : launch_stream_one<D, NK, DV, true, 2, 2, CM>(A, grid, lds);
   }
-  return rg == 4 ? launch_stream_one<D, NK, DV, false, 4>(A, grid, lds)
-                 : launch_stream_one<D, NK, DV, false, 2>(A, grid, lds);
+  return rg == 4 ? launch_stream_one<D, NK, DV, false, 4, 2, CM>(A, grid, lds)
+                 : launch_stream_one<D, NK, DV, false, 2, 2, CM>(A, grid, lds);
 }
 
 }  // namespace
@@ -1791,8 +1938,8 @@ static bool choose_direct(DevProgram const &P, Match const &M, DirectShape &d, i
     return false;
   }
   AttnParams none{};
-  return (M.has_div ? launch_direct<true>(none, dim3(1, 1, 1), d, lds, true)
-                    : launch_direct<false>(none, dim3(1, 1, 1), d, lds, true)) == 1;
+  return (M.has_div ? launch_direct<true, false>(none, dim3(1, 1, 1), d, lds, true)
+                    : launch_direct<false, false>(none, dim3(1, 1, 1), d, lds, true)) == 1;
 }
 
 bool attention_applicable(DevProgram const &P) {
@@ -1900,8 +2047,14 @@ int try_launch_attention(DevProgram const &P0) {
         if (!set_grid_magics(A, grid)) {
           return 0;
         }
-        int rc = M.D == 64 ? launch_stream<64, 64, 64>(A, M.has_div, grid, rgs, lds, wide)
-                           : launch_stream<128, 64, 128>(A, M.has_div, grid, rgs, lds);
+        int rc;
+        if (M.kv_colmajor) {
+          rc = M.D == 64 ? launch_stream<64, 64, 64, true>(A, M.has_div, grid, rgs, lds, wide)
+                         : launch_stream<128, 64, 128, true>(A, M.has_div, grid, rgs, lds);
+        } else {
+          rc = M.D == 64 ? launch_stream<64, 64, 64, false>(A, M.has_div, grid, rgs, lds, wide)
+                         : launch_stream<128, 64, 128, false>(A, M.has_div, grid, rgs, lds);
+        }
         if (rc == 1) {
           s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
           s.last().workgroups = grid.x * grid.y * grid.z;
@@ -1935,8 +2088,11 @@ int try_launch_attention(DevProgram const &P0) {
                                     s.phase_trace_bytes) {
         B.trace = nullptr;
       }
-      int const rc = M.has_div ? launch_direct<true>(B, direct_grid, dshape, direct_lds)
-                               : launch_direct<false>(B, direct_grid, dshape, direct_lds);
+      int const rc = M.kv_colmajor
+                         ? (M.has_div ? launch_direct<true, true>(B, direct_grid, dshape, direct_lds)
+                                      : launch_direct<false, true>(B, direct_grid, dshape, direct_lds))
+                         : (M.has_div ? launch_direct<true, false>(B, direct_grid, dshape, direct_lds)
+                                      : launch_direct<false, false>(B, direct_grid, dshape, direct_lds));
       if (rc != 0) {
         if (rc == 1) {
           s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
@@ -1996,13 +2152,13 @@ int try_launch_attention(DevProgram const &P0) {
     return 0;
   }
   if (M.D == 64 && M.NK == 64) {
-    rc = launch_shape<64, 64, 64>(A, M.has_div, grid, rg, ip, lds);
+    rc = launch_shape<64, 64, 64>(A, M.has_div, M.kv_colmajor, grid, rg, ip, lds);
   } else if (M.D == 64 && M.NK == 128) {
-    rc = launch_shape<64, 128, 64>(A, M.has_div, grid, rg, ip, lds);
+    rc = launch_shape<64, 128, 64>(A, M.has_div, M.kv_colmajor, grid, rg, ip, lds);
   } else if (M.D == 64 && M.NK == 256) {
-    rc = launch_shape<64, 256, 64>(A, M.has_div, grid, rg, ip, lds);
+    rc = launch_shape<64, 256, 64>(A, M.has_div, M.kv_colmajor, grid, rg, ip, lds);
   } else {
-    rc = launch_shape<128, 64, 128>(A, M.has_div, grid, rg, ip, lds);
+    rc = launch_shape<128, 64, 128>(A, M.has_div, M.kv_colmajor, grid, rg, ip, lds);
   }
   if (rc == 1) {
     s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;

@@ -126,6 +126,12 @@ bool aligned(CTile const &t, int vec) {
 }
 
 bool cmatch(DevProgram const &P, CMatch &M) {
+  // (both inputs are read as row-major matrices: a column-major one takes the interpreter)
+  for (int o = 0; o < P.num_ops && P.ops[o].kind == DOP_LOAD; o++) {
+    if (P.ops[o].sub == 1) {
+      return false;
+    }
+  }
   int const last = P.num_ops - 1, F = P.forloop_range;
   if (P.num_ops < 4 || P.num_ops > 6 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
       P.ops[last].kind != DOP_OUTPUT) {

@@ -1,7 +1,10 @@
 // Kernel-level fp16 operators (the un-fused ops a kernel graph runs outside its
-// customized ops).  All tensors are row-major; arithmetic is fp32 with one fp16
-// rounding per stored element, the rule the reference's generated programs
-// follow (src/kernel/triton_code_gen.cc:246-268).
+// customized ops).  Arithmetic is fp32 with one fp16 rounding per stored element, the rule
+// the reference's generated programs follow (src/kernel/triton_code_gen.cc:246-268).
+// Results are row-major; the matmul reads either storage order of its operands (as the
+// reference's GEMM call does, src/kernel/cuda/matmul_kernel.cu:61-76), the element-wise
+// operators and reductions index their inputs flat, so their callers hand them row-major
+// buffers (mi355_f16_transpose makes one from a column-major tensor).
 #include "common.h"
 
 namespace mi355 {
@@ -39,15 +42,16 @@ __global__ void f16_fill_normal_kernel(_Float16 *x, size_t n, float std, uint64_
   }
 }
 
-// Batched row-major GEMM on the matrix cores: 64x64 output tile per workgroup,
-// four wavefronts each owning a 32x32 quadrant, k advanced 32 at a time through
-// LDS.  A is staged k-contiguous per row, B is transposed while staging so both
-// operands are read as 16-byte k-runs; rows are padded by 8 halfs so the 16-byte
-// reads of 32 consecutive rows spread over the LDS banks.
+// Batched GEMM on the matrix cores, any shape and either storage order of the operands
+// (element (r, c) of A at r * a_rs + c * a_cs, likewise B): 64x64 output tile per workgroup,
+// four wavefronts each owning a 32x32 quadrant, k advanced 32 at a time through LDS, both
+// tiles staged k-contiguous with rows padded by 8 halfs.  The general-purpose kernel: ragged
+// extents, unaligned bases.
 __global__ __launch_bounds__(kThreads) void f16_matmul_kernel(_Float16 const *__restrict__ A,
                                                              _Float16 const *__restrict__ B,
                                                              _Float16 *__restrict__ C, int m,
-                                                             int n, int k) {
+                                                             int n, int k, int a_rs, int a_cs,
+                                                             int b_rs, int b_cs) {
   constexpr int T = 64, TK = 32, LD = TK + 8;
   __shared__ __attribute__((aligned(16))) _Float16 As[T][LD];
   __shared__ __attribute__((aligned(16))) _Float16 Bs[T][LD];
@@ -63,25 +67,27 @@ __global__ __launch_bounds__(kThreads) void f16_matmul_kernel(_Float16 const *__
   for (int i = 0; i < 16; i++) {
     acc[i] = 0.0f;
   }
+  // a thread stages 8 elements of each tile per step, walking the direction that is
+  // contiguous in memory: along k (8 consecutive k of one row) or along the rows / columns
+  // (one k of 8 consecutive rows / columns)
+  bool const a_along_k = a_cs == 1, b_along_k = b_rs == 1;
   for (int k0 = 0; k0 < k; k0 += TK) {
-    // A tile: 64 rows x 32 k, 8 halfs per thread
     {
-      int r = tid / 4, kk = (tid % 4) * 8;
-      int gr = row0 + r;
+      int const r = a_along_k ? tid / 4 : (tid % 8) * 8, kk = a_along_k ? (tid % 4) * 8 : tid / 8;
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        int gk = k0 + kk + j;
-        As[r][kk + j] = (gr < m && gk < k) ? A[(size_t)gr * k + gk] : (_Float16)0.0f;
+        int const rr = a_along_k ? r : r + j, kj = a_along_k ? kk + j : kk;
+        int const gr = row0 + rr, gk = k0 + kj;
+        As[rr][kj] = (gr < m && gk < k) ? A[(size_t)gr * a_rs + (size_t)gk * a_cs] : (_Float16)0.0f;
       }
     }
-    // B tile: 32 k x 64 n read along n, written transposed
     {
-      int kk = tid / 8, c = (tid % 8) * 8;
-      int gk = k0 + kk;
+      int const c = b_along_k ? tid / 4 : (tid % 8) * 8, kk = b_along_k ? (tid % 4) * 8 : tid / 8;
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        int gc = col0 + c + j;
-        Bs[c + j][kk] = (gk < k && gc < n) ? B[(size_t)gk * n + gc] : (_Float16)0.0f;
+        int const cc = b_along_k ? c : c + j, kj = b_along_k ? kk + j : kk;
+        int const gc = col0 + cc, gk = k0 + kj;
+        Bs[cc][kj] = (gk < k && gc < n) ? B[(size_t)gk * b_rs + (size_t)gc * b_cs] : (_Float16)0.0f;
       }
     }
     __syncthreads();
@@ -99,6 +105,31 @@ __global__ __launch_bounds__(kThreads) void f16_matmul_kernel(_Float16 const *__
     int col = col0 + wc + lane % 32;
     if (row < m && col < n) {
       C[(size_t)row * n + col] = static_cast<_Float16>(acc[r]);
+    }
+  }
+}
+
+// out[b][c][r] = in[b][r][c] through a 64 x 64 LDS tile: the row-major copy of a column-major
+// tensor (or the other way round) for the operators that index their inputs flat.
+__global__ __launch_bounds__(kThreads) void f16_transpose_kernel(_Float16 const *__restrict__ in,
+                                                                _Float16 *__restrict__ out, int rows,
+                                                                int cols) {
+  __shared__ _Float16 tile[64][66];
+  size_t const b = blockIdx.z;
+  in += b * (size_t)rows * cols;
+  out += b * (size_t)rows * cols;
+  int const r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  for (int e = threadIdx.x; e < 64 * 64; e += kThreads) {
+    int const r = e / 64, c = e % 64;
+    if (r0 + r < rows && c0 + c < cols) {
+      tile[r][c] = in[(size_t)(r0 + r) * cols + c0 + c];
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 64 * 64; e += kThreads) {
+    int const c = e / 64, r = e % 64;
+    if (r0 + r < rows && c0 + c < cols) {
+      out[(size_t)(c0 + c) * rows + r0 + r] = tile[r][c];
     }
   }
 }
@@ -207,8 +238,8 @@ extern "C" int mi355_f16_fill_normal(void *x, size_t n, float std, uint64_t seed
   return MI355_OK;
 }
 
-extern "C" int mi355_f16_matmul(void const *A, void const *B, void *C, int batch, int m, int n,
-                                int k) {
+extern "C" int mi355_f16_matmul_layout(void const *A, void const *B, void *C, int batch, int m,
+                                       int n, int k, int a_column_major, int b_column_major) {
   MI355_REQUIRE_INIT();
   if (batch < 0 || m < 0 || n < 0 || k < 0) {
     return fail(MI355_ERR_INVALID, "negative matmul extent");
@@ -222,7 +253,34 @@ extern "C" int mi355_f16_matmul(void const *A, void const *B, void *C, int batch
   dim3 grid((n + 63) / 64, (m + 63) / 64, batch);
   f16_matmul_kernel<<<grid, kThreads, 0, state().stream()>>>(
       static_cast<_Float16 const *>(A), static_cast<_Float16 const *>(B),
-      static_cast<_Float16 *>(C), m, n, k);
+      static_cast<_Float16 *>(C), m, n, k, a_column_major ? 1 : k, a_column_major ? m : 1,
+      b_column_major ? 1 : n, b_column_major ? k : 1);
+  MI355_HIP(hipGetLastError());
+  return MI355_OK;
+}
+
+extern "C" int mi355_f16_matmul(void const *A, void const *B, void *C, int batch, int m, int n,
+                                int k) {
+  return mi355_f16_matmul_layout(A, B, C, batch, m, n, k, 0, 0);
+}
+
+extern "C" int mi355_f16_transpose(void const *in, void *out, int batch, int rows, int cols) {
+  MI355_REQUIRE_INIT();
+  if (batch < 0 || rows < 0 || cols < 0) {
+    return fail(MI355_ERR_INVALID, "negative transpose extent");
+  }
+  if (batch == 0 || rows == 0 || cols == 0) {
+    return MI355_OK;
+  }
+  if (batch > 65535 || (rows + 63) / 64 > 65535) {
+    return fail(MI355_ERR_UNSUPPORTED, "transpose grid out of range");
+  }
+  if (in == out) {
+    return fail(MI355_ERR_INVALID, "transpose in place");
+  }
+  dim3 grid((cols + 63) / 64, (rows + 63) / 64, batch);
+  f16_transpose_kernel<<<grid, kThreads, 0, state().stream()>>>(
+      static_cast<_Float16 const *>(in), static_cast<_Float16 *>(out), rows, cols);
   MI355_HIP(hipGetLastError());
   return MI355_OK;
 }

@@ -174,9 +174,48 @@ __device__ __forceinline__ void store_weight(uint4v const (&x)[PPT][4], int R, i
   }
 }
 
+// Column-major weights (a [R][C] tile stored column by column: C rows of R contiguous halfs,
+// `ld` halfs apart) already have k contiguous: the same two halves without the transpose.
+// Patch p is four consecutive 16-byte chunks of dst[C][R] (R / 8 chunks per row).
+template <int PPT>
+__device__ __forceinline__ void load_weight_cm(_Float16 const *__restrict__ src, int ld, int R, int C,
+                                               uint4v (&x)[PPT][4], int tid, int nthreads) {
+  int const cpr = R / 8, patches = C * cpr / 4;
+#pragma unroll
+  for (int i = 0; i < PPT; i++) {
+    int p = tid + i * nthreads;
+    if (p < patches) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        int const q = 4 * p + j;
+        x[i][j] = *reinterpret_cast<uint4v const *>(src + (long long)(q / cpr) * ld + 8 * (q % cpr));
+      }
+    }
+  }
+}
+
+template <int PPT>
+__device__ __forceinline__ void store_weight_cm(uint4v const (&x)[PPT][4], int R, int C,
+                                                _Float16 *__restrict__ dst, int tid, int nthreads) {
+  int const cpr = R / 8, patches = C * cpr / 4;
+  int const mask = (cpr - 1) & 7;
+#pragma unroll
+  for (int i = 0; i < PPT; i++) {
+    int p = tid + i * nthreads;
+    if (p < patches) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        int const q = 4 * p + j;
+        *reinterpret_cast<uint4v *>(dst + sw_chunk(q / cpr, q % cpr, R, mask)) = x[i][j];
+      }
+    }
+  }
+}
+
 // MT m-tiles of 16 rows, NB weight matrices, 4 wavefronts = the 4 column tiles of a
-// 64-column weight tile.  KTMAX bounds the staging register arrays.
-template <int MT, int NB, int PRO, bool LORA, int KTMAX>
+// 64-column weight tile.  KTMAX bounds the staging register arrays.  WCM: every weight-side
+// operand (weights, lora A and B) is a column-major tensor.
+template <int MT, int NB, int PRO, bool LORA, int KTMAX, bool WCM>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
   constexpr int NT = 256;
   constexpr int WPPT = ((KTMAX / 4) * 8 + NT - 1) / NT;  // weight patches per thread
@@ -204,7 +243,13 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
   if (LORA) {
     // B [16][64] -> B^T [64][16], loop invariant: 32 patches
     _Float16 const *src = static_cast<_Float16 const *>(P.lb.ptr) + gtile_offset(P.lb, bx, by, bz, 0);
-    stage_weight<1>(src, P.lb.d_cols, 16, 64, lb_lds, tid, NT);
+    if (WCM) {  // already B^T [64][16]: 128 chunks, copied as they are
+      uint4v x[1][4];
+      load_weight_cm<1>(src, P.lb.d_cols, 16, 64, x, tid, NT);
+      store_weight_cm<1>(x, 16, 64, lb_lds, tid, NT);
+    } else {
+      stage_weight<1>(src, P.lb.d_cols, 16, 64, lb_lds, tid, NT);
+    }
   }
 
   _Float16 acc16[NB][MT][4];  // O[16mt + c][16*wave + 4g + r], used when ksplit == 1
@@ -246,11 +291,19 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
     for (int b = 0; b < NB; b++) {
       GTile const &bt = b == 0 ? P.b0 : P.b1;
       _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it);
-      load_weight<WPPT>(src, bt.d_cols, KT, 64, wreg[b], tid, NT);
+      if (WCM) {
+        load_weight_cm<WPPT>(src, bt.d_cols, KT, 64, wreg[b], tid, NT);
+      } else {
+        load_weight<WPPT>(src, bt.d_cols, KT, 64, wreg[b], tid, NT);
+      }
     }
     if (LORA) {
       _Float16 const *src = static_cast<_Float16 const *>(P.la.ptr) + gtile_offset(P.la, bx, by, bz, it);
-      load_weight<LORA ? LPPT : 1>(src, P.la.d_cols, KT, 16, lreg, tid, NT);
+      if (WCM) {
+        load_weight_cm<LORA ? LPPT : 1>(src, P.la.d_cols, KT, 16, lreg, tid, NT);
+      } else {
+        load_weight<LORA ? LPPT : 1>(src, P.la.d_cols, KT, 16, lreg, tid, NT);
+      }
     }
   };
   // registers -> LDS: activation tile as it is (prologue applied), weights transposed
@@ -287,10 +340,18 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
     }
 #pragma unroll
     for (int b = 0; b < NB; b++) {
-      store_weight<WPPT>(wreg[b], KT, 64, b_lds + b * 64 * KT, tid, NT);
+      if (WCM) {
+        store_weight_cm<WPPT>(wreg[b], KT, 64, b_lds + b * 64 * KT, tid, NT);
+      } else {
+        store_weight<WPPT>(wreg[b], KT, 64, b_lds + b * 64 * KT, tid, NT);
+      }
     }
     if (LORA) {
-      store_weight<LORA ? LPPT : 1>(lreg, KT, 16, la_lds, tid, NT);
+      if (WCM) {
+        store_weight_cm<LORA ? LPPT : 1>(lreg, KT, 16, la_lds, tid, NT);
+      } else {
+        store_weight<LORA ? LPPT : 1>(lreg, KT, 16, la_lds, tid, NT);
+      }
     }
   };
   bool const split = P.ksplit > 1;
@@ -535,13 +596,19 @@ __device__ __forceinline__ half4 lane_tr16(_Float16 const *p) {
   return __builtin_bit_cast(half4, v);
 }
 
-template <int KT, int NB, int PRO, bool LORA>
+// Column-major weights (WCM): column n of a weight tile is KT contiguous halfs, so a lane's
+// operand -- eight consecutive k of one column -- is 16 contiguous bytes of global memory, like
+// its activation rows: every operand goes straight into registers, the strips and the
+// transposing reads disappear, LDS holds the product slots only, and a piece's sixteen columns
+// are sixteen streams of whole cache lines that no other workgroup touches.
+template <int KT, int NB, int PRO, bool LORA, bool WCM>
 __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
   GemmParams const &P = L.g;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   constexpr int KS = KT / 32;                                // MFMA steps (and 1 KB loads) per strip
   constexpr int STRIPS = NB + (LORA ? 1 : 0);
-  constexpr int WAVE_BYTES = STRIPS * KT * 32 + (LORA ? 512 : 0);  // + the [16][16] piece of lora B
+  // (row-major weights: the strips, + the [16][16] piece of lora B)
+  constexpr int WAVE_BYTES = WCM ? 0 : STRIPS * KT * 32 + (LORA ? 512 : 0);
   int const tid = threadIdx.x, lane = tid % 64, IP = blockDim.x / 64;
   int const ip = __builtin_amdgcn_readfirstlane(tid / 64);  // (wave-uniform: addresses stay scalar)
   int const g = lane / 16, c = lane % 16;
@@ -581,11 +648,15 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
   bool const row_ok = row < M;
   int const row_ld = row_ok ? row : M - 1;
 
+  half4 lb_frag = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
   if (LORA) {
-    // lora B [16][64], loop invariant: this piece's 16 columns, rows of 32 bytes
-    _Float16 const *src = static_cast<_Float16 const *>(P.lb.ptr) + gtile_offset(P.lb, bx, by, bz, 0) + n0;
-    if (lane < 32) {
-      lane_dma16(src, (uint32_t)((ld_row * P.lb.d_cols + 8 * ld_half) * 2), lane_lds_address(lb_piece));
+    _Float16 const *src = static_cast<_Float16 const *>(P.lb.ptr) + gtile_offset(P.lb, bx, by, bz, 0);
+    if (WCM) {
+      // lora B^T[n0 + c][k = 4g .. + 3]: 8 bytes, loop invariant
+      lb_frag = *reinterpret_cast<half4 const *>(src + (long long)(n0 + c) * P.lb.d_cols + 4 * g);
+    } else if (lane < 32) {
+      // lora B [16][64], loop invariant: this piece's 16 columns, rows of 32 bytes
+      lane_dma16(src + n0, (uint32_t)((ld_row * P.lb.d_cols + 8 * ld_half) * 2), lane_lds_address(lb_piece));
     }
   }
 
@@ -596,15 +667,26 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     // ---- issue everything this iteration needs -------------------------------------------
+    uint4v wr[WCM ? STRIPS : 1][KS];  // column-major weights: the operands themselves
 #pragma unroll
     for (int b = 0; b < STRIPS; b++) {
       GTile const &bt = b == NB ? P.la : (b == 0 ? P.b0 : P.b1);
       int const col0 = b == NB ? 0 : n0;  // the lora A tile is [KT][16]: whole
-      _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it) + col0;
-      uint32_t const off = (uint32_t)((ld_row * bt.d_cols + 8 * ld_half) * 2);
+      if (WCM) {
+        // W^T[col0 + c][32j + 8g + 0..7]
+        _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it) +
+                              (long long)(col0 + c) * bt.d_cols + 8 * g;
 #pragma unroll
-      for (int j = 0; j < KS; j++) {
-        lane_dma16(src + (long long)(32 * j) * bt.d_cols, off, lane_lds_address(strip[b]) + j * 1024);
+        for (int j = 0; j < KS; j++) {
+          wr[b][j] = *reinterpret_cast<uint4v const *>(src + 32 * j);
+        }
+      } else {
+        _Float16 const *src = static_cast<_Float16 const *>(bt.ptr) + gtile_offset(bt, bx, by, bz, it) + col0;
+        uint32_t const off = (uint32_t)((ld_row * bt.d_cols + 8 * ld_half) * 2);
+#pragma unroll
+        for (int j = 0; j < KS; j++) {
+          lane_dma16(src + (long long)(32 * j) * bt.d_cols, off, lane_lds_address(strip[b]) + j * 1024);
+        }
       }
     }
     _Float16 const *a0 = static_cast<_Float16 const *>(P.a0.ptr) + gtile_offset(P.a0, bx, by, bz, it) +
@@ -632,6 +714,12 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
       asm volatile("" : "+v"(xr[j]));  // (no use of a fragment moves above the wait)
       if (PRO == PRO_SILU_MUL) {
         asm volatile("" : "+v"(ur[j]));
+      }
+      if (WCM) {
+#pragma unroll
+        for (int b = 0; b < STRIPS; b++) {
+          asm volatile("" : "+v"(wr[b][j]));
+        }
       }
     }
 #pragma clang diagnostic pop
@@ -667,9 +755,14 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
       float4v d = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int j = 0; j < KS; j++) {
-        _Float16 const *ap = strip[NB] + (32 * j + 8 * g) * 16 + tr_off;
-        half4 const lo = lane_tr16(ap), hi = lane_tr16(ap + 64);
-        half8 const a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        half8 a;
+        if (WCM) {
+          a = __builtin_bit_cast(half8, wr[WCM ? NB : 0][j]);
+        } else {
+          _Float16 const *ap = strip[NB] + (32 * j + 8 * g) * 16 + tr_off;
+          half4 const lo = lane_tr16(ap), hi = lane_tr16(ap + 64);
+          a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
         d = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, x[j], d, 0, 0, 0);
       }
 #pragma unroll
@@ -683,13 +776,18 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
       float4v o = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int j = 0; j < KS; j++) {
-        _Float16 const *wp = strip[b] + (32 * j + 8 * g) * 16 + tr_off;
-        half4 const lo = lane_tr16(wp), hi = lane_tr16(wp + 64);
-        half8 const w = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        half8 w;
+        if (WCM) {
+          w = __builtin_bit_cast(half8, wr[WCM ? b : 0][j]);
+        } else {
+          _Float16 const *wp = strip[b] + (32 * j + 8 * g) * 16 + tr_off;
+          half4 const lo = lane_tr16(wp), hi = lane_tr16(wp + 64);
+          w = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
         o = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, x[j], o, 0, 0, 0);
       }
       if (LORA) {
-        half4 const w = lane_tr16(lb_piece + (4 * g) * 16 + tr_off);  // B[k = 4g ..][n = c]
+        half4 const w = WCM ? lb_frag : lane_tr16(lb_piece + (4 * g) * 16 + tr_off);  // B[k = 4g ..][n = c]
         o = __builtin_amdgcn_mfma_f32_16x16x16f16(w, dfrag, o, 0, 0, 0);
       }
       half4 p16;
@@ -741,14 +839,19 @@ __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
 // ---------------------------------------------------------------------------------------
 namespace {
 
+// (a column-major tensor -- DevOp::sub == 1 on its loader -- holds element (r, c) at
+// c * d_rows + r: a step along the rows is one element, a step along the columns d_rows, and
+// `d_cols` of the result is that leading dimension)
 GTile gtile(DevOp const &op, void const *ptr) {
   GTile t;
   t.ptr = ptr;
+  bool const cm = op.kind == DOP_LOAD && op.sub == 1;
+  long long const rstep = cm ? 1 : op.d_cols, cstep = cm ? op.d_rows : 1;
   for (int i = 0; i < 3; i++) {
-    t.lin[i] = op.g_bs[i] + (long long)op.row_bs[i] * op.d_cols + op.col_bs[i];
+    t.lin[i] = op.g_bs[i] + op.row_bs[i] * rstep + op.col_bs[i] * cstep;
   }
-  t.lin[3] = op.g_fs + (long long)op.row_fs * op.d_cols + op.col_fs;
-  t.d_cols = op.d_cols;
+  t.lin[3] = op.g_fs + op.row_fs * rstep + op.col_fs * cstep;
+  t.d_cols = cm ? op.d_rows : op.d_cols;
   return t;
 }
 
@@ -758,6 +861,9 @@ struct GMatch {
   int a0, a1, b0, b1, la, lb;  // load op indices (-1 when absent)
   int o0, o1;                  // output op indices
   int M, KT;
+  // every weight-side operand (b0, b1, la, lb) is a DmemColumnMajor tensor, as the reference's
+  // plans declare their weights (cpp_examples/lora.cc:36-41): k is contiguous in memory
+  bool wcm;
 };
 
 int loader_of(DevProgram const &P, int nloads, int tensor) {
@@ -841,6 +947,18 @@ bool gmatch(DevProgram const &P, GMatch &G) {
   if (G.a0 < 0 || G.b0 < 0 || (G.nb == 2 && G.b1 < 0)) {
     return false;
   }
+  // activations row-major; the weight-side operands all in one storage order
+  G.wcm = P.ops[G.b0].sub == 1;
+  for (int i : {G.a0, G.a1}) {
+    if (i >= 0 && P.ops[i].sub == 1) {
+      return false;
+    }
+  }
+  for (int i : {G.b0, G.b1, G.la, G.lb}) {
+    if (i >= 0 && (P.ops[i].sub == 1) != G.wcm) {
+      return false;
+    }
+  }
   DevTensor const &ta = P.t[P.ops[G.a0].dst], &tb = P.t[P.ops[G.b0].dst];
   G.M = ta.rows;
   G.KT = ta.cols;
@@ -870,7 +988,7 @@ bool gmatch(DevProgram const &P, GMatch &G) {
   return true;
 }
 
-template <int MT, int NB, int PRO, bool LORA>
+template <int MT, int NB, int PRO, bool LORA, bool WCM>
 int launch_kt(GemmParams const &A, dim3 grid, int lds) {
   State &s = state();
   auto go = [&](auto *fn) -> int {
@@ -883,17 +1001,17 @@ int launch_kt(GemmParams const &A, dim3 grid, int lds) {
     return 1;
   };
   if (A.KT <= 64) {
-    return go(gemm_fused_kernel<MT, NB, PRO, LORA, 64>);
+    return go(gemm_fused_kernel<MT, NB, PRO, LORA, 64, WCM>);
   }
   if (A.KT <= 256) {
-    return go(gemm_fused_kernel<MT, NB, PRO, LORA, 256>);
+    return go(gemm_fused_kernel<MT, NB, PRO, LORA, 256, WCM>);
   }
-  return go(gemm_fused_kernel<MT, NB, PRO, LORA, 512>);
+  return go(gemm_fused_kernel<MT, NB, PRO, LORA, 512, WCM>);
 }
 
 // gemm_lanes_kernel for this plan, or 0 when it is not the better choice (see the rule in
 // try_launch_lanes); k extents 64 / 128 / 256.
-template <int NB, int PRO, bool LORA>
+template <int NB, int PRO, bool LORA, bool WCM>
 int launch_lanes_kt(LaneParams const &L, int grid, int threads, int lds) {
   State &s = state();
   auto go = [&](auto *fn) -> int {
@@ -907,11 +1025,11 @@ int launch_lanes_kt(LaneParams const &L, int grid, int threads, int lds) {
   };
   switch (L.g.KT) {
     case 64:
-      return go(gemm_lanes_kernel<64, NB, PRO, LORA>);
+      return go(gemm_lanes_kernel<64, NB, PRO, LORA, WCM>);
     case 128:
-      return go(gemm_lanes_kernel<128, NB, PRO, LORA>);
+      return go(gemm_lanes_kernel<128, NB, PRO, LORA, WCM>);
     case 256:
-      return go(gemm_lanes_kernel<256, NB, PRO, LORA>);
+      return go(gemm_lanes_kernel<256, NB, PRO, LORA, WCM>);
     default:
       return 0;
   }
@@ -935,12 +1053,17 @@ int try_launch_lanes(DevProgram const &P, GMatch const &G, GemmParams const &A) 
   // every piece re-reads the activation rows, so the L2 -> L1 traffic is 4-5 x the bytes of the
   // plan (measured on the LoRA plan: 202 MB of requests for 34 MB), which is what bounds a plan
   // of tens of MB; the range-splitting kernel moves whole lines once.
+  // Column-major weights have neither cost (a piece's columns are whole lines of its own, read
+  // straight into registers), so the one launch also serves plans of tens of MB.
   long long const weight_bytes = blocks * F * (long long)(G.nb * G.KT * 64 + (G.lora ? G.KT * 16 : 0)) * 2;
-  if (s.gemm_mode == 0 && (blocks * S > 1024 || weight_bytes > (8LL << 20))) {
+  if (s.gemm_mode == 0 && !G.wcm && (blocks * S > 1024 || weight_bytes > (8LL << 20))) {
+    return 0;
+  }
+  if (s.gemm_mode == 0 && G.wcm && (blocks * S > 4096 || weight_bytes > (64LL << 20))) {
     return 0;
   }
   int const strips = G.nb + (G.lora ? 1 : 0);
-  int const wave_bytes = strips * G.KT * 32 + (G.lora ? 512 : 0);
+  int const wave_bytes = G.wcm ? 0 : strips * G.KT * 32 + (G.lora ? 512 : 0);
   int const slot_bytes = F * G.nb * 512;
   int ip = F < 16 ? F : 16;
   while (ip > 1 && ip * wave_bytes + slot_bytes > s.max_lds) {
@@ -964,7 +1087,8 @@ int try_launch_lanes(DevProgram const &P, GMatch const &G, GemmParams const &A) 
   int rc = 0;
 #define MI355_LANES_CASE(NBV, PROV, LORAV)                                  \
   if (G.nb == NBV && G.pro == PROV && G.lora == LORAV) {                    \
-    rc = launch_lanes_kt<NBV, PROV, LORAV>(L, grid, ip * 64, lds);          \
+    rc = G.wcm ? launch_lanes_kt<NBV, PROV, LORAV, true>(L, grid, ip * 64, lds)   \
+               : launch_lanes_kt<NBV, PROV, LORAV, false>(L, grid, ip * 64, lds); \
   }
   MI355_LANES_CASE(1, PRO_NONE, false)
   MI355_LANES_CASE(1, PRO_EXP, false)
@@ -1049,7 +1173,8 @@ int try_launch_gemm(DevProgram const &P) {
   int rc = 0;
 #define MI355_GEMM_CASE(MTV, NBV, PROV, LORAV)                                        \
   if (mt == MTV && G.nb == NBV && G.pro == PROV && G.lora == LORAV) {                 \
-    rc = launch_kt<MTV, NBV, PROV, LORAV>(A, grid, lds);                              \
+    rc = G.wcm ? launch_kt<MTV, NBV, PROV, LORAV, true>(A, grid, lds)                 \
+               : launch_kt<MTV, NBV, PROV, LORAV, false>(A, grid, lds);               \
   }
   MI355_GEMM_CASE(1, 1, PRO_NONE, false)
   MI355_GEMM_CASE(2, 1, PRO_NONE, false)

@@ -19,12 +19,14 @@ struct TensorInfo {
   bool persistent = false;
   bool as_a = false, as_b = false;
   int declared = 299;  // loader tiles: the plan's stensor layout word (SmemUnknownLayout otherwise)
+  bool dmem_colmajor = false;  // loader tiles (fp16): the device tensor is stored column by column
   int bytes = 0;
 };
 
 // Declared thread-block layouts (values of the reference's include/mirage/layout.h:37-47):
 // 200 / 202-204 are the row-major family, 201 / 205-207 the column-major one; the
 // TensorOpMultiplicand_Crosswise{16,32,64} members pad by 4 / 8 / 16 halfs.
+constexpr int kDmemColumnMajor = 101;  // include/mirage/layout.h:28-34
 bool declared_known(int l) { return l >= 200 && l <= 207; }
 bool declared_column_major(int l) { return l == 201 || (l >= 205 && l <= 207); }
 int declared_pad(int l) {
@@ -154,12 +156,21 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       d.dst = define(q[18], rows, cols, o);
       if (d.dst >= 0) {
         T[d.dst].declared = q[17];
+        T[d.dst].dmem_colmajor = f16 && q[16] == kDmemColumnMajor;
       }
       d.hoist = (F == 1) || (d.row_fs == 0 && d.col_fs == 0 && d.g_fs == 0);
+      // The fp16 data of a DmemColumnMajor tensor is stored column by column (element (r, c)
+      // of a [R, C] matrix at c * R + r), as the reference's fp16 loader reads it
+      // (include/mirage/threadblock/cuda/input_loader.h:221-247); fingerprint buffers are
+      // row-major whatever the declaration (input_loader.h:457-467).
+      bool const colmajor = f16 && q[16] == kDmemColumnMajor;
+      d.sub = colmajor ? 1 : 0;
       long long max_row = (long long)(F - 1) * d.row_fs + rows - 1;
       long long max_col = (long long)(F - 1) * d.col_fs + cols - 1;
       long long max_g = (long long)(F - 1) * d.g_fs;
-      bool al = cols % 8 == 0 && d.d_cols % 8 == 0 && d.col_fs % 8 == 0 && d.g_fs % 8 == 0;
+      // 16-byte pieces run along the contiguous direction: columns, or rows when column-major
+      bool al = colmajor ? (rows % 8 == 0 && d.d_rows % 8 == 0 && d.row_fs % 8 == 0 && d.g_fs % 8 == 0)
+                         : (cols % 8 == 0 && d.d_cols % 8 == 0 && d.col_fs % 8 == 0 && d.g_fs % 8 == 0);
       for (int g = 0; g < 3; g++) {
         long long b = plan.grid_dim[g] - 1;
         if (d.row_bs[g] < 0 || d.col_bs[g] < 0 || d.g_bs[g] < 0) {
@@ -169,7 +180,7 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
         max_row += b * d.row_bs[g];
         max_col += b * d.col_bs[g];
         max_g += b * d.g_bs[g];
-        al = al && d.col_bs[g] % 8 == 0 && d.g_bs[g] % 8 == 0;
+        al = al && (colmajor ? d.row_bs[g] : d.col_bs[g]) % 8 == 0 && d.g_bs[g] % 8 == 0;
       }
       if (d.row_fs < 0 || d.col_fs < 0 || d.g_fs < 0) {
         err = "negative loader stride";
@@ -181,7 +192,8 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       }
       d.vec8 = al ? 1 : 0;
       d.galign = d.vec8;
-      ext.in_elems[d.io] = max_g + max_row * d.d_cols + max_col + 1;
+      ext.in_elems[d.io] = colmajor ? max_g + max_col * d.d_rows + max_row + 1
+                                    : max_g + max_row * d.d_cols + max_col + 1;
     } else if (t == TB_OUTPUT_OP) {
       if (!need(17) || o < out_start) {
         err = "output saver out of place or truncated";
@@ -393,7 +405,10 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
     } else {
       // every tile row-major with padded rows, as it is loaded (the matrix-core B operand is
       // gathered with transposing LDS reads) -- unless the plan's declaration rules
-      bool column_major = false;
+      // A tile of a column-major device tensor stays column-major in LDS (16-byte pieces
+      // then move as they are, and a matmul reads it k-contiguous as its B operand) unless
+      // a matmul wants it as its A operand.
+      bool column_major = ti.dmem_colmajor && !ti.as_a;
       int p = pad;
       if (declared_layouts && declared_known(ti.declared)) {
         column_major = declared_column_major(ti.declared);
@@ -563,6 +578,10 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       d.mg0 = fast_div_magic(d.mm_kc / 4);
       d.mg1 = fast_div_magic(n / 2);
       d.mg2 = fast_div_magic(n / 4);
+    } else if (d.kind == DOP_LOAD && d.sub == 1) {
+      // a column-major tensor is walked as the row-major matrix of its transpose
+      d.mg0 = fast_div_magic(prog.t[d.dst].rows);
+      d.mg1 = fast_div_magic(prog.t[d.dst].rows / 8);
     } else if (d.kind == DOP_REDUCE) {
       d.mg0 = fast_div_magic(d.red_inner);
     } else if (d.kind == DOP_CONCAT) {
@@ -573,8 +592,13 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
   // LDS writes of 16 bytes need 8-element row strides on the destination
   for (int o = 0; o < prog.num_ops; o++) {
     DevOp &d = prog.ops[o];
-    if (d.kind == DOP_LOAD && f16 && (prog.t[d.dst].cs != 1 || prog.t[d.dst].rs % 8 != 0)) {
-      d.vec8 = d.vec8 ? 2 : 0;  // 2: vector global read, scalar LDS scatter
+    if (d.kind == DOP_LOAD && f16) {
+      // (for a column-major device tensor the 16-byte pieces run down a column of the tile)
+      DevTensor const &t = prog.t[d.dst];
+      int const along = d.sub == 1 ? t.rs : t.cs, across = d.sub == 1 ? t.cs : t.rs;
+      if (along != 1 || across % 8 != 0) {
+        d.vec8 = d.vec8 ? 2 : 0;  // 2: vector global read, scalar LDS scatter
+      }
     }
     if (d.kind == DOP_OUTPUT && f16 && (prog.t[d.dst].cs != 1 || prog.t[d.dst].rs % 8 != 0)) {
       d.vec8 = 0;

@@ -754,26 +754,35 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
           _Float16 *s = tile_ptr(lds, t);
           TileOrigin org = tile_origin(op, it, blockIdx.x);
           _Float16 const *g = static_cast<_Float16 const *>(P.in[op.io]) + org.base;
+          // A column-major device tensor (element (r, c) at c * d_rows + r) is walked as the
+          // row-major matrix of its transpose: rows and columns, origins and the tile's LDS
+          // strides swap roles, and the 16-byte pieces run down the tile's columns.
+          bool const cm = op.sub == 1;
+          int const vrows = cm ? t.cols : t.rows, vcols = cm ? t.rows : t.cols;
+          int const ld = cm ? op.d_rows : op.d_cols;
+          int const r0 = cm ? org.col0 : org.row0, c0 = cm ? org.row0 : org.col0;
+          int const srs = cm ? t.cs : t.rs, scs = cm ? t.rs : t.cs;
           if (op.vec8) {
-            int const cpr = t.cols / 8, n = t.rows * cpr;
+            int const cpr = vcols / 8, n = vrows * cpr;
+            uint32_t const magic = cm ? op.mg1 : t.mcpr;
             for (int e = tid; e < n; e += kInterpThreads) {
-              int const r = fdiv(e, t.mcpr), c = (e - r * cpr) * 8;
-              half8 v = *reinterpret_cast<half8 const *>(
-                  g + (long long)(org.row0 + r) * op.d_cols + org.col0 + c);
+              int const r = fdiv(e, magic), c = (e - r * cpr) * 8;
+              half8 v = *reinterpret_cast<half8 const *>(g + (long long)(r0 + r) * ld + c0 + c);
               if (op.vec8 == 1) {
-                *reinterpret_cast<half8 *>(s + r * t.rs + c) = v;
+                *reinterpret_cast<half8 *>(s + r * srs + c) = v;
               } else {
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
-                  s[r * t.rs + (c + j) * t.cs] = v[j];
+                  s[r * srs + (c + j) * scs] = v[j];
                 }
               }
             }
           } else {
-            int const n = t.rows * t.cols;
+            int const n = vrows * vcols;
+            uint32_t const magic = cm ? op.mg0 : t.mcols;
             for (int e = tid; e < n; e += kInterpThreads) {
-              int const r = fdiv(e, t.mcols), c = e - r * t.cols;
-              s[r * t.rs + c * t.cs] = g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c];
+              int const r = fdiv(e, magic), c = e - r * vcols;
+              s[r * srs + c * scs] = g[(long long)(r0 + r) * ld + c0 + c];
             }
           }
           break;

@@ -43,12 +43,15 @@ inline uint32_t fast_div_magic(int d) {
 
 struct DevOp {
   int kind;
-  int sub;             // UNARY / BINARY: the TB_* operator code
+  int sub;             // UNARY / BINARY: the TB_* operator code; LOAD (fp16): 1 = the device tensor
+                       // is DmemColumnMajor, element (r, c) of its [d_rows, d_cols] matrix at
+                       // c * d_rows + r (fingerprint tensors are always row-major)
   int src0, src1, dst; // tensor ids (-1 when unused)
   int io;              // LOAD: input slot; OUTPUT: output slot
   int hoist;           // LOAD: loop invariant, executed at iteration 0 only
   int vec8;            // LOAD / OUTPUT: 16-byte accesses usable on both the global and LDS side
-  int galign;          // LOAD / OUTPUT: every row segment is 16-byte aligned in global memory
+  int galign;          // LOAD / OUTPUT: every row segment (column segment of a column-major tensor)
+                       // is 16-byte aligned in global memory
   int row_bs[3], col_bs[3], row_fs, col_fs;  // block / for-loop strides of the tile origin
   int g_bs[3], g_fs;                         // block / for-loop strides of the batch offset
   int d_rows, d_cols;                        // matrix shape of the device tensor
@@ -57,6 +60,7 @@ struct DevOp {
   int mm_kc;  // MATMUL, uint16 interpreter: k chunk of the packed-residue path, 0 = scalar path
   int mm_mb;  // MATMUL, matrix-core variant (sub == 1): rows of A packed at a time
   // division magics.  MATMUL: kc / 4, n / 2, n / 4.  REDUCE: inner.  CONCAT: inner, a + b.
+  // LOAD of a column-major tensor: the tile's rows, rows / 8.
   uint32_t mg0, mg1, mg2;
 };
 

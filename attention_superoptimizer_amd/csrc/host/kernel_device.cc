@@ -7,6 +7,7 @@
 #include "mi355_abi.h"
 #include "mirage/kernel/device_memory_manager.h"
 #include "mirage/kernel/graph.h"
+#include "mirage/layout.h"
 #include "mirage/utils/hip_types.h"
 
 #include <cstring>
@@ -70,17 +71,59 @@ static void matmul_extents(DTensor const &A, DTensor const &B, int &batch, int &
   }
 }
 
+// The fp16 data of a DmemColumnMajor tensor holds each matrix column by column.  The GEMM reads
+// either order (as the reference's does, matmul_kernel.cu:61-76); the element-wise operators
+// and reductions index their inputs flat, so a column-major input is first copied row-major
+// into a temporary at the top of the arena (freed again before the call returns: LIFO).
+static bool column_major(DTensor const &t) {
+  return t.layout == mirage::layout::DmemColumnMajor && t.num_dims >= 2;
+}
+
+namespace {
+struct RowMajorCopy {
+  void *ptr = nullptr;  // what the operator reads
+  DTensor temp;
+  bool held = false;
+  explicit RowMajorCopy(DTensor const &t) : ptr(t.data_ptr) {
+    if (!column_major(t)) {
+      return;
+    }
+    temp = t;
+    temp.layout = mirage::layout::DmemRowMajor;
+    DeviceMemoryManager::get_instance()->allocate(temp, false);
+    held = true;
+    int batch = 1;
+    for (int i = 0; i < t.num_dims - 2; i++) {
+      batch *= t.dim[i];
+    }
+    // the buffer is `batch` matrices of [cols][rows]
+    MI355_CALL(mi355_f16_transpose(t.data_ptr, temp.data_ptr, batch, t.dim[t.num_dims - 1],
+                                   t.dim[t.num_dims - 2]));
+    ptr = temp.data_ptr;
+  }
+  RowMajorCopy(RowMajorCopy const &) = delete;
+  RowMajorCopy &operator=(RowMajorCopy const &) = delete;
+  ~RowMajorCopy() {
+    if (held) {
+      mi355_sync();
+      DeviceMemoryManager::get_instance()->free(temp);
+    }
+  }
+};
+}  // namespace
+
 bool KNMatmulOp::profile(ProfileResult &result) {
   require_device("KNMatmulOp::profile");
   int batch, m, n, k;
   matmul_extents(input_tensors[0], input_tensors[1], batch, m, n, k);
   int const iters = 16;
-  MI355_CALL(mi355_f16_matmul(input_tensors[0].data_ptr, input_tensors[1].data_ptr,
-                              output_tensors[0].data_ptr, batch, m, n, k));
+  int const a_cm = column_major(input_tensors[0]) ? 1 : 0, b_cm = column_major(input_tensors[1]) ? 1 : 0;
+  MI355_CALL(mi355_f16_matmul_layout(input_tensors[0].data_ptr, input_tensors[1].data_ptr,
+                                     output_tensors[0].data_ptr, batch, m, n, k, a_cm, b_cm));
   MI355_CALL(mi355_timer_start());
   for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_matmul(input_tensors[0].data_ptr, input_tensors[1].data_ptr,
-                                output_tensors[0].data_ptr, batch, m, n, k));
+    MI355_CALL(mi355_f16_matmul_layout(input_tensors[0].data_ptr, input_tensors[1].data_ptr,
+                                       output_tensors[0].data_ptr, batch, m, n, k, a_cm, b_cm));
   }
   float ms = 0.0f;
   MI355_CALL(mi355_timer_stop(&ms));
@@ -102,11 +145,11 @@ bool KNElementUnaryOp::profile(ProfileResult &result) {
   require_device("KNElementUnaryOp::profile");
   size_t const n = input_tensors[0].num_elements();
   int const iters = ProfileResult::NUM_ITERATIONS;
-  MI355_CALL(mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
+  RowMajorCopy const in(input_tensors[0]);
+  MI355_CALL(mi355_f16_unary(op_type, in.ptr, output_tensors[0].data_ptr, n));
   MI355_CALL(mi355_timer_start());
   for (int i = 0; i < iters; i++) {
-    MI355_CALL(
-        mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
+    MI355_CALL(mi355_f16_unary(op_type, in.ptr, output_tensors[0].data_ptr, n));
   }
   float ms = 0.0f;
   MI355_CALL(mi355_timer_stop(&ms));
@@ -126,12 +169,12 @@ bool KNElementBinaryOp::profile(ProfileResult &result) {
   require_device("KNElementBinaryOp::profile");
   DTensor const &a = input_tensors[0], &b = input_tensors[1], &o = output_tensors[0];
   int const iters = 16;
-  MI355_CALL(mi355_f16_binary(op_type, a.data_ptr, a.dim, b.data_ptr, b.dim, o.data_ptr, o.dim,
-                              o.num_dims));
+  RowMajorCopy const ra(a);
+  RowMajorCopy const rb(b);
+  MI355_CALL(mi355_f16_binary(op_type, ra.ptr, a.dim, rb.ptr, b.dim, o.data_ptr, o.dim, o.num_dims));
   MI355_CALL(mi355_timer_start());
   for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_binary(op_type, a.data_ptr, a.dim, b.data_ptr, b.dim, o.data_ptr,
-                                o.dim, o.num_dims));
+    MI355_CALL(mi355_f16_binary(op_type, ra.ptr, a.dim, rb.ptr, b.dim, o.data_ptr, o.dim, o.num_dims));
   }
   float ms = 0.0f;
   MI355_CALL(mi355_timer_stop(&ms));
@@ -166,12 +209,11 @@ bool KNReductionOp::profile(ProfileResult &result) {
   reduction_strides(input_tensors[0], output_tensors[0], reduction_dim_idx, factor, is, os);
   size_t const n = output_tensors[0].num_elements();
   int const iters = ProfileResult::NUM_ITERATIONS;
-  MI355_CALL(mi355_f16_reduce(input_tensors[0].data_ptr, output_tensors[0].data_ptr, n, factor,
-                              is, os));
+  RowMajorCopy const in(input_tensors[0]);
+  MI355_CALL(mi355_f16_reduce(in.ptr, output_tensors[0].data_ptr, n, factor, is, os));
   MI355_CALL(mi355_timer_start());
   for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_reduce(input_tensors[0].data_ptr, output_tensors[0].data_ptr, n,
-                                factor, is, os));
+    MI355_CALL(mi355_f16_reduce(in.ptr, output_tensors[0].data_ptr, n, factor, is, os));
   }
   float ms = 0.0f;
   MI355_CALL(mi355_timer_stop(&ms));

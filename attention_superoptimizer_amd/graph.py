@@ -83,17 +83,33 @@ class DTensor:
         assert rc == 0, N.last_error()
         return a
 
+    @property
+    def column_major(self) -> bool:
+        return self.layout == DMEM_LAYOUT["DmemColumnMajor"] and len(self.dims) >= 2
+
     def write_data(self, a: np.ndarray) -> None:
-        a = np.ascontiguousarray(a, dtype=np.float16)
+        """Uploads the LOGICAL values `a` (shape = dims).  The fp16 buffer of a DmemColumnMajor
+        tensor holds each [rows, cols] matrix column by column, as the reference's fp16 loader
+        reads it (include/mirage/threadblock/cuda/input_loader.h:221-247); the fingerprint
+        buffer is row-major whatever the layout (input_loader.h:457-467)."""
+        a = np.asarray(a, dtype=np.float16)
         assert a.size == self.num_elements
+        a = a.reshape(self.dims)
+        if self.column_major:
+            a = a.swapaxes(-1, -2)
+        a = np.ascontiguousarray(a)
         rc = N.runtime().mirage_tensor_write(self._h, 0, a.ctypes.data_as(ctypes.c_void_p), a.nbytes)
         assert rc == 0, N.last_error()
 
     def read_data(self) -> np.ndarray:
-        a = np.empty(self.dims, np.float16)
+        """The logical values (shape = dims), whatever the buffer's layout."""
+        dims = list(self.dims)
+        if self.column_major:
+            dims[-1], dims[-2] = dims[-2], dims[-1]
+        a = np.empty(dims, np.float16)
         rc = N.runtime().mirage_tensor_read(self._h, 0, a.ctypes.data_as(ctypes.c_void_p), a.nbytes)
         assert rc == 0, N.last_error()
-        return a
+        return np.ascontiguousarray(a.swapaxes(-1, -2)) if self.column_major else a
 
     def has_same_fingerprint(self, other: "DTensor") -> bool:
         return bool(N.runtime().mirage_tensor_same_fingerprint(self._h, other._h))

@@ -317,6 +317,16 @@ int mi355_f16_fill_iota(void *x, size_t n, int last_dim);
 int mi355_f16_fill_normal(void *x, size_t n, float std, uint64_t seed);
 /* KNMatmulOp::profile's GEMM, src/kernel/cuda/matmul_kernel.cu:28-143 (row-major) */
 int mi355_f16_matmul(void const *A, void const *B, void *C, int batch, int m, int n, int k);
+/* The same with the operands' storage order stated, as matmul_kernel.cu:61-76 turns
+ * DmemColumnMajor operands into transposed GEMM arguments: a column-major [rows, cols]
+ * matrix holds element (r, c) at c * rows + r.  C is row-major (matmul_kernel.cu:74-75). */
+int mi355_f16_matmul_layout(void const *A, void const *B, void *C, int batch, int m, int n, int k,
+                            int a_column_major, int b_column_major);
+/* out[b][c][r] = in[b][r][c] for `batch` [rows, cols] matrices: the row-major copy of a
+ * DmemColumnMajor tensor (call it with rows = the tensor's columns and cols = its rows) for
+ * the element-wise operators and reductions, which index their inputs flat as
+ * element_unary_kernel.cu:30-42 and element_binary_kernel.cu:30-51 do. */
+int mi355_f16_transpose(void const *in, void *out, int batch, int rows, int cols);
 /* execute_elementunary, src/kernel/cuda/element_unary_kernel.cu:30-42 */
 int mi355_f16_unary(int op, void const *in, void *out, size_t n);
 /* execute_elementbinary, src/kernel/cuda/element_binary_kernel.cu:30-51, with the
