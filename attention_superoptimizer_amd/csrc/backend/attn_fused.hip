@@ -539,8 +539,18 @@ __device__ __forceinline__ constexpr int stream_swizzle_key(int r) {
   return RowHalfs == 128 ? (r & 7) : (IsK ? (((r >> 1) & 1) | (((r >> 3) & 1) << 1)) : ((r >> 1) & 3));
 }
 
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW, bool CM = false>
+// Key tiles wider than 64 keys (SPI strips of 64 keys per for-loop iteration; the form without the
+// division only, which needs no whole row sum before P.V): the strips of an iteration go through
+// the same pipeline one after the other, P.V and the row sums run on in fp32 across them and are
+// rounded to fp16 and added to the for-loop accumulators once per ITERATION -- the roundings of
+// the sequential program for that tile width, an eighth of the conversion work at SPI = 8.
+// MSUM (the form without the division): the row sums are one more column block of P.V, against
+// a B operand of ones, instead of a packed dot product and two cross-lane adds per key block on
+// the vector pipe (v_dot2 shares the matrix pipe and stalls it more than the two MFMAs cost).
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW, bool CM = false, int SPI = 1>
 __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams const P) {
+  static_assert(SPI == 1 || !HAS_DIV, "strips of one iteration need the form without the division");
+  constexpr bool MSUM = !HAS_DIV;
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
   constexpr int NT = 64 * RG;
@@ -572,8 +582,7 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   int const kc_row = 8 * a4 + b4, kc_key = cm_swizzle_key<D, true>(8 * a4 + b4);
   int const vc_key = cm_swizzle_key<NK, false>(c);
   int const row_base = (slice * RG + wave) * RPW * 16;
-  int const F = P.forloop_range;
-
+  int const F = P.forloop_range * SPI;  // passes: strips of 64 keys
   half8 qf[RPW][DK];
   {
     _Float16 const *q = static_cast<_Float16 const *>(P.q.ptr) + tile_offset(P.q, bx, by, bz, 0) +
@@ -590,10 +599,23 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   // is one packed fp16 add (the exact sum of two fp16 numbers rounded once, which is
   // what adding in fp32 and rounding gives)
   half2v oacc[RPW][DB][2];
-  _Float16 racc[RPW];
+  // row-sum accumulators: lane (g, c) holds the sum of query row c (dot-product form: [0]), or of
+  // rows 4g .. 4g + 3 (MSUM: the accumulator layout of the matrix instruction)
+  _Float16 racc[RPW][MSUM ? 4 : 1];
+  // running fp32 sums of the iteration in progress: P.V (SPI > 1 only; with one strip per
+  // iteration they are transient) and, MSUM, the row sums
+  float4v o_run[SPI > 1 ? DB : 1][RPW], s_run[RPW];
 #pragma unroll
   for (int rp = 0; rp < RPW; rp++) {
-    racc[rp] = (_Float16)0.0f;
+#pragma unroll
+    for (int r = 0; r < (MSUM ? 4 : 1); r++) {
+      racc[rp][r] = (_Float16)0.0f;
+    }
+    s_run[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int t = 0; t < (SPI > 1 ? DB : 1); t++) {
+      o_run[t][rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 #pragma unroll
     for (int t = 0; t < DB; t++) {
       oacc[rp][t][0] = half2v{(_Float16)0.0f, (_Float16)0.0f};
@@ -630,15 +652,19 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       v_goff[i] = 2u * (uint32_t)(r * P.v.d_cols + 8 * (pos ^ (2 * stream_swizzle_key<DV, false>(r))));
     }
   }
+  // (strip `it` is strip it % SPI of iteration it / SPI: 64 keys further is 64 columns of K and 64
+  // rows of V, or 64 rows of K^T and 64 columns of V^T)
   auto fetch_k = [&](int it, int b) {
-    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it);
+    _Float16 const *kg = static_cast<_Float16 const *>(P.k.ptr) + tile_offset(P.k, bx, by, bz, it / SPI) +
+                         (CM ? (long long)(64 * (it % SPI)) * P.k.d_cols : (long long)(64 * (it % SPI)));
 #pragma unroll
     for (int i = 0; i < KI; i++) {
       lds_dma16(kg, k_goff[i], lds_k + 2u * (uint32_t)(b * NK * D + (wave * KI + i) * 512));
     }
   };
   auto fetch_v = [&](int it, int b) {
-    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it);
+    _Float16 const *vg = static_cast<_Float16 const *>(P.v.ptr) + tile_offset(P.v, bx, by, bz, it / SPI) +
+                         (CM ? (long long)(64 * (it % SPI)) : (long long)(64 * (it % SPI)) * P.v.d_cols);
 #pragma unroll
     for (int i = 0; i < VI; i++) {
       lds_dma16(vg, v_goff[i], lds_v + 2u * (uint32_t)(b * DV * NK + (wave * VI + i) * 512));
@@ -696,7 +722,9 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
         float const x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[0]), LOG2E, 0.0f));
         float const x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(static_cast<float>(s2[1]), LOG2E, 0.0f));
         half2v const e2 = {static_cast<_Float16>(x0), static_cast<_Float16>(x1)};
-        rs[rp] = __builtin_amdgcn_fdot2(e2, ones, rs[rp], false);
+        if (!MSUM) {
+          rs[rp] = __builtin_amdgcn_fdot2(e2, ones, rs[rp], false);
+        }
         pk[rp][j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
       }
     }
@@ -712,27 +740,57 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   // After the last key block: the row sum across the four lane groups, then either the
   // normalisation of P (form with div) or the accumulation of the denominator.
   auto s_finish = [&](uint32_t (&pk)[RPW][KB / 2][4], float (&rs)[RPW]) {
+    if (MSUM) {
+      return;  // the row sums come out of the matrix cores with P.V
+    }
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       rs[rp] += __shfl_xor(rs[rp], 16, 64);
       rs[rp] += __shfl_xor(rs[rp], 32, 64);
       _Float16 const r16 = static_cast<_Float16>(rs[rp]);
-      if (HAS_DIV) {
-        float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
+      float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
 #pragma unroll
-        for (int jj = 0; jj < KB / 2; jj++) {
+      for (int jj = 0; jj < KB / 2; jj++) {
 #pragma unroll
-          for (int w = 0; w < 4; w++) {
-            half2v const e2 = __builtin_bit_cast(half2v, pk[rp][jj][w]);
-            // (a fused multiply-add with +0: maps to the mixed-precision FMA that reads and
-            // writes fp16; exp values are positive, so the +0 changes nothing)
-            half2v const p2 = {static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[0]), inv, 0.0f)),
-                               static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[1]), inv, 0.0f))};
-            pk[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
-          }
+        for (int w = 0; w < 4; w++) {
+          half2v const e2 = __builtin_bit_cast(half2v, pk[rp][jj][w]);
+          // (a fused multiply-add with +0: maps to the mixed-precision FMA that reads and
+          // writes fp16; exp values are positive, so the +0 changes nothing)
+          half2v const p2 = {static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[0]), inv, 0.0f)),
+                             static_cast<_Float16>(__builtin_fmaf(static_cast<float>(e2[1]), inv, 0.0f))};
+          pk[rp][jj][w] = __builtin_bit_cast(uint32_t, p2);
         }
-      } else {
-        racc[rp] = static_cast<_Float16>(static_cast<float>(racc[rp]) + static_cast<float>(r16));
+      }
+    }
+  };
+  // MSUM: the row sums of P(it) join the running sums; after an iteration's last strip they are
+  // rounded to fp16 and added to the for-loop accumulators
+  half8 ones8;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    ones8[e] = (_Float16)1.0f;
+  }
+  auto sum_mfma = [&](uint32_t const (&pk)[RPW][KB / 2][4], bool last_strip) {
+    if (!MSUM) {
+      return;
+    }
+#pragma unroll
+    for (int jj = 0; jj < KB / 2; jj++) {
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+        uint4v const a = {pk[rp][jj][0], pk[rp][jj][1], pk[rp][jj][2], pk[rp][jj][3]};
+        s_run[rp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), ones8, s_run[rp], 0, 0, 0);
+      }
+    }
+    if (last_strip) {
+#pragma unroll
+      for (int rp = 0; rp < RPW; rp++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          _Float16 const r16 = static_cast<_Float16>(s_run[rp][r]);
+          racc[rp][MSUM ? r : 0] = static_cast<_Float16>(static_cast<float>(racc[rp][MSUM ? r : 0]) + static_cast<float>(r16));
+        }
+        s_run[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
       }
     }
   };
@@ -752,10 +810,14 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       }
     }
   };
+  // (SPI > 1: `o` is the column block's running sum of the iteration, zeroed when the iteration's
+  // last strip has been added to the accumulators; SPI == 1: a fresh sum per pass)
   auto pv_mfma = [&](half8 const (&b)[KB / 2], uint32_t const (&pk)[RPW][KB / 2][4], float4v (&o)[RPW]) {
+    if (SPI == 1) {
 #pragma unroll
-    for (int rp = 0; rp < RPW; rp++) {
-      o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int rp = 0; rp < RPW; rp++) {
+        o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+      }
     }
 #pragma unroll
     for (int jj = 0; jj < KB / 2; jj++) {
@@ -767,21 +829,32 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       }
     }
   };
-  auto pv_post = [&](float4v const (&o)[RPW], int t) {
+  auto pv_post = [&](float4v (&o)[RPW], int t, bool last_strip) {
+    if (SPI > 1 && !last_strip) {
+      return;
+    }
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
       half2v lo = {static_cast<_Float16>(o[rp][0]), static_cast<_Float16>(o[rp][1])};
       half2v hi = {static_cast<_Float16>(o[rp][2]), static_cast<_Float16>(o[rp][3])};
       oacc[rp][t][0] = oacc[rp][t][0] + lo;
       oacc[rp][t][1] = oacc[rp][t][1] + hi;
+      if (SPI > 1) {
+        o[rp] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+      }
     }
   };
-  auto pv_block = [&](_Float16 const *vt, int t, uint32_t const (&pk)[RPW][KB / 2][4]) {
+  auto pv_block = [&](_Float16 const *vt, int t, uint32_t const (&pk)[RPW][KB / 2][4], bool last_strip) {
     half8 b[KB / 2];
-    float4v o[RPW];
     pv_fetch(vt, t, b);
-    pv_mfma(b, pk, o);
-    pv_post(o, t);
+    if (SPI > 1) {
+      pv_mfma(b, pk, o_run[SPI > 1 ? t : 0]);
+      pv_post(o_run[SPI > 1 ? t : 0], t, last_strip);
+    } else {
+      float4v o[RPW];
+      pv_mfma(b, pk, o);
+      pv_post(o, t, true);
+    }
   };
 
   // The loop is skewed by one phase: pass `it` multiplies P(it) with V(it) while it
@@ -816,7 +889,7 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
   // by this wavefront's own work; the scheduling barriers keep that order.
   constexpr int TPU = DB / KB;  // P.V column blocks per S block
   auto skewed_pass = [&](int it, uint32_t const (&pcur)[RPW][KB / 2][4],
-                         uint32_t (&pnext)[RPW][KB / 2][4]) {
+                         uint32_t (&pnext)[RPW][KB / 2][4], bool last_strip) {
     _Float16 const *vt = vbuf + (it & 1) * DV * NK;
     _Float16 const *kt = kbuf + ((it + 1) & 1) * NK * D;
     float rs[RPW];
@@ -841,14 +914,31 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
         s_fetch(kt, u + 1, ka);
       }
       __builtin_amdgcn_sched_barrier(0);
-      float4v o[TPU][RPW];
+      if (SPI > 1) {
 #pragma unroll
-      for (int x = 0; x < TPU; x++) {
-        pv_mfma(vb[x], pcur, o[x]);
-      }
+        for (int x = 0; x < TPU; x++) {
+          pv_mfma(vb[x], pcur, o_run[SPI > 1 ? u * TPU + x : 0]);
+        }
+        if (u == KB - 1) {
+          sum_mfma(pcur, last_strip);
+        }
 #pragma unroll
-      for (int x = 0; x < TPU; x++) {
-        pv_post(o[x], u * TPU + x);
+        for (int x = 0; x < TPU; x++) {
+          pv_post(o_run[SPI > 1 ? u * TPU + x : 0], u * TPU + x, last_strip);
+        }
+      } else {
+        float4v o[TPU][RPW];
+#pragma unroll
+        for (int x = 0; x < TPU; x++) {
+          pv_mfma(vb[x], pcur, o[x]);
+        }
+        if (u == KB - 1) {
+          sum_mfma(pcur, true);
+        }
+#pragma unroll
+        for (int x = 0; x < TPU; x++) {
+          pv_post(o[x], u * TPU + x, true);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -862,13 +952,13 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     fetch_k(it + 2, 0);
     fetch_v(it + 1, 1);
     __builtin_amdgcn_sched_barrier(0);
-    skewed_pass(0, pa, pb);
+    skewed_pass(0, pa, pb, (it & (SPI - 1)) == SPI - 1);
     fetched();
     __syncthreads();
     fetch_k(it + 3, 1);
     fetch_v(it + 2, 0);
     __builtin_amdgcn_sched_barrier(0);
-    skewed_pass(1, pb, pa);
+    skewed_pass(1, pb, pa, ((it + 1) & (SPI - 1)) == SPI - 1);
     fetched();
     __syncthreads();
   }
@@ -878,7 +968,7 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     }
     fetch_v(it + 1, (it + 1) & 1);
     __builtin_amdgcn_sched_barrier(0);
-    skewed_pass(it, pa, pb);
+    skewed_pass(it, pa, pb, (it & (SPI - 1)) == SPI - 1);
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
 #pragma unroll
@@ -896,8 +986,9 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     _Float16 const *vt = vbuf + (it & 1) * DV * NK;
 #pragma unroll
     for (int t = 0; t < DB; t++) {
-      pv_block(vt, t, pa);
+      pv_block(vt, t, pa, true);
     }
+    sum_mfma(pa, true);
     __syncthreads();
   }
 
@@ -923,12 +1014,14 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
       *reinterpret_cast<uint4v *>(og + (long long)rr * P.o.d_cols + cc) =
           *reinterpret_cast<uint4v const *>(ow + rr * LDO + cc);
     }
-    if (!HAS_DIV && g == 0) {
+    if (MSUM && c < 4) {
+      // every lane of a group holds the sums of rows 4g .. 4g + 3: lane c < 4 stores row 4g + c
       _Float16 *rgp = static_cast<_Float16 *>(const_cast<void *>(P.r.ptr)) +
                       tile_offset(P.r, bx, by, bz, 0);
 #pragma unroll
       for (int rp = 0; rp < RPW; rp++) {
-        rgp[(long long)(row_base + 16 * rp + c) * P.r.d_cols] = racc[rp];
+        _Float16 const v = c == 0 ? racc[rp][0] : (c == 1 ? racc[rp][MSUM ? 1 : 0] : (c == 2 ? racc[rp][MSUM ? 2 : 0] : racc[rp][MSUM ? 3 : 0]));
+        rgp[(long long)(row_base + 16 * rp + 4 * g + c) * P.r.d_cols] = v;
       }
     }
   }
@@ -1809,9 +1902,9 @@ int launch_shape(AttnParams const &A, bool has_div, bool cm, dim3 grid, int rg, 
                  : launch_waves<D, NK, DV, false, false>(A, grid, rg, ip, lds);
 }
 
-template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW, bool CM>
+template <int D, int NK, int DV, bool HAS_DIV, int RG, int RPW, bool CM, int SPI = 1>
 int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
-  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, RPW, CM>;
+  auto *fn = attn_stream_kernel<D, NK, DV, HAS_DIV, RG, RPW, CM, SPI>;
   if (lds > 65536) {
     MI355_HIP(hipFuncSetAttribute(reinterpret_cast<void const *>(fn),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -1822,7 +1915,18 @@ int launch_stream_one(AttnParams const &A, dim3 grid, int lds) {
 }
 
 template <int D, int NK, int DV, bool CM>
-int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds, bool wide = false) {
+int launch_stream(AttnParams const &A, bool has_div, dim3 grid, int rg, int lds, bool wide = false, int spi = 1) {
+  if (spi > 1) {  // wider key tiles: four wavefronts of 32 rows, the form without the division
+    if (has_div || rg != 4 || wide) {
+      return 0;
+    }
+    switch (spi) {
+      case 2: return launch_stream_one<D, NK, DV, false, 4, 2, CM, 2>(A, grid, lds);
+      case 4: return launch_stream_one<D, NK, DV, false, 4, 2, CM, 4>(A, grid, lds);
+      case 8: return launch_stream_one<D, NK, DV, false, 4, 2, CM, 8>(A, grid, lds);
+      default: return 0;
+    }
+  }
   if constexpr (D == 64) {
     if (wide) {  // four wavefronts of 64 rows
       return has_div ? launch_stream_one<D, NK, DV, true, 4, 4, CM>(A, grid, lds)
@@ -1942,11 +2046,57 @@ static bool choose_direct(DevProgram const &P, Match const &M, DirectShape &d, i
                     : launch_direct<false, false>(none, dim3(1, 1, 1), d, lds, true)) == 1;
 }
 
+// Whether (and in which shape) the throughput variant takes the plan: query tiles of whole
+// 64- or 128-row slabs, enough of them to fill the chip twice over, a for-loop long enough to
+// pipeline; key tiles of 64 keys, or (the form without the division, 128-row slabs) of 128 / 256 /
+// 512 keys walked as strips of 64.
+struct StreamShape {
+  int rgs = 0, spi = 1;
+  bool wide = false;
+};
+static bool choose_stream(DevProgram const &P, Match const &M, StreamShape &st) {
+  State &s = state();
+  st = StreamShape{};
+  if (s.attention_mode == 1 || s.attention_mode == 3) {
+    return false;
+  }
+  long long const blocks_all = (long long)P.grid[0] * P.grid[1] * P.grid[2];
+  int const slabs = M.m / 32;
+  st.rgs = (M.m % 128 == 0) ? 4 : ((M.m % 64 == 0) ? 2 : 0);
+  bool const heads = (M.D == 64 && M.DV == 64) || (M.D == 128 && M.DV == 128);
+  if (st.rgs == 0 || !heads) {
+    return false;
+  }
+  if (M.NK == 128 || M.NK == 256 || M.NK == 512) {
+    st.spi = M.NK / 64;
+    if (M.has_div || st.rgs != 4) {
+      return false;
+    }
+  } else if (M.NK != 64) {
+    return false;
+  }
+  if (s.attention_mode != 2 &&
+      !(P.forloop_range * st.spi >= 2 && blocks_all * (slabs / st.rgs) >= 512)) {
+    return false;
+  }
+  // Head size 64 with 256-row query tiles and enough of them for two wavefronts per SIMD:
+  // wavefronts of 64 rows (half the LDS operand reads per MFMA; at head size 64 the registers
+  // still fit two wavefronts per SIMD).  Measured on the 32-group x 16,384-key decode plan:
+  // 68.8 -> 67.0 us.
+  st.wide = st.spi == 1 && M.D == 64 && M.m % 256 == 0 &&
+            (s.attention_mode == 2 || blocks_all * (M.m / 64) >= 2048);
+  if (st.wide) {
+    st.rgs = 8;
+  }
+  return true;
+}
+
 bool attention_applicable(DevProgram const &P) {
   Match M;
   DirectShape d;
+  StreamShape st;
   int lds = 0;
-  if (match(P, M) && (shape_supported(M) || choose_direct(P, M, d, lds))) {
+  if (match(P, M) && (shape_supported(M) || choose_stream(P, M, st) || choose_direct(P, M, d, lds))) {
     return true;
   }
   DevProgram merged;
@@ -1963,8 +2113,10 @@ int try_launch_attention(DevProgram const &P0) {
   bool pieces = !match(P0, M);
   if (!pieces) {
     DirectShape probe;
+    StreamShape probe_stream;
     int probe_lds = 0;
-    pieces = !shape_supported(M) && !choose_direct(P0, M, probe, probe_lds);
+    pieces = !shape_supported(M) && !choose_stream(P0, M, probe_stream) &&
+             !choose_direct(P0, M, probe, probe_lds);
   }
   if (pieces) {
     if (!merge_column_pieces(P0, M, merged, r_copies, r_copy_stride)) {
@@ -1976,7 +2128,9 @@ int try_launch_attention(DevProgram const &P0) {
   DirectShape dshape;
   int direct_lds = 0;
   bool const direct = choose_direct(P, M, dshape, direct_lds);
-  if (!direct && (pieces || !shape_supported(M))) {
+  StreamShape stream_probe;
+  bool const stream = !pieces && choose_stream(P, M, stream_probe);
+  if (!direct && !stream && (pieces || !shape_supported(M))) {
     return 0;  // (only the direct-staging variant stores copies of the row sums)
   }
   State &s = state();
@@ -2010,35 +2164,14 @@ int try_launch_attention(DevProgram const &P0) {
       }
     }
   }
-  long long const blocks_all = (long long)P.grid[0] * P.grid[1] * P.grid[2];
-  // ---- throughput variant: enough independent 32-row wavefront slabs to fill the chip
-  // twice over, and a for-loop long enough to pipeline
+  // ---- throughput variant
   {
-    int const slabs = M.m / 32;
-    int rgs = (M.m % 128 == 0) ? 4 : ((M.m % 64 == 0) ? 2 : 0);
-    bool const shape = (M.D == 64 && M.NK == 64 && M.DV == 64) || (M.D == 128 && M.NK == 64 && M.DV == 128);
-    bool want = rgs != 0 && shape && P.forloop_range >= 2 && blocks_all * (slabs / rgs) >= 512 && !pieces;
-    // Head size 64 with 256-row query tiles and enough of them for two wavefronts per SIMD:
-    // wavefronts of 64 rows.  The transposing LDS operand reads are the largest share of a pass
-    // (every wavefront reads the whole K and V tile), and a 64-row wavefront reads half as
-    // much per MFMA; at head size 64 its registers still fit two wavefronts per SIMD.
-    bool wide = false;
-    if (s.attention_mode == 1 || s.attention_mode == 3) {
-      want = false;
-    } else if (s.attention_mode == 2) {
-      want = rgs != 0 && shape;
-    }
-    // (measured on the 32-group x 16,384-key decode plan: 68.8 -> 67.0 us; at head size 64 the
-    // exp / rounding work, not the LDS, is the larger share)
-    wide = want && M.D == 64 && M.m % 256 == 0 &&
-           (s.attention_mode == 2 || blocks_all * (M.m / 64) >= 2048);
-    if (wide) {
-      rgs = 8;
-    }
-    if (want) {
+    StreamShape st;
+    if (!pieces && choose_stream(P, M, st)) {
+      int const slabs = M.m / 32, rgs = st.rgs;
       A.split = slabs / rgs;
       A.stages = 2;
-      A.lds_stage_bytes = (M.NK * M.D + M.DV * M.NK) * 2;
+      A.lds_stage_bytes = (64 * M.D + M.DV * 64) * 2;  // one strip of 64 keys of K and of V
       int const out_bytes = rgs * 32 * (M.DV + 8) * 2;
       int lds = 2 * A.lds_stage_bytes;
       lds = lds > out_bytes ? lds : out_bytes;
@@ -2049,20 +2182,22 @@ int try_launch_attention(DevProgram const &P0) {
         }
         int rc;
         if (M.kv_colmajor) {
-          rc = M.D == 64 ? launch_stream<64, 64, 64, true>(A, M.has_div, grid, rgs, lds, wide)
-                         : launch_stream<128, 64, 128, true>(A, M.has_div, grid, rgs, lds);
+          rc = M.D == 64 ? launch_stream<64, 64, 64, true>(A, M.has_div, grid, rgs, lds, st.wide, st.spi)
+                         : launch_stream<128, 64, 128, true>(A, M.has_div, grid, rgs, lds, false, st.spi);
         } else {
-          rc = M.D == 64 ? launch_stream<64, 64, 64, false>(A, M.has_div, grid, rgs, lds, wide)
-                         : launch_stream<128, 64, 128, false>(A, M.has_div, grid, rgs, lds);
+          rc = M.D == 64 ? launch_stream<64, 64, 64, false>(A, M.has_div, grid, rgs, lds, st.wide, st.spi)
+                         : launch_stream<128, 64, 128, false>(A, M.has_div, grid, rgs, lds, false, st.spi);
         }
         if (rc == 1) {
           s.last().kernel_id = MI355_KERNEL_F16_ATTENTION;
           s.last().workgroups = grid.x * grid.y * grid.z;
-          s.last().threads = wide ? 256 : rgs * 64;
+          s.last().threads = st.wide ? 256 : rgs * 64;
           s.last().lds_bytes = lds;
           s.last().row_split = A.split;
         }
-        return rc;
+        if (rc != 0) {
+          return rc;
+        }
       }
     }
   }
@@ -2109,6 +2244,9 @@ int try_launch_attention(DevProgram const &P0) {
     }
   }
 
+  if (pieces || !shape_supported(M)) {
+    return 0;  // (a shape only the throughput variant is built for)
+  }
   // Row groups per workgroup: up to 4, fewer when that is what it takes to put a
   // workgroup on every compute unit.  Iteration lanes: whatever is left of 8
   // wavefronts, at most the for-loop range.

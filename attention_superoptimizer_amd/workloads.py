@@ -330,10 +330,20 @@ BASELINE_CONFIGS = {
     "C5a_gated_mlp": config5_gated_mlp,
 }
 
+def config3_mha_prefill_keys(keys_per_tile):
+    """Config C3 with the key range walked in tiles of `keys_per_tile` keys (for-loop
+    2048 / keys_per_tile): the same problem and plan shape, fewer and longer iterations, so the
+    numerator / denominator tiles are rounded to fp16 and accumulated less often."""
+    return lambda: config3_mha_prefill(F=2048 // keys_per_tile)
+
+
 # the same plans at other sizes (reported beside the baseline configurations, not instead)
 SCALED_CONFIGS = {
     "C2_gqa_decode_long": config2_gqa_decode_long,
     "gqa_inc_decode_long": gqa_inc_decode_long,
+    "C3_mha_prefill_keys128": config3_mha_prefill_keys(128),
+    "C3_mha_prefill_keys256": config3_mha_prefill_keys(256),
+    "C3_mha_prefill_keys512": config3_mha_prefill_keys(512),
 }
 
 # fp16 input distributions per config (std of N(0, std)), keyed by input op index
@@ -343,6 +353,9 @@ INPUT_STD = {
     "C2_gqa_decode_long": {0: 0.125, 1: 0.125, 2: 0.125},
     "gqa_inc_decode_long": {0: 0.125, 1: 0.125, 2: 0.125},
     "C3_mha_prefill": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
+    "C3_mha_prefill_keys128": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
+    "C3_mha_prefill_keys256": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
+    "C3_mha_prefill_keys512": {0: 128 ** -0.5, 1: 128 ** -0.5, 2: 128 ** -0.5},
     # the configurations leave X's distribution open; N(0, 0.25) keeps every partial
     # sum below 2, where one fp16 ulp is still under the 1e-3 absolute tolerance
     "C4_lora": {0: 0.25, 1: 0.02, 2: 0.02, 3: 0.02},
