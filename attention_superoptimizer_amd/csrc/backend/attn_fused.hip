@@ -2075,8 +2075,10 @@ static bool choose_stream(DevProgram const &P, Match const &M, StreamShape &st) 
   } else if (M.NK != 64) {
     return false;
   }
-  if (s.attention_mode != 2 &&
-      !(P.forloop_range * st.spi >= 2 && blocks_all * (slabs / st.rgs) >= 512)) {
+  // (64-key tiles on a small grid are better served by the latency variants; wider key tiles
+  // have no other kernel, so they take this one whatever the grid)
+  if (s.attention_mode != 2 && st.spi == 1 &&
+      !(P.forloop_range >= 2 && blocks_all * (slabs / st.rgs) >= 512)) {
     return false;
   }
   // Head size 64 with 256-row query tiles and enough of them for two wavefronts per SIMD:

@@ -176,18 +176,19 @@ __device__ __forceinline__ void store_weight(uint4v const (&x)[PPT][4], int R, i
 
 // Column-major weights (a [R][C] tile stored column by column: C rows of R contiguous halfs,
 // `ld` halfs apart) already have k contiguous: the same two halves without the transpose.
-// Patch p is four consecutive 16-byte chunks of dst[C][R] (R / 8 chunks per row).
+// The tile is dst[C][R], R / 8 chunks of 16 bytes per row; slot (i, j) of thread `tid` is chunk
+// (4 i + j) * nthreads + tid, so that the lanes of one load or store instruction walk
+// consecutive chunks of a row (whole cache lines per instruction).
 template <int PPT>
 __device__ __forceinline__ void load_weight_cm(_Float16 const *__restrict__ src, int ld, int R, int C,
                                                uint4v (&x)[PPT][4], int tid, int nthreads) {
-  int const cpr = R / 8, patches = C * cpr / 4;
+  int const cpr = R / 8, chunks = C * cpr;
 #pragma unroll
   for (int i = 0; i < PPT; i++) {
-    int p = tid + i * nthreads;
-    if (p < patches) {
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        int const q = 4 * p + j;
+    for (int j = 0; j < 4; j++) {
+      int const q = (4 * i + j) * nthreads + tid;
+      if (q < chunks) {
         x[i][j] = *reinterpret_cast<uint4v const *>(src + (long long)(q / cpr) * ld + 8 * (q % cpr));
       }
     }
@@ -197,15 +198,14 @@ __device__ __forceinline__ void load_weight_cm(_Float16 const *__restrict__ src,
 template <int PPT>
 __device__ __forceinline__ void store_weight_cm(uint4v const (&x)[PPT][4], int R, int C,
                                                 _Float16 *__restrict__ dst, int tid, int nthreads) {
-  int const cpr = R / 8, patches = C * cpr / 4;
+  int const cpr = R / 8, chunks = C * cpr;
   int const mask = (cpr - 1) & 7;
 #pragma unroll
   for (int i = 0; i < PPT; i++) {
-    int p = tid + i * nthreads;
-    if (p < patches) {
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        int const q = 4 * p + j;
+    for (int j = 0; j < 4; j++) {
+      int const q = (4 * i + j) * nthreads + tid;
+      if (q < chunks) {
         *reinterpret_cast<uint4v *>(dst + sw_chunk(q / cpr, q % cpr, R, mask)) = x[i][j];
       }
     }
@@ -1053,13 +1053,15 @@ int try_launch_lanes(DevProgram const &P, GMatch const &G, GemmParams const &A) 
   // every piece re-reads the activation rows, so the L2 -> L1 traffic is 4-5 x the bytes of the
   // plan (measured on the LoRA plan: 202 MB of requests for 34 MB), which is what bounds a plan
   // of tens of MB; the range-splitting kernel moves whole lines once.
-  // Column-major weights have neither cost (a piece's columns are whole lines of its own, read
-  // straight into registers), so the one launch also serves plans of tens of MB.
+  // With column-major weights a piece's columns are whole lines of its own, read straight into
+  // registers, so the first cost is gone; measured on the configurations of the benchmark the one
+  // launch then also wins for the two-weight plan (gated MLP, first half, 235 MB: 45.8 against
+  // 49.0 us) but not for the others (LoRA, 34 MB: 14.0 against 12.4 us; gated MLP, second half,
+  // 117 MB: 36.2 against 24.7 us), where each wavefront's loads of its activation rows and of the
+  // lora A tile outnumber its weight loads.
   long long const weight_bytes = blocks * F * (long long)(G.nb * G.KT * 64 + (G.lora ? G.KT * 16 : 0)) * 2;
-  if (s.gemm_mode == 0 && !G.wcm && (blocks * S > 1024 || weight_bytes > (8LL << 20))) {
-    return 0;
-  }
-  if (s.gemm_mode == 0 && G.wcm && (blocks * S > 4096 || weight_bytes > (64LL << 20))) {
+  bool const two_weights_cm = G.wcm && G.nb == 2 && blocks * S <= 4096;
+  if (s.gemm_mode == 0 && !two_weights_cm && (blocks * S > 1024 || weight_bytes > (8LL << 20))) {
     return 0;
   }
   int const strips = G.nb + (G.lora ? 1 : 0);

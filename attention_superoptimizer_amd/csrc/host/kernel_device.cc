@@ -110,7 +110,62 @@ struct RowMajorCopy {
     }
   }
 };
+// The result side of the same: an element-wise operator or reduction hands its output tensor
+// the layout of its first input (src/kernel/element_unary.cc:57, element_binary.cc:97,
+// reduction.cc:63), so the output of an operator on a column-major tensor is column-major too.
+// The kernel writes a row-major temporary; finish() stores it column by column.
+struct RowMajorResult {
+  void *ptr = nullptr;  // what the operator writes
+  DTensor const &out;
+  DTensor temp;
+  bool held = false;
+  explicit RowMajorResult(DTensor const &t) : ptr(t.data_ptr), out(t) {
+    if (!column_major(t)) {
+      return;
+    }
+    temp = t;
+    temp.layout = mirage::layout::DmemRowMajor;
+    DeviceMemoryManager::get_instance()->allocate(temp, false);
+    held = true;
+    ptr = temp.data_ptr;
+  }
+  RowMajorResult(RowMajorResult const &) = delete;
+  RowMajorResult &operator=(RowMajorResult const &) = delete;
+  void finish() {
+    if (held) {
+      int batch = 1;
+      for (int i = 0; i < out.num_dims - 2; i++) {
+        batch *= out.dim[i];
+      }
+      MI355_CALL(mi355_f16_transpose(temp.data_ptr, out.data_ptr, batch, out.dim[out.num_dims - 2],
+                                     out.dim[out.num_dims - 1]));
+    }
+  }
+  ~RowMajorResult() {
+    if (held) {
+      mi355_sync();
+      DeviceMemoryManager::get_instance()->free(temp);
+    }
+  }
+};
 }  // namespace
+
+// One run of an element-wise operator or reduction on row-major views of its tensors.
+template <typename Launch>
+static void on_row_major(std::vector<DTensor> const &inputs, DTensor const &output, Launch launch) {
+  // (temporaries are freed in reverse order of their allocation: the arena is a stack)
+  RowMajorCopy const a(inputs[0]);
+  if (inputs.size() > 1) {
+    RowMajorCopy const b(inputs[1]);
+    RowMajorResult o(output);
+    launch(a.ptr, b.ptr, o.ptr);
+    o.finish();
+  } else {
+    RowMajorResult o(output);
+    launch(a.ptr, nullptr, o.ptr);
+    o.finish();
+  }
+}
 
 bool KNMatmulOp::profile(ProfileResult &result) {
   require_device("KNMatmulOp::profile");
@@ -145,11 +200,11 @@ bool KNElementUnaryOp::profile(ProfileResult &result) {
   require_device("KNElementUnaryOp::profile");
   size_t const n = input_tensors[0].num_elements();
   int const iters = ProfileResult::NUM_ITERATIONS;
-  RowMajorCopy const in(input_tensors[0]);
-  MI355_CALL(mi355_f16_unary(op_type, in.ptr, output_tensors[0].data_ptr, n));
+  // (input and output share a layout and the operator is element-wise: flat in either order)
+  MI355_CALL(mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
   MI355_CALL(mi355_timer_start());
   for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_unary(op_type, in.ptr, output_tensors[0].data_ptr, n));
+    MI355_CALL(mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
   }
   float ms = 0.0f;
   MI355_CALL(mi355_timer_stop(&ms));
@@ -169,15 +224,15 @@ bool KNElementBinaryOp::profile(ProfileResult &result) {
   require_device("KNElementBinaryOp::profile");
   DTensor const &a = input_tensors[0], &b = input_tensors[1], &o = output_tensors[0];
   int const iters = 16;
-  RowMajorCopy const ra(a);
-  RowMajorCopy const rb(b);
-  MI355_CALL(mi355_f16_binary(op_type, ra.ptr, a.dim, rb.ptr, b.dim, o.data_ptr, o.dim, o.num_dims));
-  MI355_CALL(mi355_timer_start());
-  for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_binary(op_type, ra.ptr, a.dim, rb.ptr, b.dim, o.data_ptr, o.dim, o.num_dims));
-  }
   float ms = 0.0f;
-  MI355_CALL(mi355_timer_stop(&ms));
+  on_row_major(input_tensors, o, [&](void *pa, void *pb, void *po) {
+    MI355_CALL(mi355_f16_binary(op_type, pa, a.dim, pb, b.dim, po, o.dim, o.num_dims));
+    MI355_CALL(mi355_timer_start());
+    for (int i = 0; i < iters; i++) {
+      MI355_CALL(mi355_f16_binary(op_type, pa, a.dim, pb, b.dim, po, o.dim, o.num_dims));
+    }
+    MI355_CALL(mi355_timer_stop(&ms));
+  });
   result.run_time = ms / iters;
   return true;
 }
@@ -209,14 +264,15 @@ bool KNReductionOp::profile(ProfileResult &result) {
   reduction_strides(input_tensors[0], output_tensors[0], reduction_dim_idx, factor, is, os);
   size_t const n = output_tensors[0].num_elements();
   int const iters = ProfileResult::NUM_ITERATIONS;
-  RowMajorCopy const in(input_tensors[0]);
-  MI355_CALL(mi355_f16_reduce(in.ptr, output_tensors[0].data_ptr, n, factor, is, os));
-  MI355_CALL(mi355_timer_start());
-  for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_reduce(in.ptr, output_tensors[0].data_ptr, n, factor, is, os));
-  }
   float ms = 0.0f;
-  MI355_CALL(mi355_timer_stop(&ms));
+  on_row_major(input_tensors, output_tensors[0], [&](void *pi, void *, void *po) {
+    MI355_CALL(mi355_f16_reduce(pi, po, n, factor, is, os));
+    MI355_CALL(mi355_timer_start());
+    for (int i = 0; i < iters; i++) {
+      MI355_CALL(mi355_f16_reduce(pi, po, n, factor, is, os));
+    }
+    MI355_CALL(mi355_timer_stop(&ms));
+  });
   result.run_time = ms / iters;
   return true;
 }
@@ -452,14 +508,16 @@ void execute_once(KNOperator *op) {
     case KN_MATMUL_OP: {
       int batch, m, n, k;
       matmul_extents(op->input_tensors[0], op->input_tensors[1], batch, m, n, k);
-      MI355_CALL(mi355_f16_matmul(op->input_tensors[0].data_ptr, op->input_tensors[1].data_ptr,
-                                  op->output_tensors[0].data_ptr, batch, m, n, k));
+      MI355_CALL(mi355_f16_matmul_layout(op->input_tensors[0].data_ptr, op->input_tensors[1].data_ptr,
+                                         op->output_tensors[0].data_ptr, batch, m, n, k,
+                                         column_major(op->input_tensors[0]) ? 1 : 0,
+                                         column_major(op->input_tensors[1]) ? 1 : 0));
       break;
     }
     case KN_EXP_OP:
     case KN_SILU_OP:
-      MI355_CALL(mi355_f16_unary(op->op_type, op->input_tensors[0].data_ptr,
-                                 op->output_tensors[0].data_ptr,
+      // (input and output share a layout: flat in either storage order)
+      MI355_CALL(mi355_f16_unary(op->op_type, op->input_tensors[0].data_ptr, op->output_tensors[0].data_ptr,
                                  op->input_tensors[0].num_elements()));
       break;
     case KN_ADD_OP:
@@ -467,8 +525,9 @@ void execute_once(KNOperator *op) {
     case KN_DIV_OP: {
       DTensor const &a = op->input_tensors[0], &b = op->input_tensors[1],
                     &o = op->output_tensors[0];
-      MI355_CALL(mi355_f16_binary(op->op_type, a.data_ptr, a.dim, b.data_ptr, b.dim, o.data_ptr,
-                                  o.dim, o.num_dims));
+      on_row_major(op->input_tensors, o, [&](void *pa, void *pb, void *po) {
+        MI355_CALL(mi355_f16_binary(op->op_type, pa, a.dim, pb, b.dim, po, o.dim, o.num_dims));
+      });
       break;
     }
     case KN_REDUCTION_0_OP:
@@ -478,8 +537,9 @@ void execute_once(KNOperator *op) {
       int factor, is, os;
       reduction_strides(op->input_tensors[0], op->output_tensors[0], r->reduction_dim_idx,
                         factor, is, os);
-      MI355_CALL(mi355_f16_reduce(op->input_tensors[0].data_ptr, op->output_tensors[0].data_ptr,
-                                  op->output_tensors[0].num_elements(), factor, is, os));
+      on_row_major(op->input_tensors, op->output_tensors[0], [&](void *pi, void *, void *po) {
+        MI355_CALL(mi355_f16_reduce(pi, po, op->output_tensors[0].num_elements(), factor, is, os));
+      });
       break;
     }
     case KN_CUSTOMIZED_OP:

@@ -34,6 +34,13 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0
 HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "attn_direct_kernel_C2_gqa_decode.md")
 
 
+# One step of the headline measurement: this many back-to-back launches of the customized op
+# (the reference times an op over 1024 launches, customized_kernel.cu:631-648).  The wall clock
+# of a step therefore amortises the one synchronisation that ends the timed region over
+# thousands of launches, and `value` (microseconds per launch) does not depend on --steps.
+LAUNCHES_PER_STEP = 1024
+
+
 def headline_traffic_bytes():
     """HBM bytes per launch of the headline kernel from hardware counters (rocprofv3 --pmc
     FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain device
@@ -290,8 +297,11 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=1024)
-    ap.add_argument("--warmup", type=int, default=1024)
+    ap.add_argument("--steps", type=int, default=4,
+                    help="timed steps; one step = %d back-to-back launches of the headline op" % LAUNCHES_PER_STEP)
+    ap.add_argument("--warmup", type=int, default=1, help="untimed steps before them")
+    ap.add_argument("--launches-per-step", type=int, default=LAUNCHES_PER_STEP,
+                    help="launches that make one step (1 for a run under hardware counters)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fingerprints", action="store_true",
                     help="skip the batched candidate-verification throughput leg")
@@ -324,6 +334,7 @@ def main() -> int:
                     help="run 16 plain device copies of MIB MiB and exit: the known-size "
                          "traffic that hardware byte counters are scaled against")
     args = ap.parse_args()
+    per_step = max(1, args.launches_per_step)
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (a customized op's grid does not span "
               "devices); run with --gpus 1", file=sys.stderr)
@@ -350,7 +361,8 @@ def main() -> int:
 
     if args.fp_matmul:
         shape = tuple(int(x) for x in args.fp_matmul.split(","))
-        print(json.dumps(fp_matmul_rate(G, abi, shape, args.steps, args.warmup, True)), flush=True)
+        print(json.dumps(fp_matmul_rate(G, abi, shape, args.steps * per_step, args.warmup * per_step, True)),
+              flush=True)
         return 0
 
     if args.calibrate_copy:
@@ -421,7 +433,8 @@ def main() -> int:
             i_p = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(False) for a, b in op["in"]])
             o_p = (ctypes.c_void_p * 4)(*[t.device_ptr(False) for t in vals[i]])
             ms = ctypes.c_float()
-            assert abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, args.warmup, args.steps,
+            assert abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, args.warmup * per_step,
+                                                args.steps * per_step,
                                                 ctypes.byref(ms)) == 0, N.last_error()
             out[f"op{i}_us"] = round(ms.value * 1e3, 3)
         print(json.dumps({"config": args.only, **out}))
@@ -435,23 +448,23 @@ def main() -> int:
     outs = (ctypes.c_void_p * 4)(*[t.device_ptr(False) for t in vals[op_idx]])
     plan = g.lowered(op_idx, fingerprint=False)
 
+    # W untimed warm-up steps, then exactly K timed steps of LAUNCHES_PER_STEP launches each,
+    # bracketed by a synchronisation on both sides (host wall clock), with the launching queue's
+    # own events around the same launches (mean per launch: the kernel's duration)
     ms_ev = ctypes.c_float()
-    assert abi.mi355_sync() == 0
-    t0 = time.perf_counter()
-    rc = abi.mi355_customized_profile(ctypes.byref(plan), ins, outs, 0, args.warmup, 0 + args.steps,
-                                      ctypes.byref(ms_ev))
-    assert rc == 0, N.last_error()
-    assert abi.mi355_sync() == 0
-    t1 = time.perf_counter()
-    # wall clock over exactly K steps: a second, warm, timed-only pass
+    if args.warmup > 0:
+        rc = abi.mi355_customized_profile(ctypes.byref(plan), ins, outs, 0, 0,
+                                          args.warmup * per_step, ctypes.byref(ms_ev))
+        assert rc == 0, N.last_error()
     assert abi.mi355_sync() == 0
     w0 = time.perf_counter()
-    rc = abi.mi355_customized_profile(ctypes.byref(plan), ins, outs, 0, 0, args.steps,
+    rc = abi.mi355_customized_profile(ctypes.byref(plan), ins, outs, 0, 0, args.steps * per_step,
                                       ctypes.byref(ms_ev))
     assert rc == 0, N.last_error()
     assert abi.mi355_sync() == 0
     w1 = time.perf_counter()
-    ms_wall = (w1 - w0) * 1e3 / args.steps
+    ms_step = (w1 - w0) * 1e3 / args.steps
+    ms_wall = ms_step / per_step  # per launch
     ms_kernel = float(ms_ev.value)
     launch = N.Mi355LaunchInfo()
     abi.mi355_last_launch(ctypes.byref(launch))
@@ -468,7 +481,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_wall, 6),
+        "ms_per_step": round(ms_step, 6),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
@@ -476,8 +489,11 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": "C2 GQA incremental decode, one customized op: Q[2,256,64] K[2,64,4096] "
-                        "V[2,4096,64] fp16 N(0,1)/8, grid (2,16,1), forloop 4, "
-                        "matmul-exp-reduce-div-matmul, out [2,256,1024]",
+                        "V[2,4096,64] fp16 N(0,1)/8 (K and V DmemColumnMajor as the reference's plans "
+                        "declare them), grid (2,16,1), forloop 4, matmul-exp-reduce-div-matmul, "
+                        "out [2,256,1024]",
+            "launches_per_step": per_step,
+            "value_is": "host wall clock per launch over steps x launches_per_step back-to-back launches",
             "device": info.name.decode(), "arch": info.arch.decode(),
             "compute_units": info.compute_units,
             # the device's reported maximum engine clock, not the clock sustained under load
@@ -513,8 +529,9 @@ def main() -> int:
         # launch floor no longer dominates (32 groups x 16,384 keys), then the reference's
         # incremental-decode plan (8 query rows) over 268 MB of K and V -- more than the 256 MB
         # last-level cache holds, so its rate is an HBM rate
-        for name in ("C1_fused_matmul", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp",
-                     "C2_gqa_decode_long", "gqa_inc_decode_long"):
+        # (C3 also with its key range walked in tiles of 512 keys: same problem, for-loop 4)
+        for name in ("C1_fused_matmul", "C3_mha_prefill", "C3_mha_prefill_keys512", "C4_lora",
+                     "C5a_gated_mlp", "C2_gqa_decode_long", "gqa_inc_decode_long"):
             g.close()
             spec2, g, vals2 = setup(name)
             rec = {"config": name, "ops": []}
@@ -556,7 +573,14 @@ def main() -> int:
     if not args.headline_only and not args.no_fingerprints:
         g.close()
         result["fingerprint_throughput"] = fingerprint_throughput(G, not args.no_cpu_baseline)
-        result["fingerprint_matmul"] = [fp_matmul_rate(G, abi, sh, steps, 1024, False)
+        # the same 4096 candidates with every fingerprint matmul on packed 8-bit dot products
+        # on the vector ALUs (no matrix instruction anywhere in the fingerprint path)
+        assert abi.mi355_set_option(4, 1) == 0
+        vd = fingerprint_throughput(G, False, other_shapes=False)
+        assert abi.mi355_set_option(4, 0) == 0
+        result["fingerprint_throughput"]["vector_dot_route"] = {k: vd[k] for k in (
+            "candidates_per_s", "verify_s", "verdicts_as_constructed", "candidates_per_s_by_family")}
+        result["fingerprint_matmul"] = [fp_matmul_rate(G, abi, sh, steps, 1024, True)
                                         for sh, steps in (((1, 1024, 1024, 1024), 2048),
                                                           ((1, 4096, 4096, 4096), 256))]
         spec, g, vals = setup("C2_gqa_decode")
