@@ -177,6 +177,85 @@ def fp_matmul_rate(G, abi, shape, steps: int, warmup: int, both_routes: bool):
     return rec
 
 
+def kernel_level_ops(G, N, abi, W):
+    """The kernel-level fp16 operators (what the reference's KN*Op::profile run: a library GEMM,
+    element-wise kernels, a reduction; src/kernel/cuda/matmul_kernel.cu:28-143): one 4096^3 GEMM
+    in the layout the reference's plans declare (A row-major, B column-major) and with B
+    row-major (one extra launch transposes it), element-wise operators and a row reduction over
+    256 MB, and the un-fused graph of every benchmark configuration timed the way every
+    cpp_examples/*.cc times it first (sum over operators of KNOperator::profile)."""
+    rec = {}
+
+    def timed(call, iters):
+        for _ in range(max(2, iters // 8)):
+            assert call() == 0, N.last_error()
+        assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
+        for _ in range(iters):
+            assert call() == 0, N.last_error()
+        ms = ctypes.c_float()
+        assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
+        return ms.value * 1e3 / iters
+
+    n = 4096
+    g = G.KNGraph()
+    A, B, C = g.new_input((1, n, n)), g.new_input((1, n, n)), g.new_input((1, n, n))
+    for t, seed in ((A, 1), (B, 2)):
+        assert abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
+                                         ctypes.c_float(0.1), seed) == 0
+    pa, pb, pc = (ctypes.c_void_p(t.device_ptr(False)) for t in (A, B, C))
+    flops = 2.0 * n * n * n
+    rec["matmul_4096"] = {}
+    for name, b_cm in (("B_column_major", 1), ("B_row_major", 0)):
+        us = timed(lambda: abi.mi355_f16_matmul_layout(pa, pb, pc, 1, n, n, n, 0, b_cm), 256)
+        rec["matmul_4096"][name] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                                    "mfma_frac": round(flops / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+    g.close()
+    # element-wise over 128 Mi halfs: 256 MB read (512 MB for the binary operator) + 256 MB written
+    m = 128 << 20
+    g = G.KNGraph()
+    X, Y, Z = g.new_input((m,)), g.new_input((m,)), g.new_input((m,))
+    for t, seed in ((X, 3), (Y, 4)):
+        assert abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
+                                         ctypes.c_float(0.5), seed) == 0
+    px, py, pz = (ctypes.c_void_p(t.device_ptr(False)) for t in (X, Y, Z))
+    dims = (ctypes.c_int * 4)(m, 0, 0, 0)
+    rows = (ctypes.c_int * 4)(m // 4096, 4096, 0, 0)
+    ew = {}
+    us = timed(lambda: abi.mi355_f16_unary(1007, px, pz, m), 32)
+    ew["exp_256MB"] = {"us": round(us, 1), "GBps": round(4.0 * m / us / 1e3, 1)}
+    us = timed(lambda: abi.mi355_f16_binary(1008, px, dims, py, dims, pz, dims, 1), 32)
+    ew["add_256MB"] = {"us": round(us, 1), "GBps": round(6.0 * m / us / 1e3, 1)}
+    us = timed(lambda: abi.mi355_f16_reduce(px, pz, m // 4096, 4096, 4096, 1), 32)
+    ew["row_sums_256MB"] = {"us": round(us, 1), "GBps": round(2.0 * m / us / 1e3, 1)}
+    for v in ew.values():
+        v["hbm_frac"] = round(v["GBps"] / HBM_PEAK_GBS, 4)
+    rec["elementwise"] = ew
+    del rows
+    g.close()
+    # the un-fused graphs (the 128 MiB tensors above are released: the arena is a stack)
+    un = {}
+    for name, make in W.BASELINE_CONFIGS.items():
+        _, ref = make()
+        if ref is None:
+            from attention_superoptimizer_amd.workloads import attention_reference
+            ref = attention_reference([2, 256, 64], [2, 64, 4096], [2, 4096, 64]) if name == "C2_gqa_decode" else None
+        if ref is None:
+            continue
+        g2, vals2 = G.build_from_spec(ref)
+        for i, op in enumerate(ref):
+            if op["op"] == "input":
+                t = vals2[i][0]
+                assert abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
+                                                 ctypes.c_float(W.INPUT_STD[name].get(i, 0.1)), 0xC0FFEE00 + i) == 0
+        tot_ms, per_op = g2.profile_all()
+        un[name] = {"us": round(tot_ms * 1e3, 2),
+                    "ops_us": {f"{i}:{ref[i]['op']}": round(per_op[i] * 1e3, 2) for i in range(len(ref))
+                               if ref[i]["op"] != "input"}}
+        g2.close()
+    rec["unfused_graphs"] = un
+    return rec
+
+
 def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_problem: int = 64,
                            in_flight: int = 16, queues_per_submission: int = 1,
                            other_shapes: bool = True):
@@ -566,6 +645,10 @@ def main() -> int:
                         "mfma_frac": round(tot_flops / tot_us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)})
             others.append(rec)
         result["other_configs"] = others
+    if not args.headline_only:
+        g.close()
+        result["kernel_level_ops"] = kernel_level_ops(G, N, abi, W)
+        spec, g, vals = setup("C2_gqa_decode")
     if not args.headline_only and not args.no_recorded_programs:
         g.close()
         result["recorded_programs"] = recorded_programs(G, N, abi, not args.no_cpu_baseline)

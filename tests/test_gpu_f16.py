@@ -560,3 +560,81 @@ def test_full_size_configs_routes_agree(rt, abi):
             p = np.exp(s - s.max(axis=-1, keepdims=True))
             att = (p / p.sum(axis=-1, keepdims=True)) @ V
             assert_f16_close(outs["fused"][:4], att, rtol=1e-2, atol=2e-3, what="C3 vs softmax attention")
+
+
+# ---- kernel-level fp16 operators (the un-fused graphs every example of the reference times first) --
+def _abi_matmul(rt, abi, batch, m, n, k, a_cm, b_cm, seed):
+    """C = A . B through mi355_f16_matmul_layout on tensors of the arena; returns (A, B, C) as
+    logical arrays."""
+    from attention_superoptimizer_amd import graph as G
+    g = G.KNGraph()
+    try:
+        lay = {0: "DmemRowMajor", 1: "DmemColumnMajor"}
+        A = g.new_input((batch, m, k), layout=lay[a_cm])
+        B = g.new_input((batch, k, n), layout=lay[b_cm])
+        C = g.new_input((batch, m, n))
+        a, b = normal_f16([batch, m, k], 0.1, seed), normal_f16([batch, k, n], 0.1, seed + 1)
+        A.write_data(a)
+        B.write_data(b)
+        C.write_data(np.full((batch, m, n), np.nan, np.float16))
+        import ctypes
+        assert abi.mi355_f16_matmul_layout(ctypes.c_void_p(A.device_ptr(False)), ctypes.c_void_p(B.device_ptr(False)),
+                                           ctypes.c_void_p(C.device_ptr(False)), batch, m, n, k, a_cm, b_cm) == 0
+        assert abi.mi355_sync() == 0
+        return a, b, C.read_data()
+    finally:
+        g.close()
+
+
+@pytest.mark.parametrize("batch,m,n,k", [
+    (3, 70, 130, 96),      # streaming kernel, 128 x 128 tiles, ragged edges
+    (1, 33, 47, 50),       # k not a multiple of 8: the general-purpose kernel
+    (2, 257, 300, 64),     # n not a multiple of 8: masked scalar stores at the edge
+    (1, 16, 4096, 4096),   # the skinny product of the un-fused LoRA graph: k cut into ranges
+    (1, 16, 16, 4096),     # its rank-16 factor: one tile, sixteen ranges
+    (2, 256, 64, 4096),    # P . V of the un-fused decode graph: four tiles, long k
+    (1, 3600, 3700, 256),  # 256 x 256 tiles with ragged edges on both sides
+])
+def test_kernel_level_matmul_shapes_and_layouts(rt, abi, batch, m, n, k):
+    """mi355_f16_matmul_layout against fp32 numpy rounded once, every storage order of A and B."""
+    for a_cm, b_cm in ((0, 1), (0, 0), (1, 1), (1, 0)):
+        a, b, got = _abi_matmul(rt, abi, batch, m, n, k, a_cm, b_cm, 31)
+        want = orc.f16_matmul(a, b)
+        assert_f16_close(got, want, what=f"[{batch},{m},{k}] . [{batch},{k},{n}], A cm {a_cm}, B cm {b_cm}")
+
+
+def test_kernel_level_matmul_4096_cubed_by_samples_and_checksums(rt, abi):
+    """4096^3 (the size the streaming kernel is measured on): 4096 sampled elements against
+    float64 dot products at the fp16 tolerance, and every row / column sum of C against
+    A . (B . 1) and (1 . A) . B (a dropped or doubled k step, a misplaced tile or a wrong edge
+    shows in a sum even where no sample falls)."""
+    n = 4096
+    a, b, got = _abi_matmul(rt, abi, 1, n, n, n, 0, 1, 77)
+    a64, b64, c64 = a[0].astype(np.float64), b[0].astype(np.float64), got[0].astype(np.float64)
+    rng = np.random.default_rng(5)
+    ii, jj = rng.integers(0, n, 4096), rng.integers(0, n, 4096)
+    want = np.einsum("sk,ks->s", a64[ii], b64[:, jj])
+    assert_f16_close(got[0][ii, jj], want.astype(np.float16), what="4096^3 samples")
+    # sums of 4096 outputs each rounded to fp16 (|c| ~ 0.64, ulp ~ 5e-4): allow 4096 * 3e-4
+    assert np.abs(c64.sum(1) - a64 @ b64.sum(1)).max() < 1.3
+    assert np.abs(c64.sum(0) - a64.sum(0) @ b64).max() < 1.3
+
+
+def test_kernel_level_elementwise_and_reductions_large_and_ragged(rt):
+    """The vector paths (16 bytes per lane) and their scalar tails: large tensors, row lengths
+    that are not multiples of 8, one value per row as the second operand, sums along rows and
+    columns."""
+    for dims in ([4, 1000, 1024], [3, 70, 130], [2, 513, 1001]):
+        b, r, c = dims
+        spec = [
+            {"op": "input", "dims": dims}, {"op": "input", "dims": dims}, {"op": "input", "dims": [b, r, 1]},
+            {"op": "exp", "in": [[0, 0]]},
+            {"op": "silu", "in": [[1, 0]]},
+            {"op": "add", "in": [[3, 0], [4, 0]]},
+            {"op": "reduction", "in": [[3, 0]], "dim": 2, "size": 1},
+            {"op": "div", "in": [[3, 0], [6, 0]]},
+            {"op": "mul", "in": [[7, 0], [2, 0]]},
+            {"op": "reduction", "in": [[5, 0]], "dim": 1, "size": 1},
+            {"op": "reduction", "in": [[0, 0]], "dim": 0, "size": 1},
+        ]
+        _check(rt, spec, _inputs(spec, 0.5, seed=11), f"kernel ops {dims}")
