@@ -19,17 +19,27 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -ffp-contract=on: with the default (fast) the compiler may pair the terms of a short,
 # fully unrolled multiply-add chain into two-element dot products, which round differently
 # from the fp16 interpreter's chain; "on" keeps every fused multiply-add as written
+# -I include: a customized operator of one of the fused families (attention, skinny GEMM,
+# fold-and-divide) is emitted as an instantiation of that family's kernel from
+# include/mi355_kernels/*.h
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on",
+         "-I", os.path.join(os.path.dirname(HERE), "include"),
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-mllvm", "-amdgpu-mfma-vgpr-form",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
-# graphs whose programs the build generates and the GPU tests run
-EXAMPLES = ["C1_fused_matmul", "C2_gqa_decode", "C4_lora", "mlp"]
+# graphs whose programs the build generates and the GPU tests run; each in two forms: as the
+# backend itself would run it (fused-family kernels where one applies) and, under the name
+# with INTERPRETER_SUFFIX, every customized operator as the specialised interpreter
+EXAMPLES = ["C1_fused_matmul", "C2_gqa_decode", "C3_mha_prefill", "C4_lora", "C5a_gated_mlp", "mlp"]
+INTERPRETER_SUFFIX = "_interp"
+OPT_FORCE_INTERPRETER = 1
 
 
 def example_spec(name: str) -> List[dict]:
     from . import workloads as W
+    if name.endswith(INTERPRETER_SUFFIX):
+        name = name[:-len(INTERPRETER_SUFFIX)]
     if name in W.BASELINE_CONFIGS:
         return W.BASELINE_CONFIGS[name]()[0]
     return W.REFERENCE_EXAMPLES[name][0]
@@ -49,14 +59,19 @@ def program_path(name: str) -> str:
 
 def generate(name: str) -> str:
     """Builds the example graph through the host API and writes its HIP program."""
+    from . import _native as N
     from . import graph as G
     G.set_smem_budget(1 << 20)
     os.makedirs(GENERATED, exist_ok=True)
+    forced = 1 if name.endswith(INTERPRETER_SUFFIX) else 0
+    if N.backend().mi355_set_option(OPT_FORCE_INTERPRETER, forced) != 0:
+        raise RuntimeError("mi355_set_option failed")
     g, _ = G.build_from_spec(example_spec(name))
     try:
         g.generate_hip_program(source_path(name))
     finally:
         g.close()
+        N.backend().mi355_set_option(OPT_FORCE_INTERPRETER, 0)
     return source_path(name)
 
 
@@ -70,7 +85,7 @@ def compile_program(src: str, out: str) -> None:
 
 
 def build_examples() -> None:
-    for name in EXAMPLES:
+    for name in EXAMPLES + [e + INTERPRETER_SUFFIX for e in EXAMPLES]:
         src = generate(name)
         compile_library(src, library_path(name))
         compile_program(src, program_path(name))

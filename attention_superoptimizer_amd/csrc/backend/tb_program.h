@@ -159,6 +159,29 @@ inline long long fp_program_blocks(DevProgram const &p) {
   return (long long)(p.grid[0] / gx) * p.splits * (p.grid[1] / gy) * p.grid[2];
 }
 
+// ---- source emission of the fused families (emit_hip.cc) ---------------------------------------
+// While a sink is installed on the calling thread, try_launch_attention / _gemm / _combine go
+// through their whole choice of kernel and launch shape and then PRINT the launches they would
+// make -- the kernel template with its literal arguments, grid, LDS and the parameter block
+// with literal values, as statements of a C++ function body -- instead of making them.  The
+// printed code names the kernels of include/mi355_kernels/*.h.  Device pointers bound to the
+// program while printing are tags that print as `in[i]`, `out[i]` or `scratch`.
+struct EmitSink {
+  std::string text;          // statements of the launcher body
+  unsigned headers = 0;      // bit 0: attention.h, bit 1: gemm.h, bit 2: combine.h
+  size_t scratch_bytes = 0;  // workspace the printed launches share (0: none)
+};
+EmitSink *&emit_sink();
+constexpr uintptr_t kEmitInBase = 0x100000, kEmitOutBase = 0x200000, kEmitScratch = 0x300000, kEmitStep = 0x1000;
+constexpr size_t kEmitScratchBytes = (size_t)64 << 20;  // what a printed program may ask for
+inline void *emit_in_tag(int i) { return reinterpret_cast<void *>(kEmitInBase + kEmitStep * (uintptr_t)i); }
+inline void *emit_out_tag(int i) { return reinterpret_cast<void *>(kEmitOutBase + kEmitStep * (uintptr_t)i); }
+std::string emit_pointer(void const *p);  // "in[2]", "out[0]", "scratch", "nullptr"
+std::string emit_fmt(char const *f, ...);
+// One printed launch: `params` declares the parameter block `P`.
+void emit_launch(EmitSink &sink, char const *kernel, std::string const &template_args, dim3 grid, int threads,
+                 int lds, std::string const &params);
+
 // `declared_layouts`: fp16 loader tiles take the LDS layout the plan declares for them
 // (see MI355_OPT_PLAN_SMEM_LAYOUT) instead of the one their consumers want.
 int compile_plan(mi355_plan const &plan, bool f16, int max_lds, DevProgram &prog,
