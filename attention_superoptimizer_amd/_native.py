@@ -131,11 +131,12 @@ ABI = {
 
 class MirageLayoutStats(ctypes.Structure):
     _fields_ = [("assignments", ctypes.c_longlong), ("measurements", ctypes.c_longlong),
+                ("unrunnable", ctypes.c_longlong),
                 ("truncated", ctypes.c_int), ("first_ms", ctypes.c_float),
                 ("best_ms", ctypes.c_float), ("worst_ms", ctypes.c_float)]
 
 
-# float cost(void *user, int op_index, int const *loader_layouts, int n)
+# float cost(void *user, int op_index, int const *layouts, int n)
 LAYOUT_COST_FN = ctypes.CFUNCTYPE(ctypes.c_float, ctypes.c_void_p, ctypes.c_int,
                                   ctypes.POINTER(ctypes.c_int), ctypes.c_int)
 

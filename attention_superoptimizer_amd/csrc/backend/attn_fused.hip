@@ -102,7 +102,7 @@ struct Match {
 
 // `pieces`: the value tile may be narrower than 16 bytes (checked by merge_column_pieces)
 bool match(DevProgram const &P, Match &M, bool pieces = false) {
-  if (P.num_ops < 9 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
+  if (has_column_major_saver(P) || P.num_ops < 9 || P.ops[0].kind != DOP_LOAD || P.ops[1].kind != DOP_LOAD ||
       P.ops[2].kind != DOP_LOAD || P.ops[3].kind != DOP_MATMUL) {
     return false;
   }

@@ -58,7 +58,11 @@ bool aligned(CTile const &t, int vec) {
 }
 
 bool cmatch(DevProgram const &P, CMatch &M) {
-  // (both inputs are read as row-major matrices: a column-major one takes the interpreter)
+  // (inputs are read and the result stored as row-major matrices: a column-major one takes
+  // the interpreter)
+  if (has_column_major_saver(P)) {
+    return false;
+  }
   for (int o = 0; o < P.num_ops && P.ops[o].kind == DOP_LOAD; o++) {
     if (P.ops[o].sub == 1) {
       return false;

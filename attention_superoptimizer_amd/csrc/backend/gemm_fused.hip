@@ -118,6 +118,9 @@ int loader_of(DevProgram const &P, int nloads, int tensor) {
 }
 
 bool gmatch(DevProgram const &P, GMatch &G) {
+  if (has_column_major_saver(P)) {
+    return false;
+  }
   int nl = 0;
   while (nl < P.num_ops && P.ops[nl].kind == DOP_LOAD) {
     nl++;

@@ -217,8 +217,12 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
         return MI355_ERR_INVALID;
       }
       d.dst = define(q[16], rows, cols, o);
+      // a DmemColumnMajor result is stored column by column, as the reference's fp16 saver does
+      // (include/mirage/threadblock/cuda/output_saver.h:252-290); element by element here
+      bool const colmajor = f16 && q[13] == kDmemColumnMajor;
+      d.sub = colmajor ? 1 : 0;
       long long max_row = rows - 1, max_col = cols - 1, max_g = 0;
-      bool al = cols % 8 == 0 && d.d_cols % 8 == 0;
+      bool al = !colmajor && cols % 8 == 0 && d.d_cols % 8 == 0;
       for (int g = 0; g < 3; g++) {
         long long b = plan.grid_dim[g] - 1;
         if (d.row_bs[g] < 0 || d.col_bs[g] < 0 || d.g_bs[g] < 0) {
@@ -236,7 +240,8 @@ static int compile_plan_padded(mi355_plan const &plan, bool f16, int pad, int ma
       }
       d.vec8 = al ? 1 : 0;
       d.galign = d.vec8;
-      ext.out_elems[d.io] = max_g + max_row * d.d_cols + max_col + 1;
+      ext.out_elems[d.io] = colmajor ? max_g + max_col * d.d_rows + max_row + 1
+                                     : max_g + max_row * d.d_cols + max_col + 1;
     } else if (t == TB_MATMUL_OP) {
       if (!need(6)) {
         err = "matmul truncated";

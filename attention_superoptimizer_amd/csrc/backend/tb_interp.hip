@@ -1041,7 +1041,9 @@ __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram c
             }
             _Float16 h = static_cast<_Float16>(v);
             if (last) {
-              g[(long long)(org.row0 + r) * op.d_cols + org.col0 + c] = h;
+              // (op.sub == 1: a column-major device tensor, element (r, c) at c * d_rows + r)
+              g[op.sub == 1 ? (long long)(org.col0 + c) * op.d_rows + org.row0 + r
+                            : (long long)(org.row0 + r) * op.d_cols + org.col0 + c] = h;
             } else {
               acc[r * ta.rs + c * ta.cs] = h;
             }

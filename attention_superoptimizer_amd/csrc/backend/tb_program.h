@@ -43,7 +43,7 @@ inline uint32_t fast_div_magic(int d) {
 
 struct DevOp {
   int kind;
-  int sub;             // UNARY / BINARY: the TB_* operator code; LOAD (fp16): 1 = the device tensor
+  int sub;             // UNARY / BINARY: the TB_* operator code; LOAD / OUTPUT (fp16): 1 = the device tensor
                        // is DmemColumnMajor, element (r, c) of its [d_rows, d_cols] matrix at
                        // c * d_rows + r (fingerprint tensors are always row-major)
   int src0, src1, dst; // tensor ids (-1 when unused)
@@ -166,6 +166,17 @@ inline long long fp_program_blocks(DevProgram const &p) {
 // with literal values, as statements of a C++ function body -- instead of making them.  The
 // printed code names the kernels of include/mi355_kernels/*.h.  Device pointers bound to the
 // program while printing are tags that print as `in[i]`, `out[i]` or `scratch`.
+// True when a saver of `P` writes a column-major device tensor: the fused kernels store rows,
+// such a program runs on the interpreter.
+inline bool has_column_major_saver(DevProgram const &P) {
+  for (int o = 0; o < P.num_ops; o++) {
+    if (P.ops[o].kind == DOP_OUTPUT && P.ops[o].sub == 1) {
+      return true;
+    }
+  }
+  return false;
+}
+
 struct EmitSink {
   std::string text;          // statements of the launcher body
   unsigned headers = 0;      // bit 0: attention.h, bit 1: gemm.h, bit 2: combine.h

@@ -196,15 +196,28 @@ bool KNMatmulOp::fingerprint(void) {
 }
 
 // ---- element-wise unary (reference src/kernel/cuda/element_unary_kernel.cu:44-112) -------
+// Element-wise, so flat in either storage order while input and output share a layout (what the
+// operator's constructor sets up); a layout search may declare them differently, and then the
+// result is stored in the order its tensor declares.
+static void run_unary(mirage::type::KNOperatorType type, std::vector<DTensor> const &inputs,
+                      DTensor const &output, size_t n) {
+  if (column_major(inputs[0]) == column_major(output)) {
+    MI355_CALL(mi355_f16_unary(type, inputs[0].data_ptr, output.data_ptr, n));
+    return;
+  }
+  on_row_major(inputs, output,
+               [&](void *pa, void *, void *po) { MI355_CALL(mi355_f16_unary(type, pa, po, n)); });
+}
+
 bool KNElementUnaryOp::profile(ProfileResult &result) {
   require_device("KNElementUnaryOp::profile");
   size_t const n = input_tensors[0].num_elements();
   int const iters = ProfileResult::NUM_ITERATIONS;
-  // (input and output share a layout and the operator is element-wise: flat in either order)
-  MI355_CALL(mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
+  auto once = [&]() { run_unary(op_type, input_tensors, output_tensors[0], n); };
+  once();
   MI355_CALL(mi355_timer_start());
   for (int i = 0; i < iters; i++) {
-    MI355_CALL(mi355_f16_unary(op_type, input_tensors[0].data_ptr, output_tensors[0].data_ptr, n));
+    once();
   }
   float ms = 0.0f;
   MI355_CALL(mi355_timer_stop(&ms));
@@ -359,9 +372,15 @@ bool KNCustomizedOp::profile(ProfileResult &result) {
   require_device("KNCustomizedOp::profile");
   LoweredOp l = lower(*this, false);
   float ms = 0.0f;
-  MI355_CALL(mi355_customized_profile(&l.plan, l.inputs, l.outputs, 0,
-                                      ProfileResult::NUM_WARPUP_ITERATIONS,
-                                      ProfileResult::NUM_ITERATIONS, &ms));
+  int const rc = mi355_customized_profile(&l.plan, l.inputs, l.outputs, 0, ProfileResult::NUM_WARPUP_ITERATIONS,
+                                          ProfileResult::NUM_ITERATIONS, &ms);
+  if (rc == MI355_ERR_UNSUPPORTED) {
+    // no kernel of this backend runs the program as declared (say, tiles that only a fused
+    // kernel keeps out of LDS, under layouts the fused kernels do not take): not a candidate
+    result = ProfileResult::infinity();
+    return false;
+  }
+  MIRAGE_CHECK(rc == MI355_OK, mi355_last_error());
   result.run_time = ms;
   return true;
 }
@@ -516,9 +535,7 @@ void execute_once(KNOperator *op) {
     }
     case KN_EXP_OP:
     case KN_SILU_OP:
-      // (input and output share a layout: flat in either storage order)
-      MI355_CALL(mi355_f16_unary(op->op_type, op->input_tensors[0].data_ptr, op->output_tensors[0].data_ptr,
-                                 op->input_tensors[0].num_elements()));
+      run_unary(op->op_type, op->input_tensors, op->output_tensors[0], op->input_tensors[0].num_elements());
       break;
     case KN_ADD_OP:
     case KN_MUL_OP:

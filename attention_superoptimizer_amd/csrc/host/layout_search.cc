@@ -79,14 +79,46 @@ std::vector<SmemLayout> get_valid_output_layout(TBOperator const *op, int idx) {
   }
 }
 
+// What the cost of `op` may depend on: the layouts of the device tensors it reads, of those it
+// writes (an input operator only publishes its tensor: none) and, for a customized operator,
+// of its loaders' tiles.
+std::vector<int> cost_layouts(KNOperator const *op) {
+  std::vector<int> key;
+  if (op->op_type == KN_INPUT_OP) {
+    return key;
+  }
+  for (DTensor const &t : op->input_tensors) {
+    key.push_back((int)t.layout);
+  }
+  for (DTensor const &t : op->output_tensors) {
+    key.push_back((int)t.layout);
+  }
+  if (op->op_type == KN_CUSTOMIZED_OP) {
+    auto const *c = static_cast<KNCustomizedOp const *>(op);
+    for (TBOperator *bop : c->bgraph.operators) {
+      if (bop->op_type == TB_INPUT_OP) {
+        key.push_back((int)bop->output_tensors[0].layout);
+      }
+    }
+  }
+  return key;
+}
+
 namespace {
+
+// cost of an operator whose profile() reports that nothing runs it
+constexpr float kUnrunnable = -1.0f;
 
 struct Searcher {
   mirage::kernel::Graph &g;
   LayoutSearchConfig const &cfg;
   LayoutSearchResult res;
-  std::map<std::pair<int, std::vector<int>>, float> known;  // (operator, loader layouts) -> ms
-  std::map<int, float> fused_cost;  // operators that took a fused kernel: their (only) time
+  // (operator, layouts its time depends on) -> ms.  The layouts: those of the device tensors
+  // it reads and writes, then those of its loaders' tiles.
+  std::map<std::pair<int, std::vector<int>>, float> known;
+  // Customized operators that took a fused kernel under given device-tensor layouts: the
+  // kernel stages operands its own way, so the tiles' layouts cannot change that time.
+  std::map<std::pair<int, std::vector<int>>, float> fused_cost;
   std::vector<int> best;                                    // snapshot of every layout
   bool have_best = false;
 
@@ -119,6 +151,23 @@ struct Searcher {
           in.layout = l;
         }
       }
+      // the loaders and savers of a customized operator keep their own copies of the device
+      // tensors; the lowered program takes the layouts from those
+      if (op->op_type == KN_CUSTOMIZED_OP) {
+        for (TBOperator *bop : static_cast<KNCustomizedOp *>(op)->bgraph.operators) {
+          if (bop->op_type == TB_INPUT_OP) {
+            auto *in = static_cast<mirage::threadblock::TBInputOp *>(bop);
+            if (in->dtensor.guid == t.guid) {
+              in->dtensor.layout = l;
+            }
+          } else if (bop->op_type == TB_OUTPUT_OP) {
+            auto *out = static_cast<mirage::threadblock::TBOutputOp *>(bop);
+            if (out->dtensor.guid == t.guid) {
+              out->dtensor.layout = l;
+            }
+          }
+        }
+      }
     }
   }
 
@@ -136,22 +185,18 @@ struct Searcher {
 
   float op_cost(int op_idx) {
     KNOperator *op = g.operators[op_idx];
-    std::vector<int> key;
-    if (op->op_type == KN_CUSTOMIZED_OP) {
-      auto *c = static_cast<KNCustomizedOp *>(op);
-      for (TBOperator *bop : c->bgraph.operators) {
-        if (bop->op_type == TB_INPUT_OP) {
-          key.push_back((int)bop->output_tensors[0].layout);
-        }
-      }
-    }
+    std::vector<int> key = cost_layouts(op);
     auto it = known.find({op_idx, key});
     if (it != known.end()) {
       return it->second;
     }
-    // an operator that ran on a fused kernel keeps its tiles in registers / its own LDS
-    // layout: no declared layout can change its time, one measurement stands for all
-    auto fl = fused_cost.find(op_idx);
+    std::vector<int> device_key;
+    for (int l : key) {
+      if (l < (int)SmemRowMajor) {
+        device_key.push_back(l);
+      }
+    }
+    auto fl = fused_cost.find({op_idx, device_key});
     if (fl != fused_cost.end()) {
       return fl->second;
     }
@@ -160,12 +205,12 @@ struct Searcher {
       ms = cfg.cost(op);
     } else {
       ProfileResult r;
-      op->profile(r);
-      ms = r.run_time;
+      bool const ran = op->profile(r);
+      ms = ran ? r.run_time : kUnrunnable;
       mi355_launch_info li{};
-      if (op->op_type == KN_CUSTOMIZED_OP && mi355_last_launch(&li) == MI355_OK &&
+      if (ran && op->op_type == KN_CUSTOMIZED_OP && mi355_last_launch(&li) == MI355_OK &&
           li.kernel_id != MI355_KERNEL_F16_INTERP) {
-        fused_cost[op_idx] = ms;
+        fused_cost[{op_idx, device_key}] = ms;
       }
     }
     res.measurements++;
@@ -180,13 +225,21 @@ struct Searcher {
       return;
     }
     float total = 0.0f;
+    bool runnable = true;
     for (int i = 0; i < (int)g.operators.size(); i++) {
-      total += op_cost(i);
-    }
-    if (res.assignments == 0) {
-      res.first_run_time = res.worst_run_time = total;
+      float const ms = op_cost(i);
+      runnable = runnable && ms != kUnrunnable;
+      total += ms;
     }
     res.assignments++;
+    if (!runnable) {
+      // an operator no kernel of the backend runs under these layouts: not a candidate
+      res.unrunnable++;
+      return;
+    }
+    if (!have_best) {
+      res.first_run_time = res.worst_run_time = total;
+    }
     res.worst_run_time = total > res.worst_run_time ? total : res.worst_run_time;
     if (!have_best || total < res.best_run_time) {
       have_best = true;
@@ -300,13 +353,16 @@ extern "C" {
 struct mirage_layout_stats {
   long long assignments;
   long long measurements;
+  long long unrunnable;
   int truncated;
   float first_ms, best_ms, worst_ms;
 };
 
-// cost(user, operator index, layouts of the operator's loader tiles, their count) in ms;
-// NULL measures with KNOperator::profile.
-typedef float (*mirage_layout_cost_fn)(void *user, int op_index, int const *loader_layouts, int n);
+// cost(user, operator index, the layouts the operator's cost may depend on, their count) in
+// ms; NULL measures with KNOperator::profile.  The layouts: those of the device tensors the
+// operator reads, then of those it writes (DmemLayout values), then of its loaders' tiles
+// (SmemLayout values); none for an input operator.
+typedef float (*mirage_layout_cost_fn)(void *user, int op_index, int const *layouts, int n);
 
 int mirage_optimize_layout(void *graph, long long max_assignments, mirage_layout_cost_fn cost,
                            void *user, mirage_layout_stats *out) {
@@ -321,16 +377,8 @@ int mirage_optimize_layout(void *graph, long long max_assignments, mirage_layout
       while (G.operators[index] != op) {
         index++;
       }
-      std::vector<int> loaders;
-      if (op->op_type == mirage::type::KN_CUSTOMIZED_OP) {
-        auto *c = static_cast<mirage::kernel::KNCustomizedOp *>(op);
-        for (mirage::threadblock::TBOperator *bop : c->bgraph.operators) {
-          if (bop->op_type == mirage::type::TB_INPUT_OP) {
-            loaders.push_back((int)bop->output_tensors[0].layout);
-          }
-        }
-      }
-      return cost(user, index, loaders.data(), (int)loaders.size());
+      std::vector<int> const layouts = mirage::search::cost_layouts(op);
+      return cost(user, index, layouts.data(), (int)layouts.size());
     };
   }
   mirage::search::LayoutSearchResult r;
@@ -338,6 +386,7 @@ int mirage_optimize_layout(void *graph, long long max_assignments, mirage_layout
   if (out != nullptr) {
     out->assignments = r.assignments;
     out->measurements = r.measurements;
+    out->unrunnable = r.unrunnable;
     out->truncated = r.truncated ? 1 : 0;
     out->first_ms = r.first_run_time;
     out->best_ms = r.best_run_time;

@@ -62,7 +62,16 @@ class DTensor:
         guid = ctypes.c_longlong()
         N.runtime().mirage_tensor_info(self._h, nd, dims, dt, lay, guid)
         self.dims = tuple(dims[i] for i in range(nd.value))
-        self.data_type, self.layout, self.guid = dt.value, lay.value, guid.value
+        self.data_type, self.guid = dt.value, guid.value
+
+    @property
+    def layout(self) -> int:
+        """The tensor's DmemLayout now (a layout search may have changed it)."""
+        nd, dt, lay = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        dims = (ctypes.c_int * 4)()
+        guid = ctypes.c_longlong()
+        N.runtime().mirage_tensor_info(self._h, nd, dims, dt, lay, guid)
+        return lay.value
 
     @property
     def num_elements(self) -> int:
@@ -340,8 +349,11 @@ def optimize_layout(graph: "KNGraph", cost=None, max_assignments: int = 0) -> di
     """KernelGraphGenerator::optimize_layout (reference src/search/search.cc:699-777):
     enumerates the layouts of every kernel-level output tensor and of every tile inside
     the customized operators, costs each complete assignment and leaves `graph` under the
-    cheapest one.  `cost(op_index, loader_layouts) -> ms` replaces the measurement by
-    KNOperator::profile (which needs the device)."""
+    cheapest one.  `cost(op_index, layouts) -> ms` replaces the measurement by
+    KNOperator::profile (which needs the device); `layouts` are the ones the operator's cost
+    may depend on: DmemLayout values of the device tensors it reads, then of those it writes,
+    then SmemLayout values of its loaders' tiles (none for an input operator).  Device tensors
+    whose layout changed hold their old contents in the old order: write their data again."""
     st = N.MirageLayoutStats()
     if cost is None:
         cb = N.LAYOUT_COST_FN()
@@ -350,7 +362,7 @@ def optimize_layout(graph: "KNGraph", cost=None, max_assignments: int = 0) -> di
     rc = N.runtime().mirage_optimize_layout(graph._g, max_assignments, cb, None, ctypes.byref(st))
     assert rc == 0
     return {"assignments": st.assignments, "measurements": st.measurements,
-            "truncated": bool(st.truncated), "first_ms": st.first_ms, "best_ms": st.best_ms,
+            "unrunnable": st.unrunnable, "truncated": bool(st.truncated), "first_ms": st.first_ms, "best_ms": st.best_ms,
             "worst_ms": st.worst_ms}
 
 

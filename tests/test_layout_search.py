@@ -18,6 +18,14 @@ NAMES = {ROW: "SmemRowMajor", COL: "SmemColumnMajor",
          COL64: "SmemColumnMajorTensorOpMultiplicand_Crosswise64"}
 
 
+DROW, DCOL = 100, 101
+
+
+def _split(layouts):
+    """(device-tensor layouts, loader tile layouts) of a cost callback's list."""
+    return tuple(l for l in layouts if l < 200), tuple(l for l in layouts if l >= 200)
+
+
 def _matmul_graph():
     spec, _ = W.BASELINE_CONFIGS["C1_fused_matmul"]()
     return G.build_from_spec(spec)[0]
@@ -33,13 +41,14 @@ def test_matmul_plan_enumeration_matches_an_independent_count():
     """A . B as one customized op: device tensors A, B, C take 2 layouts each; the loaders'
     tiles 6 each, of which the matmul admits 3 pairs; its result 6, of which the saver
     admits the 3 row-major ones.  2^3 * 3 * 3 = 72 complete assignments, and the operator
-    is costed once per distinct pair of loader layouts."""
+    is costed once per distinct set of layouts its time can depend on: those of A, B and C
+    and the pair of loader layouts (an input operator's cost depends on none)."""
     g = _matmul_graph()
     try:
         seen = []
 
-        def cost(op, loaders):
-            seen.append((op, tuple(loaders)))
+        def cost(op, layouts):
+            seen.append((op, tuple(layouts)))
             return 1.0
 
         st = G.optimize_layout(g, cost)
@@ -49,9 +58,11 @@ def test_matmul_plan_enumeration_matches_an_independent_count():
                 brute += 1
         assert st["assignments"] == 8 * brute == 72
         assert not st["truncated"]
-        # inputs A and B once each, the customized op once per admissible pair
-        assert sorted(seen) == sorted([(0, ()), (1, ())] + [(2, p) for p in MATMUL_PAIRS])
-        assert st["measurements"] == len(seen) == 5
+        # inputs A and B once each, the customized op once per (A, B, C, admissible pair)
+        want = [(0, ()), (1, ())] + [(2, d + p) for d in itertools.product((DROW, DCOL), repeat=3)
+                                     for p in MATMUL_PAIRS]
+        assert sorted(seen) == sorted(want)
+        assert st["measurements"] == len(seen) == 26 and st["unrunnable"] == 0
     finally:
         g.close()
 
@@ -61,14 +72,23 @@ def test_the_cheapest_assignment_is_left_on_the_graph():
     try:
         want = (ROW64, COL64)
 
-        def cost(op, loaders):
+        def cost(op, layouts):
             if op != 2:
                 return 0.0
-            return 1.0 if tuple(loaders) == want else 3.0
+            device, loaders = _split(layouts)
+            # B column-major is worth one unit, the right pair of tile layouts two
+            return 4.0 - (1.0 if device == (DROW, DCOL, DROW) else 0.0) - (2.0 if loaders == want else 0.0)
 
         st = G.optimize_layout(g, cost)
-        assert st["best_ms"] == 1.0 and st["worst_ms"] == 3.0
+        assert st["best_ms"] == 1.0 and st["worst_ms"] == 4.0
         assert _loader_layouts(g, 2) == [NAMES[l] for l in want]
+        # the device tensors carry the chosen layouts, and so do the copies the customized
+        # operator, its loaders and its saver hold
+        ops = json.loads(g.to_json())
+        assert [o["output_tensors"][0]["layout"] for o in ops] == ["DmemRowMajor", "DmemColumnMajor", "DmemRowMajor"]
+        assert [t["layout"] for t in ops[2]["input_tensors"]] == ["DmemRowMajor", "DmemColumnMajor"]
+        held = [o["dtensor"]["layout"] for o in ops[2]["bgraph"]["operators"] if "dtensor" in o]
+        assert held == ["DmemRowMajor", "DmemColumnMajor", "DmemRowMajor"]
         # the copies the consumers hold follow: the matmul's operands carry the same layouts
         tb = json.loads(g.to_json())[2]["bgraph"]["operators"]
         mm = [o for o in tb if o["op_type"] == "tb_matmul_op"][0]
@@ -88,9 +108,9 @@ def test_attention_plan_rules_prune_the_search():
     try:
         costed = set()
 
-        def cost(op, loaders):
-            if loaders:
-                costed.add(tuple(loaders))
+        def cost(op, layouts):
+            if _split(layouts)[1]:
+                costed.add(_split(layouts)[1])
             return 1.0
 
         st = G.optimize_layout(g, cost)
