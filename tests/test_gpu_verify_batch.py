@@ -133,6 +133,36 @@ def test_verify_batch_full_size_verdicts(rt):
         assert verdicts == [c["expect_equal"] for c in prob["candidates"]], prob["family"]
 
 
+def test_the_whole_benchmark_batch_verifies_as_constructed(rt):
+    """The batch the fingerprint benchmark times -- 64 problems of 64 candidates at full dims,
+    4096 candidate mugraphs -- through the same batched verify: every verdict is the one the
+    generator constructed (a fused rewrite equals its reference, a mutant does not), and for
+    every eighth candidate each output fingerprint and the verdict equal the oracle's."""
+    probs = C.generate(num_problems=64, per_problem=64)
+    assert sum(len(p["candidates"]) for p in probs) == 4096
+    checked = 0
+    for n, prob in enumerate(probs):
+        verdicts, outs, ref_out = _verify_problem(rt, prob)
+        assert verdicts == [c["expect_equal"] for c in prob["candidates"]], (n, prob["family"])
+        seed = prob["input_seed"]
+        want_ref = _outputs(prob["reference"],
+                            orc.eval_graph(prob["reference"], "fp", _inputs(prob["reference"], seed), threads=8))
+        assert len(ref_out) == len(want_ref) and all(np.array_equal(a, b) for a, b in zip(ref_out, want_ref))
+        for k in range(n % 8, len(prob["candidates"]), 8):
+            c = prob["candidates"][k]
+            want = _outputs(c["spec"], orc.eval_graph(c["spec"], "fp", _inputs(c["spec"], seed), threads=8))
+            assert len(outs[k]) == len(want)
+            for a, b in zip(outs[k], want):
+                assert np.array_equal(a, b), (n, k, prob["family"])
+            oracle_verdict = len(want) == len(want_ref) and all(
+                a.shape == b.shape and np.array_equal(a, b) for a, b in zip(want_ref, want))
+            assert verdicts[k] == oracle_verdict, (n, k, prob["family"])
+            checked += 1
+        if n % 8 == 7:
+            print("problems verified:", n + 1, "candidates checked against the oracle:", checked, flush=True)
+    assert checked == 512
+
+
 def test_verify_batches_in_flight_match_one_at_a_time(rt):
     """Four submissions in flight (verify_batch_begin x 4, then verify_batch_end x 4, the
     reference graphs fingerprinted as part of their batches): same verdicts and the same
