@@ -97,6 +97,7 @@ ABI = {
     "mi355_fp_binary_many": (_ci, [_pi, _pvp, _pi, _pvp, _pi, _pvp, _pi, _pi, _ci]),
     "mi355_fp_reduce": (_ci, [_vp, _vp, _sz, _ci, _ci, _ci]),
     "mi355_fp_equal": (_ci, [_vp, _vp, _sz, _pi]),
+    "mi355_fp_big_tiles_check": (_ci, [_pi]),
     "mi355_fp_equal_reset": (_ci, [_ci, _ci]),
     "mi355_fp_equal_enqueue": (_ci, [_vp, _vp, _sz, _ci]),
     "mi355_fp_equal_enqueue_many": (_ci, [_pvp, _pvp, ctypes.POINTER(_sz), _pi, _ci]),

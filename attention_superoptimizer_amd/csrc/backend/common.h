@@ -81,6 +81,8 @@ struct State {
   int attention_mode = 0;  // 0 auto, 1 latency kernel only, 2 throughput kernel when it fits
   int fp_vector_dot_only = 0;  // 1: fingerprint matmuls never take the matrix-core kernels
   int fp_big_tiles = 1;        // 0: large kernel-level matmuls keep 64 x 64 tiles
+  int fp_big_tiles_ok = 1;     // 0: the self-check of the 128-row tile kernels failed on this
+                               // device / build: they stay off whatever fp_big_tiles says
   int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
   int direct_lanes = 0;      // MI355_OPT_DIRECT_LANES
   int gemm_mode = 0;         // MI355_OPT_GEMM_MODE

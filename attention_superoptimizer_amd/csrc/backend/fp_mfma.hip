@@ -1084,7 +1084,7 @@ static int launch_mfma_group(uint16_t const *const *A, uint16_t const *const *B,
     // 32-bit there); below that 128 x 64 tiles if there is one of those for every compute unit
     // (1536^3: 26.7 us against 33.2 on 64 x 64 tiles; 1536 x 2048 x 1024: 23.2 against 25.7 on
     // 128 x 128; from 256 wide tiles on the narrow ones are no faster or slower)
-    bool const fits_big = state().fp_big_tiles && kp <= kBigMaxK &&
+    bool const fits_big = state().fp_big_tiles && state().fp_big_tiles_ok && kp <= kBigMaxK &&
                           (size_t)std::max(mp, np) * (size_t)kp < ((size_t)1 << 31);
     bool const narrow = fits_big && tiles128 < kBigMinTiles && tiles128x64 >= kBigMinTiles;
     bool const large = fits_big && (tiles128 >= kBigMinTiles || narrow);
@@ -1156,6 +1156,72 @@ bool mfma_matmul_pays(int batch, int m, int n, int k) {
 int launch_mfma_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m, int n,
                        int k) {
   return launch_mfma_group(&A, &B, &C, &batch, &m, &n, &k, 1);
+}
+
+// fp_mfma_matmul_big_kernel prefetches B^T with loads that land in registers behind the
+// compiler's back (plane_load16 / landed): correct as long as the compiler neither spills nor
+// copies those registers between the load and its wait, which the build checks for (no
+// scratch, the recorded occupancy) but cannot prove.  So the kernels are also checked where
+// they run: one product that takes the 128 x 128 tiles and one that takes the 128 x 64 tiles,
+// 8 k steps each, against the 64 x 64-tile kernel that uses ordinary loads.  The ring makes
+// the results bit-identical; on a difference the 128-row kernels stay off for this process.
+extern "C" int mi355_fp_big_tiles_check(int *passed) {
+  MI355_REQUIRE_INIT();
+  State &s = state();
+  constexpr int M = 2048, N = 2048, NN = 1024, K = 512;
+  size_t const a_elems = (size_t)M * K, b_elems = (size_t)K * N, c_elems = (size_t)M * N,
+               cn_elems = (size_t)M * NN;
+  uint16_t *buf = nullptr;
+  MI355_HIP(hipMalloc(reinterpret_cast<void **>(&buf), (a_elems + b_elems + 2 * c_elems + 2 * cn_elems) * 2));
+  uint16_t *A = buf, *B = A + a_elems, *C1 = B + b_elems, *C2 = C1 + c_elems, *D1 = C2 + c_elems,
+           *D2 = D1 + cn_elems;
+  std::vector<uint16_t> host(a_elems + b_elems);
+  uint64_t x = 0x9E3779B97F4A7C15ull;
+  for (uint16_t &v : host) {
+    x = x * 6364136223846793005ull + 1442695040888963407ull;
+    v = (uint16_t)((x >> 33) % FP_PQ);
+  }
+  int rc = MI355_OK, eq_big = 0, eq_narrow = 0;
+  int const asked = s.fp_big_tiles, ok_before = s.fp_big_tiles_ok;
+  auto run = [&](int big, uint16_t *c, uint16_t *d) {
+    s.fp_big_tiles = big;
+    s.fp_big_tiles_ok = 1;
+    if (rc == MI355_OK) {
+      rc = mi355_fp_matmul(A, B, c, 1, M, N, K);
+    }
+    if (rc == MI355_OK) {
+      rc = mi355_fp_matmul(A, B, d, 1, M, NN, K);  // the first K x NN elements of B, as a matrix
+    }
+  };
+  if (hipMemcpy(A, host.data(), host.size() * 2, hipMemcpyHostToDevice) != hipSuccess) {
+    rc = fail(MI355_ERR_HIP, "self-check upload failed");
+  }
+  run(1, C1, D1);
+  run(0, C2, D2);
+  s.fp_big_tiles = asked;
+  s.fp_big_tiles_ok = ok_before;
+  if (rc == MI355_OK) {
+    rc = mi355_fp_equal(C1, C2, c_elems, &eq_big);
+  }
+  if (rc == MI355_OK) {
+    rc = mi355_fp_equal(D1, D2, cn_elems, &eq_narrow);
+  }
+  hipError_t const freed = hipFree(buf);
+  if (rc != MI355_OK) {
+    return rc;
+  }
+  MI355_HIP(freed);
+  s.fp_big_tiles_ok = (eq_big && eq_narrow) ? 1 : 0;
+  if (!s.fp_big_tiles_ok) {
+    fprintf(stderr,
+            "mi355: the 128-row fingerprint matmul kernels disagree with the 64 x 64-tile kernel on this "
+            "device (128 x 128 tiles %s, 128 x 64 tiles %s); large matmuls keep 64 x 64 tiles\n",
+            eq_big ? "equal" : "DIFFER", eq_narrow ? "equal" : "DIFFER");
+  }
+  if (passed != nullptr) {
+    *passed = s.fp_big_tiles_ok;
+  }
+  return MI355_OK;
 }
 
 extern "C" int mi355_fp_matmul_many(uint16_t const *const *A, uint16_t const *const *B,

@@ -149,7 +149,8 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
   if (arena_base != nullptr) {
     *arena_base = s.arena;
   }
-  return MI355_OK;
+  // the kernels whose loads the compiler cannot see are checked once on the device they run on
+  return mi355_fp_big_tiles_check(nullptr);
 }
 
 extern "C" int mi355_shutdown(void) {

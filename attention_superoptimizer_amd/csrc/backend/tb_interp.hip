@@ -1474,21 +1474,26 @@ extern "C" int mi355_customized_fp_static(mi355_plan const *plan, void const *co
       d.vec8 = 0;
     }
   }
-  // the split rule of mi355_customized_fp; what it needs must fit the array
+  // The split rule of mi355_customized_fp (set_splits): as many ranges as it would take, fewer
+  // while their partial sums do not fit the array (any split gives the same ring sum).  A
+  // for-loop it would split but of which not even two ranges fit is refused rather than run
+  // unsplit on a fraction of the device.
   prog.splits = 1;
   long long const blocks = (long long)prog.grid[0] * prog.grid[1] * prog.grid[2];
   int const F = prog.forloop_range;
   if (F >= 2 && blocks < 192) {
-    int const splits = (int)std::min<long long>(std::min(F, 64), (256 + blocks - 1) / blocks);
+    int splits = (int)std::min<long long>(std::min(F, 64), (256 + blocks - 1) / blocks);
     long long elems = 0;
     for (int i = 0; i < plan->num_dmem_outputs; i++) {
       elems += (ext.out_elems[i] + 7) / 8 * 8;
     }
-    long long const need = elems * splits * 2;
-    if (splits >= 2 && need > (long long)MI355_STATIC_SCRATCH_BYTES) {
+    while (splits > 2 && elems * splits * 2 > (long long)MI355_STATIC_SCRATCH_BYTES) {
+      splits--;
+    }
+    if (splits >= 2 && elems * splits * 2 > (long long)MI355_STATIC_SCRATCH_BYTES) {
       return fail(MI355_ERR_UNSUPPORTED,
-                  "plan needs %lld bytes of partial sums (%d ranges of its for-loop); the static "
-                  "scratch holds %d", need, splits, (int)MI355_STATIC_SCRATCH_BYTES);
+                  "plan needs %lld bytes of partial sums for two ranges of its for-loop; the static "
+                  "scratch holds %d", elems * splits * 2, (int)MI355_STATIC_SCRATCH_BYTES);
     }
     if (splits >= 2) {
       prog.splits = splits;

@@ -222,6 +222,17 @@ int mi355_fp_unary(int op, uint16_t const *in, uint16_t *out, size_t n);
  * op = KN_ADD_OP / KN_MUL_OP / KN_DIV_OP (1008 / 1009 / 1010) */
 int mi355_fp_binary(int op, uint16_t const *in1, int const *dims1, uint16_t const *in2,
                     int const *dims2, uint16_t *out, int const *dims_out, int num_dims);
+/* Self-check of the two fingerprint-matmul kernels that work on 128-row tiles.  They prefetch
+ * one operand with loads issued from inline assembly, whose completion the compiler does not
+ * track; the build verifies that they use no scratch memory and keep their occupancy, this call
+ * verifies the results where they run: a [2048, 512] x [512, 2048] and a [2048, 512] x [512, 1024]
+ * product on those kernels against the 64 x 64-tile kernel (ordinary loads), which must agree
+ * bit for bit.  mi355_init runs it once; on a difference the 128-row kernels stay off for the
+ * process (MI355_OPT_FP_MATMUL_ROUTE cannot switch them back on) and a line goes to stderr.
+ * *passed (may be NULL): 1 = equal.  Allocates and frees 30 MB of device memory; blocking.
+ * No counterpart in the reference, whose matmul fingerprint is one scalar kernel
+ * (src/kernel/cuda/matmul_kernel.cu:133-203). */
+int mi355_fp_big_tiles_check(int *passed);
 /* `count` <= MI355_MAX_BINARY_OPS independent operators of the kind above in one launch (a
  * verification batch holds one per candidate): operator e uses ops[e], in1[e], in2[e], out[e],
  * num_dims[e] and the dims at dims1 / dims2 / dims_out + 4 * e.  Every dim <= 65535. */
@@ -268,9 +279,11 @@ int mi355_customized_fp(mi355_plan const *plan, void const *const *inputs,
  * the lookup tables: the partial sums of a split for-loop go to a file-scope device array
  * of MI355_STATIC_SCRATCH_BYTES instead of the backend's scratch slab, and the plan always
  * runs on the generic interpreter (the matrix-core route needs residue planes in allocated
- * memory).  Bit-identical to mi355_customized_fp.  A plan whose partial sums do not fit
- * (for-loop ranges x output elements x 2 bytes, ranges chosen as in mi355_customized_fp)
- * is refused with MI355_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array:
+ * memory).  Bit-identical to mi355_customized_fp.  The for-loop is cut into the ranges
+ * mi355_customized_fp would take, or into fewer while their partial sums (ranges x output
+ * elements x 2 bytes) do not fit the array -- any split gives the same sum in the ring.  A
+ * plan of which not even two ranges fit (more than 2 Mi output elements, on a grid small
+ * enough to be split) is refused with MI355_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array:
  * calls that overlap on one GPU (different queues or host threads) race; calls on one
  * queue are ordered.  Nothing in the array needs clearing between calls. */
 #define MI355_STATIC_SCRATCH_BYTES (8 << 20)

@@ -409,6 +409,60 @@ def test_large_matmuls_on_128_tiles_match_oracle(rt, abi):
     assert np.all(ext[0] == (8192 * x * x) % FP_PQ)
 
 
+@pytest.mark.parametrize("n,k", [(2048, 640), (2048, 600), (1024, 640), (1024, 1000)],
+                         ids=["128x128 tiles", "128x128 tiles, ragged k", "128x64 tiles", "128x64 tiles, ragged k"])
+def test_128_row_tiles_take_every_operand_of_the_last_k_step(rt, abi, n, k):
+    """The kernels on 128-row tiles prefetch B^T with loads that complete behind the compiler's
+    back.  An operand read before it landed would be the one of an earlier step, or of the call
+    before: so the same device buffers are multiplied three times in a row -- as filled, then
+    with only the last 64 of k changed in B, then with only those changed in A -- and every
+    product must equal the oracle's on slices of rows and columns from every corner, and the
+    64 x 64-tile kernel's (ordinary loads) everywhere."""
+    m = 2048
+    A = uniform_fp((1, m, k), 3100 + k)
+    B = uniform_fp((1, k, n), 3200 + k)
+    A2, B2 = A.copy(), B.copy()
+    B2[:, k - 64:, :] = uniform_fp((1, 64, n), 3300 + k)
+    A2[:, :, k - 64:] = uniform_fp((1, m, 64), 3400 + k)
+    spec = [{"op": "input", "dims": [1, m, k]}, {"op": "input", "dims": [1, k, n]},
+            {"op": "input", "dims": [1, m, n]}]
+    rows = np.r_[0:8, 1016:1032, m - 8:m]
+    cols = np.r_[0:8, n // 2 - 8:n // 2 + 8, n - 8:n]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        a, b, c = (vals[i][0] for i in range(3))
+        products = []
+        for step, (x, y) in enumerate([(A, B), (A, B2), (A2, B2)]):
+            a.write_fingerprint(x)
+            b.write_fingerprint(y)
+            got = {}
+            for route in (0, 2):
+                c.write_fingerprint(np.full((1, m, n), 7, np.uint16))
+                assert abi.mi355_set_option(4, route) == 0
+                try:
+                    assert abi.mi355_fp_matmul(ctypes.c_void_p(a.device_ptr(True)), ctypes.c_void_p(b.device_ptr(True)),
+                                               ctypes.c_void_p(c.device_ptr(True)), 1, m, n, k) == 0
+                finally:
+                    assert abi.mi355_set_option(4, 0) == 0
+                got[route] = c.read_fingerprint()
+            assert np.array_equal(got[0][0, rows, :], orc.fp_matmul(x[:, rows, :], y)[0]), step
+            assert np.array_equal(got[0][0][:, cols], orc.fp_matmul(x, y[:, :, cols])[0]), step
+            assert np.array_equal(got[0], got[2]), step
+            products.append(got[0])
+        # (the changes are seen: they alter the products)
+        assert not np.array_equal(products[0], products[1]) and not np.array_equal(products[1], products[2])
+    finally:
+        g.close()
+
+
+def test_the_self_check_of_the_128_row_tile_kernels_passes(rt, abi):
+    """What mi355_init ran once on this device; on demand it gives the same verdict and leaves
+    the routes as they were."""
+    passed = ctypes.c_int(-1)
+    assert abi.mi355_fp_big_tiles_check(ctypes.byref(passed)) == 0
+    assert passed.value == 1
+
+
 def test_full_size_matmul_checksum_of_checksums(rt, abi):
     """4096 x 4096 x 4096, uniform inputs: too large for the oracle as a whole, so the check is
     linear algebra in the ring: (1^T A) B = 1^T (A B) and A (B 1) = (A B) 1.  The two vector

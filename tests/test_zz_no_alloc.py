@@ -1,8 +1,9 @@
 """mi355_customized_fp_static -- the entry point that allocates nothing -- against
 mi355_customized_fp, through the C ABI, bit for bit: two calls in a row, the second with a
 smaller input (the static scratch keeps the first call's contents), then a plan without a
-split for-loop, a third call on the first plan again, and the refusal of a plan whose partial
-sums exceed the array."""
+split for-loop, a third call on the first plan again, a plan that gets fewer ranges than
+mi355_customized_fp gives it because theirs would not fit the array, and the refusal of a plan
+of which not even two ranges fit."""
 import ctypes
 
 import numpy as np
@@ -66,11 +67,33 @@ def test_static_scratch_entry_point_matches_the_allocating_one(rt, abi):
             assert np.array_equal(x, y), what + ": static entry point vs mi355_customized_fp"
 
 
+def test_static_scratch_entry_point_takes_fewer_ranges_when_four_do_not_fit(rt, abi):
+    """64 blocks -> mi355_customized_fp cuts the for-loop into 4 ranges: 4 x 256 x 8192 outputs
+    x 2 bytes = 16 MiB of partial sums.  The static array holds 8 MiB: two ranges, same bits."""
+    from attention_superoptimizer_amd import workloads as W
+    spec = W.tiled_matmul(256, 8192, 64, (64, 1, 1), 4, (-1, -1, -1), (1, -1, -1), (1, -1, -1))[0]
+    g, vals = rt.build_from_spec(spec)
+    try:
+        for i in (0, 1):
+            vals[i][0].write_fingerprint(uniform_fp(spec[i]["dims"], 500 + i))
+        plan = g.lowered(2, True)
+        i_p = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(True) for a, b in spec[2]["in"]])
+        o_p = (ctypes.c_void_p * 4)(*[t.device_ptr(True) for t in vals[2]])
+        assert abi.mi355_customized_fp(ctypes.byref(plan), i_p, o_p) == 0
+        want = vals[2][0].read_fingerprint()
+        vals[2][0].write_fingerprint(np.full(want.shape, 7, np.uint16))
+        assert abi.mi355_customized_fp_static(ctypes.byref(plan), i_p, o_p) == 0
+        assert abi.mi355_sync() == 0
+        assert np.array_equal(vals[2][0].read_fingerprint(), want)
+    finally:
+        g.close()
+
+
 def test_static_scratch_entry_point_refuses_what_does_not_fit(rt, abi):
     from attention_superoptimizer_amd import _native as N
     from attention_superoptimizer_amd import workloads as W
-    # 64 blocks -> 4 ranges x 256 x 8192 outputs x 2 bytes = 16 MiB of partial sums
-    spec = W.tiled_matmul(256, 8192, 64, (64, 1, 1), 4, (-1, -1, -1), (1, -1, -1), (1, -1, -1))[0]
+    # 128 blocks -> 2 ranges x 256 x 16384 outputs x 2 bytes = 16 MiB of partial sums
+    spec = W.tiled_matmul(256, 16384, 64, (128, 1, 1), 4, (-1, -1, -1), (1, -1, -1), (1, -1, -1))[0]
     g, vals = rt.build_from_spec(spec)
     try:
         plan = g.lowered(2, True)
