@@ -177,6 +177,33 @@ def fp_matmul_rate(G, abi, shape, steps: int, warmup: int, both_routes: bool):
     return rec
 
 
+def f16_matmul_rate(G, N, abi, m, n, k, operands, iters, warmup):
+    """One kernel-level fp16 GEMM [m, k] x [k, n], A row-major and B column-major (the layout
+    the reference's plans declare), by the launching queue's events.  `operands`: "normal" =
+    N(0, 0.1) values, "zeros" = all-zero operands (same instructions, nothing toggles)."""
+    g = G.KNGraph()
+    A, B, C = g.new_input((1, m, k)), g.new_input((1, k, n)), g.new_input((1, m, n))
+    for t, seed in ((A, 1), (B, 2)):
+        if operands == "zeros":
+            t.write_data(np.zeros(t.dims, np.float16))
+        else:
+            assert abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
+                                             ctypes.c_float(0.1), seed) == 0
+    pa, pb, pc = (ctypes.c_void_p(t.device_ptr(False)) for t in (A, B, C))
+    for _ in range(warmup):
+        assert abi.mi355_f16_matmul_layout(pa, pb, pc, 1, m, n, k, 0, 1) == 0, N.last_error()
+    assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
+    for _ in range(iters):
+        assert abi.mi355_f16_matmul_layout(pa, pb, pc, 1, m, n, k, 0, 1) == 0, N.last_error()
+    ms = ctypes.c_float()
+    assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
+    g.close()
+    us = ms.value * 1e3 / max(1, iters)
+    flops = 2.0 * m * n * k
+    return {"shape": [m, n, k], "operands": operands, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+            "mfma_frac": round(flops / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+
+
 def kernel_level_ops(G, N, abi, W):
     """The kernel-level fp16 operators (what the reference's KN*Op::profile run: a library GEMM,
     element-wise kernels, a reduction; src/kernel/cuda/matmul_kernel.cu:28-143): one 4096^3 GEMM
@@ -210,6 +237,11 @@ def kernel_level_ops(G, N, abi, W):
         rec["matmul_4096"][name] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
                                     "mfma_frac": round(flops / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
     g.close()
+    # the same GEMM on all-zero operands: the same instruction stream with no bits toggling in
+    # operand fetch, MFMA inputs and results; what it gains is clock the power management
+    # takes away under random operands, not anything the kernel does differently
+    z = f16_matmul_rate(G, N, abi, n, n, n, "zeros", 256, 32)
+    rec["matmul_4096"]["B_column_major_zero_operands"] = {k2: z[k2] for k2 in ("us", "TFLOPs", "mfma_frac")}
     # element-wise over 128 Mi halfs: 256 MB read (512 MB for the binary operator) + 256 MB written
     m = 128 << 20
     g = G.KNGraph()
@@ -409,6 +441,16 @@ def main() -> int:
     ap.add_argument("--fp-matmul", default="", metavar="B,M,N,K",
                     help="time the kernel-level fingerprint matmul of that shape on the matrix-core "
                          "route and on the vector-dot route and print both (used under the profiler)")
+    ap.add_argument("--f16-matmul", default="", metavar="M,N,K",
+                    help="time the kernel-level fp16 GEMM of that shape (A row-major, B column-major) "
+                         "and print it (used under the profiler)")
+    ap.add_argument("--operands", default="normal", choices=("normal", "zeros"),
+                    help="with --only and --f16-matmul: N(0, std) inputs (default) or all zeros, which "
+                         "run the same instructions with no bits toggling: the difference is the "
+                         "clock the power management grants")
+    ap.add_argument("--row-major", action="store_true",
+                    help="with --only: declare every input tensor DmemRowMajor instead of the storage "
+                         "order the plan declares (the other alternative a layout search costs)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run 16 plain device copies of MIB MiB and exit: the known-size "
                          "traffic that hardware byte counters are scaled against")
@@ -444,6 +486,12 @@ def main() -> int:
               flush=True)
         return 0
 
+    if args.f16_matmul:
+        m, n, k = (int(x) for x in args.f16_matmul.split(","))
+        print(json.dumps(f16_matmul_rate(G, N, abi, m, n, k, args.operands, args.steps * per_step,
+                                         args.warmup * per_step)), flush=True)
+        return 0
+
     if args.calibrate_copy:
         n = args.calibrate_copy << 20
         g = G.KNGraph()
@@ -459,10 +507,15 @@ def main() -> int:
 
     def setup(name):
         spec, _ = (W.BASELINE_CONFIGS.get(name) or W.SCALED_CONFIGS[name])()
+        if args.row_major:
+            spec = [dict(op, layout="DmemRowMajor") if op["op"] == "input" else op for op in spec]
         g, vals = G.build_from_spec(spec)
         for i, op in enumerate(spec):
             if op["op"] == "input":
                 t = vals[i][0]
+                if args.operands == "zeros":
+                    t.write_data(np.zeros(t.dims, np.float16))
+                    continue
                 rc = abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
                                                ctypes.c_float(W.INPUT_STD[name][i]), 0xC0FFEE00 + i)
                 assert rc == 0, N.last_error()

@@ -398,19 +398,30 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
   // Steady state is branch-free: the next iteration's loads are issued as soon as this
   // iteration's tiles are in LDS and stay in flight while it is multiplied; the last
   // iteration is peeled.
-  fetch(it_begin);
-  for (int it = it_begin; it + 1 < it_end; it++) {
+  // A split for-loop leaves every iteration's tile in its own slot of the slab, so a workgroup
+  // may walk its range in any order: each starts at a different iteration (rotating through the
+  // range), so that at any moment the workgroups of the chip read at many different offsets
+  // along k.  Started in step they would all sit at the same one or two offsets within the
+  // operand's power-of-two row or column stride, i.e. on a fraction of the memory channels.
+  int const n_it = it_end - it_begin;
+  int const rot = split ? (int)((blockIdx.x / P.ksplit * 5u + blockIdx.y * 3u + blockIdx.z) % (unsigned)n_it) : 0;
+  auto nth = [&](int i) {
+    int const j = i + rot;
+    return it_begin + (j >= n_it ? j - n_it : j);
+  };
+  fetch(nth(0));
+  for (int i = 0; i + 1 < n_it; i++) {
     __syncthreads();  // previous iteration's tiles fully consumed
     stash();
     __syncthreads();
-    fetch(it + 1);
+    fetch(nth(i + 1));
     __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the products
-    compute(it);
+    compute(nth(i));
   }
   __syncthreads();
   stash();
   __syncthreads();
-  compute(it_end - 1);
+  compute(nth(n_it - 1));
 
   // ---- finish ---------------------------------------------------------------------------
   // A split for-loop has left every iteration's tile in the scratch slab.  Otherwise the
