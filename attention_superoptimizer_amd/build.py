@@ -102,7 +102,10 @@ def build_backend():
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         list(pool.map(compile_one, zip(srcs, objs)))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", BACKEND_LIB] + objs)
+    # -Bsymbolic: kernel handles are weak global symbols named after the kernel; a generated
+    # program loaded into the same process instantiates some of the same templates, and each
+    # library must launch through its own handles
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", BACKEND_LIB] + objs)
 
 
 def build_runtime():

@@ -77,7 +77,11 @@ def generate(name: str) -> str:
 
 def compile_library(src: str, out: str) -> None:
     """The program without its main(), as a shared library exporting graphdef_launch."""
-    subprocess.check_call([HIPCC] + FLAGS + ["-DGRAPHDEF_NO_MAIN", "-shared", "-fPIC", src, "-o", out])
+    # -Bsymbolic: the program's kernels are instantiations of templates the backend library
+    # instantiates too, and a kernel's host-side handle is a weak global symbol of that name;
+    # loaded into one process, each library must launch through its own handles
+    subprocess.check_call([HIPCC] + FLAGS + ["-DGRAPHDEF_NO_MAIN", "-shared", "-fPIC", "-fvisibility=hidden",
+                                             "-Wl,-Bsymbolic", src, "-o", out])
 
 
 def compile_program(src: str, out: str) -> None:

@@ -417,7 +417,7 @@ void Graph::generate_hip_program(char const *file_path) {
   std::stringstream launcher;
   launcher << "// Launches every customized operator of the graph in order.  dtensors[i] is device\n"
               "// tensor i in creation order (see graphdef_tensor_elements).\n"
-              "extern \"C\" int graphdef_launch(void *const *dtensors, hipStream_t stream) {\n";
+              "GRAPHDEF_API int graphdef_launch(void *const *dtensors, hipStream_t stream) {\n";
   int kernels = 0;
   for (KNOperator *op : operators) {
     if (op->op_type != mirage::type::KN_CUSTOMIZED_OP) {
@@ -451,9 +451,9 @@ void Graph::generate_hip_program(char const *file_path) {
     file << (i ? ", " : "") << (is_input[i] ? 1 : 0);
   }
   file << "};\n"
-          "extern \"C\" int graphdef_num_tensors(void) { return " << elements.size() << "; }\n"
-          "extern \"C\" long long graphdef_tensor_elements(int i) { return kTensorElements[i]; }\n"
-          "extern \"C\" int graphdef_sync(void) { return (int)hipDeviceSynchronize(); }\n\n";
+          "GRAPHDEF_API int graphdef_num_tensors(void) { return " << elements.size() << "; }\n"
+          "GRAPHDEF_API long long graphdef_tensor_elements(int i) { return kTensorElements[i]; }\n"
+          "GRAPHDEF_API int graphdef_sync(void) { return (int)hipDeviceSynchronize(); }\n\n";
   file << launcher.str();
   // the profiling main: random fp16 tensors, 1000 warm-up launches, 1000 timed
   file << R"HIP(#ifndef GRAPHDEF_NO_MAIN

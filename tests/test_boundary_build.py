@@ -27,6 +27,10 @@ def test_header_symbols_are_exported_by_the_in_tree_library():
     have = set(re.findall(r" T (mi355_[a-z0-9_]+)", syms))
     missing = [s for s in _abi_symbols() if s not in have]
     assert not missing, missing
+    # kernel handles are weak global symbols named after the kernel: the library binds its own
+    # (a generated program in the same process instantiates some of the same templates)
+    assert "SYMBOLIC" in subprocess.check_output(
+        ["readelf", "-d", os.path.join(PKG, "libmi355_backend.so")]).decode()
 
 
 @pytest.mark.skipif(shutil.which("cmake") is None, reason="cmake not installed")
@@ -49,6 +53,7 @@ def test_cmake_configures_and_builds_for_gfx950(tmp_path):
     syms = subprocess.check_output(["nm", "-D", "--defined-only", str(backend)]).decode()
     have = set(re.findall(r" T (mi355_[a-z0-9_]+)", syms))
     assert not [s for s in _abi_symbols() if s not in have]
+    assert "SYMBOLIC" in subprocess.check_output(["readelf", "-d", str(backend)]).decode()
     # the code object is gfx950 and nothing else
     notes = subprocess.check_output(["strings", "-n", "8", str(backend)]).decode()
     assert "gfx950" in notes and "gfx90a" not in notes and "gfx942" not in notes

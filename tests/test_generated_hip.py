@@ -114,3 +114,7 @@ def test_hipcc_compiles_the_program_for_gfx950(tmp_path):
         for name in ("graphdef_launch", "graphdef_kernel_0_launch", "graphdef_num_tensors",
                      "graphdef_tensor_elements", "graphdef_sync"):
             assert f" T {name}" in syms
+        # a kernel's host-side handle is a weak global symbol named after the kernel, and the
+        # backend library instantiates the same templates: each library binds its own
+        dyn = subprocess.check_output(["readelf", "-d", str(tmp_path / "libc1.so")]).decode()
+        assert "SYMBOLIC" in dyn
