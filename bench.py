@@ -444,6 +444,10 @@ def main() -> int:
     ap.add_argument("--f16-matmul", default="", metavar="M,N,K",
                     help="time the kernel-level fp16 GEMM of that shape (A row-major, B column-major) "
                          "and print it (used under the profiler)")
+    ap.add_argument("--vendor-gemm", default="", metavar="M,N,K",
+                    help="time the vendor library's fp16 GEMM of that shape (torch.matmul, which calls "
+                         "hipBLASLt / rocBLAS; A row-major, B column-major) with --operands and print it: "
+                         "the scale the kernel-level GEMM of this backend is read against")
     ap.add_argument("--operands", default="normal", choices=("normal", "zeros"),
                     help="with --only and --f16-matmul: N(0, std) inputs (default) or all zeros, which "
                          "run the same instructions with no bits toggling: the difference is the "
@@ -460,6 +464,34 @@ def main() -> int:
         print("bench.py: this path runs on ONE GPU (a customized op's grid does not span "
               "devices); run with --gpus 1", file=sys.stderr)
         return 2
+
+    if args.vendor_gemm:
+        # (nothing of this backend runs here: the library call through torch, events on torch's stream)
+        import torch
+        m, n, k = (int(x) for x in args.vendor_gemm.split(","))
+        gen = torch.Generator(device="cuda").manual_seed(1)
+        if args.operands == "zeros":
+            a = torch.zeros(m, k, device="cuda", dtype=torch.half)
+            b = torch.zeros(n, k, device="cuda", dtype=torch.half)
+        else:
+            a = (torch.randn(m, k, device="cuda", generator=gen) * 0.1).half()
+            b = (torch.randn(n, k, device="cuda", generator=gen) * 0.1).half()
+        iters, warm = max(1, args.steps * per_step), max(1, args.warmup * per_step)
+        for _ in range(warm):
+            c = a @ b.t()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            c = a @ b.t()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / iters
+        del c
+        print(json.dumps({"vendor_library_gemm": [m, n, k], "operands": args.operands, "us": round(us, 2),
+                          "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1),
+                          "mfma_frac": round(2.0 * m * n * k / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}), flush=True)
+        return 0
 
     from attention_superoptimizer_amd import _native as N
     from attention_superoptimizer_amd import graph as G
