@@ -105,7 +105,7 @@ def build_backend():
     # -Bsymbolic: kernel handles are weak global symbols named after the kernel; a generated
     # program loaded into the same process instantiates some of the same templates, and each
     # library must launch through its own handles
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", BACKEND_LIB] + objs)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", BACKEND_LIB] + objs + ["-ldl"])
 
 
 def build_runtime():

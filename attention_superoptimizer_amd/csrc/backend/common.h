@@ -86,6 +86,7 @@ struct State {
   int plan_smem_layout = 0;  // 1: loader tiles take the LDS layout their plan declares
   int direct_lanes = 0;      // MI355_OPT_DIRECT_LANES
   int gemm_mode = 0;         // MI355_OPT_GEMM_MODE
+  int f16_matmul_route = 0;  // MI355_OPT_F16_MATMUL_ROUTE
   // phase timestamps of the direct-staging attention kernel (MI355_OPT_PHASE_TRACE): while
   // set, launches of that kernel record six wall-clock stamps per wavefront here
   unsigned long long *phase_trace = nullptr;        // null while tracing is off
@@ -114,6 +115,12 @@ bool mfma_matmul_pays(int batch, int m, int n, int k);
 int launch_mfma_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m, int n,
                        int k);
 int sync_all_queues();
+// The vendor library's GEMM on the calling thread's queue (vendor_gemm.cc): row-major C =
+// A . B for `batch` matrices, each operand in either storage order; MI355_ERR_UNSUPPORTED
+// when the library cannot be loaded.  vendor_gemm_release drops its per-queue handles.
+int vendor_gemm(void const *A, void const *B, void *C, int batch, int m, int n, int k, int a_column_major,
+                int b_column_major);
+int vendor_gemm_release();
 // Looks up the device address of the file-scope scratch array behind
 // mi355_customized_fp_static (tb_interp.hip); called by mi355_init with `device` current.
 int static_scratch_setup(int device);

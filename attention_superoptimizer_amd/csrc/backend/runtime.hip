@@ -161,6 +161,7 @@ extern "C" int mi355_shutdown(void) {
   if (int rc = sync_all_queues()) {
     return rc;
   }
+  vendor_gemm_release();  // its handles are bound to the queues destroyed below
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     MI355_HIP(hipEventDestroy(s.ev0[q]));
     MI355_HIP(hipEventDestroy(s.ev1[q]));
@@ -273,6 +274,10 @@ extern "C" int mi355_set_option(int option, int value) {
   }
   if (option == MI355_OPT_GEMM_MODE && value >= 0 && value <= 2) {
     state().gemm_mode = value;
+    return MI355_OK;
+  }
+  if (option == MI355_OPT_F16_MATMUL_ROUTE && (value == 0 || value == 1)) {
+    state().f16_matmul_route = value;
     return MI355_OK;
   }
   if (option == MI355_OPT_PHASE_TRACE && (value == 0 || value == 1)) {

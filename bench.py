@@ -31,6 +31,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_FP16_PEAK_TFLOPS = 2500.0
+OPT_F16_MATMUL_ROUTE = 8  # include/mi355_abi.h
 HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "attn_direct_kernel_C2_gqa_decode.md")
 
 
@@ -242,6 +243,14 @@ def kernel_level_ops(G, N, abi, W):
     # takes away under random operands, not anything the kernel does differently
     z = f16_matmul_rate(G, N, abi, n, n, n, "zeros", 256, 32)
     rec["matmul_4096"]["B_column_major_zero_operands"] = {k2: z[k2] for k2 in ("us", "TFLOPs", "mfma_frac")}
+    # the same product on the backend's other route: the vendor's BLAS, as the reference calls its own
+    assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 1) == 0
+    try:
+        for name, operands in (("vendor_route", "normal"), ("vendor_route_zero_operands", "zeros")):
+            v = f16_matmul_rate(G, N, abi, n, n, n, operands, 256, 32)
+            rec["matmul_4096"][name] = {k2: v[k2] for k2 in ("us", "TFLOPs", "mfma_frac")}
+    finally:
+        assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 0) == 0
     # element-wise over 128 Mi halfs: 256 MB read (512 MB for the binary operator) + 256 MB written
     m = 128 << 20
     g = G.KNGraph()
@@ -444,6 +453,9 @@ def main() -> int:
     ap.add_argument("--f16-matmul", default="", metavar="M,N,K",
                     help="time the kernel-level fp16 GEMM of that shape (A row-major, B column-major) "
                          "and print it (used under the profiler)")
+    ap.add_argument("--f16-route", default="own", choices=("own", "vendor"),
+                    help="with --f16-matmul: this backend's kernels (default) or its vendor-library "
+                         "route (MI355_OPT_F16_MATMUL_ROUTE = 1: rocBLAS opened at run time)")
     ap.add_argument("--vendor-gemm", default="", metavar="M,N,K",
                     help="time the vendor library's fp16 GEMM of that shape (torch.matmul, which calls "
                          "hipBLASLt / rocBLAS; A row-major, B column-major) with --operands and print it: "
@@ -520,8 +532,10 @@ def main() -> int:
 
     if args.f16_matmul:
         m, n, k = (int(x) for x in args.f16_matmul.split(","))
-        print(json.dumps(f16_matmul_rate(G, N, abi, m, n, k, args.operands, args.steps * per_step,
-                                         args.warmup * per_step)), flush=True)
+        assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 1 if args.f16_route == "vendor" else 0) == 0
+        rec = f16_matmul_rate(G, N, abi, m, n, k, args.operands, args.steps * per_step, args.warmup * per_step)
+        rec["route"] = args.f16_route
+        print(json.dumps(rec), flush=True)
         return 0
 
     if args.calibrate_copy:

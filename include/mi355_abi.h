@@ -133,6 +133,15 @@ typedef struct mi355_launch_info {
  * kernel wherever it applies.  Both keep the accumulation order of the sequential loop;
  * results agree to the last bit.  A measurement knob that the tests use to cover both. */
 #define MI355_OPT_GEMM_MODE 7
+/* F16_MATMUL_ROUTE: what runs a kernel-level fp16 matmul (mi355_f16_matmul,
+ * mi355_f16_matmul_layout).  0 = this library's kernels (default); 1 = the vendor's BLAS
+ * (rocblas_gemm_strided_batched_ex, fp16 in and out, fp32 accumulation, atomics off), which
+ * is what the reference calls on its side (cublasGemmStridedBatchedEx,
+ * src/kernel/cuda/matmul_kernel.cu:86-131).  rocBLAS is opened at run time on the first
+ * such call; when it cannot be, the call fails with MI355_ERR_UNSUPPORTED and nothing else
+ * runs in its place.  Both routes accumulate in fp32 and round once; their sums differ in
+ * order, so results agree to fp16 rounding, not to the bit. */
+#define MI355_OPT_F16_MATMUL_ROUTE 8
 
 /* ---- lifetime ------------------------------------------------------------
  * Replaces DeviceMemoryManager's constructor / destructor

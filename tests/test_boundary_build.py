@@ -33,6 +33,23 @@ def test_header_symbols_are_exported_by_the_in_tree_library():
         ["readelf", "-d", os.path.join(PKG, "libmi355_backend.so")]).decode()
 
 
+def test_options_take_their_documented_values_only():
+    """mi355_set_option needs no device: every option of the header accepts its documented
+    values and refuses the next one; the vendor's BLAS is not a link dependency (it is opened
+    when the option that asks for it is used)."""
+    lib = ctypes.CDLL(os.path.join(PKG, "libmi355_backend.so"))
+    text = open(os.path.join(ROOT, "include", "mi355_abi.h")).read()
+    opts = dict((name, int(v)) for name, v in re.findall(r"#define (MI355_OPT_[A-Z0-9_]+) (\d+)", text))
+    assert sorted(opts.values()) == list(range(1, len(opts) + 1))
+    assert lib.mi355_set_option(opts["MI355_OPT_F16_MATMUL_ROUTE"], 1) == 0
+    assert lib.mi355_set_option(opts["MI355_OPT_F16_MATMUL_ROUTE"], 0) == 0
+    assert lib.mi355_set_option(opts["MI355_OPT_F16_MATMUL_ROUTE"], 2) != 0
+    assert lib.mi355_set_option(opts["MI355_OPT_GEMM_MODE"], 3) != 0
+    assert lib.mi355_set_option(len(opts) + 1, 0) != 0
+    needed = subprocess.check_output(["readelf", "-d", os.path.join(PKG, "libmi355_backend.so")]).decode()
+    assert "rocblas" not in needed
+
+
 @pytest.mark.skipif(shutil.which("cmake") is None, reason="cmake not installed")
 def test_cmake_configures_and_builds_for_gfx950(tmp_path):
     """project(... LANGUAGES CXX HIP), CMAKE_HIP_ARCHITECTURES gfx950, targets mi355_backend,

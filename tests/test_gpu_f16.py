@@ -620,6 +620,49 @@ def test_kernel_level_matmul_4096_cubed_by_samples_and_checksums(rt, abi):
     assert np.abs(c64.sum(0) - a64.sum(0) @ b64).max() < 1.3
 
 
+OPT_F16_MATMUL_ROUTE = 8
+
+
+@pytest.fixture
+def vendor_route(abi):
+    assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 1) == 0
+    yield
+    assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 0) == 0
+
+
+@pytest.mark.parametrize("batch,m,n,k", [
+    (3, 70, 130, 96),
+    (1, 33, 47, 50),
+    (1, 16, 4096, 4096),
+    (2, 256, 64, 4096),
+    (1, 1024, 1024, 1024),
+])
+def test_kernel_level_matmul_on_the_vendor_library(rt, abi, vendor_route, batch, m, n, k):
+    """The second route of mi355_f16_matmul_layout (the vendor's BLAS, opened at run time) in
+    every storage order of A and B: the operand order, transposes and leading dimensions it
+    hands to a column-major library are what a wrong storage order would break."""
+    for a_cm, b_cm in ((0, 1), (0, 0), (1, 1), (1, 0)):
+        a, b, got = _abi_matmul(rt, abi, batch, m, n, k, a_cm, b_cm, 41)
+        want = orc.f16_matmul(a, b)
+        assert_f16_close(got, want, what=f"vendor [{batch},{m},{k}] . [{batch},{k},{n}], A cm {a_cm}, B cm {b_cm}")
+
+
+def test_the_vendor_route_runs_the_matmul_operators_of_a_graph(rt, abi, vendor_route):
+    """KNMatmulOp::run reaches the same entry point: an un-fused attention graph (Q . K^T with K
+    column-major, exp, row sums, division, P . V) on the vendor route against the oracle."""
+    spec = [
+        {"op": "input", "dims": [2, 256, 64]},
+        {"op": "input", "dims": [2, 64, 512], "layout": "DmemColumnMajor"},
+        {"op": "input", "dims": [2, 512, 64]},
+        {"op": "matmul", "in": [[0, 0], [1, 0]]},
+        {"op": "exp", "in": [[3, 0]]},
+        {"op": "reduction", "in": [[4, 0]], "dim": 2, "size": 1},
+        {"op": "div", "in": [[4, 0], [5, 0]]},
+        {"op": "matmul", "in": [[6, 0], [2, 0]]},
+    ]
+    _check(rt, spec, _inputs(spec, {0: 0.1, 1: 0.1, 2: 1.0}), "vendor route, un-fused attention")
+
+
 def test_kernel_level_elementwise_and_reductions_large_and_ragged(rt):
     """The vector paths (16 bytes per lane) and their scalar tails: large tensors, row lengths
     that are not multiples of 8, one value per row as the second operand, sums along rows and
