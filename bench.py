@@ -183,22 +183,24 @@ def f16_matmul_rate(G, N, abi, m, n, k, operands, iters, warmup):
     the reference's plans declare), by the launching queue's events.  `operands`: "normal" =
     N(0, 0.1) values, "zeros" = all-zero operands (same instructions, nothing toggles)."""
     g = G.KNGraph()
-    A, B, C = g.new_input((1, m, k)), g.new_input((1, k, n)), g.new_input((1, m, n))
-    for t, seed in ((A, 1), (B, 2)):
-        if operands == "zeros":
-            t.write_data(np.zeros(t.dims, np.float16))
-        else:
-            assert abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
-                                             ctypes.c_float(0.1), seed) == 0
-    pa, pb, pc = (ctypes.c_void_p(t.device_ptr(False)) for t in (A, B, C))
-    for _ in range(warmup):
-        assert abi.mi355_f16_matmul_layout(pa, pb, pc, 1, m, n, k, 0, 1) == 0, N.last_error()
-    assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
-    for _ in range(iters):
-        assert abi.mi355_f16_matmul_layout(pa, pb, pc, 1, m, n, k, 0, 1) == 0, N.last_error()
-    ms = ctypes.c_float()
-    assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
-    g.close()
+    try:
+        A, B, C = g.new_input((1, m, k)), g.new_input((1, k, n)), g.new_input((1, m, n))
+        for t, seed in ((A, 1), (B, 2)):
+            if operands == "zeros":
+                t.write_data(np.zeros(t.dims, np.float16))
+            else:
+                assert abi.mi355_f16_fill_normal(ctypes.c_void_p(t.device_ptr(False)), t.num_elements,
+                                                 ctypes.c_float(0.1), seed) == 0
+        pa, pb, pc = (ctypes.c_void_p(t.device_ptr(False)) for t in (A, B, C))
+        for _ in range(warmup):
+            assert abi.mi355_f16_matmul_layout(pa, pb, pc, 1, m, n, k, 0, 1) == 0, N.last_error()
+        assert abi.mi355_sync() == 0 and abi.mi355_timer_start() == 0
+        for _ in range(iters):
+            assert abi.mi355_f16_matmul_layout(pa, pb, pc, 1, m, n, k, 0, 1) == 0, N.last_error()
+        ms = ctypes.c_float()
+        assert abi.mi355_timer_stop(ctypes.byref(ms)) == 0
+    finally:
+        g.close()
     us = ms.value * 1e3 / max(1, iters)
     flops = 2.0 * m * n * k
     return {"shape": [m, n, k], "operands": operands, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
@@ -244,11 +246,14 @@ def kernel_level_ops(G, N, abi, W):
     z = f16_matmul_rate(G, N, abi, n, n, n, "zeros", 256, 32)
     rec["matmul_4096"]["B_column_major_zero_operands"] = {k2: z[k2] for k2 in ("us", "TFLOPs", "mfma_frac")}
     # the same product on the backend's other route: the vendor's BLAS, as the reference calls its own
+    # (an optional route: where rocBLAS cannot be opened the record says so and the run goes on)
     assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 1) == 0
     try:
         for name, operands in (("vendor_route", "normal"), ("vendor_route_zero_operands", "zeros")):
             v = f16_matmul_rate(G, N, abi, n, n, n, operands, 256, 32)
             rec["matmul_4096"][name] = {k2: v[k2] for k2 in ("us", "TFLOPs", "mfma_frac")}
+    except AssertionError as e:
+        rec["matmul_4096"]["vendor_route"] = {"error": str(e) or N.last_error()}
     finally:
         assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 0) == 0
     # element-wise over 128 Mi halfs: 256 MB read (512 MB for the binary operator) + 256 MB written

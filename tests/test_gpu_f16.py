@@ -625,6 +625,14 @@ OPT_F16_MATMUL_ROUTE = 8
 
 @pytest.fixture
 def vendor_route(abi):
+    import ctypes
+    try:
+        ctypes.CDLL("librocblas.so.5")
+    except OSError:
+        try:
+            ctypes.CDLL("/opt/rocm/lib/librocblas.so.5")
+        except OSError:
+            pytest.skip("rocBLAS is not installed: the vendor route of the fp16 matmul cannot run")
     assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 1) == 0
     yield
     assert abi.mi355_set_option(OPT_F16_MATMUL_ROUTE, 0) == 0
