@@ -9,6 +9,7 @@
 //                       arithmetic the reference's generated programs define,
 //                       src/kernel/triton_code_gen.cc:223-333)
 #include "common.h"
+#include "mi355_kernels/kernarg.h"
 #include "tb_program.h"
 #include <atomic>
 
@@ -570,6 +571,9 @@ __global__ __launch_bounds__(kInterpThreads) void fp_interp_kernel(
     DevProgram const P, uint16_t const *__restrict__ g_exp, uint16_t const *__restrict__ g_divp,
     uint16_t const *__restrict__ g_divq) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  // (the program record is an argument of 3 KB that the block walks operator by operator: all
+  // of its lines in one trip)
+  fetch_kernel_arguments_large<sizeof(DevProgram)>();
   fp_load_tables(lds, g_exp, g_divp, g_divq);
   __syncthreads();
   fp_interp_block(P, lds, blockIdx.x % P.grid[0], blockIdx.y, blockIdx.z, blockIdx.x / P.grid[0]);
@@ -735,6 +739,7 @@ __device__ __forceinline__ half8 splat8(_Float16 x) {
 __global__ __launch_bounds__(kInterpThreads) void f16_interp_kernel(DevProgram const P,
                                                                     unsigned long long *trace) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  fetch_kernel_arguments_large<sizeof(DevProgram)>();  // (the program record, walked operator by operator)
   int const tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   int const F = P.forloop_range;
   bool const tracing = trace != nullptr && tid == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;

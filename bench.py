@@ -449,6 +449,11 @@ def main() -> int:
     ap.add_argument("--gemm-mode", type=int, default=0, choices=(0, 1, 2),
                     help="with --only: which fused skinny-GEMM kernel runs (0 the backend's choice, 1 the "
                          "range-splitting kernel, 2 the one-launch kernel)")
+    ap.add_argument("--interpreter", action="store_true",
+                    help="with --only: every customized op on the generic LDS interpreter "
+                         "(MI355_OPT_FORCE_INTERPRETER) instead of the fused kernel its shape selects")
+    ap.add_argument("--fingerprint", action="store_true",
+                    help="with --only: time the fingerprint run of every customized op instead of its fp16 run")
     ap.add_argument("--attention-mode", type=int, default=0, choices=(0, 1, 2, 3),
                     help="with --only: which fused attention kernel runs (0 the backend's choice; see "
                          "MI355_OPT_ATTENTION_MODE)")
@@ -608,15 +613,17 @@ def main() -> int:
         spec, g, vals = setup(args.only)
         assert abi.mi355_set_option(7, args.gemm_mode) == 0
         assert abi.mi355_set_option(2, args.attention_mode) == 0
+        assert abi.mi355_set_option(1, 1 if args.interpreter else 0) == 0
         out = {}
+        fp = bool(args.fingerprint)
         for i, op in enumerate(spec):
             if op["op"] != "customized":
                 continue
-            pl = g.lowered(i, fingerprint=False)
-            i_p = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(False) for a, b in op["in"]])
-            o_p = (ctypes.c_void_p * 4)(*[t.device_ptr(False) for t in vals[i]])
+            pl = g.lowered(i, fingerprint=fp)
+            i_p = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(fp) for a, b in op["in"]])
+            o_p = (ctypes.c_void_p * 4)(*[t.device_ptr(fp) for t in vals[i]])
             ms = ctypes.c_float()
-            assert abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, args.warmup * per_step,
+            assert abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 1 if fp else 0, args.warmup * per_step,
                                                 args.steps * per_step,
                                                 ctypes.byref(ms)) == 0, N.last_error()
             out[f"op{i}_us"] = round(ms.value * 1e3, 3)

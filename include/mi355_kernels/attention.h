@@ -13,6 +13,8 @@
 
 #include <cstdint>
 
+#include "kernarg.h"
+
 namespace mi355 {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -213,6 +215,7 @@ __device__ __forceinline__ constexpr int cm_swizzle_key(int r) {
 // consecutive for-loop iterations.
 template <int D, int NK, int DV, bool HAS_DIV, int RG, int IP, bool CM = false>
 __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams const P) {
+  fetch_kernel_arguments<sizeof(AttnParams), 3>();  // every line of the block, one trip (decode_block reads gridDim.z)
   constexpr int LDO = DV + 8;
   constexpr int KB = NK / 16, DB = DV / 16, DK = D / 32;
   constexpr int NW = RG * IP, NT = 64 * NW;
@@ -1050,7 +1053,10 @@ __device__ __forceinline__ void wait_vm() {
 // their V^T operand as two 8-byte reads.
 template <int D, int NK, int DV, bool HAS_DIV, int IP, int RPW, int NBUF, int NIT, int SPI, int IPS,
           bool TRACE, bool CM>
-__global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const P) {
+__global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const) {
+  // (the argument block is read by hand, all of it at once; decode_block reads gridDim.z, so
+  // the block counts behind the arguments exist and are fetched with them)
+  AttnParams const P = load_kernel_arguments<AttnParams, 3>();
   constexpr bool PERM = CM && IPS != 4;  // permuted key order inside pairs of S^T blocks
   static_assert(D == 64 && NK == 64 && DV == 64, "the chunk swizzles assume rows of 128 bytes");
   static_assert((SPI == 1 || IPS == 1) && (SPI == 1 || SPI == 2 || SPI == 4) &&

@@ -9,6 +9,8 @@
 
 #include <cstdint>
 
+#include "kernarg.h"
+
 namespace mi355 {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -36,7 +38,8 @@ __device__ __forceinline__ long long ctile_origin(CTile const &t) {
 }
 
 template <int VEC, int MODE>
-__global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const P) {
+__global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const) {
+  CombineParams const P = load_kernel_arguments<CombineParams, 0>();  // the whole block, one trip
   typedef _Float16 halfv __attribute__((ext_vector_type(VEC)));
   _Float16 const *n = static_cast<_Float16 const *>(P.n.ptr) + ctile_origin(P.n);
   _Float16 const *d = static_cast<_Float16 const *>(P.d.ptr) + ctile_origin(P.d);

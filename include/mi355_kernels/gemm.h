@@ -10,6 +10,8 @@
 
 #include <cstdint>
 
+#include "kernarg.h"
+
 namespace mi355 {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -187,6 +189,7 @@ __device__ __forceinline__ void store_weight_cm(uint4v const (&x)[PPT][4], int R
 // operand (weights, lora A and B) is a column-major tensor.
 template <int MT, int NB, int PRO, bool LORA, int KTMAX, bool WCM>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
+  fetch_kernel_arguments<sizeof(GemmParams), 2>();  // every line of the block, one trip (gridDim.x, .y are read)
   constexpr int NT = 256;
   constexpr int WPPT = ((KTMAX / 4) * 8 + NT - 1) / NT;  // weight patches per thread
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -466,6 +469,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(GemmParams const P) {
 // workgroup the LoRA plan took 77 us instead of 13).
 template <int NB>
 __global__ __launch_bounds__(256) void gemm_combine_kernel(GemmParams const P) {
+  fetch_kernel_arguments<sizeof(GemmParams), 2>();  // (gridDim.x, .y are read)
   int const tid = threadIdx.x, M = P.M, F = P.forloop_range;
   int const bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
   int const block_linear = bx + gridDim.x * (by + gridDim.y * bz);
@@ -584,6 +588,7 @@ __device__ __forceinline__ half4 lane_tr16(_Float16 const *p) {
 // are sixteen streams of whole cache lines that no other workgroup touches.
 template <int KT, int NB, int PRO, bool LORA, bool WCM>
 __global__ __launch_bounds__(1024) void gemm_lanes_kernel(LaneParams const L) {
+  fetch_kernel_arguments<sizeof(LaneParams), 4>();  // every line of the block, one trip (blockDim.x is read)
   GemmParams const &P = L.g;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   constexpr int KS = KT / 32;                                // MFMA steps (and 1 KB loads) per strip
