@@ -1168,9 +1168,12 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const) 
   constexpr int EPT = ROWS * DV / (64 * IP);  // elements per thread (16 rows: 8 / 4 / 2 for IP = 2 / 4 / 8)
   static_assert(EPT == 2 || EPT == 4 || EPT == 8, "2, 4 or 8 wavefronts");
   int const out_row = tid / (DV / EPT), out_col = (tid % (DV / EPT)) * EPT;
-  _Float16 *const og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
-                       tile_offset(P.o, bx, by, bz, 0) +
-                       (long long)(row_base + out_row) * P.o.d_cols + out_col;
+  _Float16 *og = static_cast<_Float16 *>(const_cast<void *>(P.o.ptr)) +
+                 tile_offset(P.o, bx, by, bz, 0) +
+                 (long long)(row_base + out_row) * P.o.d_cols + out_col;
+  // (the address is made opaque here so that it IS computed here, while the wavefront waits for
+  // its tiles: left alone the compiler computes it where it is used, after the last barrier)
+  asm volatile("" : "+v"(og));
 
   // results of this wavefront's iterations, packed fp16: keep[j][rp][2t], [2t+1] =
   // O[row 16rp + c][16t + 4g + r] for r = 0,1 / 2,3; keep[j][rp][2 DB] = the row sum of row c
@@ -1184,10 +1187,13 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const) 
       int const b = NBUF == 2 ? (q & 1) : 0;
       // the tile pair of iteration j (and everything older) has landed when at most the next
       // pair's loads are outstanding
+      // (a pair's K loads go out before its V loads, and loads complete in order: the K tile,
+      // and the Q tile before it, are there when the V loads are the oldest still outstanding;
+      // the V tile is waited for where it is first read, after the S^T products are issued)
       if (NBUF == 2 && q + 1 < nstrips) {
-        wait_vm<KI + VI>();
+        wait_vm<KI + 2 * VI>();
       } else {
-        wait_vm<0>();
+        wait_vm<VI>();
       }
       if (q == 0) {
         // Q fragments (B operand of S^T): Q[row c][32kk + 8g .. +7]
@@ -1253,6 +1259,11 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const) 
             acc[rp][jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[jb][kk], qf[rp][kk], acc[rp][jb], 0, 0, 0);
           }
         }
+      }
+      if (NBUF == 2 && q + 1 < nstrips) {
+        wait_vm<KI + VI>();
+      } else {
+        wait_vm<0>();
       }
       half8 vb[DB][KB / 2];
 #pragma unroll
