@@ -61,6 +61,7 @@ struct State {
   int *cmp_slots = nullptr;   // the same memory as the device addresses it
   hipEvent_t marks[MI355_NUM_MARKS][MI355_NUM_QUEUES] = {};
   hipEvent_t ev0[MI355_NUM_QUEUES] = {}, ev1[MI355_NUM_QUEUES] = {};  // timer pair per queue
+  hipEvent_t pace[MI355_NUM_QUEUES][2] = {};  // markers that bound how far a timed loop runs ahead
   int max_lds = 65536;
   // staging of batched launches (mi355_customized_fp_batch): per queue a small ring of
   // pinned host / device buffer pairs that carry the program records of one call

@@ -128,6 +128,8 @@ extern "C" int mi355_init(size_t arena_bytes, void **arena_base) {
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     MI355_HIP(hipEventCreate(&s.ev0[q]));
     MI355_HIP(hipEventCreate(&s.ev1[q]));
+    MI355_HIP(hipEventCreateWithFlags(&s.pace[q][0], hipEventDisableTiming));
+    MI355_HIP(hipEventCreateWithFlags(&s.pace[q][1], hipEventDisableTiming));
   }
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     for (int b = 0; b < State::kBatchSlots; b++) {
@@ -165,6 +167,8 @@ extern "C" int mi355_shutdown(void) {
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     MI355_HIP(hipEventDestroy(s.ev0[q]));
     MI355_HIP(hipEventDestroy(s.ev1[q]));
+    MI355_HIP(hipEventDestroy(s.pace[q][0]));
+    MI355_HIP(hipEventDestroy(s.pace[q][1]));
   }
   MI355_HIP(hipFree(s.arena));
   MI355_HIP(hipFree(s.exp_tbl));

@@ -1884,18 +1884,36 @@ extern "C" int mi355_customized_profile(mi355_plan const *plan, void const *cons
     return rc;
   }
   State &s = state();
-  for (int i = 0; i < warmup; i++) {
-    rc = launch(prog, fingerprint == 0);
-    if (rc != MI355_OK) {
-      return rc;
+  // The host enqueues faster than the device runs, and a queue several thousand launches deep
+  // runs each of them slower (4096 launches of a 3.8 us kernel in flight: 4.2 us each; the
+  // runtime's pool of argument blocks wraps and the queue drains while it does).  So the loop
+  // is paced: a marker after every batch, and the host waits for the batch before the one it
+  // has just enqueued, which leaves between one and two batches in flight and the device never
+  // idle.
+  constexpr int kPaceBatch = 1024;
+  long long enqueued = 0;
+  auto launch_paced = [&](int count) -> int {
+    for (int i = 0; i < count; i++) {
+      int const r = launch(prog, fingerprint == 0);
+      if (r != MI355_OK) {
+        return r;
+      }
+      if (++enqueued % kPaceBatch == 0) {
+        long long const batch = enqueued / kPaceBatch;
+        MI355_HIP(hipEventRecord(s.pace[tls_queue][batch & 1], s.stream()));
+        if (batch > 1) {
+          MI355_HIP(hipEventSynchronize(s.pace[tls_queue][(batch - 1) & 1]));
+        }
+      }
     }
+    return MI355_OK;
+  };
+  if ((rc = launch_paced(warmup)) != MI355_OK) {
+    return rc;
   }
   MI355_HIP(hipEventRecord(s.ev0[tls_queue], s.stream()));
-  for (int i = 0; i < iters; i++) {
-    rc = launch(prog, fingerprint == 0);
-    if (rc != MI355_OK) {
-      return rc;
-    }
+  if ((rc = launch_paced(iters)) != MI355_OK) {
+    return rc;
   }
   MI355_HIP(hipEventRecord(s.ev1[tls_queue], s.stream()));
   MI355_HIP(hipEventSynchronize(s.ev1[tls_queue]));

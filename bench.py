@@ -331,42 +331,51 @@ def fingerprint_throughput(G, cpu_baseline: bool, num_problems: int = 64, per_pr
             for gph in reversed(graphs):
                 gph.close()
             ref_g.close()
-    t_build = t_verify = 0.0
-    tot = {"kernel_ops": 0, "customized_ops": 0, "compares": 0, "fp_bytes": 0, "matmul_macs": 0,
-           "enqueue_seconds": 0.0, "wait_seconds": 0.0}
-    n = wrong = 0
-    fam = {}
-    pos = 0
-    while pos < len(order):
-        family = probs[order[pos]]["family"]
-        group = [probs[i] for i in order[pos:pos + in_flight] if probs[i]["family"] == family]
-        pos += len(group)
-        b0 = time.perf_counter()
-        built = []
-        for prob in group:
-            ref_g, _ = G.build_from_spec(prob["reference"])
-            built.append((ref_g, [G.build_from_spec(c["spec"])[0] for c in prob["candidates"]]))
-        b1 = time.perf_counter()
-        tickets = [G.verify_batch_begin(graphs, ref_g, prob["input_seed"])
-                   for prob, (ref_g, graphs) in zip(group, built)]
-        results = [G.verify_batch_end(t) for t in tickets]
-        b2 = time.perf_counter()
-        t_build += b1 - b0
-        t_verify += b2 - b1
-        f = fam.setdefault(family, [0, 0.0])
-        f[1] += b2 - b1
-        for prob, (verdicts, st) in zip(group, results):
-            f[0] += len(verdicts)
-            for k in tot:
-                tot[k] += st[k]
-            n += len(verdicts)
-            wrong += sum(v != c["expect_equal"] for v, c in zip(verdicts, prob["candidates"]))
-        for ref_g, graphs in reversed(built):
-            for gph in reversed(graphs):
-                gph.close()
-            ref_g.close()
+    def one_pass():
+        t_build = t_verify = 0.0
+        tot = {"kernel_ops": 0, "customized_ops": 0, "compares": 0, "fp_bytes": 0, "matmul_macs": 0,
+               "enqueue_seconds": 0.0, "wait_seconds": 0.0}
+        n = wrong = 0
+        fam = {}
+        pos = 0
+        while pos < len(order):
+            family = probs[order[pos]]["family"]
+            group = [probs[i] for i in order[pos:pos + in_flight] if probs[i]["family"] == family]
+            pos += len(group)
+            b0 = time.perf_counter()
+            built = []
+            for prob in group:
+                ref_g, _ = G.build_from_spec(prob["reference"])
+                built.append((ref_g, [G.build_from_spec(c["spec"])[0] for c in prob["candidates"]]))
+            b1 = time.perf_counter()
+            tickets = [G.verify_batch_begin(graphs, ref_g, prob["input_seed"])
+                       for prob, (ref_g, graphs) in zip(group, built)]
+            results = [G.verify_batch_end(t) for t in tickets]
+            b2 = time.perf_counter()
+            t_build += b1 - b0
+            t_verify += b2 - b1
+            f = fam.setdefault(family, [0, 0.0])
+            f[1] += b2 - b1
+            for prob, (verdicts, st) in zip(group, results):
+                f[0] += len(verdicts)
+                for k in tot:
+                    tot[k] += st[k]
+                n += len(verdicts)
+                wrong += sum(v != c["expect_equal"] for v, c in zip(verdicts, prob["candidates"]))
+            for ref_g, graphs in reversed(built):
+                for gph in reversed(graphs):
+                    gph.close()
+                ref_g.close()
+        return t_verify, t_build, tot, n, wrong, fam
+
+    # a pass is a few milliseconds of wall clock with host threads in it: three passes, the one
+    # with the median time is reported (all three rates are listed)
+    passes = sorted((one_pass() for _ in range(3)), key=lambda r: r[0])
+    t_verify, t_build, tot, n, wrong, fam = passes[1]
+    wrong = max(r[4] for r in passes)
     rec = {
         "candidates": n, "problems": len(probs), "candidates_per_s": round(n / t_verify, 1),
+        "candidates_per_s_of_each_pass": [round(r[3] / r[0], 1) for r in passes],
         "verify_s": round(t_verify, 4), "host_enqueue_s": round(tot["enqueue_seconds"], 4),
         "final_wait_s": round(tot["wait_seconds"], 4), "host_graph_build_s": round(t_build, 4),
         "kernel_ops": tot["kernel_ops"], "customized_ops": tot["customized_ops"],
