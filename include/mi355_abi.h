@@ -323,7 +323,10 @@ int mi355_plan_extents(mi355_plan const *plan, long long *in_elems, long long *o
 int mi355_customized_run(mi355_plan const *plan, void const *const *inputs,
                          void *const *outputs);
 /* KNCustomizedOp::profile, customized_kernel.cu:615-653: `warmup` untimed then
- * `iters` timed launches between two events on the backend stream; *ms = mean. */
+ * `iters` timed launches between two events on the backend stream; *ms = mean.
+ * The host never runs more than two batches of 1024 launches ahead of the device (a
+ * marker per batch, waited for one batch later): with several thousand launches queued
+ * every launch takes longer, so an unpaced loop would time the depth of its own queue. */
 int mi355_customized_profile(mi355_plan const *plan, void const *const *inputs,
                              void *const *outputs, int fingerprint, int warmup, int iters,
                              float *ms);
