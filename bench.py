@@ -104,6 +104,7 @@ def recorded_programs(G, N, abi, with_oracle: bool):
     rec = {
         "programs": len(ts), "min_us": round(ts[0], 2), "median_us": round(ts[len(ts) // 2], 2),
         "max_us": round(ts[-1], 2), "sum_us": round(sum(ts), 1), "customized_op_kernels": kernels,
+        "per_program_us": [round(t, 2) for t in totals],
         "timing": "per program: sum over operators of the mean time of 16 launches after one warm-up, events on the launching queue",
         "reference_published_us": {"min": 29.2, "max": 91.9, "hardware": "A100 (other hardware: context, not a baseline)"},
         "inputs": "fp16 N(0, 0.05), seeded",

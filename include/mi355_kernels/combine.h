@@ -37,7 +37,10 @@ __device__ __forceinline__ long long ctile_origin(CTile const &t) {
   return (long long)blockIdx.x * t.lin[0] + (long long)blockIdx.y * t.lin[1] + (long long)blockIdx.z * t.lin[2];
 }
 
-template <int VEC, int MODE>
+// BATCH: pieces a thread keeps in flight: 16 for a small fold (latency sets its time), 4 for a
+// large one (bandwidth does, and sixteen pieces a power of two apart in flight per thread halve
+// the rate).
+template <int VEC, int MODE, int BATCH>
 __global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const) {
   CombineParams const P = load_kernel_arguments<CombineParams, 0>();  // the whole block, one trip
   typedef _Float16 halfv __attribute__((ext_vector_type(VEC)));
@@ -50,9 +53,40 @@ __global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const)
     int const x = (e - r * xv) * VEC;
     _Float16 const *nr = n + (long long)r * P.n.d_cols + x;
     _Float16 const *dr = d + (long long)r * P.d.d_cols;
+    // Whole batches of pieces are loaded together and consumed in order afterwards: piece by
+    // piece (a load, its wait, an add) a fold of 16 denominators and 16 numerator pieces is 32
+    // trips to the L2 in a row, several microseconds for a kilobyte of data.  The first
+    // numerator batch is in flight while the denominators are added; what is left over after
+    // the whole batches is folded piece by piece.
+    halfv v[BATCH];
+    auto load_pieces = [&](int s0) {
+      _Float16 const *first = nr + s0 * P.step;
+#pragma unroll
+      for (int u = 0; u < BATCH; u++) {
+        v[u] = *reinterpret_cast<halfv const *>(first + u * P.step);
+      }
+    };
+    halfv lone = {};  // (a fold of fewer pieces than a batch: its first piece, loaded as early)
+    if (P.S >= BATCH) {
+      load_pieces(0);
+    } else if (P.S > 0) {
+      lone = *reinterpret_cast<halfv const *>(nr);
+    }
     float den = 0.0f;
-    for (int s = 0; s < P.SD; s++) {
-      den += static_cast<float>(dr[s]);
+    int sd = 0;
+    for (; sd + BATCH <= P.SD; sd += BATCH) {
+      _Float16 dv[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; u++) {
+        dv[u] = dr[sd + u];
+      }
+#pragma unroll
+      for (int u = 0; u < BATCH; u++) {
+        den += static_cast<float>(dv[u]);
+      }
+    }
+    for (; sd < P.SD; sd++) {
+      den += static_cast<float>(dr[sd]);
     }
     float const den16 = static_cast<float>(static_cast<_Float16>(den));
     float acc[VEC];
@@ -60,12 +94,10 @@ __global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const)
     for (int j = 0; j < VEC; j++) {
       acc[j] = 0.0f;
     }
-#pragma unroll 4
-    for (int s = 0; s < P.S; s++) {
-      halfv const v = *reinterpret_cast<halfv const *>(nr + s * P.step);
+    auto add_piece = [&](halfv const &piece) {
 #pragma unroll
       for (int j = 0; j < VEC; j++) {
-        float const t = static_cast<float>(v[j]);
+        float const t = static_cast<float>(piece[j]);
         if (MODE == SUM_THEN_DIV) {
           acc[j] += t;
         } else if (MODE == DIV_THEN_SUM) {
@@ -75,6 +107,20 @@ __global__ __launch_bounds__(256) void combine_fused_kernel(CombineParams const)
               static_cast<_Float16>(acc[j] + static_cast<float>(static_cast<_Float16>(t / den16))));
         }
       }
+    };
+    int sn = 0;
+    for (; sn + BATCH <= P.S; sn += BATCH) {
+      if (sn > 0) {
+        load_pieces(sn);
+      }
+#pragma unroll
+      for (int u = 0; u < BATCH; u++) {
+        add_piece(v[u]);
+      }
+    }
+#pragma unroll 4
+    for (; sn < P.S; sn++) {
+      add_piece(sn == 0 ? lone : *reinterpret_cast<halfv const *>(nr + sn * P.step));
     }
     halfv out;
 #pragma unroll

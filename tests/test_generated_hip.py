@@ -49,7 +49,7 @@ def test_fused_families_are_emitted_as_their_kernels(tmp_path):
     text = _emit(spec, tmp_path / "c3.hip")
     assert text.count("__global__") == 0
     assert "mi355::attn_stream_kernel<128, 64, 128, false, 4, 2, true, 1><<<dim3(32, 1, 16), 256, 65536, stream>>>(P);" in text
-    assert '#include "mi355_kernels/combine.h"' in text and "mi355::combine_fused_kernel<8, 0><<<dim3(32, 64, 1), 256, 0, stream>>>(P);" in text
+    assert '#include "mi355_kernels/combine.h"' in text and "mi355::combine_fused_kernel<8, 0, 4><<<dim3(32, 64, 1), 256, 0, stream>>>(P);" in text
     # C4: the range kernel and its fold share a workspace the program allocates once
     spec, _ = W.config4_lora()
     text = _emit(spec, tmp_path / "c4.hip")
