@@ -745,6 +745,12 @@ def main() -> int:
                 ms = ctypes.c_float()
                 rc = abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, 32, 128, ctypes.byref(ms))
                 assert rc == 0, N.last_error()
+                if ms.value < 0.02:
+                    # a short operator right behind a long one of another kind: 160 launches are
+                    # over before the clocks have settled (the fold of the long decode plan read
+                    # 6.3 us this way and 2.8 us over 512 launches), so it is timed again, longer
+                    rc = abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, 512, 1024, ctypes.byref(ms))
+                    assert rc == 0, N.last_error()
                 li = N.Mi355LaunchInfo()
                 abi.mi355_last_launch(ctypes.byref(li))
                 nbytes = 2 * (sum(vals2[a][b].num_elements for a, b in op["in"]) +
