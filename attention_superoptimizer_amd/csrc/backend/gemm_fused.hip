@@ -57,23 +57,39 @@ namespace {
 // (a column-major tensor -- DevOp::sub == 1 on its loader -- holds element (r, c) at
 // c * d_rows + r: a step along the rows is one element, a step along the columns d_rows, and
 // `d_cols` of the result is that leading dimension)
-GTile gtile(DevOp const &op, void const *ptr) {
+// The tile origin of a loader / saver as one stride per block coordinate and per iteration.
+// `fits` is cleared when an origin could leave 31 bits (the kernels multiply and add these
+// strides in 32 bits): `extents` = the grid and the for-loop range.
+GTile gtile(DevOp const &op, void const *ptr, int const (&extents)[4], bool &fits) {
   GTile t;
   t.ptr = ptr;
   bool const cm = op.kind == DOP_LOAD && op.sub == 1;
   long long const rstep = cm ? 1 : op.d_cols, cstep = cm ? op.d_rows : 1;
+  long long lin[4];
   for (int i = 0; i < 3; i++) {
-    t.lin[i] = op.g_bs[i] + op.row_bs[i] * rstep + op.col_bs[i] * cstep;
+    lin[i] = op.g_bs[i] + op.row_bs[i] * rstep + op.col_bs[i] * cstep;
   }
-  t.lin[3] = op.g_fs + op.row_fs * rstep + op.col_fs * cstep;
+  lin[3] = op.g_fs + op.row_fs * rstep + op.col_fs * cstep;
+  long long reach = 0;
+  for (int i = 0; i < 4; i++) {
+    long long const a = lin[i] < 0 ? -lin[i] : lin[i];
+    if (a >= (1LL << 31)) {
+      fits = false;
+    }
+    reach += a * (extents[i] > 0 ? extents[i] - 1 : 0);
+    t.lin[i] = (int)lin[i];
+  }
+  if (reach >= (1LL << 31)) {
+    fits = false;
+  }
   t.d_cols = cm ? op.d_rows : op.d_cols;
   return t;
 }
 
 // The parameter blocks as C++ source (for programs that Graph::generate_hip_program writes).
 std::string literal(GTile const &t) {
-  return emit_fmt("mi355::GTile{%s, {%lldLL, %lldLL, %lldLL, %lldLL}, %d}", emit_pointer(t.ptr).c_str(), t.lin[0],
-                  t.lin[1], t.lin[2], t.lin[3], t.d_cols);
+  return emit_fmt("mi355::GTile{%s, {%d, %d, %d, %d}, %d}", emit_pointer(t.ptr).c_str(), t.lin[0], t.lin[1],
+                  t.lin[2], t.lin[3], t.d_cols);
 }
 std::string literal(GemmParams const &A, char const *var) {
   std::string t = emit_fmt("    mi355::GemmParams %s{};\n", var);
@@ -384,15 +400,20 @@ int try_launch_gemm(DevProgram const &P) {
   }
   State &s = state();
   GemmParams A{};
-  auto in_tile = [&](int i) { return gtile(P.ops[i], P.in[P.ops[i].io]); };
+  int const extents[4] = {P.grid[0], P.grid[1], P.grid[2], P.forloop_range};
+  bool fits = true;
+  auto in_tile = [&](int i) { return gtile(P.ops[i], P.in[P.ops[i].io], extents, fits); };
   A.a0 = in_tile(G.a0);
   A.a1 = G.a1 >= 0 ? in_tile(G.a1) : A.a0;
   A.b0 = in_tile(G.b0);
   A.b1 = G.b1 >= 0 ? in_tile(G.b1) : A.b0;
   A.la = G.la >= 0 ? in_tile(G.la) : A.a0;
   A.lb = G.lb >= 0 ? in_tile(G.lb) : A.a0;
-  A.o0 = gtile(P.ops[G.o0], P.out[P.ops[G.o0].io]);
-  A.o1 = G.o1 >= 0 ? gtile(P.ops[G.o1], P.out[P.ops[G.o1].io]) : A.o0;
+  A.o0 = gtile(P.ops[G.o0], P.out[P.ops[G.o0].io], extents, fits);
+  A.o1 = G.o1 >= 0 ? gtile(P.ops[G.o1], P.out[P.ops[G.o1].io], extents, fits) : A.o0;
+  if (!fits) {
+    return 0;  // a tensor of more than 2^31 elements: the generic interpreter takes the plan
+  }
   A.M = G.M;
   A.KT = G.KT;
   A.forloop_range = P.forloop_range;

@@ -27,8 +27,11 @@ enum { PRO_NONE = 0, PRO_EXP = 1, PRO_SILU = 2, PRO_SILU_MUL = 3 };
 // strides into one stride per coordinate (a few scalar multiplies per tile address).
 struct GTile {
   void const *ptr;
-  long long lin[4];  // elements per step of bx, by, bz and of the iteration
-  int d_cols;        // row stride of the tensor
+  int lin[4];  // elements per step of bx, by, bz and of the iteration (the host takes a plan on
+               // these kernels only when every tile origin fits 31 bits: the parameter block
+               // of the one-launch kernel then fits the scalar registers, and a tile address is
+               // four 32-bit multiplies)
+  int d_cols;  // row stride of the tensor
 };
 
 struct GemmParams {
@@ -43,7 +46,7 @@ struct GemmParams {
 };
 
 __device__ __forceinline__ long long gtile_offset(GTile const &t, int bx, int by, int bz, int it) {
-  return bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3];
+  return (long long)(bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3]);
 }
 
 // 16-byte chunk `chunk` of row `row` in a swizzled LDS tile with LD halfs per row.
