@@ -93,6 +93,23 @@ __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int 
   return bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3];
 }
 
+// x[l] + x[l ^ 16] + x[l ^ 32] + x[l ^ 48] in every lane l: the sum over the four groups of 16
+// lanes, in the order ((l, l ^ 16), (l ^ 32, l ^ 48)) that two shuffles would add them in.  The
+// two lane-swap instructions of this part exchange rows of 16 lanes and halves of the
+// wavefront between two registers in a few cycles; a shuffle is a trip through the LDS
+// crossbar, and two of them in a row sit in the middle of the softmax's dependent chain.
+// (Inline assembly: the compiler's own builtin for these instructions returns the first result
+// twice here.  The wait states cover a vector write to either register just before.)
+__device__ __forceinline__ float sum_lane_groups(float x) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  float const pair = a + b;
+  a = pair;
+  b = pair;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+
 // Element offset of 16-byte chunk `chunk` of row `row` in a swizzled LDS tile whose
 // rows hold LD halfs (LD a multiple of 64).
 __device__ __forceinline__ int swz_chunk(int row, int chunk, int LD) {
@@ -372,8 +389,7 @@ __global__ __launch_bounds__(64 * RG * IP) void attn_fused_kernel(AttnParams con
             pk[j / 2][2 * (j & 1) + h] = __builtin_bit_cast(uint32_t, e2);
           }
         }
-        rs += __shfl_xor(rs, 16, 64);
-        rs += __shfl_xor(rs, 32, 64);
+        rs = sum_lane_groups(rs);
         r16 = static_cast<_Float16>(rs);  // row-sum tile (fp16)
         if (HAS_DIV) {
           // one reciprocal per row, then multiplies: within an fp32 ulp of the division
@@ -725,8 +741,7 @@ __global__ __launch_bounds__(64 * RG, 2) void attn_stream_kernel(AttnParams cons
     }
 #pragma unroll
     for (int rp = 0; rp < RPW; rp++) {
-      rs[rp] += __shfl_xor(rs[rp], 16, 64);
-      rs[rp] += __shfl_xor(rs[rp], 32, 64);
+      rs[rp] = sum_lane_groups(rs[rp]);
       _Float16 const r16 = static_cast<_Float16>(rs[rp]);
       float const inv = __builtin_amdgcn_rcpf(static_cast<float>(r16));
 #pragma unroll
@@ -1325,8 +1340,7 @@ __global__ __launch_bounds__(64 * IP) void attn_direct_kernel(AttnParams const) 
         return rs;
       };
       auto across = [&](float rs) {
-        rs += __shfl_xor(rs, 16, 64);
-        rs += __shfl_xor(rs, 32, 64);
+        rs = sum_lane_groups(rs);
         return rs;
       };
       auto normalise = [&](int rp, int w0, int nw, _Float16 r16) {
