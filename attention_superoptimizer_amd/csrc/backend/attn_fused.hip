@@ -54,23 +54,38 @@ namespace {
 // (a column-major tensor -- DevOp::sub == 1 on its loader -- holds element (r, c) at
 // c * d_rows + r: a step along the rows is one element, a step along the columns d_rows, and
 // `d_cols` of the result is that leading dimension)
-TileAddr tile_addr(DevOp const &op, void const *ptr) {
+// `fits` is cleared when a tile origin could leave 31 bits (the kernels multiply and add the
+// strides in 32 bits); `extents` = the plan's grid and its for-loop range.
+TileAddr tile_addr(DevOp const &op, void const *ptr, int const (&extents)[4], bool &fits) {
   TileAddr t;
   t.ptr = ptr;
   bool const cm = op.kind == DOP_LOAD && op.sub == 1;
   long long const rstep = cm ? 1 : op.d_cols, cstep = cm ? op.d_rows : 1;
+  long long lin[4];
   for (int i = 0; i < 3; i++) {
-    t.lin[i] = op.g_bs[i] + op.row_bs[i] * rstep + op.col_bs[i] * cstep;
+    lin[i] = op.g_bs[i] + op.row_bs[i] * rstep + op.col_bs[i] * cstep;
   }
-  t.lin[3] = op.g_fs + op.row_fs * rstep + op.col_fs * cstep;
+  lin[3] = op.g_fs + op.row_fs * rstep + op.col_fs * cstep;
+  long long reach = 0;
+  for (int i = 0; i < 4; i++) {
+    long long const a = lin[i] < 0 ? -lin[i] : lin[i];
+    if (a >= (1LL << 31)) {
+      fits = false;
+    }
+    reach += a * (extents[i] > 0 ? extents[i] - 1 : 0);
+    t.lin[i] = (int)lin[i];
+  }
+  if (reach >= (1LL << 31)) {
+    fits = false;
+  }
   t.d_cols = cm ? op.d_rows : op.d_cols;
   return t;
 }
 
 // The parameter block as C++ source (for programs that Graph::generate_hip_program writes).
 std::string literal(TileAddr const &t) {
-  return emit_fmt("mi355::TileAddr{%s, {%lldLL, %lldLL, %lldLL, %lldLL}, %d}", emit_pointer(t.ptr).c_str(), t.lin[0],
-                  t.lin[1], t.lin[2], t.lin[3], t.d_cols);
+  return emit_fmt("mi355::TileAddr{%s, {%d, %d, %d, %d}, %d}", emit_pointer(t.ptr).c_str(), t.lin[0], t.lin[1],
+                  t.lin[2], t.lin[3], t.d_cols);
 }
 std::string literal(AttnParams const &A) {
   std::string t = "    mi355::AttnParams P{};\n";
@@ -646,11 +661,16 @@ int try_launch_attention(DevProgram const &P0) {
   AttnParams A;
   A.r_copies = r_copies;
   A.r_copy_stride = r_copy_stride;
-  A.q = tile_addr(P.ops[M.q], P.in[P.ops[M.q].io]);
-  A.k = tile_addr(P.ops[M.k], P.in[P.ops[M.k].io]);
-  A.v = tile_addr(P.ops[M.v], P.in[P.ops[M.v].io]);
-  A.o = tile_addr(P.ops[M.out_o], P.out[P.ops[M.out_o].io]);
-  A.r = M.out_r >= 0 ? tile_addr(P.ops[M.out_r], P.out[P.ops[M.out_r].io]) : A.o;
+  int const extents[4] = {P.grid[0], P.grid[1], P.grid[2], P.forloop_range};
+  bool fits = true;
+  A.q = tile_addr(P.ops[M.q], P.in[P.ops[M.q].io], extents, fits);
+  A.k = tile_addr(P.ops[M.k], P.in[P.ops[M.k].io], extents, fits);
+  A.v = tile_addr(P.ops[M.v], P.in[P.ops[M.v].io], extents, fits);
+  A.o = tile_addr(P.ops[M.out_o], P.out[P.ops[M.out_o].io], extents, fits);
+  A.r = M.out_r >= 0 ? tile_addr(P.ops[M.out_r], P.out[P.ops[M.out_r].io], extents, fits) : A.o;
+  if (!fits) {
+    return 0;  // a tensor of more than 2^31 elements: the generic interpreter takes the plan
+  }
   A.forloop_range = P.forloop_range;
   A.rows = M.m < 16 ? M.m : 16;
   A.trace = nullptr;

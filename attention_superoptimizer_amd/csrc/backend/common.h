@@ -116,6 +116,8 @@ bool mfma_matmul_pays(int batch, int m, int n, int k);
 int launch_mfma_matmul(uint16_t const *A, uint16_t const *B, uint16_t *C, int batch, int m, int n,
                        int k);
 int sync_all_queues();
+// Drops what mi355_customized_profile keeps of its last call per queue (tb_interp.hip).
+void drop_profile_replays();
 // The vendor library's GEMM on the calling thread's queue (vendor_gemm.cc): row-major C =
 // A . B for `batch` matrices, each operand in either storage order; MI355_ERR_UNSUPPORTED
 // when the library cannot be loaded.  vendor_gemm_release drops its per-queue handles.

@@ -164,6 +164,7 @@ extern "C" int mi355_shutdown(void) {
     return rc;
   }
   vendor_gemm_release();  // its handles are bound to the queues destroyed below
+  drop_profile_replays();
   for (int q = 0; q < MI355_NUM_QUEUES; q++) {
     MI355_HIP(hipEventDestroy(s.ev0[q]));
     MI355_HIP(hipEventDestroy(s.ev1[q]));
@@ -255,6 +256,7 @@ extern "C" int mi355_mark_wait_host(int mark) {
 }
 
 extern "C" int mi355_set_option(int option, int value) {
+  drop_profile_replays();
   if (option == MI355_OPT_FORCE_INTERPRETER) {
     state().force_interpreter = value;
     return MI355_OK;

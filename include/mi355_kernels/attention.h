@@ -65,8 +65,10 @@ __device__ __forceinline__ half4 lds_read_tr16(_Float16 const *p) {
 // instead of three sums of products; they sit on the path to the first load).
 struct TileAddr {
   void const *ptr;
-  long long lin[4];  // elements per step of bx, by, bz and of the iteration
-  int d_cols;        // row stride of the tensor
+  int lin[4];  // elements per step of bx, by, bz and of the iteration (the host takes a plan on
+               // these kernels only when every tile origin fits 31 bits: a tile address is then
+               // four 32-bit multiplies, and the parameter block 240 bytes of scalar registers)
+  int d_cols;  // row stride of the tensor
 };
 
 struct AttnParams {
@@ -90,7 +92,7 @@ struct AttnParams {
 
 __device__ __forceinline__ long long tile_offset(TileAddr const &t, int bx, int by, int bz,
                                                  int it) {
-  return bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3];
+  return (long long)(bx * t.lin[0] + by * t.lin[1] + bz * t.lin[2] + it * t.lin[3]);
 }
 
 // x[l] + x[l ^ 16] + x[l ^ 32] + x[l ^ 48] in every lane l: the sum over the four groups of 16

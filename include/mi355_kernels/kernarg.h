@@ -83,15 +83,18 @@ __device__ __forceinline__ void fetch_kernel_arguments_large() {
 // The whole argument block of a kernel whose only parameter is one T, read into scalar
 // registers by loads issued together: the kernel then makes one trip for its arguments instead
 // of one per place where the compiler first needs a field.  For blocks of 320 bytes (five
-// loads of 64) and of 152 (64, 64, 16, 8); a larger block does not fit the scalar registers
+// loads of 64), of 240 (64, 64, 64, 32, 16) and of 152 (64, 64, 16, 8); a larger block does not
+// fit the scalar registers
 // beside the kernel's own values and takes fetch_kernel_arguments.  The block counts behind
 // the arguments are touched as above.
 typedef uint32_t kernarg_words16 __attribute__((ext_vector_type(16)));
+typedef uint32_t kernarg_words8 __attribute__((ext_vector_type(8)));
 typedef uint32_t kernarg_words4 __attribute__((ext_vector_type(4)));
 typedef uint32_t kernarg_words2 __attribute__((ext_vector_type(2)));
 template <typename T, int HIDDEN_WORDS>
 __device__ __forceinline__ T load_kernel_arguments() {
-  static_assert((sizeof(T) == 320 || sizeof(T) == 152) && alignof(T) <= 8, "a block size this was written for");
+  static_assert((sizeof(T) == 320 || sizeof(T) == 240 || sizeof(T) == 152) && alignof(T) <= 8,
+                "a block size this was written for");
   auto const *block = __builtin_amdgcn_kernarg_segment_ptr();
   constexpr int last = kernarg_last_word<(int)sizeof(T), HIDDEN_WORDS>();
   uint32_t unused;
@@ -112,6 +115,25 @@ __device__ __forceinline__ T load_kernel_arguments() {
         : "s"(block), "i"(last)
         : "memory");
     static_assert(sizeof(regs) == sizeof(T), "no padding");
+    __builtin_memcpy(&t, &regs, sizeof(T));
+  } else if constexpr (sizeof(T) == 240) {
+    struct {
+      kernarg_words16 w[3];
+      kernarg_words8 x;
+      kernarg_words4 y;
+    } regs;
+    asm volatile(
+        "s_load_dwordx16 %0, %6, 0x0\n\t"
+        "s_load_dwordx16 %1, %6, 0x40\n\t"
+        "s_load_dwordx16 %2, %6, 0x80\n\t"
+        "s_load_dwordx8 %3, %6, 0xc0\n\t"
+        "s_load_dwordx4 %4, %6, 0xe0\n\t"
+        "s_load_dword %5, %6, %7\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&s"(regs.w[0]), "=&s"(regs.w[1]), "=&s"(regs.w[2]), "=&s"(regs.x), "=&s"(regs.y), "=&s"(unused)
+        : "s"(block), "i"(last)
+        : "memory");
+    static_assert(sizeof(regs) >= sizeof(T), "registers for the whole block");
     __builtin_memcpy(&t, &regs, sizeof(T));
   } else {
     struct {

@@ -40,8 +40,8 @@ def test_fused_families_are_emitted_as_their_kernels(tmp_path):
     assert ("mi355::attn_direct_kernel<64, 64, 64, true, 4, 2, 1, 1, 1, 1, false, true>"
             "<<<dim3(16, 16, 1), 256, 81920, stream>>>(P);") in text
     # K [2, 64, 4096] and V [2, 4096, 64] are column-major: leading dimensions 64 and 4096
-    assert "P.k = mi355::TileAddr{in[1], {262144LL, 16384LL, 0LL, 4096LL}, 64};" in text
-    assert "P.v = mi355::TileAddr{in[2], {262144LL, 256LL, 0LL, 64LL}, 4096};" in text
+    assert "P.k = mi355::TileAddr{in[1], {262144, 16384, 0, 4096}, 64};" in text
+    assert "P.v = mi355::TileAddr{in[2], {262144, 256, 0, 64}, 4096};" in text
     assert "hipFuncAttributeMaxDynamicSharedMemorySize, 81920" in text
     assert "void const *in[] = {dtensors[0], dtensors[1], dtensors[2]};" in text
     # C3: throughput attention kernel, then the fold-and-divide kernel

@@ -431,6 +431,49 @@ def test_streaming_kernels_are_deterministic(rt, abi):
             assert abi.mi355_set_option(7, 0) == 0
 
 
+def test_profile_loops_leave_the_results_of_a_plain_run(rt, abi):
+    """mi355_customized_profile captures what one call launches and repeats it (kernel by
+    kernel; for 512 launches and more as chains of 256 kernel nodes, one graph launch each).
+    Whatever the loop's length, the outputs afterwards are the bits a plain run leaves --
+    checked twice per plan, with plain runs and cleared outputs between the loops, on a
+    one-kernel plan, a two-kernel plan (range kernel + fold) and the generic interpreter."""
+    import ctypes
+    from attention_superoptimizer_amd import workloads as W
+    cases = [("C2, direct-staging attention", W.config2_gqa_decode()[0], 3, 0, 0),
+             ("LoRA, range kernel and its fold", W.config4_lora(m=16, d=1024, r=16, grid=16, F=4)[0], 4, 1, 0),
+             ("C1 on the interpreter", W.config1_fused_matmul()[0], 2, 0, 1)]
+    for what, spec, op, gemm_mode, interpreter in cases:
+        assert abi.mi355_set_option(7, gemm_mode) == 0
+        assert abi.mi355_set_option(1, interpreter) == 0
+        g, vals = rt.build_from_spec(spec)
+        try:
+            for i, o in enumerate(spec):
+                if o["op"] == "input":
+                    vals[i][0].write_data(normal_f16(o["dims"], 0.05, 900 + i))
+            g.execute(op)
+            plain = [t.read_data().view(np.uint16).copy() for t in vals[op]]
+            pl = g.lowered(op, fingerprint=False)
+            i_p = (ctypes.c_void_p * 4)(*[vals[a][b].device_ptr(False) for a, b in spec[op]["in"]])
+            o_p = (ctypes.c_void_p * 4)(*[t.device_ptr(False) for t in vals[op]])
+            ms = ctypes.c_float()
+            for warmup, iters in ((0, 3), (256, 1024), (5, 700), (0, 512)):
+                for t in vals[op]:
+                    t.write_data(np.full(t.dims, np.nan, np.float16))
+                assert abi.mi355_customized_profile(ctypes.byref(pl), i_p, o_p, 0, warmup, iters,
+                                                    ctypes.byref(ms)) == 0
+                assert ms.value > 0
+                for a, t in zip(plain, vals[op]):
+                    b = t.read_data().view(np.uint16)
+                    assert np.array_equal(a, b), f"{what}: after {warmup} + {iters} launches {int((a != b).sum())} elements differ"
+                g.execute(op)  # plain work between the loops
+                for a, t in zip(plain, vals[op]):
+                    assert np.array_equal(a, t.read_data().view(np.uint16)), what
+        finally:
+            g.close()
+            assert abi.mi355_set_option(7, 0) == 0
+            assert abi.mi355_set_option(1, 0) == 0
+
+
 def test_attention_throughput_variant(rt, abi):
     """the pipelined 32-rows-per-wavefront variant, forced on small problems: both forms,
     both head sizes"""
