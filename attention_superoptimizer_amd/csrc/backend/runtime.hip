@@ -343,18 +343,44 @@ extern "C" int mi355_launch_floor(int iters, float *us) {
     return fail(MI355_ERR_INVALID, "bad arguments");
   }
   State &s = state();
-  for (int i = 0; i < 64; i++) {
+  // The same way mi355_customized_profile repeats a call: chains of 256 kernel nodes, one graph
+  // launch each, so that the figure is the device's launch-to-launch time and not the host's
+  // time per launch call.
+  constexpr int kChain = 256;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  MI355_HIP(hipStreamBeginCapture(s.stream(), hipStreamCaptureModeThreadLocal));
+  for (int i = 0; i < kChain; i++) {
     empty_kernel<<<1, 64, 0, s.stream()>>>();
   }
-  MI355_HIP(hipEventRecord(s.ev0[tls_queue], s.stream()));
-  for (int i = 0; i < iters; i++) {
-    empty_kernel<<<1, 64, 0, s.stream()>>>();
+  MI355_HIP(hipStreamEndCapture(s.stream(), &graph));
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (e == hipSuccess) {
+    e = hipGraphLaunch(exec, s.stream());  // warm-up
   }
-  MI355_HIP(hipEventRecord(s.ev1[tls_queue], s.stream()));
-  MI355_HIP(hipEventSynchronize(s.ev1[tls_queue]));
+  int const chains = (iters + kChain - 1) / kChain;
+  if (e == hipSuccess) {
+    e = hipEventRecord(s.ev0[tls_queue], s.stream());
+  }
+  for (int i = 0; i < chains && e == hipSuccess; i++) {
+    e = hipGraphLaunch(exec, s.stream());
+  }
+  if (e == hipSuccess) {
+    e = hipEventRecord(s.ev1[tls_queue], s.stream());
+  }
+  if (e == hipSuccess) {
+    e = hipEventSynchronize(s.ev1[tls_queue]);
+  }
   float ms = 0.0f;
-  MI355_HIP(hipEventElapsedTime(&ms, s.ev0[tls_queue], s.ev1[tls_queue]));
-  *us = ms * 1000.0f / iters;
+  if (e == hipSuccess) {
+    e = hipEventElapsedTime(&ms, s.ev0[tls_queue], s.ev1[tls_queue]);
+  }
+  if (exec != nullptr) {
+    (void)hipGraphExecDestroy(exec);
+  }
+  (void)hipGraphDestroy(graph);
+  MI355_HIP(e);
+  *us = ms * 1000.0f / ((float)chains * kChain);
   return MI355_OK;
 }
 

@@ -155,8 +155,10 @@ int mi355_is_initialised(void);
 char const *mi355_last_error(void);
 int mi355_get_device_info(mi355_device_info *info);
 int mi355_set_option(int option, int value);
-/* Mean microseconds per launch of an empty kernel, `iters` launches back to back on
- * the backend stream: the floor under any per-launch figure (blocking). */
+/* Mean microseconds per launch of an empty kernel, `iters` launches (rounded up to whole
+ * chains of 256 kernel nodes, one graph launch each, as mi355_customized_profile repeats a
+ * call) back to back on the backend stream: the floor under any per-launch figure
+ * (blocking). */
 int mi355_launch_floor(int iters, float *us);
 /* Device addresses of the three uint16 tables (113, 227, 113 entries), in the
  * reference's layout: exp[i] = 3^i mod 227; div_p[i], div_q[i] = inverse of i
