@@ -1930,8 +1930,8 @@ struct LaunchReplay {
   }
 };
 
-// MI355_OK with R.kernels filled, MI355_OK with R.kernels empty when the call cannot be replayed
-// (it enqueues something other than kernels, or capture is refused), or launch()'s error.
+// R.kernels filled, or left empty when the call cannot be replayed (it enqueues something other
+// than kernels, fails under capture, or capture is refused).
 int capture_launches(DevProgram const &prog, bool fp16, LaunchReplay &R) {
   hipStream_t const q = state().stream();
   if (hipStreamBeginCapture(q, hipStreamCaptureModeThreadLocal) != hipSuccess) {
@@ -1942,10 +1942,9 @@ int capture_launches(DevProgram const &prog, bool fp16, LaunchReplay &R) {
   hipGraph_t g = nullptr;
   hipError_t const ended = hipStreamEndCapture(q, &g);  // (always: the queue must leave capture)
   R.graph = g;
-  if (rc != MI355_OK) {
-    return rc;
-  }
-  if (ended != hipSuccess || g == nullptr) {
+  if (rc != MI355_OK || ended != hipSuccess || g == nullptr) {
+    // (a call that fails under capture, e.g. because it waits for something, is made again
+    // outside it by the caller's loop, which then reports what it returns)
     (void)hipGetLastError();
     return MI355_OK;
   }
