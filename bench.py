@@ -693,7 +693,9 @@ def main() -> int:
                         "declare them), grid (2,16,1), forloop 4, matmul-exp-reduce-div-matmul, "
                         "out [2,256,1024]",
             "launches_per_step": per_step,
-            "value_is": "host wall clock per launch over steps x launches_per_step back-to-back launches",
+            "value_is": "host wall clock per launch over steps x launches_per_step back-to-back launches "
+                        "(the kernel launches of one call, captured once and enqueued as chains of 256 "
+                        "kernel nodes, each launch behind the one before)",
             "device": info.name.decode(), "arch": info.arch.decode(),
             "compute_units": info.compute_units,
             # the device's reported maximum engine clock, not the clock sustained under load
