@@ -2000,18 +2000,18 @@ int capture_launches(DevProgram const &prog, bool fp16, LaunchReplay &R) {
 // chain once, outside its timed call.
 struct KeptReplay {
   bool fp16 = false;
+  unsigned generation = 0;
   DevProgram prog;
   std::unique_ptr<LaunchReplay> replay;
 };
 KeptReplay g_kept[MI355_NUM_QUEUES];
+// what is kept from before the last drop is not used again (a queue's slot is touched only by
+// the host thread that drives the queue, so a drop from another thread just moves this on)
+std::atomic<unsigned> g_kept_generation{1};
 }  // namespace
 
 // (options change which kernels a plan runs on: what was captured under the old ones is dropped)
-void drop_profile_replays() {
-  for (KeptReplay &k : g_kept) {
-    k.replay.reset();
-  }
-}
+void drop_profile_replays() { g_kept_generation.fetch_add(1, std::memory_order_relaxed); }
 }  // namespace mi355
 
 extern "C" int mi355_customized_profile(mi355_plan const *plan, void const *const *inputs,
@@ -2038,8 +2038,11 @@ extern "C" int mi355_customized_profile(mi355_plan const *plan, void const *cons
   long long enqueued = 0;
   KeptReplay &kept = g_kept[tls_queue];
   static_assert(std::is_trivially_copyable<DevProgram>::value, "compared and kept as bytes");
-  if (kept.replay == nullptr || kept.fp16 != (fingerprint == 0) || std::memcmp(&kept.prog, &prog, sizeof(prog)) != 0) {
+  unsigned const generation = g_kept_generation.load(std::memory_order_relaxed);
+  if (kept.replay == nullptr || kept.generation != generation || kept.fp16 != (fingerprint == 0) ||
+      std::memcmp(&kept.prog, &prog, sizeof(prog)) != 0) {
     kept.replay.reset(new LaunchReplay);
+    kept.generation = generation;
     std::memcpy(&kept.prog, &prog, sizeof(prog));
     kept.fp16 = fingerprint == 0;
     if ((rc = capture_launches(prog, fingerprint == 0, *kept.replay)) != MI355_OK) {
